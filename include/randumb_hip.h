@@ -1,0 +1,162 @@
+/*
+ * randumb_hip.h - C ABI of librandumb_hip.so, the gfx950 (MI355X) implementation of RANDUMB's
+ * pseudorandom-matrix hot path.
+ *
+ * A pseudorandom tensor is  W = Noise(seed) . coef : the noise is Squirrel5 integer-hash noise in
+ * [-1, 1] addressed by (seed, index) and is never stored; only coef is trainable.
+ *
+ * Conventions shared by every entry point
+ *   - all pointers are DEVICE pointers on the current HIP device unless stated otherwise;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); work is enqueued, not awaited;
+ *   - nothing is allocated or freed inside the library; outputs and workspaces belong to the caller;
+ *   - return value: 0 = ok, < 0 = argument error (RDB_E_*), > 0 = a hipError_t from a launch;
+ *     rdb_last_error_string() describes the last non-zero return on the calling thread;
+ *   - dtype codes: RDB_F32 = 0, RDB_BF16 = 1 (rdb_dtype);
+ *   - seeds are uint32 (the reference is exercised with 0 <= seed < 2^31);
+ *   - "vector-coef" = the reference form, one coef vector c[k] for the whole tensor:
+ *         W_flat[a] = sum_m noise(PRIME*a + m) * c[m],  a = storage offset of the element;
+ *     "matrix-coef" = the row-batched form, coef C[rows x k] over a contiguous (rows, row_len) tensor:
+ *         W[o, i] = sum_m noise(PRIME*i + m) * C[o, m]
+ *     (row o alone is a vector-coef tensor of shape (row_len,) with coef C[o, :]).
+ *
+ * Reference citations are to Clyde013/randumb, paths relative to its checkout:
+ *   R.py  = src/rten_cpp/RandumbTensor.py      R.cu = src/rten_cpp/csrc/cuda/rten.cu
+ *   R.cpp = src/rten_cpp/csrc/rten.cpp
+ */
+#ifndef RANDUMB_HIP_H
+#define RANDUMB_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { RDB_F32 = 0, RDB_BF16 = 1 } rdb_dtype;
+
+enum {
+    RDB_OK = 0,
+    RDB_E_NULL = -1,        /* a required pointer is NULL */
+    RDB_E_SHAPE = -2,       /* a size is negative, zero where it must not be, or too large */
+    RDB_E_DTYPE = -3,       /* unknown or unsupported dtype code / combination */
+    RDB_E_ALIGN = -4,       /* pointer or leading dimension not aligned as required */
+    RDB_E_UNSUPPORTED = -5, /* valid request this build has no kernel for */
+    RDB_E_WORKSPACE = -6    /* workspace missing or too small */
+};
+
+/* Library identification; bumps when an entry point changes meaning. */
+int rdb_abi_version(void);
+
+/* Text for the last non-zero return code on this thread (never NULL). */
+const char *rdb_last_error_string(void);
+
+/* ------------------------------------------------------------------------------------------ noise probes
+ * Replace: squirrel5_generate_2d / squirrel5_kernel_2d (R.py:78-105), rten_cpp::sq5_gen_2d (R.cpp:37,
+ * R.cu:50-71; its store index bug for non-square shapes is not reproduced).
+ * out is fp32 [N x M] row-major, out[n*M + m] = noise(PRIME*n + m, seed). */
+int rdb_sq5_fill_2d(float *out, int64_t N, int64_t M, uint32_t seed, void *stream);
+
+/* Replace: squirrel5_generate_1d / squirrel5_kernel_1d (R.py:108-126).  out[n] = noise(n, seed). */
+int rdb_sq5_fill_1d(float *out, int64_t N, uint32_t seed, void *stream);
+
+/* ------------------------------------------------------------------------------------------ materialise
+ * Replaces: op rten::materialize_fwd + materialize_fwd_kernel (R.py:235-290, 371-381) and
+ * rten_cpp::materialize_fwd (R.cpp:38, R.cu:74-152).
+ * Writes the (P, Q) view with element strides (sP, sQ) of the pseudorandom tensor, contiguous fp32:
+ *     out[p*Q + q] = W_flat[a],  a = q*sQ + p*sP                                   (R.py:264)
+ * coef_rows == 0: vector-coef, coef is [k].  coef_rows > 0: matrix-coef, coef is [coef_rows x k]
+ * contiguous and `a` addresses a contiguous (coef_rows, row_len) tensor.
+ * scale_bias: NULL, or a device pointer to ONE value of dtype coef_dtype; adds
+ *     scale_bias[0] * noise(a, seed)  (the fused random bias, R.py:286-289).
+ * A 1-D tensor of Q elements is passed as P = 1, sP = 0 (R.py:375-377). */
+int rdb_materialize_fwd(float *out, const void *coef, int coef_dtype, int64_t coef_rows, int64_t k,
+                        int64_t row_len, int64_t P, int64_t Q, int64_t sP, int64_t sQ, uint32_t seed,
+                        const void *scale_bias, void *stream);
+
+/* Replaces: op rten::materialize_bwd + materialize_bwd_kernel (R.py:304-359, 383-390).
+ * dW is a contiguous tensor of Nw elements (dtype dw_dtype).  dcoef is fp32 and is OVERWRITTEN:
+ *   vector-coef (coef_rows == 0): dcoef[m] = sum_a noise(PRIME*a + m) * dW[a],              dcoef is [k]
+ *   matrix-coef: Nw = coef_rows*row_len, dcoef[o*k+m] = sum_i noise(PRIME*i + m) * dW[o*row_len+i].
+ * The reduction is a fixed tree (no atomics): results are bitwise reproducible run to run.
+ * workspace: device scratch of at least rdb_materialize_bwd_workspace_bytes(...) bytes (may be NULL
+ * when that returns 0). */
+int rdb_materialize_bwd(float *dcoef, const void *dW, int dw_dtype, int64_t coef_rows, int64_t k,
+                        int64_t row_len, int64_t Nw, uint32_t seed, void *workspace,
+                        int64_t workspace_bytes, void *stream);
+int64_t rdb_materialize_bwd_workspace_bytes(int64_t coef_rows, int64_t k, int64_t row_len, int64_t Nw);
+
+/* Replaces: op rten::scale_bias_bwd + scale_bias_bwd_kernel (R.py:399-420).
+ * ds[0] = sum_a dW[a] * noise(a, seed) over the contiguous dW; fp32, overwritten, deterministic.
+ * workspace: at least rdb_scale_bias_bwd_workspace_bytes(Nw) bytes. */
+int rdb_scale_bias_bwd(float *ds, const void *dW, int dw_dtype, int64_t Nw, uint32_t seed,
+                       void *workspace, int64_t workspace_bytes, void *stream);
+int64_t rdb_scale_bias_bwd_workspace_bytes(int64_t Nw);
+
+/* ------------------------------------------------------------------------------------------ embedding
+ * Replaces: op rten::embed_fwd + embed_fwd_kernel (R.py:998-1057, 1121-1126).
+ * out[j*rowsize + r] = sum_m noise(PRIME*(idx[j]*rowsize + r) + m) * coef[m];  out fp32 [n_idx x rowsize],
+ * idx int64 [n_idx], coef vector-coef [k]. */
+int rdb_embed_fwd(float *out, const int64_t *idx, int64_t n_idx, const void *coef, int coef_dtype,
+                  int64_t k, int64_t rowsize, uint32_t seed, void *stream);
+
+/* Replaces: op rten::embed_bwd + embed_bwd_kernel (R.py:1059-1108, 1128-1134).
+ * dcoef[m] = sum_{j,r} noise(PRIME*(idx[j]*rowsize + r) + m) * dout[j*rowsize + r]; fp32 [k], overwritten,
+ * deterministic.  workspace: at least rdb_embed_bwd_workspace_bytes(n_idx, rowsize, k) bytes. */
+int rdb_embed_bwd(float *dcoef, const int64_t *idx, int64_t n_idx, const void *dout, int dout_dtype,
+                  int64_t k, int64_t rowsize, uint32_t seed, void *workspace, int64_t workspace_bytes,
+                  void *stream);
+int64_t rdb_embed_bwd_workspace_bytes(int64_t n_idx, int64_t rowsize, int64_t k);
+
+/* ------------------------------------------------------------------------------------------ fused linear
+ * The pseudorandom weight W is (out_f, in_f); element (o, i) has storage offset a = o*sO + i*sI
+ * (F.linear's weight: sO = in_f, sI = 1; `mat1 @ tensor` with a contiguous (P, Q) tensor: out_f = Q,
+ * in_f = P, sO = 1, sI = Q).  W is regenerated tile by tile on chip and never written to memory.
+ * coef_rows == 0: vector-coef, coef [k];  coef_rows == out_f: matrix-coef, coef [out_f x k] (requires
+ * sO = in_f, sI = 1; the noise row is i).
+ * scale_bias: NULL or one device value of coef_dtype: W += scale_bias[0]*noise(a).
+ * act_dtype is the dtype of x / y / dy / dx: RDB_BF16 computes with bf16 MFMA and fp32 accumulation
+ * (W rounded to bf16 once, after its fp32 accumulation, as materialize().to(dtype) does, R.py:892);
+ * RDB_F32 computes with fp32 MFMA.  Leading dimensions are in elements.
+ */
+typedef struct rdb_linear_desc {
+    int64_t tokens;     /* rows of x / y / dy / dx */
+    int64_t in_f;       /* W columns, contraction dim of the forward */
+    int64_t out_f;      /* W rows */
+    int64_t k;          /* coef length */
+    int64_t coef_rows;  /* 0 = vector-coef, out_f = matrix-coef */
+    int64_t sO, sI;     /* storage strides of W's (o, i) element */
+    uint32_t seed;
+    int32_t act_dtype;  /* rdb_dtype of activations and their gradients */
+    int32_t coef_dtype; /* rdb_dtype of coef and scale_bias */
+    int32_t algo;       /* RDB_ALGO_* ; 0 = let the library choose */
+} rdb_linear_desc;
+
+enum {
+    RDB_ALGO_AUTO = 0,
+    RDB_ALGO_TILE = 1 /* regenerate W tiles in LDS, contract with MFMA (general shapes) */
+};
+
+/* Replaces the dispatch of aten.mm / aten.addmm on a pseudorandom tensor: materialize() then the dense
+ * product fakeMM (R.py:771-791, 942-952), and the experimental rt_mm (R.py:457-645).
+ * y[t, o] = sum_i x[t, i] * W[o, i]  (+ bias[o] if bias != NULL; bias has act_dtype). */
+int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef,
+                   const void *scale_bias, const void *bias, const rdb_linear_desc *desc, void *stream);
+
+/* Replaces autograd's MmBackward on the materialised weight (second materialize() + dense product).
+ * dx[t, i] = sum_o dy[t, o] * W[o, i]. */
+int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef,
+                      const void *scale_bias, const rdb_linear_desc *desc, void *stream);
+
+/* Replaces MmBackward's dW = dy^T x followed by RandumbTensorConstructor.backward ->
+ * materialize_bwd (+ scale_bias_bwd) (R.py:979-990): dW is contracted with the regenerated noise tile
+ * as it is produced and never written to memory.
+ * dcoef (fp32, [k] or [out_f x k]) and, when d_scale_bias != NULL, d_scale_bias (fp32 [1]) are
+ * OVERWRITTEN.  Partial sums from different tiles are combined with fp32 atomics (order-dependent in
+ * the last bits, like the reference's relaxed atomics, R.py:359). */
+int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const void *dy, int64_t lddy, const void *x,
+                         int64_t ldx, const rdb_linear_desc *desc, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RANDUMB_HIP_H */

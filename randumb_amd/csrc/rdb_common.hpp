@@ -1,0 +1,97 @@
+// Shared device helpers for librandumb_hip: Squirrel5 noise, bf16 conversion, MFMA fragments, errors.
+// gfx950 only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/randumb_hip.h"
+
+namespace rdb {
+
+// ----------------------------------------------------------------------------------------------- errors
+int set_error(int code, const char *fmt, ...);  // records the message for rdb_last_error_string, returns code
+int check_launch(const char *what);             // hipGetLastError -> positive code + message
+
+// ----------------------------------------------------------------------------------------------- noise
+// Squirrel5 constants and the row/column mixing prime (reference: src/rten_cpp/RandumbTensor.py:140-145,
+// src/rten_cpp/csrc/cuda/rten.cu:13-18).
+constexpr uint32_t SQ5_N1 = 0xd2a80a3fu;
+constexpr uint32_t SQ5_N2 = 0xa884f197u;
+constexpr uint32_t SQ5_N3 = 0x6C736F4Bu;
+constexpr uint32_t SQ5_N4 = 0xB79F3ABBu;
+constexpr uint32_t SQ5_N5 = 0x1b56c4f5u;
+constexpr uint32_t PRIME = 198491317u;
+// (PRIME*n + m)*N1 + seed == n*PN1 + m*N1 + seed (mod 2^32): lets a loop over n or m advance the first
+// round with one add instead of a multiply.
+constexpr uint32_t PN1 = (uint32_t)((uint64_t)PRIME * (uint64_t)SQ5_N1);
+
+// Rounds after "b = idx*N1 + seed" (reference: RandumbTensor.py:151-159).
+__device__ __forceinline__ uint32_t sq5_tail(uint32_t b)
+{
+    b ^= (b >> 9);
+    b += SQ5_N2;
+    b ^= (b >> 11);
+    b *= SQ5_N3;
+    b ^= (b >> 13);
+    b += SQ5_N4;
+    b ^= (b >> 15);
+    b *= SQ5_N5;
+    b ^= (b >> 17);
+    return b;
+}
+
+__device__ __forceinline__ uint32_t sq5_bits(uint32_t idx, uint32_t seed) { return sq5_tail(idx * SQ5_N1 + seed); }
+
+// int32 reinterpretation -> fp32 (round to nearest even) -> exact scale by 2^-31
+// (reference: RandumbTensor.py:162-163; fp32(1/0x7FFFFFFF) == 2^-31).
+__device__ __forceinline__ float sq5_unit(uint32_t bits) { return (float)(int32_t)bits * 4.656612873077392578125e-10f; }
+
+__device__ __forceinline__ float noise1d(uint32_t idx, uint32_t seed) { return sq5_unit(sq5_bits(idx, seed)); }
+__device__ __forceinline__ float noise2d(uint32_t n, uint32_t m, uint32_t seed)
+{
+    return sq5_unit(sq5_bits(PRIME * n + m, seed));
+}
+// First-round value for (n, m): pass to sq5_tail.  first(n, m+1) = first(n, m) + N1; first(n+1, m) = first(n, m) + PN1.
+__device__ __forceinline__ uint32_t sq5_first(uint32_t n, uint32_t m, uint32_t seed) { return n * PN1 + m * SQ5_N1 + seed; }
+
+// ----------------------------------------------------------------------------------------------- bf16
+typedef uint16_t bf16_t;  // storage type
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi)
+{
+    f32x2 v = {lo, hi};
+    bf16x2 r = __builtin_convertvector(v, bf16x2);  // v_cvt_pk_bf16_f32: round to nearest even
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) { return (bf16_t)(f32x2_to_bf16x2(f, 0.0f) & 0xffffu); }
+
+template <typename T> struct elem;
+template <> struct elem<float> {
+    static constexpr int dtype = RDB_F32;
+    __device__ static __forceinline__ float load(const float *p) { return *p; }
+    __device__ static __forceinline__ void store(float *p, float v) { *p = v; }
+    __device__ static __forceinline__ float round(float v) { return v; }
+};
+template <> struct elem<bf16_t> {
+    static constexpr int dtype = RDB_BF16;
+    __device__ static __forceinline__ float load(const bf16_t *p) { return bf16_to_f32(*p); }
+    __device__ static __forceinline__ void store(bf16_t *p, float v) { *p = f32_to_bf16(v); }
+    __device__ static __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+};
+
+// Reads element i of a buffer whose dtype is only known at run time.
+__device__ __forceinline__ float load_as_f32(const void *p, int dtype, int64_t i)
+{
+    return dtype == RDB_BF16 ? bf16_to_f32(((const bf16_t *)p)[i]) : ((const float *)p)[i];
+}
+
+inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace rdb

@@ -1,0 +1,389 @@
+// Fused linear layer on a pseudorandom weight, general-shape kernels ("tile" algorithm).
+//
+//   forward : y  = x  . W^T        W (out_f x in_f) is regenerated block by block in LDS
+//   bwd dx  : dx = dy . W
+//   bwd dC  : dW = dy^T . x  is produced block by block in registers and contracted at once with the
+//             regenerated noise, dcoef += dW . Noise^T; neither W nor dW is ever written to memory.
+//
+// Each 256-thread block owns a 128 x 128 output block (4 waves, 64 x 64 each, 32x32 MFMA blocks) and walks the
+// contraction in steps of 32.  Reference behaviour replaced: materialize() + dense product per aten.mm
+// (src/rten_cpp/RandumbTensor.py:942-952, 771-791), autograd's MmBackward on the dense weight, and
+// RandumbTensorConstructor.backward -> materialize_bwd / scale_bias_bwd (RandumbTensor.py:979-990).
+#include "rdb_tile.hpp"
+
+namespace rdb {
+
+constexpr int BM = 128, BN = 128, BK = 32;
+
+struct LinParams {
+    WeightSpec w;
+    const void *a;  // fwd: x, dx: dy, dcoef: dy
+    const void *b;  // dcoef: x
+    void *out;      // fwd: y, dx: dx
+    const void *bias;
+    float *dcoef;
+    float *dsb;
+    int64_t lda, ldb, ldo;
+    int64_t tokens;
+    int vec_a, vec_b;  // 16-byte vector loads allowed
+};
+
+template <typename T>
+__device__ __forceinline__ void mma_step(f32x16 (&acc)[2][2], const T *As, const T *Bs, int ld, int wm, int wn, int r, int g)
+{
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+        typename MMA<T>::Frag fa[2], fb[2];
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi) fa[mi] = MMA<T>::load(As + (wm * 64 + mi * 32 + r) * ld + ks * 16 + g * 8);
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) fb[ni] = MMA<T>::load(Bs + (wn * 64 + ni * 32 + r) * ld + ks * 16 + g * 8);
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) MMA<T>::mma(acc[mi][ni], fa[mi], fb[ni]);
+    }
+}
+
+// out[(m0+m)*ldo + n0+n] = acc (+ bias[n]) for the block's valid part.
+template <typename T>
+__device__ __forceinline__ void store_block(const f32x16 (&acc)[2][2], T *out, int64_t ldo, int64_t m0, int64_t M, int64_t n0,
+                                            int64_t N, const T *bias, int wm, int wn, int r, int g)
+{
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni) {
+        const int64_t n = n0 + wn * 64 + ni * 32 + r;
+        if (n >= N) continue;
+        const float bv = bias ? to_f32<T>(bias[n]) : 0.0f;
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int64_t m = m0 + wm * 64 + mi * 32 + 8 * (j / 4) + 4 * g + (j % 4);
+                if (m < M) out[m * ldo + n] = from_f32<T>(acc[mi][ni][j] + bv);
+            }
+    }
+}
+
+// ----------------------------------------------------------------------------------------------- forward
+// y[t, o] = sum_i x[t, i] * W[o, i].  M = tokens, N = out_f, contraction over in_f.
+template <typename T, bool MATRIX>
+__global__ __launch_bounds__(TILE_THREADS) void linear_fwd_kernel(LinParams p)
+{
+    constexpr int LD = BK + MMA<T>::PAD;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T *As = reinterpret_cast<T *>(smem_raw);
+    T *Bs = As + BM * LD;
+    T *scratch = Bs + BN * LD;
+    const int t = threadIdx.x, wave = t / 64, lane = t % 64, r = lane % 32, g = lane / 32, wm = wave / 2, wn = wave % 2;
+    const int64_t n0 = (int64_t)blockIdx.x * BN, m0 = (int64_t)blockIdx.y * BM;
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) acc[mi][ni] = zero16();
+    for (int64_t k0 = 0; k0 < p.w.in_f; k0 += BK) {
+        load_tile_rowmajor<T, BM, BK>(As, LD, (const T *)p.a, p.lda, m0, p.tokens, k0, p.w.in_f, p.vec_a);
+        gen_w_tile<T, BN, BK, true, MATRIX>(Bs, LD, scratch, p.w, n0, k0);  // Bs[o][i]
+        __syncthreads();
+        mma_step<T>(acc, As, Bs, LD, wm, wn, r, g);
+        __syncthreads();
+    }
+    store_block<T>(acc, (T *)p.out, p.ldo, m0, p.tokens, n0, p.w.out_f, (const T *)p.bias, wm, wn, r, g);
+}
+
+// ----------------------------------------------------------------------------------------------- backward dx
+// dx[t, i] = sum_o dy[t, o] * W[o, i].  M = tokens, N = in_f, contraction over out_f.
+template <typename T, bool MATRIX>
+__global__ __launch_bounds__(TILE_THREADS) void linear_dx_kernel(LinParams p)
+{
+    constexpr int LD = BK + MMA<T>::PAD;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T *As = reinterpret_cast<T *>(smem_raw);
+    T *Bs = As + BM * LD;
+    T *scratch = Bs + BN * LD;
+    const int t = threadIdx.x, wave = t / 64, lane = t % 64, r = lane % 32, g = lane / 32, wm = wave / 2, wn = wave % 2;
+    const int64_t n0 = (int64_t)blockIdx.x * BN, m0 = (int64_t)blockIdx.y * BM;
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) acc[mi][ni] = zero16();
+    for (int64_t k0 = 0; k0 < p.w.out_f; k0 += BK) {
+        load_tile_rowmajor<T, BM, BK>(As, LD, (const T *)p.a, p.lda, m0, p.tokens, k0, p.w.out_f, p.vec_a);
+        gen_w_tile<T, BK, BN, false, MATRIX>(Bs, LD, scratch, p.w, k0, n0);  // Bs[i][o]
+        __syncthreads();
+        mma_step<T>(acc, As, Bs, LD, wm, wn, r, g);
+        __syncthreads();
+    }
+    store_block<T>(acc, (T *)p.out, p.ldo, m0, p.tokens, n0, p.w.in_f, (const T *)nullptr, wm, wn, r, g);
+}
+
+// ----------------------------------------------------------------------------------------------- backward dcoef
+// dW[o, i] = sum_t dy[t, o] * x[t, i] for the block (M = out_f, N = in_f, contraction over tokens), then
+//   matrix-coef: dC[o, m]  += sum_i dW[o, i] * noise(i, m)           (matrix cores, m in chunks of 32)
+//   vector-coef: dcoef[m]  += sum_{o,i} dW[o, i] * noise(o*sO + i*sI, m)   (vector ALU)
+//   d_scale_bias           += sum_{o,i} dW[o, i] * noise(o*sO + i*sI)
+// dW is rounded to T once before the contraction (a bf16 dense product would have stored it as bf16).
+template <typename T, bool MATRIX>
+__global__ __launch_bounds__(TILE_THREADS) void linear_dcoef_kernel(LinParams p)
+{
+    constexpr int LD = BK + MMA<T>::PAD;
+    constexpr int LDW = BN + MMA<T>::PAD;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T *As = reinterpret_cast<T *>(smem_raw);
+    T *Bs = As + BM * LD;
+    const int t = threadIdx.x, wave = t / 64, lane = t % 64, r = lane % 32, g = lane / 32, wm = wave / 2, wn = wave % 2;
+    const int64_t n0 = (int64_t)blockIdx.x * BN, m0 = (int64_t)blockIdx.y * BM;  // n0: first i, m0: first o
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) acc[mi][ni] = zero16();
+    for (int64_t k0 = 0; k0 < p.tokens; k0 += BK) {
+        load_tile_transposed<T, BM, BK>(As, LD, (const T *)p.a, p.lda, m0, p.w.out_f, k0, p.tokens, p.vec_a);  // As[o][t]
+        load_tile_transposed<T, BN, BK>(Bs, LD, (const T *)p.b, p.ldb, n0, p.w.in_f, k0, p.tokens, p.vec_b);   // Bs[i][t]
+        __syncthreads();
+        mma_step<T>(acc, As, Bs, LD, wm, wn, r, g);
+        __syncthreads();
+    }
+    // stage dW as Ws[o][i] (i contiguous); entries outside the matrix are exact zeros (zero-filled operands)
+    T *Ws = reinterpret_cast<T *>(smem_raw);  // [BM][LDW], reuses the operand tiles
+    T *Ns = Ws + BM * LDW;                    // [32][LDW]  Ns[m][i]
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int o = wm * 64 + mi * 32 + 8 * (j / 4) + 4 * g + (j % 4), i = wn * 64 + ni * 32 + r;
+                Ws[o * LDW + i] = from_f32<T>(acc[mi][ni][j]);
+            }
+    __syncthreads();
+    const WeightSpec &w = p.w;
+    if constexpr (MATRIX) {
+        // E[a = m][b = o] = sum_i Ns[m][i] * Ws[o][i]; wave `wave` owns o-block `wave` (32 rows of the tile)
+        for (int64_t mc = 0; mc < w.k; mc += 32) {
+            for (int e = t; e < 32 * BN; e += TILE_THREADS) {
+                const int mm = e / BN, ii = e % BN;
+                Ns[mm * LDW + ii] = from_f32<T>(noise2d((uint32_t)(n0 + ii), (uint32_t)(mc + mm), w.seed));
+            }
+            __syncthreads();
+            f32x16 e16 = zero16();
+#pragma unroll
+            for (int ks = 0; ks < BN / 16; ++ks) {
+                typename MMA<T>::Frag fa = MMA<T>::load(Ns + r * LDW + ks * 16 + g * 8);
+                typename MMA<T>::Frag fb = MMA<T>::load(Ws + (wave * 32 + r) * LDW + ks * 16 + g * 8);
+                MMA<T>::mma(e16, fa, fb);
+            }
+            const int64_t o = m0 + wave * 32 + r;
+            if (o < w.out_f) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const int64_t m = mc + 8 * (j / 4) + 4 * g + (j % 4);
+                    if (m < w.k) unsafeAtomicAdd(p.dcoef + o * w.k + m, e16[j]);
+                }
+            }
+            __syncthreads();
+        }
+    } else {
+        // thread (ml = t % 32, grp = t / 32): coefficient mc + ml, elements grp, grp + 8, ... of the block
+        float *red = reinterpret_cast<float *>(Ns);  // [8][32]
+        const int ml = t % 32, grp = t / 32;
+        for (int64_t mc = 0; mc < w.k; mc += 32) {
+            const uint32_t mterm = (uint32_t)(mc + ml) * SQ5_N1 + w.seed;
+            float s = 0.0f;
+            for (int e = grp; e < BM * BN; e += 8) {
+                const int oo = e / BN, ii = e % BN;
+                const uint32_t a = (uint32_t)((m0 + oo) * w.sO + (n0 + ii) * w.sI);
+                s = fmaf(sq5_unit(sq5_tail(a * PN1 + mterm)), to_f32<T>(Ws[oo * LDW + ii]), s);
+            }
+            __syncthreads();
+            red[grp * 32 + ml] = s;
+            __syncthreads();
+            if (grp == 0 && mc + ml < w.k) {
+                float tot = red[ml];
+#pragma unroll
+                for (int j = 1; j < 8; ++j) tot += red[j * 32 + ml];
+                unsafeAtomicAdd(p.dcoef + mc + ml, tot);
+            }
+        }
+    }
+    if (p.dsb) {
+        float s = 0.0f;
+        for (int e = t; e < BM * BN; e += TILE_THREADS) {
+            const int oo = e / BN, ii = e % BN;
+            s = fmaf(to_f32<T>(Ws[oo * LDW + ii]), noise1d((uint32_t)((m0 + oo) * w.sO + (n0 + ii) * w.sI), w.seed), s);
+        }
+        __syncthreads();
+        float *red = reinterpret_cast<float *>(Ns);
+        red[t] = s;
+        __syncthreads();
+        for (int st = TILE_THREADS / 2; st > 0; st >>= 1) {
+            if (t < st) red[t] += red[t + st];
+            __syncthreads();
+        }
+        if (t == 0) unsafeAtomicAdd(p.dsb, red[0]);
+    }
+}
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(float *p, int64_t n)
+{
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) p[e] = 0.0f;
+}
+
+// ----------------------------------------------------------------------------------------------- host side
+template <typename T> static size_t smem_fwd() { return sizeof(T) * ((BM + BN) * (BK + MMA<T>::PAD) + gen_scratch_elems<T, BN, BK>()); }
+template <typename T> static size_t smem_dcoef()
+{
+    const size_t a = sizeof(T) * (BM + BN) * (BK + MMA<T>::PAD);
+    const size_t b = sizeof(T) * (BM + 32) * (BN + MMA<T>::PAD);
+    return a > b ? a : b;
+}
+
+static int check_desc(const char *who, const rdb_linear_desc *d)
+{
+    if (!d) return set_error(RDB_E_NULL, "%s: desc is NULL", who);
+    if (d->tokens < 0 || d->in_f < 0 || d->out_f < 0 || d->k < 0)
+        return set_error(RDB_E_SHAPE, "%s: negative size tokens=%lld in=%lld out=%lld k=%lld", who, (long long)d->tokens,
+                         (long long)d->in_f, (long long)d->out_f, (long long)d->k);
+    if (d->act_dtype != RDB_F32 && d->act_dtype != RDB_BF16) return set_error(RDB_E_DTYPE, "%s: unknown act dtype %d", who, d->act_dtype);
+    if (d->coef_dtype != RDB_F32 && d->coef_dtype != RDB_BF16) return set_error(RDB_E_DTYPE, "%s: unknown coef dtype %d", who, d->coef_dtype);
+    if (d->coef_rows != 0 && d->coef_rows != d->out_f)
+        return set_error(RDB_E_SHAPE, "%s: coef_rows must be 0 or out_f (%lld), got %lld", who, (long long)d->out_f, (long long)d->coef_rows);
+    if (d->coef_rows != 0 && (d->sO != d->in_f || d->sI != 1))
+        return set_error(RDB_E_SHAPE, "%s: matrix-coef needs strides (in_f, 1), got (%lld, %lld)", who, (long long)d->sO, (long long)d->sI);
+    if (d->sO < 0 || d->sI < 0) return set_error(RDB_E_SHAPE, "%s: negative weight stride", who);
+    if (d->algo != RDB_ALGO_AUTO && d->algo != RDB_ALGO_TILE) return set_error(RDB_E_UNSUPPORTED, "%s: unknown algo %d", who, d->algo);
+    if (d->tokens > (1ll << 31) * BM || d->in_f > (1ll << 31) || d->out_f > (1ll << 31))
+        return set_error(RDB_E_SHAPE, "%s: dimension too large", who);
+    return RDB_OK;
+}
+
+static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+static WeightSpec make_spec(const rdb_linear_desc *d, const void *coef, const void *scale_bias)
+{
+    WeightSpec w;
+    w.coef = coef;
+    w.scale_bias = scale_bias;
+    w.out_f = d->out_f;
+    w.in_f = d->in_f;
+    w.k = d->k;
+    w.sO = d->sO;
+    w.sI = d->sI;
+    w.seed = d->seed;
+    w.coef_dtype = d->coef_dtype;
+    return w;
+}
+
+template <typename K> static int launch(K kernel, dim3 grid, size_t smem, hipStream_t s, const LinParams &p, const char *name)
+{
+    if (smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return set_error((int)e, "%s: cannot reserve %zu bytes of LDS: %s", name, smem, hipGetErrorString(e));
+    }
+    kernel<<<grid, TILE_THREADS, smem, s>>>(p);
+    return check_launch(name);
+}
+
+}  // namespace rdb
+
+using namespace rdb;
+
+extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias,
+                              const void *bias, const rdb_linear_desc *d, void *stream)
+{
+    int rc = check_desc("rdb_linear_fwd", d);
+    if (rc) return rc;
+    if (d->tokens == 0 || d->out_f == 0) return RDB_OK;
+    if (!y || (!x && d->in_f > 0) || (!coef && d->k > 0)) return set_error(RDB_E_NULL, "rdb_linear_fwd: y, x or coef is NULL");
+    if (ldy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_fwd: leading dimension smaller than the row");
+    const int es = d->act_dtype == RDB_BF16 ? 2 : 4;
+    LinParams p = {};
+    p.w = make_spec(d, coef, scale_bias);
+    p.a = x;
+    p.lda = ldx;
+    p.out = y;
+    p.ldo = ldy;
+    p.bias = bias;
+    p.tokens = d->tokens;
+    p.vec_a = aligned16(x) && (ldx * es) % 16 == 0;
+    dim3 grid((unsigned)cdiv(d->out_f, BN), (unsigned)cdiv(d->tokens, BM));
+    hipStream_t s = (hipStream_t)stream;
+    const bool mat = d->coef_rows != 0;
+    if (d->act_dtype == RDB_BF16)
+        return mat ? launch(linear_fwd_kernel<bf16_t, true>, grid, smem_fwd<bf16_t>(), s, p, "linear_fwd_kernel<bf16,matrix>")
+                   : launch(linear_fwd_kernel<bf16_t, false>, grid, smem_fwd<bf16_t>(), s, p, "linear_fwd_kernel<bf16,vector>");
+    return mat ? launch(linear_fwd_kernel<float, true>, grid, smem_fwd<float>(), s, p, "linear_fwd_kernel<f32,matrix>")
+               : launch(linear_fwd_kernel<float, false>, grid, smem_fwd<float>(), s, p, "linear_fwd_kernel<f32,vector>");
+}
+
+extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias,
+                                 const rdb_linear_desc *d, void *stream)
+{
+    int rc = check_desc("rdb_linear_bwd_dx", d);
+    if (rc) return rc;
+    if (d->tokens == 0 || d->in_f == 0) return RDB_OK;
+    if (!dx || (!dy && d->out_f > 0) || (!coef && d->k > 0)) return set_error(RDB_E_NULL, "rdb_linear_bwd_dx: dx, dy or coef is NULL");
+    if (lddx < d->in_f || lddy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dx: leading dimension smaller than the row");
+    const int es = d->act_dtype == RDB_BF16 ? 2 : 4;
+    LinParams p = {};
+    p.w = make_spec(d, coef, scale_bias);
+    p.a = dy;
+    p.lda = lddy;
+    p.out = dx;
+    p.ldo = lddx;
+    p.tokens = d->tokens;
+    p.vec_a = aligned16(dy) && (lddy * es) % 16 == 0;
+    dim3 grid((unsigned)cdiv(d->in_f, BN), (unsigned)cdiv(d->tokens, BM));
+    hipStream_t s = (hipStream_t)stream;
+    const bool mat = d->coef_rows != 0;
+    if (d->act_dtype == RDB_BF16)
+        return mat ? launch(linear_dx_kernel<bf16_t, true>, grid, smem_fwd<bf16_t>(), s, p, "linear_dx_kernel<bf16,matrix>")
+                   : launch(linear_dx_kernel<bf16_t, false>, grid, smem_fwd<bf16_t>(), s, p, "linear_dx_kernel<bf16,vector>");
+    return mat ? launch(linear_dx_kernel<float, true>, grid, smem_fwd<float>(), s, p, "linear_dx_kernel<f32,matrix>")
+               : launch(linear_dx_kernel<float, false>, grid, smem_fwd<float>(), s, p, "linear_dx_kernel<f32,vector>");
+}
+
+extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const void *dy, int64_t lddy, const void *x, int64_t ldx,
+                                    const rdb_linear_desc *d, void *stream)
+{
+    int rc = check_desc("rdb_linear_bwd_dcoef", d);
+    if (rc) return rc;
+    const int64_t ncoef = (d->coef_rows ? d->coef_rows : 1) * d->k;
+    if (ncoef > 0 && !dcoef) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef: dcoef is NULL");
+    hipStream_t s = (hipStream_t)stream;
+    if (ncoef > 0) {
+        fill_zero_kernel<<<(unsigned)(cdiv(ncoef, 256) < 1024 ? cdiv(ncoef, 256) : 1024), 256, 0, s>>>(dcoef, ncoef);
+        rc = check_launch("fill_zero_kernel");
+        if (rc) return rc;
+    }
+    if (d_scale_bias) {
+        fill_zero_kernel<<<1, 256, 0, s>>>(d_scale_bias, 1);
+        rc = check_launch("fill_zero_kernel");
+        if (rc) return rc;
+    }
+    if (d->tokens == 0 || d->in_f == 0 || d->out_f == 0 || (ncoef == 0 && !d_scale_bias)) return RDB_OK;
+    if (!dy || !x) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef: dy or x is NULL");
+    if (lddy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dcoef: leading dimension smaller than the row");
+    const int es = d->act_dtype == RDB_BF16 ? 2 : 4;
+    LinParams p = {};
+    p.w = make_spec(d, nullptr, nullptr);
+    p.a = dy;
+    p.lda = lddy;
+    p.b = x;
+    p.ldb = ldx;
+    p.dcoef = dcoef;
+    p.dsb = d_scale_bias;
+    p.tokens = d->tokens;
+    p.vec_a = aligned16(dy) && (lddy * es) % 16 == 0;
+    p.vec_b = aligned16(x) && (ldx * es) % 16 == 0;
+    dim3 grid((unsigned)cdiv(d->in_f, BN), (unsigned)cdiv(d->out_f, BM));
+    const bool mat = d->coef_rows != 0;
+    if (d->act_dtype == RDB_BF16)
+        return mat ? launch(linear_dcoef_kernel<bf16_t, true>, grid, smem_dcoef<bf16_t>(), s, p, "linear_dcoef_kernel<bf16,matrix>")
+                   : launch(linear_dcoef_kernel<bf16_t, false>, grid, smem_dcoef<bf16_t>(), s, p, "linear_dcoef_kernel<bf16,vector>");
+    return mat ? launch(linear_dcoef_kernel<float, true>, grid, smem_dcoef<float>(), s, p, "linear_dcoef_kernel<f32,matrix>")
+               : launch(linear_dcoef_kernel<float, false>, grid, smem_dcoef<float>(), s, p, "linear_dcoef_kernel<f32,vector>");
+}

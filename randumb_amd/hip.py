@@ -1,0 +1,246 @@
+"""Tensor-level wrappers over the C ABI: allocate outputs with torch, pass raw device pointers and the current
+HIP stream to ``librandumb_hip.so``.  No arithmetic happens in Python and there is no CPU path: a CPU tensor
+raises ``NotImplementedError`` exactly as the reference's CPU registrations do
+(src/rten_cpp/RandumbTensor.py:438-448, 1151-1157)."""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib
+from ._lib import LinearDesc, RDB_ALGO_AUTO, RDB_BF16, RDB_F32
+
+_DT = {torch.float32: RDB_F32, torch.bfloat16: RDB_BF16}
+
+
+def _need_gpu(name: str, *tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise NotImplementedError(f"Unsupported CPU implementation of {name} called.")
+
+
+def _native(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """Contiguous tensor of a dtype the library reads directly (fp32 / bf16); other floats go through fp32."""
+    if t is None:
+        return None
+    if t.dtype not in _DT:
+        t = t.to(torch.float32)
+    return t.contiguous()
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _workspace(nbytes: int, device) -> Optional[torch.Tensor]:
+    return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes > 0 else None
+
+
+def _seed(seed: int) -> int:
+    seed = int(seed)
+    if not 0 <= seed < 2**32:
+        raise ValueError(f"seed must fit in 32 unsigned bits, got {seed}")
+    return seed
+
+
+# ------------------------------------------------------------------------------------------------ probes
+def sq5_fill_2d(N: int, M: int, seed: int, device="cuda") -> torch.Tensor:
+    """Noise matrix ``(N, M)``, ``out[n, m] = noise(PRIME*n + m)``  (RandumbTensor.py:101-105)."""
+    out = torch.empty((N, M), dtype=torch.float32, device=device)
+    _need_gpu("sq5_fill_2d", out)
+    with torch.cuda.device(out.device):
+        _lib.check(_lib.load().rdb_sq5_fill_2d(_p(out), N, M, _seed(seed), _stream(out.device)), "rdb_sq5_fill_2d")
+    return out
+
+
+def sq5_fill_1d(N: int, seed: int, device="cuda") -> torch.Tensor:
+    """1-D noise ``out[n] = noise(n)``  (RandumbTensor.py:122-126)."""
+    out = torch.empty((N,), dtype=torch.float32, device=device)
+    _need_gpu("sq5_fill_1d", out)
+    with torch.cuda.device(out.device):
+        _lib.check(_lib.load().rdb_sq5_fill_1d(_p(out), N, _seed(seed), _stream(out.device)), "rdb_sq5_fill_1d")
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ materialise
+def materialize_fwd(coefs: torch.Tensor, size: Sequence[int], strides: Sequence[int], seed: int,
+                    scale_bias: Optional[torch.Tensor], fused_bias: bool, row_len: Optional[int] = None) -> torch.Tensor:
+    """fp32 contiguous tensor of shape ``size``; the view's ``strides`` address the noise rows
+    (RandumbTensor.py:371-381).  ``coefs.dim() == 2`` selects the matrix-coef form, whose base tensor is
+    ``(coefs.shape[0], row_len)`` contiguous (``row_len`` defaults to ``numel / coefs.shape[0]``)."""
+    assert not (fused_bias and scale_bias is None), "scale_bias not initialized but fused_bias is True"
+    _need_gpu("materialize_fwd", coefs)
+    size, strides = [int(s) for s in size], [int(s) for s in strides]
+    output = torch.empty(size, dtype=torch.float32, device=coefs.device)
+    if len(size) == 1:  # RandumbTensor.py:375-377
+        size, strides = [1, size[0]], [0, strides[0]]
+    if len(size) != 2:
+        raise ValueError(f"materialize_fwd supports 1-D and 2-D shapes, got {size}")
+    c = _native(coefs)
+    sb = _native(scale_bias).to(c.dtype) if fused_bias else None
+    if c.dim() == 1:
+        rows, k, row_len = 0, c.shape[0], 0
+    elif c.dim() == 2:
+        rows, k = c.shape
+        numel = size[0] * size[1]
+        if row_len is None:
+            if rows == 0 or numel % rows:
+                raise ValueError(f"matrix-coef with {rows} rows cannot back a tensor of {numel} elements")
+            row_len = numel // rows
+    else:
+        raise ValueError("coefs must be 1-D or 2-D")
+    with torch.cuda.device(c.device):
+        rc = _lib.load().rdb_materialize_fwd(_p(output), _p(c), _DT[c.dtype], rows, k, row_len, size[0], size[1],
+                                             strides[0], strides[1], _seed(seed), _p(sb), _stream(c.device))
+    _lib.check(rc, "rdb_materialize_fwd")
+    return output
+
+
+def materialize_bwd(dout: torch.Tensor, dcoefs_size: int, seed: int, coef_rows: int = 0) -> torch.Tensor:
+    """``Noise.T @ dout`` in fp32: ``(dcoefs_size,)`` or, matrix-coef, ``(coef_rows, dcoefs_size)``
+    (RandumbTensor.py:383-390)."""
+    assert dout.is_contiguous(), "dout is not contiguous, backwards pass might give incorrect results."
+    _need_gpu("materialize_bwd", dout)
+    d = _native(dout)
+    k, Nw = int(dcoefs_size), d.numel()
+    shape = (k,) if coef_rows == 0 else (coef_rows, k)
+    row_len = 0 if coef_rows == 0 else Nw // max(coef_rows, 1)
+    dcoefs = torch.empty(shape, dtype=torch.float32, device=d.device)
+    L = _lib.load()
+    ws_bytes = L.rdb_materialize_bwd_workspace_bytes(coef_rows, k, row_len, Nw)
+    ws = _workspace(ws_bytes, d.device)
+    with torch.cuda.device(d.device):
+        rc = L.rdb_materialize_bwd(_p(dcoefs), _p(d), _DT[d.dtype], coef_rows, k, row_len, Nw, _seed(seed), _p(ws), ws_bytes,
+                                   _stream(d.device))
+    _lib.check(rc, "rdb_materialize_bwd")
+    return dcoefs
+
+
+def scale_bias_bwd(dout: torch.Tensor, seed: int) -> torch.Tensor:
+    """``sum(dout * noise_1d)`` as an fp32 ``(1,)`` tensor (RandumbTensor.py:414-420)."""
+    assert dout.is_contiguous(), "dout is not contiguous, backwards pass might give incorrect results."
+    _need_gpu("scale_bias_bwd", dout)
+    d = _native(dout)
+    ds = torch.empty((1,), dtype=torch.float32, device=d.device)
+    L = _lib.load()
+    ws_bytes = L.rdb_scale_bias_bwd_workspace_bytes(d.numel())
+    ws = _workspace(ws_bytes, d.device)
+    with torch.cuda.device(d.device):
+        rc = L.rdb_scale_bias_bwd(_p(ds), _p(d), _DT[d.dtype], d.numel(), _seed(seed), _p(ws), ws_bytes, _stream(d.device))
+    _lib.check(rc, "rdb_scale_bias_bwd")
+    return ds
+
+
+# ------------------------------------------------------------------------------------------------ embedding
+def embed_fwd(idx: torch.Tensor, coefs: torch.Tensor, rowsize: int, seed: int) -> torch.Tensor:
+    """Rows ``idx`` of a ``(*, rowsize)`` vector-coef tensor, fp32 ``(*idx.shape, rowsize)`` (RandumbTensor.py:1121-1126)."""
+    _need_gpu("embed_fwd", idx, coefs)
+    c = _native(coefs)
+    ix = idx.to(torch.int64).contiguous()
+    out = torch.empty((*idx.shape, rowsize), dtype=torch.float32, device=c.device)
+    with torch.cuda.device(c.device):
+        rc = _lib.load().rdb_embed_fwd(_p(out), _p(ix), ix.numel(), _p(c), _DT[c.dtype], c.numel(), int(rowsize), _seed(seed),
+                                       _stream(c.device))
+    _lib.check(rc, "rdb_embed_fwd")
+    return out
+
+
+def embed_bwd(idx: torch.Tensor, dout: torch.Tensor, dcoefs_size: int, rowsize: int, seed: int) -> torch.Tensor:
+    """Coefficient gradient of :func:`embed_fwd`, fp32 ``(dcoefs_size,)`` (RandumbTensor.py:1128-1134)."""
+    _need_gpu("embed_bwd", idx, dout)
+    d = _native(dout)
+    ix = idx.to(torch.int64).contiguous()
+    k = int(dcoefs_size)
+    dcoefs = torch.empty((k,), dtype=torch.float32, device=d.device)
+    L = _lib.load()
+    ws_bytes = L.rdb_embed_bwd_workspace_bytes(ix.numel(), int(rowsize), k)
+    ws = _workspace(ws_bytes, d.device)
+    with torch.cuda.device(d.device):
+        rc = L.rdb_embed_bwd(_p(dcoefs), _p(ix), ix.numel(), _p(d), _DT[d.dtype], k, int(rowsize), _seed(seed), _p(ws), ws_bytes,
+                             _stream(d.device))
+    _lib.check(rc, "rdb_embed_bwd")
+    return dcoefs
+
+
+# ------------------------------------------------------------------------------------------------ fused linear
+def _desc(tokens, in_f, out_f, coef, sO, sI, seed, act_dtype, algo) -> LinearDesc:
+    d = LinearDesc()
+    d.tokens, d.in_f, d.out_f = int(tokens), int(in_f), int(out_f)
+    d.k = int(coef.shape[-1])
+    d.coef_rows = 0 if coef.dim() == 1 else int(coef.shape[0])
+    d.sO, d.sI = int(sO), int(sI)
+    d.seed = _seed(seed)
+    d.act_dtype = _DT[act_dtype]
+    d.coef_dtype = _DT[coef.dtype]
+    d.algo = int(algo)
+    return d
+
+
+def _act(t: torch.Tensor) -> torch.Tensor:
+    """2-D activation with unit inner stride in a dtype the kernels compute in."""
+    if t.dtype not in _DT:
+        t = t.to(torch.float32)
+    if t.dim() != 2:
+        raise ValueError("activations must be 2-D (tokens, features)")
+    return t if t.stride(1) == 1 and t.stride(0) >= t.shape[1] else t.contiguous()
+
+
+def linear_fwd(x: torch.Tensor, coef: torch.Tensor, in_f: int, out_f: int, sO: int, sI: int, seed: int,
+               scale_bias: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+               algo: int = RDB_ALGO_AUTO) -> torch.Tensor:
+    """``y = x @ W.T (+ bias)`` with the ``(out_f, in_f)`` pseudorandom weight regenerated on chip."""
+    _need_gpu("linear_fwd", x, coef)
+    x = _act(x)
+    c = _native(coef)
+    sb = None if scale_bias is None else _native(scale_bias).to(c.dtype)
+    b = None if bias is None else bias.to(x.dtype).contiguous()
+    y = torch.empty((x.shape[0], out_f), dtype=x.dtype, device=x.device)
+    d = _desc(x.shape[0], in_f, out_f, c, sO, sI, seed, x.dtype, algo)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().rdb_linear_fwd(_p(y), y.stride(0), _p(x), x.stride(0), _p(c), _p(sb), _p(b), ctypes.byref(d),
+                                        _stream(x.device))
+    _lib.check(rc, "rdb_linear_fwd")
+    return y
+
+
+def linear_bwd_dx(dy: torch.Tensor, coef: torch.Tensor, in_f: int, out_f: int, sO: int, sI: int, seed: int,
+                  scale_bias: Optional[torch.Tensor] = None, algo: int = RDB_ALGO_AUTO) -> torch.Tensor:
+    """``dx = dy @ W``."""
+    _need_gpu("linear_bwd_dx", dy, coef)
+    dy = _act(dy)
+    c = _native(coef)
+    sb = None if scale_bias is None else _native(scale_bias).to(c.dtype)
+    dx = torch.empty((dy.shape[0], in_f), dtype=dy.dtype, device=dy.device)
+    d = _desc(dy.shape[0], in_f, out_f, c, sO, sI, seed, dy.dtype, algo)
+    with torch.cuda.device(dy.device):
+        rc = _lib.load().rdb_linear_bwd_dx(_p(dx), dx.stride(0), _p(dy), dy.stride(0), _p(c), _p(sb), ctypes.byref(d),
+                                           _stream(dy.device))
+    _lib.check(rc, "rdb_linear_bwd_dx")
+    return dx
+
+
+def linear_bwd_dcoef(dy: torch.Tensor, x: torch.Tensor, k: int, coef_rows: int, in_f: int, out_f: int, sO: int, sI: int,
+                     seed: int, want_scale_bias_grad: bool = False, algo: int = RDB_ALGO_AUTO):
+    """``(dcoef, d_scale_bias)`` in fp32: ``dcoef = (dy.T @ x) . Noise.T`` without storing ``dy.T @ x``."""
+    _need_gpu("linear_bwd_dcoef", dy, x)
+    dy, x = _act(dy), _act(x)
+    if x.dtype != dy.dtype:
+        x = x.to(dy.dtype)
+    shape = (k,) if coef_rows == 0 else (coef_rows, k)
+    dcoef = torch.empty(shape, dtype=torch.float32, device=dy.device)
+    dsb = torch.empty((1,), dtype=torch.float32, device=dy.device) if want_scale_bias_grad else None
+    d = LinearDesc()
+    d.tokens, d.in_f, d.out_f, d.k, d.coef_rows = dy.shape[0], int(in_f), int(out_f), int(k), int(coef_rows)
+    d.sO, d.sI, d.seed = int(sO), int(sI), _seed(seed)
+    d.act_dtype, d.coef_dtype, d.algo = _DT[dy.dtype], RDB_F32, int(algo)
+    with torch.cuda.device(dy.device):
+        rc = _lib.load().rdb_linear_bwd_dcoef(_p(dcoef), _p(dsb), _p(dy), dy.stride(0), _p(x), x.stride(0), ctypes.byref(d),
+                                              _stream(dy.device))
+    _lib.check(rc, "rdb_linear_bwd_dcoef")
+    return dcoef, dsb

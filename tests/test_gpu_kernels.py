@@ -1,0 +1,249 @@
+"""GPU parity of the HIP kernels (called through the C ABI) against the CPU oracle.
+
+Integer/noise results must be bit-exact.  Floating-point tolerances (relative L2 norm):
+fp32 paths 1e-5, bf16 paths 2e-2 - the bounds the task states for this path.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 1e-5
+BF16_TOL = 2e-2
+
+
+def rel_l2(a, b):
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+@pytest.fixture(scope="module")
+def hip():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from randumb_amd import hip as h
+
+    return h
+
+
+def cpu(t):
+    return t.detach().float().cpu().numpy()
+
+
+# ------------------------------------------------------------------------------------------------ noise
+@pytest.mark.parametrize("N,M,seed", [(1, 1, 0), (3, 6, 1337), (1000, 257, 47), (4096, 16, 2**31 - 1), (70, 1024, 0xFFFFFFFF)])
+def test_noise_2d_bit_exact(hip, oracle, N, M, seed):
+    print(f"case noise2d N={N} M={M} seed={seed}", flush=True)
+    got = cpu(hip.sq5_fill_2d(N, M, seed))
+    want = oracle.noise_2d(N, M, seed)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_noise_2d_wraparound_rows_bit_exact(hip, oracle):
+    # rows whose PRIME*n product wraps 2**32 many times: compare the tail of a tall matrix
+    N, M, seed = 3_000_000, 4, 1337
+    print("case noise2d tall", flush=True)
+    got = cpu(hip.sq5_fill_2d(N, M, seed)[-1000:])
+    want = oracle.noise_2d_np(np.arange(N - 1000, N), np.arange(M), seed)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("N,seed", [(1, 0), (1000003, 1337)])
+def test_noise_1d_bit_exact(hip, oracle, N, seed):
+    got = cpu(hip.sq5_fill_1d(N, seed))
+    assert np.array_equal(got.view(np.uint32), oracle.noise_1d(N, seed).view(np.uint32))
+
+
+def test_empty_shapes(hip):
+    assert hip.sq5_fill_2d(0, 5, 1).shape == (0, 5)
+    assert hip.sq5_fill_1d(0, 1).shape == (0,)
+    c = torch.randn(4, device="cuda")
+    assert hip.materialize_fwd(c, (0, 3), (3, 1), 1, None, False).shape == (0, 3)
+
+
+# ------------------------------------------------------------------------------------------------ materialise
+@pytest.mark.parametrize("P,Q,k,seed", [(3, 6, 18, 1337), (256, 784, 64, 1337), (10, 256, 64, 1338), (1, 37, 5, 0), (129, 65, 2049, 3)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_materialize_fwd_vector_coef(hip, oracle, P, Q, k, seed, dtype):
+    print(f"case mat_fwd vec P={P} Q={Q} k={k} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(0)
+    c = torch.randn(k, generator=g).to(dtype)
+    sb = torch.tensor([0.37]).to(dtype)
+    for fused in (False, True):
+        got = cpu(hip.materialize_fwd(c.cuda(), (P, Q), (Q, 1), seed, sb.cuda() if fused else None, fused))
+        want = oracle.materialize_fwd(c.float().numpy(), (P, Q), (Q, 1), seed, float(sb.float()) if fused else None)
+        assert got.dtype == np.float32 and rel_l2(got, want) < F32_TOL
+    # transposed view: same values, transposed
+    got_t = cpu(hip.materialize_fwd(c.cuda(), (Q, P), (1, Q), seed, None, False))
+    got = cpu(hip.materialize_fwd(c.cuda(), (P, Q), (Q, 1), seed, None, False))
+    assert np.array_equal(got_t, got.T)
+
+
+def test_materialize_fwd_unit_coef_is_noise_bit_exact(hip, oracle):
+    P, Q, k, seed = 33, 65, 40, 1337
+    noise = oracle.noise_2d(P * Q, k, seed)
+    for j in (0, 17, 39):
+        c = torch.zeros(k)
+        c[j] = 1.0
+        got = cpu(hip.materialize_fwd(c.cuda(), (P, Q), (Q, 1), seed, None, False)).reshape(-1)
+        assert np.array_equal(got, noise[:, j])
+    one_d = cpu(hip.materialize_fwd(c.cuda(), (Q,), (1,), seed, None, False))
+    assert np.array_equal(one_d, noise[:Q, 39])
+
+
+@pytest.mark.parametrize("out_f,in_f,k,seed", [(7, 13, 24, 47), (256, 784, 64, 1337), (10, 256, 64, 1338), (100, 200, 33, 5)])
+def test_materialize_fwd_matrix_coef(hip, oracle, out_f, in_f, k, seed):
+    print(f"case mat_fwd mat out={out_f} in={in_f} k={k}", flush=True)
+    g = torch.Generator().manual_seed(1)
+    C = torch.randn(out_f, k, generator=g)
+    sb = torch.tensor([0.5])
+    want = oracle.materialize_fwd(C.numpy(), (out_f, in_f), (in_f, 1), seed, row_len=in_f)
+    got = cpu(hip.materialize_fwd(C.cuda(), (out_f, in_f), (in_f, 1), seed, None, False))
+    assert rel_l2(got, want) < F32_TOL
+    got_t = cpu(hip.materialize_fwd(C.cuda(), (in_f, out_f), (1, in_f), seed, None, False))
+    assert np.array_equal(got_t, got.T)
+    want_b = oracle.materialize_fwd(C.numpy(), (out_f, in_f), (in_f, 1), seed, 0.5, row_len=in_f)
+    got_b = cpu(hip.materialize_fwd(C.cuda(), (out_f, in_f), (in_f, 1), seed, sb.cuda(), True))
+    assert rel_l2(got_b, want_b) < F32_TOL
+    # a view that is neither the base nor its transpose goes through the per-element kernel: first two rows only
+    got_v = cpu(hip.materialize_fwd(C.cuda(), (2, in_f), (in_f, 1), seed, None, False, row_len=in_f))
+    assert rel_l2(got_v, want[:2]) < F32_TOL
+
+
+@pytest.mark.parametrize("Nw,k,seed", [(18, 18, 1337), (200704, 64, 1337), (2560, 64, 1338), (5000, 300, 9), (1, 7, 0)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_materialize_bwd_vector_coef(hip, oracle, Nw, k, seed, dtype):
+    print(f"case mat_bwd vec Nw={Nw} k={k} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(2)
+    d = torch.randn(Nw, generator=g).to(dtype)
+    got = cpu(hip.materialize_bwd(d.cuda(), k, seed))
+    want = oracle.materialize_bwd(d.float().numpy(), k, seed)
+    assert got.shape == (k,) and rel_l2(got, want) < F32_TOL
+    again = cpu(hip.materialize_bwd(d.cuda(), k, seed))
+    assert np.array_equal(got, again)  # fixed reduction tree: reproducible
+
+
+def test_materialize_bwd_unit_vector_bit_exact(hip, oracle):
+    Nw, k, seed = 5000, 70, 1337
+    noise = oracle.noise_2d(Nw, k, seed)
+    for n in (0, 2049, Nw - 1):
+        d = torch.zeros(Nw)
+        d[n] = 1.0
+        assert np.array_equal(cpu(hip.materialize_bwd(d.cuda(), k, seed)), noise[n])
+
+
+@pytest.mark.parametrize("out_f,in_f,k,seed", [(7, 13, 24, 47), (256, 784, 64, 1337), (100, 200, 33, 5)])
+def test_materialize_bwd_matrix_coef(hip, oracle, out_f, in_f, k, seed):
+    g = torch.Generator().manual_seed(3)
+    d = torch.randn(out_f, in_f, generator=g)
+    got = cpu(hip.materialize_bwd(d.cuda(), k, seed, coef_rows=out_f))
+    want = oracle.materialize_bwd(d.numpy(), k, seed, coef_rows=out_f)
+    assert got.shape == (out_f, k) and rel_l2(got, want) < F32_TOL
+
+
+@pytest.mark.parametrize("Nw", [1, 501, 300000])
+def test_scale_bias_bwd(hip, oracle, Nw):
+    g = torch.Generator().manual_seed(4)
+    d = torch.randn(Nw, generator=g)
+    got = cpu(hip.scale_bias_bwd(d.cuda(), 77))
+    want = oracle.scale_bias_bwd(d.numpy(), 77)
+    assert got.shape == (1,) and abs(got[0] - want[0]) < 1e-4 * max(1.0, abs(want[0]))
+
+
+def test_embedding(hip, oracle):
+    g = torch.Generator().manual_seed(5)
+    rows, rowsize, k, seed = 50304, 768, 32, 1337
+    c = torch.randn(k, generator=g)
+    idx = torch.randint(0, rows, (3, 17), generator=g)
+    idx[0, 0], idx[0, 1] = rows - 1, rows - 1  # repeated index, last row
+    got = cpu(hip.embed_fwd(idx.cuda(), c.cuda(), rowsize, seed))
+    want = oracle.embed_fwd(idx.numpy(), c.numpy(), rowsize, seed)
+    assert got.shape == (3, 17, rowsize) and rel_l2(got, want) < F32_TOL
+    D = torch.randn(3, 17, rowsize, generator=g)
+    gotb = cpu(hip.embed_bwd(idx.cuda(), D.cuda(), k, rowsize, seed))
+    wantb = oracle.embed_bwd(idx.numpy(), D.numpy(), k, rowsize, seed)
+    assert rel_l2(gotb, wantb) < F32_TOL
+
+
+# ------------------------------------------------------------------------------------------------ fused linear
+LIN_SHAPES = [
+    # tokens, in_f, out_f, k, seed
+    (9, 12, 5, 18, 1337),
+    (128, 784, 256, 64, 1337),   # MNIST-shaped layer 1
+    (128, 256, 10, 64, 1338),    # MNIST-shaped layer 2
+    (200, 100, 130, 40, 7),      # ragged everything
+    (256, 768, 384, 256, 0),     # a slice of the GPT-2 MLP shape
+]
+
+
+def _inputs(T, in_f, out_f, k, matrix, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, in_f, generator=g).to(dtype)
+    dy = torch.randn(T, out_f, generator=g).to(dtype)
+    std = (3.0 / k) ** 0.5 * 0.05
+    coef = (torch.randn((out_f, k) if matrix else (k,), generator=g) * std).to(dtype)
+    return x, dy, coef
+
+
+@pytest.mark.parametrize("T,in_f,out_f,k,seed", LIN_SHAPES)
+@pytest.mark.parametrize("matrix", [True, False])
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, F32_TOL), (torch.bfloat16, BF16_TOL)])
+def test_linear_fwd_bwd(hip, oracle, T, in_f, out_f, k, seed, matrix, dtype, tol):
+    print(f"case linear T={T} in={in_f} out={out_f} k={k} matrix={matrix} {dtype}", flush=True)
+    x, dy, coef = _inputs(T, in_f, out_f, k, matrix, dtype, seed)
+    xn, dyn, cn = x.float().numpy(), dy.float().numpy(), coef.float().numpy()
+    want_y = oracle.linear_fwd(xn, cn, in_f, out_f, seed)
+    want_dx, want_dc, _ = oracle.linear_bwd(xn, dyn, cn, in_f, out_f, seed)
+    xc, dyc, cc = x.cuda(), dy.cuda(), coef.cuda()
+    y = hip.linear_fwd(xc, cc, in_f, out_f, in_f, 1, seed)
+    assert y.dtype == dtype and y.shape == (T, out_f)
+    assert rel_l2(cpu(y), want_y) < tol
+    dx = hip.linear_bwd_dx(dyc, cc, in_f, out_f, in_f, 1, seed)
+    assert dx.dtype == dtype and rel_l2(cpu(dx), want_dx) < tol
+    dc, dsb = hip.linear_bwd_dcoef(dyc, xc, k, out_f if matrix else 0, in_f, out_f, in_f, 1, seed)
+    assert dsb is None and dc.dtype == torch.float32 and dc.shape == coef.shape
+    assert rel_l2(cpu(dc), want_dc) < tol
+
+
+def test_linear_bias_and_scale_bias(hip, oracle):
+    T, in_f, out_f, k, seed = 64, 96, 48, 32, 1337
+    for matrix in (True, False):
+        x, dy, coef = _inputs(T, in_f, out_f, k, matrix, torch.float32, 11)
+        bias = torch.randn(out_f)
+        sb = torch.tensor([0.02])
+        want = oracle.linear_fwd(x.numpy(), coef.numpy(), in_f, out_f, seed, bias=bias.numpy(), scale_bias=0.02)
+        got = hip.linear_fwd(x.cuda(), coef.cuda(), in_f, out_f, in_f, 1, seed, scale_bias=sb.cuda(), bias=bias.cuda())
+        assert rel_l2(cpu(got), want) < F32_TOL
+        want_dx, want_dc, dW = oracle.linear_bwd(x.numpy(), dy.numpy(), coef.numpy(), in_f, out_f, seed, scale_bias=0.02)
+        dx = hip.linear_bwd_dx(dy.cuda(), coef.cuda(), in_f, out_f, in_f, 1, seed, scale_bias=sb.cuda())
+        assert rel_l2(cpu(dx), want_dx) < F32_TOL
+        dc, dsb = hip.linear_bwd_dcoef(dy.cuda(), x.cuda(), k, out_f if matrix else 0, in_f, out_f, in_f, 1, seed,
+                                       want_scale_bias_grad=True)
+        assert rel_l2(cpu(dc), want_dc) < F32_TOL
+        want_ds = oracle.scale_bias_bwd(dW.astype(np.float32), seed)
+        assert abs(cpu(dsb)[0] - want_ds[0]) < 1e-4 * max(1.0, abs(want_ds[0]))
+
+
+def test_linear_strided_weight_vector_coef(hip, oracle):
+    """`mat1 @ tensor` with a contiguous (P, Q) tensor: out_f = Q, in_f = P, strides (1, Q)  (rt_mm's case)."""
+    L, P, Q, k, seed = 40, 24, 36, 16, 1337
+    g = torch.Generator().manual_seed(6)
+    mat1 = torch.randn(L, P, generator=g)
+    c = torch.randn(k, generator=g)
+    W = oracle.materialize_fwd(c.numpy(), (P, Q), (Q, 1), seed).astype(np.float64)
+    got = hip.linear_fwd(mat1.cuda(), c.cuda(), P, Q, 1, Q, seed)
+    assert rel_l2(cpu(got), mat1.double().numpy() @ W) < F32_TOL
+
+
+def test_argument_errors(hip):
+    from randumb_amd._lib import RandumbHipError
+
+    x = torch.randn(4, 8, device="cuda")
+    C = torch.randn(6, 3, device="cuda")
+    with pytest.raises(RandumbHipError):  # matrix-coef with a transposed weight layout
+        hip.linear_fwd(x, C, 8, 6, 1, 6, 0)
+    with pytest.raises(ValueError):
+        hip.sq5_fill_1d(4, -1)
+    with pytest.raises(NotImplementedError):
+        hip.materialize_fwd(torch.randn(4), (2, 2), (2, 1), 0, None, False)
