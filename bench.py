@@ -1,0 +1,201 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused pseudorandom-matrix linear layer (forward + both backward products) on one MI355X.
+
+Workload (the configuration the headline metric is quoted on): one layer at the GPT-2 small MLP up-projection
+shape, in = 768 -> out = 3072, coef dim k = 256 (matrix-coef, C is [3072 x 256]), 8192 tokens, bf16
+activations with fp32 accumulation, x ~ N(0,1), dy ~ N(0,1), C ~ N(0, 3*0.02^2/k), seed 0.  Synthetic data.
+
+A "step" is one pass of the hot path: y = x W^T, dx = dy W, dC = (dy^T x) N^T, all three through the C ABI of
+librandumb_hip.so with inputs already resident in HBM.  The printed JSON line reports
+  value        algorithmic TFLOP/s of the whole step, F = 6*T*in*out + 6*out*in*k
+  roofline     the slowest of the three kernels against the dense bf16 MFMA peak, from HIP-event timing
+  cpu_baseline the CPU restatement (materialise-then-matmul: oracle C + torch.matmul fp32) on the host cores
+  compare      the same products done as materialise-to-HBM + dense GEMM on the GPU, and a plain dense GEMM
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+T, IN_F, OUT_F, K, SEED = 8192, 768, 3072, 256, 0
+
+
+def flops_fwd():
+    return 2.0 * T * IN_F * OUT_F + 2.0 * OUT_F * IN_F * K
+
+
+def flops_dx():
+    return 2.0 * T * IN_F * OUT_F + 2.0 * OUT_F * IN_F * K
+
+
+def flops_dcoef():
+    return 2.0 * T * IN_F * OUT_F + 2.0 * OUT_F * IN_F * K
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
+    ap.add_argument("--no-compare", action="store_true", help="skip the materialise+GEMM comparison legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from randumb_amd import _lib, hip
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L = _lib.load()
+
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(T, IN_F, generator=g).bfloat16().to(dev)
+    dy = torch.randn(T, OUT_F, generator=g).bfloat16().to(dev)
+    C = (torch.randn(OUT_F, K, generator=g) * (3 * 0.02**2 / K) ** 0.5).bfloat16().to(dev)
+    y = torch.empty(T, OUT_F, dtype=torch.bfloat16, device=dev)
+    dx = torch.empty(T, IN_F, dtype=torch.bfloat16, device=dev)
+    dC = torch.empty(OUT_F, K, dtype=torch.float32, device=dev)
+
+    d = _lib.LinearDesc()
+    d.tokens, d.in_f, d.out_f, d.k, d.coef_rows = T, IN_F, OUT_F, K, OUT_F
+    d.sO, d.sI, d.seed = IN_F, 1, SEED
+    d.act_dtype, d.coef_dtype, d.algo = _lib.RDB_BF16, _lib.RDB_BF16, _lib.RDB_ALGO_AUTO
+    dref = ctypes.byref(d)
+    vp = ctypes.c_void_p
+    stream = vp(torch.cuda.current_stream().cuda_stream)
+    px, pdy, pC, py, pdx, pdC = (vp(t.data_ptr()) for t in (x, dy, C, y, dx, dC))
+
+    def k_fwd():
+        _lib.check(L.rdb_linear_fwd(py, OUT_F, px, IN_F, pC, None, None, dref, stream), "rdb_linear_fwd")
+
+    def k_dx():
+        _lib.check(L.rdb_linear_bwd_dx(pdx, IN_F, pdy, OUT_F, pC, None, dref, stream), "rdb_linear_bwd_dx")
+
+    def k_dcoef():
+        _lib.check(L.rdb_linear_bwd_dcoef(pdC, None, pdy, OUT_F, px, IN_F, dref, stream), "rdb_linear_bwd_dcoef")
+
+    def step():
+        k_fwd()
+        k_dx()
+        k_dcoef()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    F = flops_fwd() + flops_dx() + flops_dcoef()
+    value = F / (ms_per_step * 1e-3) / 1e12
+
+    # per-kernel durations from HIP events recorded on the stream the kernels are launched on
+    def event_ms(fn, iters):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters
+
+    iters = max(10, min(args.steps, 50))
+    kern = {
+        "linear_fwd": (event_ms(k_fwd, iters), flops_fwd()),
+        "linear_bwd_dx": (event_ms(k_dx, iters), flops_dx()),
+        "linear_bwd_dcoef": (event_ms(k_dcoef, iters), flops_dcoef()),
+    }
+    dom = max(kern, key=lambda n: kern[n][0])
+    dom_ms, dom_flops = kern[dom]
+    achieved = dom_flops / (dom_ms * 1e-3) / 1e12
+    roofline = {
+        "bound": "mfma", "kernel": dom, "achieved": round(achieved, 3), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 5), "traffic": None, "avg_kernel_ms": round(dom_ms, 5),
+        "kernels_ms": {n: round(v[0], 5) for n, v in kern.items()},
+    }
+
+    compare = None
+    if not args.no_compare:
+        def mat_gemm_step():
+            # the reference's data flow on the GPU: W to HBM (twice per step), three dense GEMMs, dW to HBM
+            W = hip.materialize_fwd(C, (OUT_F, IN_F), (IN_F, 1), SEED, None, False).to(torch.bfloat16)
+            yy = x @ W.t()
+            W2 = hip.materialize_fwd(C, (OUT_F, IN_F), (IN_F, 1), SEED, None, False).to(torch.bfloat16)
+            dxx = dy @ W2
+            dW = dy.t() @ x
+            dCC = hip.materialize_bwd(dW, K, SEED, coef_rows=OUT_F)
+            return yy, dxx, dCC
+
+        Wd = torch.randn(OUT_F, IN_F, device=dev).bfloat16()
+
+        def dense_step():
+            return x @ Wd.t(), dy @ Wd, dy.t() @ x
+
+        compare = {
+            "materialize_then_gemm_ms": round(event_ms(mat_gemm_step, 10), 4),
+            "dense_gemm_only_ms": round(event_ms(dense_step, 20), 4),
+        }
+
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        from oracle import oracle
+
+        oracle.build()
+        torch.set_num_threads(min(os.cpu_count() or 1, 16))
+        os.environ.setdefault("OMP_NUM_THREADS", "16")
+        xc, dyc, Cc = x.float().cpu(), dy.float().cpu(), C.float().cpu().numpy()
+
+        def cpu_step():
+            W = torch.from_numpy(oracle.materialize_fwd(Cc, (OUT_F, IN_F), (IN_F, 1), SEED, row_len=IN_F, acc_double=False))
+            yy = xc @ W.t()
+            W2 = torch.from_numpy(oracle.materialize_fwd(Cc, (OUT_F, IN_F), (IN_F, 1), SEED, row_len=IN_F, acc_double=False))
+            dxx = dyc @ W2
+            dW = dyc.t() @ xc
+            dCC = oracle.materialize_bwd(dW.numpy(), K, SEED, coef_rows=OUT_F)
+            return yy, dxx, dCC
+
+        cpu_step()  # warm-up
+        n_cpu = 3
+        c0 = time.perf_counter()
+        for _ in range(n_cpu):
+            cpu_step()
+        c_ms = (time.perf_counter() - c0) * 1e3 / n_cpu
+        cpu_baseline = {
+            "value": round(F / (c_ms * 1e-3) / 1e12, 5), "unit": "TFLOP/s", "cores": int(oracle.lib().rdbo_num_threads()),
+            "kind": "port", "ms_per_step": round(c_ms, 2),
+            "sample": f"{n_cpu} full fwd+bwd steps of the same workload, fp32: oracle C materialise (OpenMP) + torch.matmul",
+        }
+
+    out = {
+        "metric": "fused PRNG-GEMM fwd+bwd TFLOP/s & % MFMA peak at 768->3072,k=256,8192 tok",
+        "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "single fused layer 768->3072, k=256 matrix-coef, 8192 tokens, bf16 act / fp32 accumulate, fwd+dx+dcoef",
+                   "tokens": T, "in": IN_F, "out": OUT_F, "k": K, "seed": SEED, "algorithmic_gflop_per_step": round(F / 1e9, 3)},
+        "frac_of_mfma_peak": round(value / MFMA_BF16_PEAK_TFLOPS, 5),
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "compare": compare,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -3,6 +3,12 @@
 Python surface mirroring the reference package ``rten_cpp`` (Clyde013/randumb) over hand-written HIP kernels
 reached through the C ABI of ``librandumb_hip.so``.
 """
-from . import _lib, hip  # noqa: F401
+from . import _lib, hip, ops  # noqa: F401
+from .RandumbTensor import CreateRandumbTensor, RandumbTensor, RandumbTensorConstructor, rt_mm  # noqa: F401
+from .SillyLayers import (SillyEmbedding, SillyLinear, SillyModuleMixin, init_coef_normal, init_kaiming_uniform,  # noqa: F401
+                          init_zeros, listgen, stepgen)
 
-__all__ = ["hip"]
+__all__ = [
+    "CreateRandumbTensor", "RandumbTensor", "RandumbTensorConstructor", "rt_mm", "SillyLinear", "SillyEmbedding",
+    "SillyModuleMixin", "init_kaiming_uniform", "init_coef_normal", "init_zeros", "stepgen", "listgen", "ops", "hip",
+]

@@ -1,0 +1,229 @@
+"""``torch.library`` operators of the pseudorandom tensor, same names and argument meaning as the reference's
+``rten::`` ops (src/rten_cpp/RandumbTensor.py:371-448, 1121-1157) and ``rten_cpp::`` ops
+(src/rten_cpp/csrc/rten.cpp:36-39, src/rten_cpp/ops.py:9-13), implemented by the HIP kernels in
+``librandumb_hip.so``.  CPU tensors raise ``NotImplementedError`` as they do in the reference.
+
+Additive to the reference surface:
+* ``materialize_fwd`` accepts a 2-D ``coefs`` (matrix-coef form) and declares ``scale_bias`` optional
+  (the reference types it ``Tensor`` yet documents ``None`` as the default, RandumbTensor.py:993);
+* ``materialize_bwd`` takes an optional ``coef_rows``;
+* ``rten::linear_fwd`` / ``linear_bwd_dx`` / ``linear_bwd_dcoef``: the fused products that never write the
+  weight (or its gradient) to memory.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+from torch import Tensor
+from torch.library import custom_op
+
+from . import hip
+
+__all__ = [
+    "materialize_fwd", "materialize_bwd", "scale_bias_bwd", "embed_fwd", "embed_bwd",
+    "linear_fwd", "linear_bwd_dx", "linear_bwd_dcoef", "sq5_gen_2d", "sq5_gen_1d",
+]
+
+
+# ------------------------------------------------------------------------------------------------ rten::materialize_*
+@custom_op("rten::materialize_fwd", mutates_args=())
+def materialize_fwd(coefs: Tensor, size: List[int], strides: List[int], seed: int, scale_bias: Optional[Tensor],
+                    fused_bias: bool, row_len: int = 0) -> Tensor:
+    return hip.materialize_fwd(coefs, size, strides, seed, scale_bias, fused_bias, row_len if row_len > 0 else None)
+
+
+@materialize_fwd.register_fake
+def _(coefs, size, strides, seed, scale_bias, fused_bias, row_len=0):
+    return coefs.new_empty(list(size), dtype=torch.float32)
+
+
+@custom_op("rten::materialize_bwd", mutates_args=())
+def materialize_bwd(dout: Tensor, dcoefs_size: int, seed: int, coef_rows: int = 0) -> Tensor:
+    return hip.materialize_bwd(dout, dcoefs_size, seed, coef_rows)
+
+
+@materialize_bwd.register_fake
+def _(dout, dcoefs_size, seed, coef_rows=0):
+    shape = [dcoefs_size] if coef_rows == 0 else [coef_rows, dcoefs_size]
+    return dout.new_empty(shape, dtype=torch.float32)
+
+
+@custom_op("rten::scale_bias_bwd", mutates_args=())
+def scale_bias_bwd(dout: Tensor, seed: int) -> Tensor:
+    return hip.scale_bias_bwd(dout, seed)
+
+
+@scale_bias_bwd.register_fake
+def _(dout, seed):
+    return dout.new_empty([1], dtype=torch.float32)
+
+
+def _to_base_layout(grad: Tensor, size, strides) -> Tensor:
+    """Gradient of a strided view scattered back to the storage order the noise rows are numbered in."""
+    size, strides = list(size), list(strides)
+    contiguous = [1] * len(size)
+    for i in range(len(size) - 2, -1, -1):
+        contiguous[i] = contiguous[i + 1] * size[i + 1]
+    if strides == contiguous or grad.numel() == 0:
+        return grad.contiguous().flatten()
+    extent = 1 + sum((s - 1) * st for s, st in zip(size, strides))
+    base = grad.new_zeros(extent)
+    base.as_strided(size, strides).copy_(grad)
+    return base
+
+
+def _mat_setup_context(ctx, inputs, output):
+    coefs, size, strides, seed, scale_bias, fused_bias, row_len = inputs
+    ctx.k = coefs.shape[-1]
+    ctx.coef_rows = 0 if coefs.dim() == 1 else coefs.shape[0]
+    ctx.coef_dtype = coefs.dtype
+    ctx.size, ctx.strides, ctx.seed, ctx.fused_bias = list(size), list(strides), seed, fused_bias
+    ctx.sb_dtype = None if scale_bias is None else scale_bias.dtype
+
+
+def _mat_backward(ctx, grad):
+    # only coefs and scale_bias are differentiable (RandumbTensor.py:423-428)
+    g = _to_base_layout(grad, ctx.size, ctx.strides)
+    dcoefs = materialize_bwd(g, ctx.k, ctx.seed, ctx.coef_rows).to(ctx.coef_dtype)
+    dscale_bias = scale_bias_bwd(g, ctx.seed).to(ctx.sb_dtype) if ctx.fused_bias else None
+    return dcoefs, None, None, None, dscale_bias, None, None
+
+
+materialize_fwd.register_autograd(_mat_backward, setup_context=_mat_setup_context)
+
+
+# ------------------------------------------------------------------------------------------------ rten::embed_*
+@custom_op("rten::embed_fwd", mutates_args=())
+def embed_fwd(idx: Tensor, coefs: Tensor, rowsize: int, seed: int) -> Tensor:
+    return hip.embed_fwd(idx, coefs, rowsize, seed)
+
+
+@embed_fwd.register_fake
+def _(idx, coefs, rowsize, seed):
+    return coefs.new_empty([*idx.shape, rowsize], dtype=torch.float32)
+
+
+@custom_op("rten::embed_bwd", mutates_args=())
+def embed_bwd(idx: Tensor, dout: Tensor, dcoefs_size: int, rowsize: int, seed: int) -> Tensor:
+    return hip.embed_bwd(idx, dout.contiguous(), dcoefs_size, rowsize, seed)
+
+
+@embed_bwd.register_fake
+def _(idx, dout, dcoefs_size, rowsize, seed):
+    return dout.new_empty([dcoefs_size], dtype=torch.float32)
+
+
+def _embed_setup_context(ctx, inputs, output):
+    idx, coefs, rowsize, seed = inputs
+    ctx.save_for_backward(idx)
+    ctx.dcoefs_size, ctx.rowsize, ctx.seed, ctx.coef_dtype = coefs.numel(), rowsize, seed, coefs.dtype
+
+
+def _embed_backward(ctx, grad):
+    (idx,) = ctx.saved_tensors
+    return None, embed_bwd(idx, grad, ctx.dcoefs_size, ctx.rowsize, ctx.seed).to(ctx.coef_dtype), None, None
+
+
+embed_fwd.register_autograd(_embed_backward, setup_context=_embed_setup_context)
+
+
+# ------------------------------------------------------------------------------------------------ rten::linear_*
+@custom_op("rten::linear_fwd", mutates_args=())
+def linear_fwd(x: Tensor, coefs: Tensor, in_features: int, out_features: int, stride_o: int, stride_i: int, seed: int,
+               scale_bias: Optional[Tensor], bias: Optional[Tensor]) -> Tensor:
+    return hip.linear_fwd(x, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias, bias)
+
+
+@linear_fwd.register_fake
+def _(x, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias, bias):
+    return x.new_empty([x.shape[0], out_features])
+
+
+@custom_op("rten::linear_bwd_dx", mutates_args=())
+def linear_bwd_dx(dy: Tensor, coefs: Tensor, in_features: int, out_features: int, stride_o: int, stride_i: int, seed: int,
+                  scale_bias: Optional[Tensor]) -> Tensor:
+    return hip.linear_bwd_dx(dy, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias)
+
+
+@linear_bwd_dx.register_fake
+def _(dy, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias):
+    return dy.new_empty([dy.shape[0], in_features])
+
+
+@custom_op("rten::linear_bwd_dcoef", mutates_args=())
+def linear_bwd_dcoef(dy: Tensor, x: Tensor, dcoefs_size: int, coef_rows: int, in_features: int, out_features: int,
+                     stride_o: int, stride_i: int, seed: int, want_scale_bias_grad: bool) -> List[Tensor]:
+    dcoef, dsb = hip.linear_bwd_dcoef(dy, x, dcoefs_size, coef_rows, in_features, out_features, stride_o, stride_i, seed,
+                                      want_scale_bias_grad)
+    return [dcoef] if dsb is None else [dcoef, dsb]
+
+
+@linear_bwd_dcoef.register_fake
+def _(dy, x, dcoefs_size, coef_rows, in_features, out_features, stride_o, stride_i, seed, want_scale_bias_grad):
+    shape = [dcoefs_size] if coef_rows == 0 else [coef_rows, dcoefs_size]
+    out = [dy.new_empty(shape, dtype=torch.float32)]
+    if want_scale_bias_grad:
+        out.append(dy.new_empty([1], dtype=torch.float32))
+    return out
+
+
+def _lin_setup_context(ctx, inputs, output):
+    x, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias, bias = inputs
+    ctx.save_for_backward(x, coefs, scale_bias)
+    ctx.meta = (in_features, out_features, stride_o, stride_i, seed)
+    ctx.has_bias = bias is not None
+    ctx.bias_dtype = None if bias is None else bias.dtype
+
+
+def _lin_backward(ctx, dy):
+    x, coefs, scale_bias = ctx.saved_tensors
+    in_f, out_f, sO, sI, seed = ctx.meta
+    dy = dy.contiguous()
+    dx = dcoefs = dsb = dbias = None
+    if ctx.needs_input_grad[0]:
+        dx = linear_bwd_dx(dy, coefs, in_f, out_f, sO, sI, seed, scale_bias)
+    want_sb = scale_bias is not None and ctx.needs_input_grad[7]
+    if ctx.needs_input_grad[1] or want_sb:
+        res = linear_bwd_dcoef(dy, x, coefs.shape[-1], 0 if coefs.dim() == 1 else coefs.shape[0], in_f, out_f, sO, sI, seed,
+                               want_sb)
+        dcoefs = res[0].to(coefs.dtype)
+        if want_sb:
+            dsb = res[1].to(scale_bias.dtype)
+    if ctx.has_bias and ctx.needs_input_grad[8]:
+        dbias = dy.sum(0).to(ctx.bias_dtype)
+    return dx, dcoefs, None, None, None, None, None, dsb, dbias
+
+
+linear_fwd.register_autograd(_lin_backward, setup_context=_lin_setup_context)
+
+
+# ------------------------------------------------------------------------------------------------ rten_cpp::*
+@custom_op("rten_cpp::sq5_gen_2d", mutates_args=())
+def _sq5_gen_2d(M: int, N: int, seed: int) -> Tensor:
+    return hip.sq5_fill_2d(M, N, seed)
+
+
+@_sq5_gen_2d.register_fake
+def _(M, N, seed):
+    return torch.empty([M, N], dtype=torch.float32, device="cuda")
+
+
+@custom_op("rten_cpp::materialize_fwd", mutates_args=())
+def _cpp_materialize_fwd(coef: Tensor, seed: int, P: int, Q: int, stride_P: int, stride_Q: int) -> Tensor:
+    assert coef.dim() == 1 and coef.is_contiguous()  # rten.cu:130-131
+    return hip.materialize_fwd(coef, (P, Q), (stride_P, stride_Q), seed, None, False)
+
+
+@_cpp_materialize_fwd.register_fake
+def _(coef, seed, P, Q, stride_P, stride_Q):
+    return coef.new_empty([P, Q], dtype=torch.float32)
+
+
+def sq5_gen_2d(M: int, N: int, seed: int) -> Tensor:
+    """Noise matrix ``(M, N)``; wrapper with the reference's name (src/rten_cpp/ops.py:9-10)."""
+    return torch.ops.rten_cpp.sq5_gen_2d.default(M, N, seed)
+
+
+def sq5_gen_1d(N: int, seed: int) -> Tensor:
+    return hip.sq5_fill_1d(N, seed)

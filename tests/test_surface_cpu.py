@@ -1,0 +1,144 @@
+"""Host-side behaviour of the Python surface that needs no GPU: lazy view ops, constructor contract, layer
+parameter/buffer names, init formulas, seed generators, C-ABI symbol table.  Written from the reference's source
+text (src/rten_cpp/RandumbTensor.py:794-994, src/rten_cpp/SillyLayers.py)."""
+import ctypes
+import math
+import os
+import re
+
+import pytest
+import torch
+
+import randumb_amd as ra
+from randumb_amd import CreateRandumbTensor, RandumbTensor, SillyLinear, listgen, stepgen
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    """The shared library loads without a GPU and exports exactly what include/randumb_hip.h declares."""
+    from randumb_amd import _lib
+
+    hdr = open(os.path.join(ROOT, "include", "randumb_hip.h")).read()
+    declared = set(re.findall(r"\b(rdb_[a-z0-9_]+)\s*\(", hdr))
+    assert declared == set(_lib.EXPORTS), declared ^ set(_lib.EXPORTS)
+    lib = ctypes.CDLL(_lib.SO_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert _lib.load().rdb_abi_version() == 1
+    assert ctypes.sizeof(_lib.LinearDesc) == 7 * 8 + 4 * 4
+
+
+def test_argument_errors_come_back_as_codes_without_a_gpu():
+    from randumb_amd import _lib
+
+    L = _lib.load()
+    assert L.rdb_sq5_fill_2d(None, -1, 4, 0, None) == -2
+    assert b"negative" in L.rdb_last_error_string()
+    assert L.rdb_sq5_fill_2d(None, 4, 4, 0, None) == -1
+    assert L.rdb_sq5_fill_2d(None, 0, 4, 0, None) == 0  # empty: nothing to do, no pointer needed
+    assert L.rdb_materialize_fwd(None, None, 7, 0, 4, 0, 2, 2, 2, 1, 0, None, None) == -3
+    d = _lib.LinearDesc()
+    d.tokens, d.in_f, d.out_f, d.k, d.coef_rows, d.sO, d.sI = 4, 8, 6, 3, 5, 8, 1
+    assert L.rdb_linear_fwd(None, 6, None, 8, None, None, None, ctypes.byref(d), None) == -2  # coef_rows != out_f
+    assert L.rdb_linear_fwd(None, 6, None, 8, None, None, None, None, None) == -1
+    assert L.rdb_materialize_bwd_workspace_bytes(0, 256, 0, 2359296) > 0
+    assert L.rdb_materialize_bwd_workspace_bytes(3072, 256, 768, 2359296) == 0
+
+
+def test_view_ops_stay_lazy_and_only_change_shape_and_stride():
+    c = torch.nn.Parameter(torch.randn(18))
+    rt = CreateRandumbTensor(c, 1337, (3, 6))
+    assert isinstance(rt, RandumbTensor) and rt.shape == (3, 6) and rt.stride() == (6, 1)
+    assert rt.int_dim == 18 and rt.noise_matrix_shape == (18, 18) and rt.seed == 1337 and rt._coef is c
+    t = rt.t()
+    assert isinstance(t, RandumbTensor) and t.shape == (6, 3) and t.stride() == (1, 6) and t._coef is c
+    assert rt.transpose(0, 1).stride() == (1, 6)
+    assert rt.view(6, 3).stride() == (3, 1)
+    assert rt.view(2, 3, 3).permute(2, 0, 1).shape == (3, 2, 3)
+    assert rt.permute(1, 0).stride() == (1, 6)
+    with pytest.raises(RuntimeError, match="view size is not compatible"):
+        rt.t().view(18)
+    b = rt.to(torch.bfloat16)
+    assert isinstance(b, RandumbTensor) and b.dtype == torch.bfloat16 and b._coef is c
+    assert rt._tensor is None
+
+
+def test_constructor_contract():
+    c = torch.nn.Parameter(torch.randn(5))
+    rt = CreateRandumbTensor(c, 3, (4, 2))
+    assert rt.requires_grad and rt.grad_fn is not None and rt.dtype == c.dtype and rt.device == c.device
+    with pytest.raises(AssertionError):
+        CreateRandumbTensor(torch.randn(2, 3, 4), 0, (4, 2))
+    with pytest.raises(AssertionError):  # matrix-coef needs (rows, row_len)
+        CreateRandumbTensor(torch.randn(3, 4), 0, (4, 2))
+    m = CreateRandumbTensor(torch.randn(4, 7), 0, (4, 9))
+    assert m.coef_rows == 4 and m.row_len == 9 and m.noise_matrix_shape == (9, 7)
+    assert m.t().row_len == 9
+    with pytest.raises(NotImplementedError):  # no CPU implementation, as in the reference
+        rt + 1
+
+
+def test_seed_generators():
+    g = stepgen(10, 3)
+    assert [next(g) for _ in range(4)] == [10, 13, 16, 19]
+    assert list(listgen([5, 7, 9])) == [5, 7, 9]
+
+
+def test_silly_linear_surface():
+    ints, seeds = stepgen(64, 0), stepgen(1337, 1)
+    l1 = SillyLinear(784, 256, ints, seeds)
+    l2 = SillyLinear(256, 10, ints, seeds, bias=False)
+    assert l1.seed == [1337, 1338] and l2.seed == [1339, 1340] and l1.int_dim == [64, 64]  # two draws per layer, bias or not
+    assert sorted(n for n, _ in l1.named_parameters()) == ["bias_coef", "bias_scale_bias", "weight_coef", "weight_scale_bias"]
+    assert sorted(n for n, _ in l1.named_buffers()) == ["bias", "weight"]
+    assert sorted(l1.state_dict().keys()) == ["bias", "bias_coef", "bias_scale_bias", "weight", "weight_coef", "weight_scale_bias"]
+    assert l2.bias is None and sorted(n for n, _ in l2.named_parameters()) == ["weight_coef", "weight_scale_bias"]
+    assert l1.weight.shape == (256, 784) and l1.bias.shape == (256,) and l1.weight_coef.shape == (64,)
+    # default init: zero coefficients, scale_bias = sqrt(3) * gain / sqrt(fan_in), gain = sqrt(2 / (1 + 5)) (SillyLayers.py:122-133)
+    assert not l1.weight_coef.any() and not l1.bias_coef.any()
+    want = math.sqrt(3.0) * math.sqrt(1.0 / 3.0) / math.sqrt(784)
+    assert abs(float(l1.weight_scale_bias) - want) < 1e-7 and abs(float(l1.bias_scale_bias) - want) < 1e-7
+    assert l1.weight.scale_bias is l1.weight_scale_bias and l1.weight._coef is l1.weight_coef
+    m = SillyLinear(12, 5, [8, 8], [1, 2], matrix_coef=True)
+    assert m.weight_coef.shape == (5, 8) and m.fused and m.weight.coef_rows == 5
+
+
+def test_apply_rebuilds_tensors_on_the_converted_parameters():
+    l = SillyLinear(12, 5, [8, 8], [1, 2])
+    l = l.to(torch.bfloat16)
+    assert l.weight.dtype == torch.bfloat16 and l.weight._coef is l.weight_coef and l.weight.scale_bias is l.weight_scale_bias
+    assert l.bias._coef is l.bias_coef and isinstance(l.weight, RandumbTensor) and l.weight.requires_grad
+    l = l.float()
+    assert l.weight.dtype == torch.float32 and l.weight._coef is l.weight_coef
+
+
+def test_init_variance_scaling():
+    """var(coef) = 3 * std^2 / k  (uniform bound = 3 * std / sqrt(k)); bias uses the weight's fan-in and its own k."""
+    l = SillyLinear(300, 50, [4096, 1024], [7, 8])
+    ra.init_kaiming_uniform(l.weight, l.bias, 7)
+    out_std = math.sqrt(1.0 / 3.0) / math.sqrt(300)
+    for coef, k in ((l.weight_coef, 4096), (l.bias_coef, 1024)):
+        bound = 3.0 * out_std / math.sqrt(k)
+        assert float(coef.abs().max()) <= bound and float(coef.abs().max()) > 0.97 * bound
+        assert abs(float(coef.var()) / (3 * out_std**2 / k) - 1) < 0.1
+    l2 = SillyLinear(300, 50, [4096, 1024], [7, 8])
+    ra.init_kaiming_uniform(l2.weight, l2.bias, 7)
+    assert torch.equal(l.weight_coef, l2.weight_coef)  # seeded generator: reproducible
+    m = SillyLinear(768, 64, [256, 256], [0, 1], matrix_coef=True, bias=False)
+    ra.init_coef_normal(m.weight, 0.02, 0)
+    assert abs(float(m.weight_coef.var()) / (3 * 0.02**2 / 256) - 1) < 0.05
+    l.init_uniform_coef_zero_bias()
+    assert float(l.weight_scale_bias) == 0.0 and l.weight_coef.any()
+
+
+def test_materialised_weight_has_the_target_std(oracle):
+    """README derivation: with var(coef) = 3 std^2 / k the weight entries have standard deviation std."""
+    g = torch.Generator().manual_seed(0)
+    k, std = 256, 0.02
+    C = torch.randn(64, k, generator=g) * math.sqrt(3 * std**2 / k)
+    W = oracle.materialize_fwd(C.numpy(), (64, 768), (768, 1), 5, row_len=768)
+    assert abs(W.std() / std - 1) < 0.05
+    c = torch.randn(k, generator=g) * math.sqrt(3 * std**2 / k)
+    W1 = oracle.materialize_fwd(c.numpy(), (64, 768), (768, 1), 5)
+    assert abs(W1.std() / std - 1) < 0.1
