@@ -133,7 +133,9 @@ typedef struct rdb_linear_desc {
 
 enum {
     RDB_ALGO_AUTO = 0,
-    RDB_ALGO_TILE = 1 /* regenerate W tiles in LDS, contract with MFMA (general shapes) */
+    RDB_ALGO_TILE = 1, /* regenerate W blocks in LDS per output block, contract with MFMA (any shape/dtype) */
+    RDB_ALGO_STRIP = 2 /* forward only: build a whole strip W[strip, 0:in] in LDS once per workgroup, then stream the
+                          tokens through it (matrix-coef, bf16, strip must fit LDS) */
 };
 
 /* Replaces the dispatch of aten.mm / aten.addmm on a pseudorandom tensor: materialize() then the dense

@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(_HERE, "librandumb_hip.so")
 
 RDB_F32, RDB_BF16 = 0, 1
-RDB_ALGO_AUTO, RDB_ALGO_TILE = 0, 1
+RDB_ALGO_AUTO, RDB_ALGO_TILE, RDB_ALGO_STRIP = 0, 1, 2
 
 # every exported entry point, in header order; tests check the list against the built library
 EXPORTS = [

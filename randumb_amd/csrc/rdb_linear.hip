@@ -254,10 +254,29 @@ static int check_desc(const char *who, const rdb_linear_desc *d)
     if (d->coef_rows != 0 && (d->sO != d->in_f || d->sI != 1))
         return set_error(RDB_E_SHAPE, "%s: matrix-coef needs strides (in_f, 1), got (%lld, %lld)", who, (long long)d->sO, (long long)d->sI);
     if (d->sO < 0 || d->sI < 0) return set_error(RDB_E_SHAPE, "%s: negative weight stride", who);
-    if (d->algo != RDB_ALGO_AUTO && d->algo != RDB_ALGO_TILE) return set_error(RDB_E_UNSUPPORTED, "%s: unknown algo %d", who, d->algo);
+    if (d->algo != RDB_ALGO_AUTO && d->algo != RDB_ALGO_TILE && d->algo != RDB_ALGO_STRIP)
+        return set_error(RDB_E_UNSUPPORTED, "%s: unknown algo %d", who, d->algo);
     if (d->tokens > (1ll << 31) * BM || d->in_f > (1ll << 31) || d->out_f > (1ll << 31))
         return set_error(RDB_E_SHAPE, "%s: dimension too large", who);
     return RDB_OK;
+}
+
+// rdb_strip.hip
+int linear_fwd_strip(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
+                     const rdb_linear_desc *d, int num_cus, hipStream_t s);
+
+// Compute units of the current device (cached per device id).
+static int num_compute_units()
+{
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
 }
 
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
@@ -299,6 +318,14 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
     if (d->tokens == 0 || d->out_f == 0) return RDB_OK;
     if (!y || (!x && d->in_f > 0) || (!coef && d->k > 0)) return set_error(RDB_E_NULL, "rdb_linear_fwd: y, x or coef is NULL");
     if (ldy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_fwd: leading dimension smaller than the row");
+    hipStream_t s = (hipStream_t)stream;
+    if (d->algo != RDB_ALGO_TILE) {
+        rc = linear_fwd_strip(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+        if (d->algo == RDB_ALGO_STRIP)
+            return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd: the strip algorithm needs matrix-coef, bf16 activations, in_f %% 8 == 0, "
+                                                "16-byte aligned x rows and a weight strip that fits LDS");
+    }
     const int es = d->act_dtype == RDB_BF16 ? 2 : 4;
     LinParams p = {};
     p.w = make_spec(d, coef, scale_bias);
@@ -310,7 +337,6 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
     p.tokens = d->tokens;
     p.vec_a = aligned16(x) && (ldx * es) % 16 == 0;
     dim3 grid((unsigned)cdiv(d->out_f, BN), (unsigned)cdiv(d->tokens, BM));
-    hipStream_t s = (hipStream_t)stream;
     const bool mat = d->coef_rows != 0;
     if (d->act_dtype == RDB_BF16)
         return mat ? launch(linear_fwd_kernel<bf16_t, true>, grid, smem_fwd<bf16_t>(), s, p, "linear_fwd_kernel<bf16,matrix>")

@@ -247,3 +247,46 @@ def test_argument_errors(hip):
         hip.sq5_fill_1d(4, -1)
     with pytest.raises(NotImplementedError):
         hip.materialize_fwd(torch.randn(4), (2, 2), (2, 1), 0, None, False)
+
+
+# ------------------------------------------------------------------------------------------------ strip-stationary forward
+STRIP_SHAPES = [
+    # tokens, in_f, out_f, k, seed
+    (1024, 768, 3072, 256, 0),   # full-width slice of the GPT-2 MLP shape (96-row strips)
+    (1000, 768, 200, 256, 3),    # ragged tokens and a ragged last strip
+    (77, 72, 130, 40, 7),        # in_f not a multiple of 64, k not a multiple of 16
+    (4096, 1536, 96, 64, 11),    # 32-row strips (a 64-row strip of 1536 columns does not fit next to nothing else)
+    (33, 8, 5, 3, 1),
+]
+
+
+@pytest.mark.parametrize("T,in_f,out_f,k,seed", STRIP_SHAPES)
+@pytest.mark.parametrize("coef_dtype", [torch.bfloat16, torch.float32])
+def test_linear_fwd_strip_algorithm(hip, oracle, T, in_f, out_f, k, seed, coef_dtype):
+    from randumb_amd._lib import RDB_ALGO_STRIP, RDB_ALGO_TILE
+
+    print(f"case strip T={T} in={in_f} out={out_f} k={k} coef={coef_dtype}", flush=True)
+    x, _, coef = _inputs(T, in_f, out_f, k, True, torch.bfloat16, seed)
+    coef = coef.float().to(coef_dtype)
+    bias = torch.randn(out_f).bfloat16()
+    sb = torch.tensor([0.01]).to(coef_dtype)
+    want = oracle.linear_fwd(x.float().numpy(), coef.float().numpy(), in_f, out_f, seed)
+    got = hip.linear_fwd(x.cuda(), coef.cuda(), in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_STRIP)
+    assert got.shape == (T, out_f) and rel_l2(cpu(got), want) < BF16_TOL
+    ref = hip.linear_fwd(x.cuda(), coef.cuda(), in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_TILE)
+    assert rel_l2(cpu(got), cpu(ref)) < 5e-3  # two on-chip schedules of the same bf16 arithmetic
+    want_b = oracle.linear_fwd(x.float().numpy(), coef.float().numpy(), in_f, out_f, seed, bias=bias.float().numpy(),
+                               scale_bias=float(sb.float()))
+    got_b = hip.linear_fwd(x.cuda(), coef.cuda(), in_f, out_f, in_f, 1, seed, scale_bias=sb.cuda(), bias=bias.cuda(),
+                           algo=RDB_ALGO_STRIP)
+    assert rel_l2(cpu(got_b), want_b) < BF16_TOL
+
+
+def test_strip_algorithm_rejects_what_it_cannot_do(hip):
+    from randumb_amd._lib import RandumbHipError, RDB_ALGO_STRIP
+
+    x = torch.randn(64, 100, device="cuda").bfloat16()   # in_f not a multiple of 8
+    C = torch.randn(32, 16, device="cuda").bfloat16()
+    with pytest.raises(RandumbHipError):
+        hip.linear_fwd(x, C, 100, 32, 100, 1, 0, algo=RDB_ALGO_STRIP)
+    assert hip.linear_fwd(x, C, 100, 32, 100, 1, 0).shape == (64, 32)  # the default falls back to the general kernel
