@@ -265,6 +265,10 @@ static int check_desc(const char *who, const rdb_linear_desc *d)
 int linear_fwd_strip(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
                      const rdb_linear_desc *d, int num_cus, hipStream_t s);
 
+// rdb_dcoef.hip
+int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d,
+                      int num_cus, hipStream_t s);
+
 // Compute units of the current device (cached per device id).
 static int num_compute_units()
 {
@@ -393,6 +397,10 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
     if (d->tokens == 0 || d->in_f == 0 || d->out_f == 0 || (ncoef == 0 && !d_scale_bias)) return RDB_OK;
     if (!dy || !x) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef: dy or x is NULL");
     if (lddy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dcoef: leading dimension smaller than the row");
+    if (d->algo != RDB_ALGO_TILE) {
+        rc = linear_dcoef_fast(dcoef, d_scale_bias, dy, lddy, x, ldx, d, num_compute_units(), s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
     const int es = d->act_dtype == RDB_BF16 ? 2 : 4;
     LinParams p = {};
     p.w = make_spec(d, nullptr, nullptr);

@@ -11,6 +11,7 @@
 //            global memory into MFMA A-operand registers (one chunk of 64 columns ahead of the math) and the W
 //            fragments from LDS.  No LDS writes and no barriers in this phase.
 // W never leaves the chip.  Replaces materialize() + dense product (src/rten_cpp/RandumbTensor.py:942-946, 771-791).
+#include <stdlib.h>
 #include "rdb_tile.hpp"
 
 namespace rdb {
@@ -28,6 +29,8 @@ struct StripParams {
     int coef_dtype;
     int coef_vec;  // 16-byte loads of coef rows allowed
     uint32_t seed;
+    int dbg;
+    long long *dbgp;
 };
 
 union Pack8 {
@@ -35,26 +38,29 @@ union Pack8 {
     uint32_t u[4];
 };
 
-// 8 consecutive coef values C[row, m0 .. m0+7] as bf16 (zero outside the matrix).
-__device__ __forceinline__ bf16x8 load_coef8(const StripParams &p, int row, int m0)
+// 8 consecutive coef values C[row, m0 .. m0+7] as bf16.
+// CMODE 0: bf16 rows, 16-byte aligned, k % 16 == 0.  CMODE 1: fp32 rows, same conditions.  Both read unconditionally:
+// the caller clamps `row` into the matrix (rows past out_f produce weight rows nobody reads).
+// CMODE 2: any layout, element by element, zero outside the matrix.
+template <int CMODE> __device__ __forceinline__ bf16x8 load_coef8(const StripParams &p, int row, int m0)
 {
     Pack8 r;
-    if (row < p.out_f && m0 + 8 <= p.k && p.coef_vec) {
-        if (p.coef_dtype == RDB_BF16) {
-            r.v = *reinterpret_cast<const bf16x8 *>((const bf16_t *)p.coef + (int64_t)row * p.k + m0);
-        } else {
-            const float *c = (const float *)p.coef + (int64_t)row * p.k + m0;
-            const f32x4 a = *reinterpret_cast<const f32x4 *>(c), b = *reinterpret_cast<const f32x4 *>(c + 4);
-            r.u[0] = f32x2_to_bf16x2(a[0], a[1]);
-            r.u[1] = f32x2_to_bf16x2(a[2], a[3]);
-            r.u[2] = f32x2_to_bf16x2(b[0], b[1]);
-            r.u[3] = f32x2_to_bf16x2(b[2], b[3]);
-        }
+    if constexpr (CMODE == 0) {
+        r.v = *reinterpret_cast<const bf16x8 *>((const bf16_t *)p.coef + (int64_t)row * p.k + m0);
+    } else if constexpr (CMODE == 1) {
+        const float *c = (const float *)p.coef + (int64_t)row * p.k + m0;
+        const f32x4 a = *reinterpret_cast<const f32x4 *>(c), b = *reinterpret_cast<const f32x4 *>(c + 4);
+        r.u[0] = f32x2_to_bf16x2(a[0], a[1]);
+        r.u[1] = f32x2_to_bf16x2(a[2], a[3]);
+        r.u[2] = f32x2_to_bf16x2(b[0], b[1]);
+        r.u[3] = f32x2_to_bf16x2(b[2], b[3]);
     } else {
         float f[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-            f[e] = (row < p.out_f && m0 + e < p.k) ? load_as_f32(p.coef, p.coef_dtype, (int64_t)row * p.k + m0 + e) : 0.0f;
+        for (int e = 0; e < 8; ++e) {
+            const float v = load_as_f32(p.coef, p.coef_dtype, (int64_t)row * p.k + (m0 + e < p.k ? m0 + e : 0));
+            f[e] = (m0 + e < p.k) ? v : 0.0f;
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) r.u[e] = f32x2_to_bf16x2(f[2 * e], f[2 * e + 1]);
     }
@@ -65,17 +71,35 @@ __device__ __forceinline__ bf16x8 load_coef8(const StripParams &p, int row, int 
 // `first` is the first-round hash state of (i, m0).
 __device__ __forceinline__ bf16x8 noise_frag(uint32_t first)
 {
+    // the eight hash chains advance in lock step so that consecutive instructions are independent
+    uint32_t b[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] = first + (uint32_t)e * SQ5_N1;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] ^= b[e] >> 9;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] += SQ5_N2;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] ^= b[e] >> 11;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] *= SQ5_N3;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] ^= b[e] >> 13;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] += SQ5_N4;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] ^= b[e] >> 15;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] *= SQ5_N5;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) b[e] ^= b[e] >> 17;
     Pack8 r;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const float a = (float)(int32_t)sq5_tail(first + (uint32_t)(2 * e) * SQ5_N1);
-        const float b = (float)(int32_t)sq5_tail(first + (uint32_t)(2 * e + 1) * SQ5_N1);
-        r.u[e] = f32x2_to_bf16x2(a, b);
-    }
+    for (int e = 0; e < 4; ++e) r.u[e] = f32x2_to_bf16x2((float)(int32_t)b[2 * e], (float)(int32_t)b[2 * e + 1]);
     return r.v;
 }
 
-template <int BO, int MI>
+template <int BO, int MI, int CMODE>
 __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
 {
     constexpr int OB = BO / 32;
@@ -87,41 +111,89 @@ __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
     const int in_pad = p.in_pad;
     const int nib = (in_pad - 8) / 32;  // 32-column blocks of the strip (in_f rounded up to 64)
 
+    long long ts[8];
+    ts[0] = __builtin_readcyclecounter();
     // ------------------------------------------------------------------ phase 1: W strip -> LDS
-    const float sb = p.scale_bias ? load_as_f32(p.scale_bias, p.coef_dtype, 0) : 0.0f;
-    for (int ib = wave; ib < nib; ib += 4) {
-        f32x16 acc[OB];
-#pragma unroll
-        for (int ob = 0; ob < OB; ++ob) acc[ob] = zero16();
-        // lane (r, g) hashes column i = ib*32 + r, coefficients m = kk*16 + g*8 + e
-        uint32_t first = (uint32_t)(ib * 32 + r) * PN1 + (uint32_t)(g * 8) * SQ5_N1 + p.seed;
-        for (int kk = 0; kk < p.k; kk += 16) {
-            bf16x8 cf[OB];
-#pragma unroll
-            for (int ob = 0; ob < OB; ++ob) cf[ob] = load_coef8(p, o0 + ob * 32 + r, kk + g * 8);
-            const bf16x8 nf = noise_frag(first);
-            first += 16u * SQ5_N1;
-#pragma unroll
-            for (int ob = 0; ob < OB; ++ob) acc[ob] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nf, cf[ob], acc[ob], 0, 0, 0);
-        }
-        // acc[ob][j] = 2^31 * W[o = o0 + ob*32 + r][i = ib*32 + 8*(j/4) + 4*g + j%4]
+    {
+        const float sb = p.scale_bias ? load_as_f32(p.scale_bias, p.coef_dtype, 0) : 0.0f;
+        // coef rows of this lane, clamped into the matrix (CMODE 2 zero-fills instead)
+        int crow[OB];
 #pragma unroll
         for (int ob = 0; ob < OB; ++ob) {
-            const int o = ob * 32 + r;
+            const int o = o0 + ob * 32 + r;
+            crow[ob] = o < p.out_f ? o : p.out_f - 1;
+        }
+        const int ksteps = (p.k + 15) / 16;
+        // CMODE 0/1: coef fragments run 4 k-steps ahead of their use in a ring of registers; the ring wraps from the last
+        // k-step of one column block to the first of the next (C does not depend on the column block).
+        constexpr bool RING = CMODE != 2;
+        bf16x8 ring[4][OB];
+        if constexpr (RING) {
 #pragma unroll
-            for (int jq = 0; jq < 4; ++jq) {
-                const int i = ib * 32 + 8 * jq + 4 * g;
-                float v[4];
+            for (int u = 0; u < 4; ++u)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    v[e] = acc[ob][jq * 4 + e] * 4.656612873077392578125e-10f;
-                    if (p.scale_bias && o0 + o < p.out_f) v[e] += sb * noise1d((uint32_t)((o0 + o) * p.in_f + i + e), p.seed);
+                for (int ob = 0; ob < OB; ++ob) ring[u][ob] = load_coef8<CMODE>(p, crow[ob], (u % ksteps) * 16 + g * 8);
+        }
+        for (int ib = wave; ib < ((p.dbg & 4) ? 0 : nib); ib += 4) {
+            f32x16 acc[OB];
+#pragma unroll
+            for (int ob = 0; ob < OB; ++ob) acc[ob] = zero16();
+            // lane (r, g) hashes column i = ib*32 + r, coefficients m = kk*16 + g*8 + e
+            uint32_t first = (uint32_t)(ib * 32 + r) * PN1 + (uint32_t)(g * 8) * SQ5_N1 + p.seed;
+            if constexpr (RING) {
+                for (int ks = 0; ks < ksteps; ks += 4) {  // ksteps % 4 == 0 (checked on the host)
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const bf16x8 nf = noise_frag(first);
+                        first += 16u * SQ5_N1;
+#pragma unroll
+                        for (int ob = 0; ob < OB; ++ob)
+                            acc[ob] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nf, ring[u][ob], acc[ob], 0, 0, 0);
+                        int nxt = ks + u + 4;
+                        if (nxt >= ksteps) nxt -= ksteps;
+#pragma unroll
+                        for (int ob = 0; ob < OB; ++ob) ring[u][ob] = load_coef8<CMODE>(p, crow[ob], nxt * 16 + g * 8);
+                    }
                 }
-                store4<bf16_t>(Wl + o * in_pad + i, v[0], v[1], v[2], v[3]);
+            } else {
+                for (int ks = 0; ks < ksteps; ++ks) {
+                    bf16x8 cf[OB];
+#pragma unroll
+                    for (int ob = 0; ob < OB; ++ob) {
+                        cf[ob] = load_coef8<2>(p, crow[ob], ks * 16 + g * 8);
+                        if (o0 + ob * 32 + r >= p.out_f) {
+                            Pack8 z;
+                            z.u[0] = z.u[1] = z.u[2] = z.u[3] = 0u;
+                            cf[ob] = z.v;
+                        }
+                    }
+                    const bf16x8 nf = noise_frag(first);
+                    first += 16u * SQ5_N1;
+#pragma unroll
+                    for (int ob = 0; ob < OB; ++ob) acc[ob] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(nf, cf[ob], acc[ob], 0, 0, 0);
+                }
+            }
+            // acc[ob][j] = 2^31 * W[o = o0 + ob*32 + r][i = ib*32 + 8*(j/4) + 4*g + j%4]
+#pragma unroll
+            for (int ob = 0; ob < OB; ++ob) {
+                const int o = ob * 32 + r;
+#pragma unroll
+                for (int jq = 0; jq < 4; ++jq) {
+                    const int i = ib * 32 + 8 * jq + 4 * g;
+                    float v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[e] = acc[ob][jq * 4 + e] * 4.656612873077392578125e-10f;
+                        if (p.scale_bias) v[e] += sb * noise1d((uint32_t)(crow[ob] * p.in_f + i + e), p.seed);
+                    }
+                    store4<bf16_t>(Wl + o * in_pad + i, v[0], v[1], v[2], v[3]);
+                }
             }
         }
     }
+    ts[1] = __builtin_readcyclecounter();
     __syncthreads();
+    ts[2] = __builtin_readcyclecounter();
 
     // ------------------------------------------------------------------ phase 2: stream tokens
     // token blocks of 32 rows: this block's range, then this wave's share of it
@@ -131,6 +203,7 @@ __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
     const int w_lo = rb_lo + wave * per_wave;
     const int w_hi = (w_lo + per_wave < rb_hi) ? w_lo + per_wave : rb_hi;
     const int nchunk = (in_pad - 8) / 64;
+    const int nfull = p.in_f / 64;  // chunks that need no column mask
 
     for (int rb = w_lo; rb < w_hi; rb += MI) {
         // row pointers; rows past the end re-read the last valid row and are never stored
@@ -139,6 +212,7 @@ __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
         for (int mi = 0; mi < MI; ++mi) {
             int row = (rb + mi) * 32 + r;
             if (rb + mi >= w_hi || row >= p.tokens) row = p.tokens - 1;
+            if (p.dbg & 1) row = row & 7;
             xrow[mi] = p.x + (int64_t)row * p.ldx + g * 32;
         }
         f32x16 acc[MI][OB];
@@ -150,20 +224,12 @@ __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
         // within a chunk of 64 columns, k-step j of lane group g covers columns g*32 + j*8 .. +7 (for x and W alike),
         // so a lane's four fragments are 64 contiguous bytes of its row
         bf16x8 xa[2][MI][4];
-        auto load_x = [&](int buf, int c) {
+        auto load_x = [&](int buf, int c) {  // chunk c lies entirely inside the row
+            if (p.dbg & 8) return;
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int col = c * 64 + g * 32 + j * 8;
-                    if (col < p.in_f) {
-                        xa[buf][mi][j] = *reinterpret_cast<const bf16x8 *>(xrow[mi] + c * 64 + j * 8);
-                    } else {
-                        Pack8 z;
-                        z.u[0] = z.u[1] = z.u[2] = z.u[3] = 0u;
-                        xa[buf][mi][j] = z.v;
-                    }
-                }
+                for (int j = 0; j < 4; ++j) xa[buf][mi][j] = *reinterpret_cast<const bf16x8 *>(xrow[mi] + c * 64 + j * 8);
         };
         auto compute = [&](int buf, int c) {
             const bf16_t *wbase = Wl + r * in_pad + c * 64 + g * 32;
@@ -179,16 +245,45 @@ __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
                         acc[mi][ob] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa[buf][mi][j], wb[ob], acc[mi][ob], 0, 0, 0);
             }
         };
-        load_x(0, 0);
-        int c = 0;
-        for (; c + 2 <= nchunk; c += 2) {
-            load_x(1, c + 1);
-            compute(0, c);
-            if (c + 2 < nchunk) load_x(0, c + 2);
-            compute(1, c + 1);
+        // full chunks, two per trip: the loads of one chunk are in flight while the other is multiplied.  The loop body has
+        // no data-dependent branch (the last prefetch re-reads a valid chunk), which keeps the load/use distance visible to
+        // the compiler's wait-count insertion.
+        if (nfull > 0) {
+            load_x(0, 0);
+            int c = 0;
+            for (; c + 2 <= nfull; c += 2) {
+                load_x(1, c + 1);
+                __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the math it overlaps with
+                compute(0, c);
+                __builtin_amdgcn_sched_barrier(0);
+                load_x(0, c + 2 < nfull ? c + 2 : nfull - 1);
+                __builtin_amdgcn_sched_barrier(0);
+                compute(1, c + 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (c < nfull) compute(0, c);
         }
-        if (c < nchunk) compute(0, c);
+        if (nchunk > nfull) {
+            // ragged last chunk: read a valid segment of the same row, then select zero (in_f % 8 == 0)
+            const int c = nfull;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int col = c * 64 + g * 32 + j * 8;
+                const bool ok = col < p.in_f;
+                const int off = ok ? c * 64 + j * 8 : -g * 32;
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi) {
+                    Pack8 v;
+                    v.v = *reinterpret_cast<const bf16x8 *>(xrow[mi] + off);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v.u[e] = ok ? v.u[e] : 0u;
+                    xa[1][mi][j] = v.v;
+                }
+            }
+            compute(1, c);
+        }
 
+        ts[3] = __builtin_readcyclecounter();
         // store: acc[mi][ob][j] = y[row = (rb+mi)*32 + 8*(j/4) + 4*g + j%4][o = o0 + ob*32 + r]
 #pragma unroll
         for (int ob = 0; ob < OB; ++ob) {
@@ -205,20 +300,35 @@ __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
                 }
             }
         }
+        ts[4] = __builtin_readcyclecounter();
+        if (p.dbgp && lane == 0 && blockIdx.x < 8) {
+            long long *d = p.dbgp + (blockIdx.x * 4 + wave) * 16 + (rb == w_lo ? 0 : 8);
+            d[0] = ts[0]; d[1] = ts[1]; d[2] = ts[2]; d[3] = ts[3]; d[4] = ts[4]; d[5] = rb; d[6] = w_hi;
+        }
+        ts[2] = ts[4];
     }
 }
 
 // LDS budget of gfx950 (160 KiB per workgroup).
 constexpr int LDS_BYTES = 160 * 1024;
 
-template <int BO> static int launch_strip(const StripParams &p, int strips, hipStream_t s)
+template <int BO, int CMODE> static int launch_strip_mode(const StripParams &p, int strips, hipStream_t s)
 {
     const size_t smem = (size_t)BO * p.in_pad * sizeof(bf16_t);
-    auto kern = linear_fwd_strip_kernel<BO, 4>;
+    auto kern = linear_fwd_strip_kernel<BO, 4, CMODE>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return set_error((int)e, "linear_fwd_strip_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
     kern<<<strips * p.splits, 256, smem, s>>>(p);
     return check_launch("linear_fwd_strip_kernel");
+}
+
+template <int BO> static int launch_strip(const StripParams &p, int strips, hipStream_t s)
+{
+    // fast coef paths need aligned rows and whole groups of four 16-wide k-steps
+    const bool fast = p.coef_vec && p.k % 64 == 0;
+    if (fast && p.coef_dtype == RDB_BF16) return launch_strip_mode<BO, 0>(p, strips, s);
+    if (fast && p.coef_dtype == RDB_F32) return launch_strip_mode<BO, 1>(p, strips, s);
+    return launch_strip_mode<BO, 2>(p, strips, s);
 }
 
 // Returns RDB_E_UNSUPPORTED (without setting an error) when the shape does not fit this algorithm.
@@ -245,6 +355,8 @@ int linear_fwd_strip(void *y, int64_t ldy, const void *x, int64_t ldx, const voi
     const int ces = d->coef_dtype == RDB_BF16 ? 2 : 4;
     p.coef_vec = (((uintptr_t)coef & 15) == 0) && ((d->k * ces) % 16 == 0);
     p.seed = d->seed;
+    p.dbg = getenv("RDB_DEBUG") ? atoi(getenv("RDB_DEBUG")) : 0;
+    p.dbgp = getenv("RDB_DBGP") ? (long long *)strtoull(getenv("RDB_DBGP"), nullptr, 0) : nullptr;
     // widest strip that fits LDS; narrower strips when that leaves compute units idle
     int bo = 0;
     for (int cand : {96, 64, 32}) {
