@@ -77,14 +77,20 @@ def main():
     stream = vp(torch.cuda.current_stream().cuda_stream)
     px, pdy, pC, py, pdx, pdC = (vp(t.data_ptr()) for t in (x, dy, C, y, dx, dC))
 
+    # caller-owned scratch, sized by the library (nothing is allocated inside the timed region)
+    ws_bytes = max(L.rdb_linear_workspace_bytes(op, dref) for op in (_lib.RDB_OP_LINEAR_FWD, _lib.RDB_OP_LINEAR_BWD_DX,
+                                                                     _lib.RDB_OP_LINEAR_BWD_DCOEF))
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    pws = vp(ws.data_ptr())
+
     def k_fwd():
-        _lib.check(L.rdb_linear_fwd(py, OUT_F, px, IN_F, pC, None, None, dref, stream), "rdb_linear_fwd")
+        _lib.check(L.rdb_linear_fwd(py, OUT_F, px, IN_F, pC, None, None, dref, pws, ws_bytes, stream), "rdb_linear_fwd")
 
     def k_dx():
-        _lib.check(L.rdb_linear_bwd_dx(pdx, IN_F, pdy, OUT_F, pC, None, dref, stream), "rdb_linear_bwd_dx")
+        _lib.check(L.rdb_linear_bwd_dx(pdx, IN_F, pdy, OUT_F, pC, None, dref, pws, ws_bytes, stream), "rdb_linear_bwd_dx")
 
     def k_dcoef():
-        _lib.check(L.rdb_linear_bwd_dcoef(pdC, None, pdy, OUT_F, px, IN_F, dref, stream), "rdb_linear_bwd_dcoef")
+        _lib.check(L.rdb_linear_bwd_dcoef(pdC, None, pdy, OUT_F, px, IN_F, dref, pws, ws_bytes, stream), "rdb_linear_bwd_dcoef")
 
     def step():
         k_fwd()

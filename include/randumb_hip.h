@@ -132,22 +132,32 @@ typedef struct rdb_linear_desc {
 } rdb_linear_desc;
 
 enum {
-    RDB_ALGO_AUTO = 0,
+    RDB_ALGO_AUTO = 0, /* fastest kernel the request qualifies for */
     RDB_ALGO_TILE = 1, /* regenerate W blocks in LDS per output block, contract with MFMA (any shape/dtype) */
-    RDB_ALGO_STRIP = 2 /* forward only: build a whole strip W[strip, 0:in] in LDS once per workgroup, then stream the
-                          tokens through it (matrix-coef, bf16, strip must fit LDS) */
+    RDB_ALGO_STRIP = 2, /* forward only: build a whole strip W[strip, 0:in] in LDS once per workgroup, then stream the
+                           tokens through it (matrix-coef, bf16, strip must fit LDS) */
+    RDB_ALGO_FACTORED = 3 /* matrix-coef only: use W = C.N associatively, e.g. dx = (dy.C).N, so that no weight tile is
+                             formed at all; the [tokens x k] intermediate lives in the caller's workspace */
 };
+
+enum { RDB_OP_LINEAR_FWD = 0, RDB_OP_LINEAR_BWD_DX = 1, RDB_OP_LINEAR_BWD_DCOEF = 2 };
+
+/* Device scratch (bytes) that entry point `op` can use for `desc`; 0 when it has no use for any.  A NULL or too small
+ * workspace is never an error with RDB_ALGO_AUTO: the library then runs a kernel that needs none. */
+int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *desc);
 
 /* Replaces the dispatch of aten.mm / aten.addmm on a pseudorandom tensor: materialize() then the dense
  * product fakeMM (R.py:771-791, 942-952), and the experimental rt_mm (R.py:457-645).
  * y[t, o] = sum_i x[t, i] * W[o, i]  (+ bias[o] if bias != NULL; bias has act_dtype). */
 int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef,
-                   const void *scale_bias, const void *bias, const rdb_linear_desc *desc, void *stream);
+                   const void *scale_bias, const void *bias, const rdb_linear_desc *desc, void *workspace,
+                   int64_t workspace_bytes, void *stream);
 
 /* Replaces autograd's MmBackward on the materialised weight (second materialize() + dense product).
  * dx[t, i] = sum_o dy[t, o] * W[o, i]. */
 int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef,
-                      const void *scale_bias, const rdb_linear_desc *desc, void *stream);
+                      const void *scale_bias, const rdb_linear_desc *desc, void *workspace,
+                      int64_t workspace_bytes, void *stream);
 
 /* Replaces MmBackward's dW = dy^T x followed by RandumbTensorConstructor.backward ->
  * materialize_bwd (+ scale_bias_bwd) (R.py:979-990): dW is contracted with the regenerated noise tile
@@ -156,7 +166,8 @@ int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t lddy, cons
  * OVERWRITTEN.  Partial sums from different tiles are combined with fp32 atomics (order-dependent in
  * the last bits, like the reference's relaxed atomics, R.py:359). */
 int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const void *dy, int64_t lddy, const void *x,
-                         int64_t ldx, const rdb_linear_desc *desc, void *stream);
+                         int64_t ldx, const rdb_linear_desc *desc, void *workspace, int64_t workspace_bytes,
+                         void *stream);
 
 #ifdef __cplusplus
 }

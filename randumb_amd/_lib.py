@@ -13,7 +13,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(_HERE, "librandumb_hip.so")
 
 RDB_F32, RDB_BF16 = 0, 1
-RDB_ALGO_AUTO, RDB_ALGO_TILE, RDB_ALGO_STRIP = 0, 1, 2
+RDB_ALGO_AUTO, RDB_ALGO_TILE, RDB_ALGO_STRIP, RDB_ALGO_FACTORED = 0, 1, 2, 3
+RDB_OP_LINEAR_FWD, RDB_OP_LINEAR_BWD_DX, RDB_OP_LINEAR_BWD_DCOEF = 0, 1, 2
 
 # every exported entry point, in header order; tests check the list against the built library
 EXPORTS = [
@@ -29,6 +30,7 @@ EXPORTS = [
     "rdb_embed_fwd",
     "rdb_embed_bwd",
     "rdb_embed_bwd_workspace_bytes",
+    "rdb_linear_workspace_bytes",
     "rdb_linear_fwd",
     "rdb_linear_bwd_dx",
     "rdb_linear_bwd_dcoef",
@@ -90,9 +92,11 @@ def load() -> ctypes.CDLL:
     L.rdb_embed_bwd_workspace_bytes.argtypes = [i64, i64, i64]
     L.rdb_embed_bwd_workspace_bytes.restype = i64
     dp = ctypes.POINTER(LinearDesc)
-    L.rdb_linear_fwd.argtypes = [vp, i64, vp, i64, vp, vp, vp, dp, vp]
-    L.rdb_linear_bwd_dx.argtypes = [vp, i64, vp, i64, vp, vp, dp, vp]
-    L.rdb_linear_bwd_dcoef.argtypes = [vp, vp, vp, i64, vp, i64, dp, vp]
+    L.rdb_linear_workspace_bytes.argtypes = [ci, dp]
+    L.rdb_linear_workspace_bytes.restype = i64
+    L.rdb_linear_fwd.argtypes = [vp, i64, vp, i64, vp, vp, vp, dp, vp, i64, vp]
+    L.rdb_linear_bwd_dx.argtypes = [vp, i64, vp, i64, vp, vp, dp, vp, i64, vp]
+    L.rdb_linear_bwd_dcoef.argtypes = [vp, vp, vp, i64, vp, i64, dp, vp, i64, vp]
     for name in ("rdb_sq5_fill_2d", "rdb_sq5_fill_1d", "rdb_materialize_fwd", "rdb_materialize_bwd", "rdb_scale_bias_bwd",
                  "rdb_embed_fwd", "rdb_embed_bwd", "rdb_linear_fwd", "rdb_linear_bwd_dx", "rdb_linear_bwd_dcoef"):
         getattr(L, name).restype = ci

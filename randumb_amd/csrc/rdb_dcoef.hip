@@ -41,8 +41,9 @@ __global__ __launch_bounds__(256, 1) void linear_dcoef_fast_kernel(DcoefParams p
     for (int mi = 0; mi < DC_BI / 64; ++mi)
 #pragma unroll
         for (int ni = 0; ni < DC_BO / 64; ++ni) acc[mi][ni] = zero16();
-    gemm_mainloop<DC_BI, DC_BO, DC_BK, M_CONT, M_CONT>(acc, lds, p.x, p.ldx, i0, p.in_f, p.dy, p.lddy, o0, p.out_f, t_begin, t_end,
-                                                       p.tokens);
+    const GlobalOperand<DC_BI, DC_BK, M_CONT> opx = {p.x, p.ldx, i0, p.in_f, t_end};
+    const GlobalOperand<DC_BO, DC_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end};
+    gemm_mainloop<DC_BI, DC_BO, DC_BK>(acc, lds, opx, opdy, t_begin, (t_end - t_begin + DC_BK - 1) / DC_BK);
 
     // dW tile -> LDS as Ws[o][i] (bf16, i contiguous).  acc[mi][ni][j]: i = wm*96 + mi*32 + 8*(j/4) + 4*g + j%4, o = wn*96 + ni*32 + r
     constexpr int LDW = DC_BI + 8;

@@ -1,0 +1,170 @@
+// Input gradient of the fused linear layer, matrix-coef + bf16, "factored" algorithm:
+//
+//   dx = dy . W = dy . (C . N) = (dy . C) . N
+//
+// With k < in*out/(in+out) the right-hand grouping needs 2*T*k*(out+in) flops instead of 2*T*out*in + 2*out*in*k and
+// forms no weight tile at all.  Two kernels on the tile engine:
+//   1. t[tok, m] = sum_o dy[tok, o] * C[o, m]            (dense; t is a bf16 [tokens x k] scratch in the workspace)
+//   2. dx[tok, i] = sum_m t[tok, m] * noise(PRIME*i + m)  (the noise operand is hashed straight into the pipeline's
+//                                                          registers, stage by stage, interleaved with the MFMAs)
+// Replaces autograd's MmBackward on the re-materialised weight (materialize() + dense product,
+// src/rten_cpp/RandumbTensor.py:942-946).
+#include "rdb_gemm.hpp"
+#include "rdb_tile.hpp"
+
+namespace rdb {
+
+// ----------------------------------------------------------------------------------------------- kernel 1: t = dy . C
+// tile: 128 coefficient columns (engine rows "m") x 128 tokens (engine rows "n"), contraction over out_f
+constexpr int K1_BC = 128, K1_BT = 128, K1_BK = 64;
+
+struct DyCParams {
+    const bf16_t *dy;
+    const bf16_t *coef;
+    bf16_t *t;
+    int64_t lddy;
+    int tokens, out_f, k;
+};
+
+__global__ __launch_bounds__(256, 1) void dx_dyc_kernel(DyCParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.x * K1_BC, tok0 = blockIdx.y * K1_BT;
+    f32x16 acc[K1_BC / 64][K1_BT / 64];
+#pragma unroll
+    for (int mi = 0; mi < K1_BC / 64; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < K1_BT / 64; ++ni) acc[mi][ni] = zero16();
+    // "A": C[o][m], tile rows = m (contiguous in memory), contraction index = o
+    const GlobalOperand<K1_BC, K1_BK, M_CONT> opc = {p.coef, (int64_t)p.k, m0, p.k, p.out_f};
+    // "B": dy[tok][o], contraction index contiguous
+    const GlobalOperand<K1_BT, K1_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f};
+    gemm_mainloop<K1_BC, K1_BT, K1_BK>(acc, lds, opc, opdy, 0, (p.out_f + K1_BK - 1) / K1_BK);
+    // acc[mi][ni][j]: m = m0 + wm*64 + mi*32 + 8*(j/4) + 4*g + j%4, tok = tok0 + wn*64 + ni*32 + r
+#pragma unroll
+    for (int ni = 0; ni < K1_BT / 64; ++ni) {
+        const int tok = tok0 + wn * 64 + ni * 32 + r;
+        if (tok >= p.tokens) continue;
+#pragma unroll
+        for (int mi = 0; mi < K1_BC / 64; ++mi)
+#pragma unroll
+            for (int jq = 0; jq < 4; ++jq) {
+                const int m = m0 + wm * 64 + mi * 32 + 8 * jq + 4 * g;
+                if (m < p.k)  // k % 8 == 0, so four consecutive coefficients are inside together
+                    store4<bf16_t>(p.t + (int64_t)tok * p.k + m, acc[mi][ni][jq * 4 + 0], acc[mi][ni][jq * 4 + 1],
+                                   acc[mi][ni][jq * 4 + 2], acc[mi][ni][jq * 4 + 3]);
+            }
+    }
+}
+
+// ----------------------------------------------------------------------------------------------- kernel 2: dx = t . N
+// tile: 192 input features (engine rows "m", hashed operand) x 128 tokens (engine rows "n"), contraction over k
+constexpr int K2_BI = 192, K2_BT = 128, K2_BK = 64;
+
+struct TNParams {
+    const bf16_t *t;
+    bf16_t *dx;
+    int64_t lddx;
+    int tokens, in_f, k;
+    uint32_t seed;
+};
+
+__global__ __launch_bounds__(256, 1) void dx_tn_kernel(TNParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
+    const int i0 = blockIdx.x * K2_BI, tok0 = blockIdx.y * K2_BT;
+    f32x16 acc[K2_BI / 64][K2_BT / 64];
+#pragma unroll
+    for (int mi = 0; mi < K2_BI / 64; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < K2_BT / 64; ++ni) acc[mi][ni] = zero16();
+    // "A": 2^31 * noise(i, m), rows = i, contraction = m; values for m >= k meet zero rows of t
+    const NoiseOperandRowsAreElements<K2_BI, K2_BK> opn = {i0, p.seed};
+    // "B": t[tok][m]
+    const GlobalOperand<K2_BT, K2_BK, K_CONT> opt = {p.t, (int64_t)p.k, tok0, p.tokens, p.k};
+    gemm_mainloop<K2_BI, K2_BT, K2_BK>(acc, lds, opn, opt, 0, (p.k + K2_BK - 1) / K2_BK);
+    // acc[mi][ni][j]: i = i0 + wm*96 + mi*32 + 8*(j/4) + 4*g + j%4, tok = tok0 + wn*64 + ni*32 + r
+#pragma unroll
+    for (int ni = 0; ni < K2_BT / 64; ++ni) {
+        const int tok = tok0 + wn * 64 + ni * 32 + r;
+        if (tok >= p.tokens) continue;
+#pragma unroll
+        for (int mi = 0; mi < K2_BI / 64; ++mi)
+#pragma unroll
+            for (int jq = 0; jq < 4; ++jq) {
+                const int i = i0 + wm * 96 + mi * 32 + 8 * jq + 4 * g;
+                if (i < p.in_f) {  // in_f % 8 == 0
+                    const float sc = 4.656612873077392578125e-10f;
+                    store4<bf16_t>(p.dx + (int64_t)tok * p.lddx + i, acc[mi][ni][jq * 4 + 0] * sc, acc[mi][ni][jq * 4 + 1] * sc,
+                                   acc[mi][ni][jq * 4 + 2] * sc, acc[mi][ni][jq * 4 + 3] * sc);
+                }
+            }
+    }
+}
+
+// ----------------------------------------------------------------------------------------------- host side
+static bool dx_factored_ok(const rdb_linear_desc *d)
+{
+    return d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16 && d->coef_rows != 0 && d->k % 8 == 0 && d->in_f % 8 == 0 &&
+           d->out_f % 8 == 0 && d->k > 0 && d->tokens > 0 && d->tokens < (1 << 30) && d->in_f < (1 << 30) && d->out_f < (1 << 30) &&
+           d->k < (1 << 24);
+}
+
+int64_t linear_dx_factored_workspace(const rdb_linear_desc *d)
+{
+    if (!dx_factored_ok(d)) return 0;
+    return d->tokens * d->k * (int64_t)sizeof(bf16_t);
+}
+
+// Returns RDB_E_UNSUPPORTED (without setting an error) when the request does not fit this algorithm.
+int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias,
+                       const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s)
+{
+    if (!dx_factored_ok(d) || scale_bias) return RDB_E_UNSUPPORTED;  // the random-bias term is not low rank
+    if (!workspace || workspace_bytes < linear_dx_factored_workspace(d) || ((uintptr_t)workspace & 15)) return RDB_E_UNSUPPORTED;
+    if (lddy % 8 || lddx % 4 || ((uintptr_t)dy & 15) || ((uintptr_t)coef & 15) || ((uintptr_t)dx & 7)) return RDB_E_UNSUPPORTED;
+    // only worth it when the factored form is cheaper than forming the weight
+    if (d->algo == RDB_ALGO_AUTO && d->k * (d->in_f + d->out_f) >= d->in_f * d->out_f) return RDB_E_UNSUPPORTED;
+
+    DyCParams p1;
+    p1.dy = (const bf16_t *)dy;
+    p1.coef = (const bf16_t *)coef;
+    p1.t = (bf16_t *)workspace;
+    p1.lddy = lddy;
+    p1.tokens = (int)d->tokens;
+    p1.out_f = (int)d->out_f;
+    p1.k = (int)d->k;
+    {
+        typedef OperandTile<K1_BC, K1_BK, M_CONT> TA;
+        typedef OperandTile<K1_BT, K1_BK, K_CONT> TB;
+        const size_t smem = 2 * (TA::LDS_ELEMS + TB::LDS_ELEMS) * sizeof(bf16_t);
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(dx_dyc_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return set_error((int)e, "dx_dyc_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+        dx_dyc_kernel<<<dim3((unsigned)cdiv(d->k, K1_BC), (unsigned)cdiv(d->tokens, K1_BT)), 256, smem, s>>>(p1);
+        int rc = check_launch("dx_dyc_kernel");
+        if (rc) return rc;
+    }
+    TNParams p2;
+    p2.t = (const bf16_t *)workspace;
+    p2.dx = (bf16_t *)dx;
+    p2.lddx = lddx;
+    p2.tokens = (int)d->tokens;
+    p2.in_f = (int)d->in_f;
+    p2.k = (int)d->k;
+    p2.seed = d->seed;
+    {
+        typedef OperandTile<K2_BI, K2_BK, K_CONT> TA;
+        typedef OperandTile<K2_BT, K2_BK, K_CONT> TB;
+        const size_t smem = 2 * (TA::LDS_ELEMS + TB::LDS_ELEMS) * sizeof(bf16_t);
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(dx_tn_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return set_error((int)e, "dx_tn_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+        dx_tn_kernel<<<dim3((unsigned)cdiv(d->in_f, K2_BI), (unsigned)cdiv(d->tokens, K2_BT)), 256, smem, s>>>(p2);
+        return check_launch("dx_tn_kernel");
+    }
+}
+
+}  // namespace rdb

@@ -119,38 +119,97 @@ __device__ __forceinline__ void mma_stage(f32x16 (&acc)[MI][NI], const bf16_t *_
     }
 }
 
-// Main loop of the tile engine over k in [k_begin, k_end).  `lds` must hold 2 * (TA::LDS_ELEMS + TB::LDS_ELEMS) elements.
-// a_row0 / b_row0: first tile rows; a_rows / b_rows: matrix extents along the tile-row axes; nk: matrix extent along k.
-template <int BM, int BN, int BK, int LA, int LB>
-__device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / 64][BN / 64], bf16_t *__restrict__ lds, const bf16_t *__restrict__ A,
-                                              int64_t lda, int a_row0, int a_rows, const bf16_t *__restrict__ B, int64_t ldb, int b_row0,
-                                              int b_rows, int k_begin, int k_end, int nk)
+// ----------------------------------------------------------------------------------------------- operand providers
+// A provider fills the registers of one pipeline stage: load(regs, k0) with k0 the stage's first contraction index.
+
+// Operand read from global memory.
+template <int ROWS, int BK, int LAYOUT> struct GlobalOperand {
+    typedef OperandTile<ROWS, BK, LAYOUT> Tile;
+    const bf16_t *src;
+    int64_t ld;
+    int row0, nrows, klim;  // klim: first contraction index that must read as zero
+    __device__ __forceinline__ void load(f32x4 (&regs)[Tile::PER_THREAD], int k0) const { Tile::load(regs, src, ld, row0, nrows, k0, klim); }
+};
+
+// Operand generated by the noise hash, tile rows = noise rows (tensor element index), contraction = coefficient index:
+// element (row, k) = 2^31 * noise(PRIME*(row0 + row) + k) as bf16 (callers fold the 2^-31 into their epilogue).
+template <int ROWS, int BK> struct NoiseOperandRowsAreElements {
+    typedef OperandTile<ROWS, BK, K_CONT> Tile;
+    int row0;
+    uint32_t seed;
+    __device__ __forceinline__ void load(f32x4 (&regs)[Tile::PER_THREAD], int k0) const
+    {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int p = 0; p < Tile::PER_THREAD; ++p) {
+            const int idx = p * 256 + t;
+            const int row = row0 + idx / (BK / 8), k = k0 + (idx % (BK / 8)) * 8;
+            const uint32_t first = (uint32_t)row * PN1 + (uint32_t)k * SQ5_N1 + seed;
+            uint32_t b[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) b[e] = sq5_tail(first + (uint32_t)e * SQ5_N1);
+            Frag8 f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) f.u[e] = f32x2_to_bf16x2((float)(int32_t)b[2 * e], (float)(int32_t)b[2 * e + 1]);
+            regs[p] = f.f4;
+        }
+    }
+};
+
+// Same noise, tile rows = coefficient index, contraction = element index: element (row, k) = 2^31 * noise(PRIME*k + row0 + row).
+template <int ROWS, int BK> struct NoiseOperandRowsAreCoefs {
+    typedef OperandTile<ROWS, BK, K_CONT> Tile;
+    int row0;
+    uint32_t seed;
+    __device__ __forceinline__ void load(f32x4 (&regs)[Tile::PER_THREAD], int k0) const
+    {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int p = 0; p < Tile::PER_THREAD; ++p) {
+            const int idx = p * 256 + t;
+            const int row = row0 + idx / (BK / 8), k = k0 + (idx % (BK / 8)) * 8;
+            const uint32_t first = (uint32_t)k * PN1 + (uint32_t)row * SQ5_N1 + seed;
+            uint32_t b[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) b[e] = sq5_tail(first + (uint32_t)e * PN1);
+            Frag8 f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) f.u[e] = f32x2_to_bf16x2((float)(int32_t)b[2 * e], (float)(int32_t)b[2 * e + 1]);
+            regs[p] = f.f4;
+        }
+    }
+};
+
+// Main loop of the tile engine over `nstage` stages of BK starting at contraction index k_begin.
+// `lds` must hold 2 * (PA::Tile::LDS_ELEMS + PB::Tile::LDS_ELEMS) elements.  On return every wave has passed a barrier
+// after its last LDS read, so the caller may reuse `lds` at once.
+template <int BM, int BN, int BK, class PA, class PB>
+__device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / 64][BN / 64], bf16_t *__restrict__ lds, const PA &pa, const PB &pb,
+                                              int k_begin, int nstage)
 {
-    typedef OperandTile<BM, BK, LA> TA;
-    typedef OperandTile<BN, BK, LB> TB;
+    typedef typename PA::Tile TA;
+    typedef typename PB::Tile TB;
     constexpr int MI = BM / 64, NI = BN / 64;
     constexpr int STAGE = TA::LDS_ELEMS + TB::LDS_ELEMS;
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, wm = wave >> 1, wn = wave & 1;
-    const int nstage = (k_end - k_begin + BK - 1) / BK;
     if (nstage <= 0) return;
 
     f32x4 ra[2][TA::PER_THREAD], rb[2][TB::PER_THREAD];
     // prologue: stage 0 -> LDS buffer 0, stage 1 -> registers (slot 1)
-    TA::load(ra[0], A, lda, a_row0, a_rows, k_begin, nk < k_end ? nk : k_end);
-    TB::load(rb[0], B, ldb, b_row0, b_rows, k_begin, nk < k_end ? nk : k_end);
-    const int klim = nk < k_end ? nk : k_end;
-    TA::load(ra[1], A, lda, a_row0, a_rows, k_begin + BK, klim);
-    TB::load(rb[1], B, ldb, b_row0, b_rows, k_begin + BK, klim);
+    pa.load(ra[0], k_begin);
+    pb.load(rb[0], k_begin);
+    pa.load(ra[1], k_begin + BK);
+    pb.load(rb[1], k_begin + BK);
     TA::store(lds, ra[0]);
     TB::store(lds + TA::LDS_ELEMS, rb[0]);
     __syncthreads();
 
     // steady state, two stages per trip so that register slots and LDS buffers are compile-time constants
     for (int s = 0; s < nstage; s += 2) {
-        // --- even stage s: compute buffer 0; registers slot 1 hold stage s+1; fetch stage s+2 into slot 0
+        // --- even stage s: compute buffer 0; register slot 1 holds stage s+1; fetch stage s+2 into slot 0
         __builtin_amdgcn_sched_barrier(0);
-        TA::load(ra[0], A, lda, a_row0, a_rows, k_begin + (s + 2) * BK, klim);
-        TB::load(rb[0], B, ldb, b_row0, b_rows, k_begin + (s + 2) * BK, klim);
+        pa.load(ra[0], k_begin + (s + 2) * BK);
+        pb.load(rb[0], k_begin + (s + 2) * BK);
         __builtin_amdgcn_sched_barrier(0);
         mma_stage<TA, TB, BK, MI, NI>(acc, lds, lds + TA::LDS_ELEMS, wm, wn, lane);
         __builtin_amdgcn_sched_barrier(0);
@@ -160,8 +219,8 @@ __device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / 64][BN / 64], b
         if (s + 1 >= nstage) break;
         // --- odd stage s+1: compute buffer 1; slot 0 holds stage s+2; fetch stage s+3 into slot 1
         __builtin_amdgcn_sched_barrier(0);
-        TA::load(ra[1], A, lda, a_row0, a_rows, k_begin + (s + 3) * BK, klim);
-        TB::load(rb[1], B, ldb, b_row0, b_rows, k_begin + (s + 3) * BK, klim);
+        pa.load(ra[1], k_begin + (s + 3) * BK);
+        pb.load(rb[1], k_begin + (s + 3) * BK);
         __builtin_amdgcn_sched_barrier(0);
         mma_stage<TA, TB, BK, MI, NI>(acc, lds + STAGE, lds + STAGE + TA::LDS_ELEMS, wm, wn, lane);
         __builtin_amdgcn_sched_barrier(0);

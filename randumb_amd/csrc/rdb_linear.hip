@@ -254,7 +254,7 @@ static int check_desc(const char *who, const rdb_linear_desc *d)
     if (d->coef_rows != 0 && (d->sO != d->in_f || d->sI != 1))
         return set_error(RDB_E_SHAPE, "%s: matrix-coef needs strides (in_f, 1), got (%lld, %lld)", who, (long long)d->sO, (long long)d->sI);
     if (d->sO < 0 || d->sI < 0) return set_error(RDB_E_SHAPE, "%s: negative weight stride", who);
-    if (d->algo != RDB_ALGO_AUTO && d->algo != RDB_ALGO_TILE && d->algo != RDB_ALGO_STRIP)
+    if (d->algo != RDB_ALGO_AUTO && d->algo != RDB_ALGO_TILE && d->algo != RDB_ALGO_STRIP && d->algo != RDB_ALGO_FACTORED)
         return set_error(RDB_E_UNSUPPORTED, "%s: unknown algo %d", who, d->algo);
     if (d->tokens > (1ll << 31) * BM || d->in_f > (1ll << 31) || d->out_f > (1ll << 31))
         return set_error(RDB_E_SHAPE, "%s: dimension too large", who);
@@ -264,6 +264,11 @@ static int check_desc(const char *who, const rdb_linear_desc *d)
 // rdb_strip.hip
 int linear_fwd_strip(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
                      const rdb_linear_desc *d, int num_cus, hipStream_t s);
+
+// rdb_dx.hip
+int64_t linear_dx_factored_workspace(const rdb_linear_desc *d);
+int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias,
+                       const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s);
 
 // rdb_dcoef.hip
 int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d,
@@ -314,9 +319,18 @@ template <typename K> static int launch(K kernel, dim3 grid, size_t smem, hipStr
 
 using namespace rdb;
 
-extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias,
-                              const void *bias, const rdb_linear_desc *d, void *stream)
+extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
 {
+    if (!d) return 0;
+    if (op == RDB_OP_LINEAR_BWD_DX && d->algo != RDB_ALGO_TILE && d->algo != RDB_ALGO_STRIP) return linear_dx_factored_workspace(d);
+    return 0;
+}
+
+extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias,
+                              const void *bias, const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    (void)workspace;
+    (void)workspace_bytes;
     int rc = check_desc("rdb_linear_fwd", d);
     if (rc) return rc;
     if (d->tokens == 0 || d->out_f == 0) return RDB_OK;
@@ -350,13 +364,21 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
 }
 
 extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias,
-                                 const rdb_linear_desc *d, void *stream)
+                                 const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
 {
     int rc = check_desc("rdb_linear_bwd_dx", d);
     if (rc) return rc;
     if (d->tokens == 0 || d->in_f == 0) return RDB_OK;
     if (!dx || (!dy && d->out_f > 0) || (!coef && d->k > 0)) return set_error(RDB_E_NULL, "rdb_linear_bwd_dx: dx, dy or coef is NULL");
     if (lddx < d->in_f || lddy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dx: leading dimension smaller than the row");
+    if (d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) {
+        rc = linear_dx_factored(dx, lddx, dy, lddy, coef, scale_bias, d, workspace, workspace_bytes, (hipStream_t)stream);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+        if (d->algo == RDB_ALGO_FACTORED)
+            return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dx: the factored algorithm needs matrix-coef in bf16, bf16 activations, no "
+                                                "scale_bias, sizes that are multiples of 8, aligned rows and a workspace of "
+                                                "rdb_linear_workspace_bytes() bytes");
+    }
     const int es = d->act_dtype == RDB_BF16 ? 2 : 4;
     LinParams p = {};
     p.w = make_spec(d, coef, scale_bias);
@@ -377,8 +399,10 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
 }
 
 extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const void *dy, int64_t lddy, const void *x, int64_t ldx,
-                                    const rdb_linear_desc *d, void *stream)
+                                    const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
 {
+    (void)workspace;
+    (void)workspace_bytes;
     int rc = check_desc("rdb_linear_bwd_dcoef", d);
     if (rc) return rc;
     const int64_t ncoef = (d->coef_rows ? d->coef_rows : 1) * d->k;

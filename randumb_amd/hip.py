@@ -10,7 +10,8 @@ from typing import Optional, Sequence
 import torch
 
 from . import _lib
-from ._lib import LinearDesc, RDB_ALGO_AUTO, RDB_BF16, RDB_F32
+from ._lib import (LinearDesc, RDB_ALGO_AUTO, RDB_BF16, RDB_F32, RDB_OP_LINEAR_BWD_DCOEF, RDB_OP_LINEAR_BWD_DX,
+                   RDB_OP_LINEAR_FWD)
 
 _DT = {torch.float32: RDB_F32, torch.bfloat16: RDB_BF16}
 
@@ -202,9 +203,12 @@ def linear_fwd(x: torch.Tensor, coef: torch.Tensor, in_f: int, out_f: int, sO: i
     b = None if bias is None else bias.to(x.dtype).contiguous()
     y = torch.empty((x.shape[0], out_f), dtype=x.dtype, device=x.device)
     d = _desc(x.shape[0], in_f, out_f, c, sO, sI, seed, x.dtype, algo)
+    L = _lib.load()
+    ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_FWD, ctypes.byref(d))
+    ws = _workspace(ws_bytes, x.device)
     with torch.cuda.device(x.device):
-        rc = _lib.load().rdb_linear_fwd(_p(y), y.stride(0), _p(x), x.stride(0), _p(c), _p(sb), _p(b), ctypes.byref(d),
-                                        _stream(x.device))
+        rc = L.rdb_linear_fwd(_p(y), y.stride(0), _p(x), x.stride(0), _p(c), _p(sb), _p(b), ctypes.byref(d), _p(ws), ws_bytes,
+                              _stream(x.device))
     _lib.check(rc, "rdb_linear_fwd")
     return y
 
@@ -218,9 +222,12 @@ def linear_bwd_dx(dy: torch.Tensor, coef: torch.Tensor, in_f: int, out_f: int, s
     sb = None if scale_bias is None else _native(scale_bias).to(c.dtype)
     dx = torch.empty((dy.shape[0], in_f), dtype=dy.dtype, device=dy.device)
     d = _desc(dy.shape[0], in_f, out_f, c, sO, sI, seed, dy.dtype, algo)
+    L = _lib.load()
+    ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX, ctypes.byref(d))
+    ws = _workspace(ws_bytes, dy.device)
     with torch.cuda.device(dy.device):
-        rc = _lib.load().rdb_linear_bwd_dx(_p(dx), dx.stride(0), _p(dy), dy.stride(0), _p(c), _p(sb), ctypes.byref(d),
-                                           _stream(dy.device))
+        rc = L.rdb_linear_bwd_dx(_p(dx), dx.stride(0), _p(dy), dy.stride(0), _p(c), _p(sb), ctypes.byref(d), _p(ws), ws_bytes,
+                                 _stream(dy.device))
     _lib.check(rc, "rdb_linear_bwd_dx")
     return dx
 
@@ -239,8 +246,11 @@ def linear_bwd_dcoef(dy: torch.Tensor, x: torch.Tensor, k: int, coef_rows: int, 
     d.tokens, d.in_f, d.out_f, d.k, d.coef_rows = dy.shape[0], int(in_f), int(out_f), int(k), int(coef_rows)
     d.sO, d.sI, d.seed = int(sO), int(sI), _seed(seed)
     d.act_dtype, d.coef_dtype, d.algo = _DT[dy.dtype], RDB_F32, int(algo)
+    L = _lib.load()
+    ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DCOEF, ctypes.byref(d))
+    ws = _workspace(ws_bytes, dy.device)
     with torch.cuda.device(dy.device):
-        rc = _lib.load().rdb_linear_bwd_dcoef(_p(dcoef), _p(dsb), _p(dy), dy.stride(0), _p(x), x.stride(0), ctypes.byref(d),
-                                              _stream(dy.device))
+        rc = L.rdb_linear_bwd_dcoef(_p(dcoef), _p(dsb), _p(dy), dy.stride(0), _p(x), x.stride(0), ctypes.byref(d), _p(ws), ws_bytes,
+                                    _stream(dy.device))
     _lib.check(rc, "rdb_linear_bwd_dcoef")
     return dcoef, dsb

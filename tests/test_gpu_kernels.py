@@ -290,3 +290,48 @@ def test_strip_algorithm_rejects_what_it_cannot_do(hip):
     with pytest.raises(RandumbHipError):
         hip.linear_fwd(x, C, 100, 32, 100, 1, 0, algo=RDB_ALGO_STRIP)
     assert hip.linear_fwd(x, C, 100, 32, 100, 1, 0).shape == (64, 32)  # the default falls back to the general kernel
+
+
+# ------------------------------------------------------------------------------------------------ optimised backward kernels
+BWD_SHAPES = [
+    # tokens, in_f, out_f, k, seed
+    (2048, 768, 3072, 256, 0),   # a quarter of the headline workload
+    (1000, 200, 328, 72, 3),     # ragged against every tile size (multiples of 8 only)
+    (64, 8, 8, 8, 5),
+    (300, 1024, 96, 512, 9),     # k larger than in*out/(in+out): the factored form is not cheaper, still exact when forced
+]
+
+
+@pytest.mark.parametrize("T,in_f,out_f,k,seed", BWD_SHAPES)
+def test_linear_bwd_fast_kernels(hip, oracle, T, in_f, out_f, k, seed):
+    from randumb_amd._lib import RDB_ALGO_FACTORED, RDB_ALGO_TILE
+
+    print(f"case bwd fast T={T} in={in_f} out={out_f} k={k}", flush=True)
+    x, dy, coef = _inputs(T, in_f, out_f, k, True, torch.bfloat16, seed)
+    want_dx, want_dc, dW = oracle.linear_bwd(x.float().numpy(), dy.float().numpy(), coef.float().numpy(), in_f, out_f, seed)
+    xc, dyc, cc = x.cuda(), dy.cuda(), coef.cuda()
+    dx = hip.linear_bwd_dx(dyc, cc, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    assert dx.shape == (T, in_f) and rel_l2(cpu(dx), want_dx) < BF16_TOL
+    dx_ref = hip.linear_bwd_dx(dyc, cc, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_TILE)
+    assert rel_l2(cpu(dx), cpu(dx_ref)) < 1e-2
+    assert rel_l2(cpu(hip.linear_bwd_dx(dyc, cc, in_f, out_f, in_f, 1, seed)), want_dx) < BF16_TOL  # whatever AUTO picks
+    dc, dsb = hip.linear_bwd_dcoef(dyc, xc, k, out_f, in_f, out_f, in_f, 1, seed, want_scale_bias_grad=True)
+    assert rel_l2(cpu(dc), want_dc) < BF16_TOL
+    dc_ref, _ = hip.linear_bwd_dcoef(dyc, xc, k, out_f, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_TILE)
+    assert rel_l2(cpu(dc), cpu(dc_ref)) < 1e-2
+    want_ds = float(oracle.scale_bias_bwd(dW.astype(np.float32), seed)[0])
+    assert abs(float(dsb) - want_ds) < 2e-2 * max(1.0, abs(want_ds), float(np.abs(dW).sum()) ** 0.5)
+
+
+def test_factored_dx_needs_what_it_says(hip):
+    from randumb_amd._lib import RandumbHipError, RDB_ALGO_FACTORED
+
+    dy = torch.randn(64, 48, device="cuda").bfloat16()
+    c = torch.randn(16, device="cuda").bfloat16()          # vector-coef has no factored form
+    with pytest.raises(RandumbHipError):
+        hip.linear_bwd_dx(dy, c, 40, 48, 40, 1, 0, algo=RDB_ALGO_FACTORED)
+    C = torch.randn(48, 16, device="cuda").bfloat16()
+    sb = torch.tensor([0.1], device="cuda").bfloat16()      # neither has the random-bias term
+    with pytest.raises(RandumbHipError):
+        hip.linear_bwd_dx(dy, C, 40, 48, 40, 1, 0, scale_bias=sb, algo=RDB_ALGO_FACTORED)
+    assert hip.linear_bwd_dx(dy, C, 40, 48, 40, 1, 0, scale_bias=sb).shape == (64, 40)

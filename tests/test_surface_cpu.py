@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_lib.SO_PATH)
     for name in declared:
         assert hasattr(lib, name), name
-    assert _lib.load().rdb_abi_version() == 1
+    assert _lib.load().rdb_abi_version() == 2
     assert ctypes.sizeof(_lib.LinearDesc) == 7 * 8 + 4 * 4
 
 
@@ -40,8 +40,8 @@ def test_argument_errors_come_back_as_codes_without_a_gpu():
     assert L.rdb_materialize_fwd(None, None, 7, 0, 4, 0, 2, 2, 2, 1, 0, None, None) == -3
     d = _lib.LinearDesc()
     d.tokens, d.in_f, d.out_f, d.k, d.coef_rows, d.sO, d.sI = 4, 8, 6, 3, 5, 8, 1
-    assert L.rdb_linear_fwd(None, 6, None, 8, None, None, None, ctypes.byref(d), None) == -2  # coef_rows != out_f
-    assert L.rdb_linear_fwd(None, 6, None, 8, None, None, None, None, None) == -1
+    assert L.rdb_linear_fwd(None, 6, None, 8, None, None, None, ctypes.byref(d), None, 0, None) == -2  # coef_rows != out_f
+    assert L.rdb_linear_fwd(None, 6, None, 8, None, None, None, None, None, 0, None) == -1
     assert L.rdb_materialize_bwd_workspace_bytes(0, 256, 0, 2359296) > 0
     assert L.rdb_materialize_bwd_workspace_bytes(3072, 256, 768, 2359296) == 0
 
