@@ -8,12 +8,13 @@
 // on the matrix cores.  Partial sums of different blocks are combined with coalesced fp32 atomics.  dW never reaches
 // memory.  Replaces MmBackward's dense dW + RandumbTensorConstructor.backward -> materialize_bwd / scale_bias_bwd
 // (src/rten_cpp/RandumbTensor.py:979-990, 304-359, 399-420).
+#include <stdlib.h>
 #include "rdb_gemm.hpp"
 #include "rdb_tile.hpp"
 
 namespace rdb {
 
-constexpr int DC_BI = 192, DC_BO = 192, DC_BK = 32, DC_MC = 64;
+constexpr int DC_BI = 192, DC_BO = 192, DC_BK = 64, DC_MC = 64;
 
 struct DcoefParams {
     const bf16_t *dy;
@@ -22,8 +23,10 @@ struct DcoefParams {
     float *dsb;
     int64_t lddy, ldx;
     int tokens, in_f, out_f, k;
-    int tok_per_split;
+    int tok_per_split, tiles_i, tiles_o, splits;
     uint32_t seed;
+    long long *dbgp;
+    int dbg;
 };
 
 __global__ __launch_bounds__(256, 1) void linear_dcoef_fast_kernel(DcoefParams p)
@@ -31,20 +34,30 @@ __global__ __launch_bounds__(256, 1) void linear_dcoef_fast_kernel(DcoefParams p
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
-    const int i0 = blockIdx.x * DC_BI, o0 = blockIdx.y * DC_BO;
-    const int t_begin = blockIdx.z * p.tok_per_split;
-    const int t_end = (t_begin + p.tok_per_split < p.tokens) ? t_begin + p.tok_per_split : p.tokens;
+    // work item = (token split, o tile, i tile), i fastest: neighbours share the dy stream, a whole die shares the x stream
+    const int w = xcd_work_item(blockIdx.x, p.tiles_i * p.tiles_o * p.splits);
+    if (w >= p.tiles_i * p.tiles_o * p.splits) return;
+    const int i0 = (w % p.tiles_i) * DC_BI, o0 = ((w / p.tiles_i) % p.tiles_o) * DC_BO, split = w / (p.tiles_i * p.tiles_o);
+    int t_begin = split * p.tok_per_split;
+    int t_end = (t_begin + p.tok_per_split < p.tokens) ? t_begin + p.tok_per_split : p.tokens;
+    int li0 = i0, lo0 = o0;
+    if (p.dbg & 1) { li0 = 0; lo0 = 0; t_end -= t_begin; t_begin = 0; }
 
+#ifdef RDB_PROFILE_MAINLOOP
+    rdb_profile_ptr = p.dbgp;
+#endif
+    long long ts0 = __builtin_readcyclecounter();
     // main product: D[m = i][n = o] (x rows as the "A" tile, dy rows as the "B" tile), contraction over tokens
     f32x16 acc[DC_BI / 64][DC_BO / 64];
 #pragma unroll
     for (int mi = 0; mi < DC_BI / 64; ++mi)
 #pragma unroll
         for (int ni = 0; ni < DC_BO / 64; ++ni) acc[mi][ni] = zero16();
-    const GlobalOperand<DC_BI, DC_BK, M_CONT> opx = {p.x, p.ldx, i0, p.in_f, t_end};
-    const GlobalOperand<DC_BO, DC_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end};
+    GlobalOperand<DC_BI, DC_BK, M_CONT> opx = {p.x, p.ldx, li0, p.in_f, t_end};
+    GlobalOperand<DC_BO, DC_BK, M_CONT> opdy = {p.dy, p.lddy, lo0, p.out_f, t_end};
     gemm_mainloop<DC_BI, DC_BO, DC_BK>(acc, lds, opx, opdy, t_begin, (t_end - t_begin + DC_BK - 1) / DC_BK);
 
+    long long ts1 = __builtin_readcyclecounter();
     // dW tile -> LDS as Ws[o][i] (bf16, i contiguous).  acc[mi][ni][j]: i = wm*96 + mi*32 + 8*(j/4) + 4*g + j%4, o = wn*96 + ni*32 + r
     constexpr int LDW = DC_BI + 8;
     bf16_t *Ws = lds;                  // [DC_BO][LDW]
@@ -108,6 +121,11 @@ __global__ __launch_bounds__(256, 1) void linear_dcoef_fast_kernel(DcoefParams p
         __syncthreads();
     }
 
+    if (p.dbgp && t == 0 && blockIdx.x == 0) {
+        long long ts2 = __builtin_readcyclecounter();
+        p.dbgp[0] = ts1 - ts0;
+        p.dbgp[1] = ts2 - ts1;
+    }
     if (p.dsb) {  // d scale_bias += sum dW[o, i] * noise(o*in_f + i)
         float s = 0.0f;
         for (int e = t; e < DC_BO * DC_BI; e += 256) {
@@ -132,7 +150,8 @@ int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, co
 {
     if (d->act_dtype != RDB_BF16 || d->coef_rows == 0) return RDB_E_UNSUPPORTED;
     if (d->in_f % 8 || d->out_f % 8 || ldx % 8 || lddy % 8 || ((uintptr_t)x & 15) || ((uintptr_t)dy & 15)) return RDB_E_UNSUPPORTED;
-    if (d->tokens < 1 || d->tokens > (1 << 30) || d->out_f > (1 << 30) || d->in_f > (1 << 30) || d->out_f * d->in_f > (1ll << 31))
+    if (d->tokens < 1 || d->tokens > (1 << 30) || d->out_f > (1 << 30) || d->in_f > (1 << 30) || d->out_f * d->in_f > (1ll << 31) ||
+        d->tokens * lddy >= (1ll << 31) || d->tokens * ldx >= (1ll << 31))
         return RDB_E_UNSUPPORTED;
     DcoefParams p;
     p.dy = (const bf16_t *)dy;
@@ -146,6 +165,8 @@ int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, co
     p.out_f = (int)d->out_f;
     p.k = (int)d->k;
     p.seed = d->seed;
+    p.dbg = getenv("RDB_DEBUG") ? atoi(getenv("RDB_DEBUG")) : 0;
+    p.dbgp = getenv("RDB_DBGP") ? (long long *)strtoull(getenv("RDB_DBGP"), nullptr, 0) : nullptr;
     const int ti = (int)cdiv(d->in_f, DC_BI), to = (int)cdiv(d->out_f, DC_BO);
     int splits = num_cus / (ti * to);
     const int max_splits = (int)cdiv(d->tokens, 256);
@@ -153,6 +174,9 @@ int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, co
     if (splits < 1) splits = 1;
     p.tok_per_split = (int)(cdiv(cdiv(d->tokens, splits), DC_BK) * DC_BK);
     splits = (int)cdiv(d->tokens, p.tok_per_split);
+    p.tiles_i = ti;
+    p.tiles_o = to;
+    p.splits = splits;
     typedef OperandTile<DC_BI, DC_BK, M_CONT> TA;
     typedef OperandTile<DC_BO, DC_BK, M_CONT> TB;
     const size_t main_bytes = 2 * (TA::LDS_ELEMS + TB::LDS_ELEMS) * sizeof(bf16_t);
@@ -161,7 +185,7 @@ int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, co
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(linear_dcoef_fast_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)smem);
     if (e != hipSuccess) return set_error((int)e, "linear_dcoef_fast_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
-    linear_dcoef_fast_kernel<<<dim3(ti, to, splits), 256, smem, s>>>(p);
+    linear_dcoef_fast_kernel<<<xcd_grid_size(ti * to * splits), 256, smem, s>>>(p);
     return check_launch("linear_dcoef_fast_kernel");
 }
 

@@ -24,6 +24,7 @@ struct DyCParams {
     bf16_t *t;
     int64_t lddy;
     int tokens, out_f, k;
+    int tiles_c, tiles_t;
 };
 
 __global__ __launch_bounds__(256, 1) void dx_dyc_kernel(DyCParams p)
@@ -31,16 +32,19 @@ __global__ __launch_bounds__(256, 1) void dx_dyc_kernel(DyCParams p)
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.x * K1_BC, tok0 = blockIdx.y * K1_BT;
+    // work item = (token tile, coefficient tile), coefficient tile fastest: neighbours share the dy tile
+    const int w = xcd_work_item(blockIdx.x, p.tiles_c * p.tiles_t);
+    if (w >= p.tiles_c * p.tiles_t) return;
+    const int m0 = (w % p.tiles_c) * K1_BC, tok0 = (w / p.tiles_c) * K1_BT;
     f32x16 acc[K1_BC / 64][K1_BT / 64];
 #pragma unroll
     for (int mi = 0; mi < K1_BC / 64; ++mi)
 #pragma unroll
         for (int ni = 0; ni < K1_BT / 64; ++ni) acc[mi][ni] = zero16();
     // "A": C[o][m], tile rows = m (contiguous in memory), contraction index = o
-    const GlobalOperand<K1_BC, K1_BK, M_CONT> opc = {p.coef, (int64_t)p.k, m0, p.k, p.out_f};
+    GlobalOperand<K1_BC, K1_BK, M_CONT> opc = {p.coef, (int64_t)p.k, m0, p.k, p.out_f};
     // "B": dy[tok][o], contraction index contiguous
-    const GlobalOperand<K1_BT, K1_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f};
+    GlobalOperand<K1_BT, K1_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f};
     gemm_mainloop<K1_BC, K1_BT, K1_BK>(acc, lds, opc, opdy, 0, (p.out_f + K1_BK - 1) / K1_BK);
     // acc[mi][ni][j]: m = m0 + wm*64 + mi*32 + 8*(j/4) + 4*g + j%4, tok = tok0 + wn*64 + ni*32 + r
 #pragma unroll
@@ -68,6 +72,7 @@ struct TNParams {
     bf16_t *dx;
     int64_t lddx;
     int tokens, in_f, k;
+    int tiles_i, tiles_t;
     uint32_t seed;
 };
 
@@ -76,16 +81,19 @@ __global__ __launch_bounds__(256, 1) void dx_tn_kernel(TNParams p)
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
-    const int i0 = blockIdx.x * K2_BI, tok0 = blockIdx.y * K2_BT;
+    // work item = (token tile, feature tile), feature tile fastest: neighbours share the t tile
+    const int w = xcd_work_item(blockIdx.x, p.tiles_i * p.tiles_t);
+    if (w >= p.tiles_i * p.tiles_t) return;
+    const int i0 = (w % p.tiles_i) * K2_BI, tok0 = (w / p.tiles_i) * K2_BT;
     f32x16 acc[K2_BI / 64][K2_BT / 64];
 #pragma unroll
     for (int mi = 0; mi < K2_BI / 64; ++mi)
 #pragma unroll
         for (int ni = 0; ni < K2_BT / 64; ++ni) acc[mi][ni] = zero16();
     // "A": 2^31 * noise(i, m), rows = i, contraction = m; values for m >= k meet zero rows of t
-    const NoiseOperandRowsAreElements<K2_BI, K2_BK> opn = {i0, p.seed};
+    NoiseOperandRowsAreElements<K2_BI, K2_BK> opn = {i0, p.seed};
     // "B": t[tok][m]
-    const GlobalOperand<K2_BT, K2_BK, K_CONT> opt = {p.t, (int64_t)p.k, tok0, p.tokens, p.k};
+    GlobalOperand<K2_BT, K2_BK, K_CONT> opt = {p.t, (int64_t)p.k, tok0, p.tokens, p.k};
     gemm_mainloop<K2_BI, K2_BT, K2_BK>(acc, lds, opn, opt, 0, (p.k + K2_BK - 1) / K2_BK);
     // acc[mi][ni][j]: i = i0 + wm*96 + mi*32 + 8*(j/4) + 4*g + j%4, tok = tok0 + wn*64 + ni*32 + r
 #pragma unroll
@@ -111,7 +119,7 @@ static bool dx_factored_ok(const rdb_linear_desc *d)
 {
     return d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16 && d->coef_rows != 0 && d->k % 8 == 0 && d->in_f % 8 == 0 &&
            d->out_f % 8 == 0 && d->k > 0 && d->tokens > 0 && d->tokens < (1 << 30) && d->in_f < (1 << 30) && d->out_f < (1 << 30) &&
-           d->k < (1 << 24);
+           d->k < (1 << 24) && d->tokens * d->k < (1ll << 31) && d->out_f * d->k < (1ll << 31);
 }
 
 int64_t linear_dx_factored_workspace(const rdb_linear_desc *d)
@@ -126,6 +134,7 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
 {
     if (!dx_factored_ok(d) || scale_bias) return RDB_E_UNSUPPORTED;  // the random-bias term is not low rank
     if (!workspace || workspace_bytes < linear_dx_factored_workspace(d) || ((uintptr_t)workspace & 15)) return RDB_E_UNSUPPORTED;
+    if (d->tokens * lddy >= (1ll << 31)) return RDB_E_UNSUPPORTED;
     if (lddy % 8 || lddx % 4 || ((uintptr_t)dy & 15) || ((uintptr_t)coef & 15) || ((uintptr_t)dx & 7)) return RDB_E_UNSUPPORTED;
     // only worth it when the factored form is cheaper than forming the weight
     if (d->algo == RDB_ALGO_AUTO && d->k * (d->in_f + d->out_f) >= d->in_f * d->out_f) return RDB_E_UNSUPPORTED;
@@ -144,7 +153,9 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
         const size_t smem = 2 * (TA::LDS_ELEMS + TB::LDS_ELEMS) * sizeof(bf16_t);
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(dx_dyc_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return set_error((int)e, "dx_dyc_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
-        dx_dyc_kernel<<<dim3((unsigned)cdiv(d->k, K1_BC), (unsigned)cdiv(d->tokens, K1_BT)), 256, smem, s>>>(p1);
+        p1.tiles_c = (int)cdiv(d->k, K1_BC);
+        p1.tiles_t = (int)cdiv(d->tokens, K1_BT);
+        dx_dyc_kernel<<<xcd_grid_size(p1.tiles_c * p1.tiles_t), 256, smem, s>>>(p1);
         int rc = check_launch("dx_dyc_kernel");
         if (rc) return rc;
     }
@@ -162,7 +173,9 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
         const size_t smem = 2 * (TA::LDS_ELEMS + TB::LDS_ELEMS) * sizeof(bf16_t);
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(dx_tn_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return set_error((int)e, "dx_tn_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
-        dx_tn_kernel<<<dim3((unsigned)cdiv(d->in_f, K2_BI), (unsigned)cdiv(d->tokens, K2_BT)), 256, smem, s>>>(p2);
+        p2.tiles_i = (int)cdiv(d->in_f, K2_BI);
+        p2.tiles_t = (int)cdiv(d->tokens, K2_BT);
+        dx_tn_kernel<<<xcd_grid_size(p2.tiles_i * p2.tiles_t), 256, smem, s>>>(p2);
         return check_launch("dx_tn_kernel");
     }
 }

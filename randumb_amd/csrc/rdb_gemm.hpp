@@ -11,11 +11,22 @@
 // Pipeline: global loads run two stages ahead in registers, one stage ahead in LDS (double buffer), one barrier per stage.
 #pragma once
 
+#ifndef RDB_SCHED_FENCE
+#define RDB_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+#endif
+
 #include "rdb_common.hpp"
 
 namespace rdb {
 
+#ifdef RDB_PROFILE_MAINLOOP
+__device__ long long *rdb_profile_ptr;
+#endif
+
 typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+// 16 bytes of zeros in device memory: the load target of operand pieces that lie outside their matrix.
+__device__ __align__(16) const uint32_t rdb_zero_piece[4] = {0u, 0u, 0u, 0u};
 
 enum OperandLayout { K_CONT = 0, M_CONT = 1 };
 
@@ -29,54 +40,81 @@ union Frag8 {
 // One operand of the tile engine.  ROWS = tile rows (BM or BN), BK = contraction depth per stage.
 template <int ROWS, int BK, int LAYOUT> struct OperandTile {
     static constexpr int PAD = 8;
+    static constexpr int LAYOUT_ID = LAYOUT;
     static constexpr int LD = (LAYOUT == K_CONT) ? (BK + PAD) : (ROWS + PAD);     // LDS row stride, elements
     static constexpr int LDS_ELEMS = (LAYOUT == K_CONT) ? ROWS * LD : BK * LD;    // per stage
     static constexpr int PIECES = ROWS * BK / 8;                                   // 16-byte pieces per stage
     static constexpr int PER_THREAD = (PIECES + 255) / 256;
     static_assert(PIECES % 256 == 0, "operand stage must split evenly over 256 threads");
 
-    // Global -> registers.  row0: first tile row; nrows: rows of the matrix; k0: first k of the stage; nk: k extent.
-    // Pieces outside the matrix read a valid address and are zeroed (rows % 8 == 0 / k % 8 == 0 is guaranteed by the host
-    // for the contiguous axis, so a 16-byte piece is entirely inside or outside).
-    __device__ static __forceinline__ void load(f32x4 (&regs)[PER_THREAD], const bf16_t *__restrict__ src, int64_t ld, int row0,
-                                                int nrows, int k0, int nk)
+    // Per-thread description of the pieces it copies from global memory: element offset of each piece at stage 0, and
+    // whether its tile row lies inside the matrix.  Built once, before the main loop.
+    struct Pieces {
+        int off[PER_THREAD];
+        int kk[PER_THREAD];    // contraction offset of the piece inside a stage
+        bool rowok[PER_THREAD];
+    };
+    __device__ static __forceinline__ Pieces pieces(int64_t ld, int row0, int nrows, int k_begin)
     {
+        Pieces q;
         const int t = threadIdx.x;
 #pragma unroll
         for (int p = 0; p < PER_THREAD; ++p) {
             const int idx = p * 256 + t;
             int row, k;
-            bool ok;
             if (LAYOUT == K_CONT) {
                 row = row0 + idx / (BK / 8);
-                k = k0 + (idx % (BK / 8)) * 8;
+                k = (idx % (BK / 8)) * 8;
             } else {
-                k = k0 + idx / (ROWS / 8);
+                k = idx / (ROWS / 8);
                 row = row0 + (idx % (ROWS / 8)) * 8;
             }
-            ok = row < nrows && k < nk;
-            const int rr = ok ? row : 0, kk = ok ? k : 0;
-            const bf16_t *ptr = (LAYOUT == K_CONT) ? src + (int64_t)rr * ld + kk : src + (int64_t)kk * ld + rr;
-            f32x4 v = *reinterpret_cast<const f32x4 *>(ptr);
-            const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-            regs[p] = ok ? v : z;
+            q.rowok[p] = row < nrows;
+            const int rr = q.rowok[p] ? row : 0;
+            q.kk[p] = k;
+            q.off[p] = (LAYOUT == K_CONT) ? (int)(rr * ld) + k_begin + k : (int)((k_begin + k) * ld) + rr;
+        }
+        return q;
+    }
+
+    // Global -> registers for the stage whose first contraction index is k0 = k_begin + stage*BK; `adv` is the element
+    // offset of that stage relative to stage 0 (stage*BK for K_CONT, stage*BK*ld for M_CONT).  Pieces outside the matrix
+    // (row >= nrows or k >= klim) are redirected to 16 bytes of zeros, so nothing downstream of the load has to wait for
+    // it; the host guarantees that the contiguous axis is a multiple of 8, so a piece is entirely inside or outside.
+    __device__ static __forceinline__ void load(f32x4 (&regs)[PER_THREAD], const bf16_t *__restrict__ src, const Pieces &q, int adv, int k0,
+                                                int klim)
+    {
+#pragma unroll
+        for (int p = 0; p < PER_THREAD; ++p) {
+            const bool ok = q.rowok[p] && (k0 + q.kk[p] < klim);
+            const bf16_t *ptr = ok ? src + (q.off[p] + adv) : reinterpret_cast<const bf16_t *>(rdb_zero_piece);
+            regs[p] = *reinterpret_cast<const f32x4 *>(ptr);
         }
     }
 
+    __device__ static __forceinline__ void load_piece(f32x4 &reg, const bf16_t *__restrict__ src, const Pieces &q, int p, int adv, int k0,
+                                                      int klim)
+    {
+        const bool ok = q.rowok[p] && (k0 + q.kk[p] < klim);
+        const bf16_t *ptr = ok ? src + (q.off[p] + adv) : reinterpret_cast<const bf16_t *>(rdb_zero_piece);
+        reg = *reinterpret_cast<const f32x4 *>(ptr);
+    }
+
     // Registers -> LDS stage.
+    __device__ static __forceinline__ void store_piece(bf16_t *__restrict__ lds, const f32x4 &reg, int p)
+    {
+        const int idx = p * 256 + threadIdx.x;
+        int off;
+        if (LAYOUT == K_CONT)
+            off = (idx / (BK / 8)) * LD + (idx % (BK / 8)) * 8;
+        else
+            off = (idx / (ROWS / 8)) * LD + (idx % (ROWS / 8)) * 8;
+        *reinterpret_cast<f32x4 *>(lds + off) = reg;
+    }
     __device__ static __forceinline__ void store(bf16_t *__restrict__ lds, const f32x4 (&regs)[PER_THREAD])
     {
-        const int t = threadIdx.x;
 #pragma unroll
-        for (int p = 0; p < PER_THREAD; ++p) {
-            const int idx = p * 256 + t;
-            int off;
-            if (LAYOUT == K_CONT)
-                off = (idx / (BK / 8)) * LD + (idx % (BK / 8)) * 8;
-            else
-                off = (idx / (ROWS / 8)) * LD + (idx % (ROWS / 8)) * 8;
-            *reinterpret_cast<f32x4 *>(lds + off) = regs[p];
-        }
+        for (int p = 0; p < PER_THREAD; ++p) store_piece(lds, regs[p], p);
     }
 
     // Fragment of the 32-row block starting at tile row `rb` for k-step ks (16 wide) of the stage:
@@ -100,35 +138,73 @@ template <int ROWS, int BK, int LAYOUT> struct OperandTile {
     }
 };
 
-// Accumulates one LDS stage into the wave's (MI x NI) 32x32 blocks.
+// Accumulates one LDS stage into the wave's (MI x NI) 32x32 blocks.  The fragments of k-step ks+1 are requested before the
+// MFMAs of k-step ks are issued, so LDS latency hides behind the matrix pipe.
 template <class TA, class TB, int BK, int MI, int NI>
 __device__ __forceinline__ void mma_stage(f32x16 (&acc)[MI][NI], const bf16_t *__restrict__ As, const bf16_t *__restrict__ Bs, int wm,
                                           int wn, int lane)
 {
+    constexpr int KS = BK / 16;
+    bf16x8 fa[2][MI], fb[2][NI];
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-        bf16x8 fa[MI], fb[NI];
+    for (int mi = 0; mi < MI; ++mi) fa[0][mi] = TA::frag(As, wm * MI * 32 + mi * 32, 0, lane);
 #pragma unroll
-        for (int mi = 0; mi < MI; ++mi) fa[mi] = TA::frag(As, wm * MI * 32 + mi * 32, ks, lane);
+    for (int ni = 0; ni < NI; ++ni) fb[0][ni] = TB::frag(Bs, wn * NI * 32 + ni * 32, 0, lane);
 #pragma unroll
-        for (int ni = 0; ni < NI; ++ni) fb[ni] = TB::frag(Bs, wn * NI * 32 + ni * 32, ks, lane);
+    for (int ks = 0; ks < KS; ++ks) {
+        const int cur = ks & 1, nxt = cur ^ 1;
+        if (ks + 1 < KS) {
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi) fa[nxt][mi] = TA::frag(As, wm * MI * 32 + mi * 32, ks + 1, lane);
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) fb[nxt][ni] = TB::frag(Bs, wn * NI * 32 + ni * 32, ks + 1, lane);
+        }
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-            for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi], fb[ni], acc[mi][ni], 0, 0, 0);
+            for (int ni = 0; ni < NI; ++ni)
+                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][mi], fb[cur][ni], acc[mi][ni], 0, 0, 0);
     }
 }
+
+// ----------------------------------------------------------------------------------------------- work distribution
+// The 8 accelerator dies (XCDs) of the chip each have their own L2 and receive workgroups round-robin by linear block id.
+// Work items that read the same operand tiles should therefore sit on one die and run at the same time: item w of `total`
+// (neighbours in w share operands) goes to block id  (w % per_die) * 8 + w / per_die,  i.e. a block decodes
+//   w = (block % 8) * per_die + block / 8,   per_die = ceil(total / 8);   w >= total means the block has nothing to do.
+__device__ __forceinline__ int xcd_work_item(int block, int total)
+{
+    const int per_die = (total + 7) >> 3;
+    return (block & 7) * per_die + (block >> 3);
+}
+inline int xcd_grid_size(int total) { return ((total + 7) / 8) * 8; }
 
 // ----------------------------------------------------------------------------------------------- operand providers
 // A provider fills the registers of one pipeline stage: load(regs, k0) with k0 the stage's first contraction index.
 
-// Operand read from global memory.
+// Operand read from global memory (offsets are 32-bit: the host checks that the matrix has fewer than 2^31 elements).
 template <int ROWS, int BK, int LAYOUT> struct GlobalOperand {
     typedef OperandTile<ROWS, BK, LAYOUT> Tile;
     const bf16_t *src;
     int64_t ld;
     int row0, nrows, klim;  // klim: first contraction index that must read as zero
-    __device__ __forceinline__ void load(f32x4 (&regs)[Tile::PER_THREAD], int k0) const { Tile::load(regs, src, ld, row0, nrows, k0, klim); }
+    typename Tile::Pieces q;
+    int k_begin;
+    __device__ __forceinline__ void init(int kb)
+    {
+        k_begin = kb;
+        q = Tile::pieces(ld, row0, nrows, kb);
+    }
+    __device__ __forceinline__ void load_piece(f32x4 &reg, int p, int stage) const
+    {
+        const int adv = (LAYOUT == K_CONT) ? stage * BK : (int)(stage * BK * ld);
+        Tile::load_piece(reg, src, q, p, adv, k_begin + stage * BK, klim);
+    }
+    __device__ __forceinline__ void load(f32x4 (&regs)[Tile::PER_THREAD], int stage) const
+    {
+#pragma unroll
+        for (int p = 0; p < Tile::PER_THREAD; ++p) load_piece(regs[p], p, stage);
+    }
 };
 
 // Operand generated by the noise hash, tile rows = noise rows (tensor element index), contraction = coefficient index:
@@ -137,22 +213,25 @@ template <int ROWS, int BK> struct NoiseOperandRowsAreElements {
     typedef OperandTile<ROWS, BK, K_CONT> Tile;
     int row0;
     uint32_t seed;
-    __device__ __forceinline__ void load(f32x4 (&regs)[Tile::PER_THREAD], int k0) const
+    int k_begin;
+    __device__ __forceinline__ void init(int kb) { k_begin = kb; }
+    __device__ __forceinline__ void load_piece(f32x4 &reg, int p, int stage) const
     {
-        const int t = threadIdx.x;
+        const int idx = p * 256 + threadIdx.x, k0 = k_begin + stage * BK;
+        const int row = row0 + idx / (BK / 8), k = k0 + (idx % (BK / 8)) * 8;
+        const uint32_t first = (uint32_t)row * PN1 + (uint32_t)k * SQ5_N1 + seed;
+        uint32_t b[8];
 #pragma unroll
-        for (int p = 0; p < Tile::PER_THREAD; ++p) {
-            const int idx = p * 256 + t;
-            const int row = row0 + idx / (BK / 8), k = k0 + (idx % (BK / 8)) * 8;
-            const uint32_t first = (uint32_t)row * PN1 + (uint32_t)k * SQ5_N1 + seed;
-            uint32_t b[8];
+        for (int e = 0; e < 8; ++e) b[e] = sq5_tail(first + (uint32_t)e * SQ5_N1);
+        Frag8 f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) b[e] = sq5_tail(first + (uint32_t)e * SQ5_N1);
-            Frag8 f;
+        for (int e = 0; e < 4; ++e) f.u[e] = f32x2_to_bf16x2((float)(int32_t)b[2 * e], (float)(int32_t)b[2 * e + 1]);
+        reg = f.f4;
+    }
+    __device__ __forceinline__ void load(f32x4 (&regs)[Tile::PER_THREAD], int stage) const
+    {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) f.u[e] = f32x2_to_bf16x2((float)(int32_t)b[2 * e], (float)(int32_t)b[2 * e + 1]);
-            regs[p] = f.f4;
-        }
+        for (int p = 0; p < Tile::PER_THREAD; ++p) load_piece(regs[p], p, stage);
     }
 };
 
@@ -161,31 +240,91 @@ template <int ROWS, int BK> struct NoiseOperandRowsAreCoefs {
     typedef OperandTile<ROWS, BK, K_CONT> Tile;
     int row0;
     uint32_t seed;
-    __device__ __forceinline__ void load(f32x4 (&regs)[Tile::PER_THREAD], int k0) const
+    int k_begin;
+    __device__ __forceinline__ void init(int kb) { k_begin = kb; }
+    __device__ __forceinline__ void load_piece(f32x4 &reg, int p, int stage) const
     {
-        const int t = threadIdx.x;
+        const int idx = p * 256 + threadIdx.x, k0 = k_begin + stage * BK;
+        const int row = row0 + idx / (BK / 8), k = k0 + (idx % (BK / 8)) * 8;
+        const uint32_t first = (uint32_t)k * PN1 + (uint32_t)row * SQ5_N1 + seed;
+        uint32_t b[8];
 #pragma unroll
-        for (int p = 0; p < Tile::PER_THREAD; ++p) {
-            const int idx = p * 256 + t;
-            const int row = row0 + idx / (BK / 8), k = k0 + (idx % (BK / 8)) * 8;
-            const uint32_t first = (uint32_t)k * PN1 + (uint32_t)row * SQ5_N1 + seed;
-            uint32_t b[8];
+        for (int e = 0; e < 8; ++e) b[e] = sq5_tail(first + (uint32_t)e * PN1);
+        Frag8 f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) b[e] = sq5_tail(first + (uint32_t)e * PN1);
-            Frag8 f;
+        for (int e = 0; e < 4; ++e) f.u[e] = f32x2_to_bf16x2((float)(int32_t)b[2 * e], (float)(int32_t)b[2 * e + 1]);
+        reg = f.f4;
+    }
+    __device__ __forceinline__ void load(f32x4 (&regs)[Tile::PER_THREAD], int stage) const
+    {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) f.u[e] = f32x2_to_bf16x2((float)(int32_t)b[2 * e], (float)(int32_t)b[2 * e + 1]);
-            regs[p] = f.f4;
-        }
+        for (int p = 0; p < Tile::PER_THREAD; ++p) load_piece(regs[p], p, stage);
     }
 };
 
+// One pipeline stage: multiplies the LDS buffer `cur` into the accumulators while, slice by slice between the MFMAs, the
+// registers loaded during the previous stage go to the idle buffer `oth` and are refilled with stage `next_stage`.
+// The copy work and the next k-step's fragment reads are paced against the MFMAs with scheduling groups: every MFMA is
+// followed by a fixed number of memory instructions, so the vector-memory and LDS pipes run in the shadow of the matrix pipe.
+template <int BK, int MI, int NI, class PA, class PB>
+__device__ __forceinline__ void pipeline_stage(f32x16 (&acc)[MI][NI], const bf16_t *__restrict__ cur, bf16_t *__restrict__ oth,
+                                               f32x4 (&ra)[PA::Tile::PER_THREAD], f32x4 (&rb)[PB::Tile::PER_THREAD], const PA &pa, const PB &pb,
+                                               int next_stage, int wm, int wn, int lane)
+{
+    typedef typename PA::Tile TA;
+    typedef typename PB::Tile TB;
+    constexpr int KS = BK / 16;
+    constexpr int FRAG_OPS = (MI * (TA::LAYOUT_ID == M_CONT ? 2 : 1)) + (NI * (TB::LAYOUT_ID == M_CONT ? 2 : 1));
+    constexpr int COPY_OPS = 2 * ((TA::PER_THREAD + TB::PER_THREAD + KS - 1) / KS);
+    constexpr int MEM_PER_MFMA = (FRAG_OPS + COPY_OPS + MI * NI - 1) / (MI * NI);
+    const bf16_t *As = cur, *Bs = cur + TA::LDS_ELEMS;
+    bf16x8 fa[2][MI], fb[2][NI];
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi) fa[0][mi] = TA::frag(As, wm * MI * 32 + mi * 32, 0, lane);
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) fb[0][ni] = TB::frag(Bs, wn * NI * 32 + ni * 32, 0, lane);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const int c = ks & 1, n = c ^ 1;
+#pragma unroll
+        for (int p = 0; p < TA::PER_THREAD; ++p)
+            if (p % KS == ks) {
+                TA::store_piece(oth, ra[p], p);
+                pa.load_piece(ra[p], p, next_stage);
+            }
+#pragma unroll
+        for (int p = 0; p < TB::PER_THREAD; ++p)
+            if ((p + TA::PER_THREAD) % KS == ks) {
+                TB::store_piece(oth + TA::LDS_ELEMS, rb[p], p);
+                pb.load_piece(rb[p], p, next_stage);
+            }
+        if (ks + 1 < KS) {
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi) fa[n][mi] = TA::frag(As, wm * MI * 32 + mi * 32, ks + 1, lane);
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) fb[n][ni] = TB::frag(Bs, wn * NI * 32 + ni * 32, ks + 1, lane);
+        }
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[c][mi], fb[c][ni], acc[mi][ni], 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < MI * NI; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // one MFMA
+            __builtin_amdgcn_sched_group_barrier(0x090, MEM_PER_MFMA, 0);  // then vector-memory / LDS instructions
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();
+}
+
 // Main loop of the tile engine over `nstage` stages of BK starting at contraction index k_begin.
 // `lds` must hold 2 * (PA::Tile::LDS_ELEMS + PB::Tile::LDS_ELEMS) elements.  On return every wave has passed a barrier
-// after its last LDS read, so the caller may reuse `lds` at once.
+// after its last LDS read, so the caller may reuse `lds` at once.  An odd stage count is rounded up (the extra stage lies
+// past klim and reads as zeros), so the two-stage loop body has a single exit.
 template <int BM, int BN, int BK, class PA, class PB>
-__device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / 64][BN / 64], bf16_t *__restrict__ lds, const PA &pa, const PB &pb,
-                                              int k_begin, int nstage)
+__device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / 64][BN / 64], bf16_t *__restrict__ lds, PA &pa, PB &pb, int k_begin,
+                                              int nstage)
 {
     typedef typename PA::Tile TA;
     typedef typename PB::Tile TB;
@@ -193,40 +332,22 @@ __device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / 64][BN / 64], b
     constexpr int STAGE = TA::LDS_ELEMS + TB::LDS_ELEMS;
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, wm = wave >> 1, wn = wave & 1;
     if (nstage <= 0) return;
+    pa.init(k_begin);
+    pb.init(k_begin);
 
-    f32x4 ra[2][TA::PER_THREAD], rb[2][TB::PER_THREAD];
-    // prologue: stage 0 -> LDS buffer 0, stage 1 -> registers (slot 1)
-    pa.load(ra[0], k_begin);
-    pb.load(rb[0], k_begin);
-    pa.load(ra[1], k_begin + BK);
-    pb.load(rb[1], k_begin + BK);
-    TA::store(lds, ra[0]);
-    TB::store(lds + TA::LDS_ELEMS, rb[0]);
+    f32x4 ra[TA::PER_THREAD], rb[TB::PER_THREAD];
+    pa.load(ra, 0);
+    pb.load(rb, 0);
+    TA::store(lds, ra);
+    TB::store(lds + TA::LDS_ELEMS, rb);
+    pa.load(ra, 1);
+    pb.load(rb, 1);
     __syncthreads();
 
-    // steady state, two stages per trip so that register slots and LDS buffers are compile-time constants
     for (int s = 0; s < nstage; s += 2) {
-        // --- even stage s: compute buffer 0; register slot 1 holds stage s+1; fetch stage s+2 into slot 0
-        __builtin_amdgcn_sched_barrier(0);
-        pa.load(ra[0], k_begin + (s + 2) * BK);
-        pb.load(rb[0], k_begin + (s + 2) * BK);
-        __builtin_amdgcn_sched_barrier(0);
-        mma_stage<TA, TB, BK, MI, NI>(acc, lds, lds + TA::LDS_ELEMS, wm, wn, lane);
-        __builtin_amdgcn_sched_barrier(0);
-        TA::store(lds + STAGE, ra[1]);
-        TB::store(lds + STAGE + TA::LDS_ELEMS, rb[1]);
-        __syncthreads();
-        if (s + 1 >= nstage) break;
-        // --- odd stage s+1: compute buffer 1; slot 0 holds stage s+2; fetch stage s+3 into slot 1
-        __builtin_amdgcn_sched_barrier(0);
-        pa.load(ra[1], k_begin + (s + 3) * BK);
-        pb.load(rb[1], k_begin + (s + 3) * BK);
-        __builtin_amdgcn_sched_barrier(0);
-        mma_stage<TA, TB, BK, MI, NI>(acc, lds + STAGE, lds + STAGE + TA::LDS_ELEMS, wm, wn, lane);
-        __builtin_amdgcn_sched_barrier(0);
-        TA::store(lds, ra[0]);
-        TB::store(lds + TA::LDS_ELEMS, rb[0]);
-        __syncthreads();
+        // stage s lives in buffer 0 and the registers hold stage s+1; then the roles of the buffers swap
+        pipeline_stage<BK, MI, NI>(acc, lds, lds + STAGE, ra, rb, pa, pb, s + 2, wm, wn, lane);
+        pipeline_stage<BK, MI, NI>(acc, lds + STAGE, lds, ra, rb, pa, pb, s + 3, wm, wn, lane);
     }
 }
 
