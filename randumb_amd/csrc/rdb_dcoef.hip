@@ -53,8 +53,8 @@ __global__ __launch_bounds__(256, 1) void linear_dcoef_fast_kernel(DcoefParams p
     for (int mi = 0; mi < DC_BI / 64; ++mi)
 #pragma unroll
         for (int ni = 0; ni < DC_BO / 64; ++ni) acc[mi][ni] = zero16();
-    GlobalOperand<DC_BI, DC_BK, M_CONT> opx = {p.x, p.ldx, li0, p.in_f, t_end};
-    GlobalOperand<DC_BO, DC_BK, M_CONT> opdy = {p.dy, p.lddy, lo0, p.out_f, t_end};
+    GlobalOperand<DC_BI, DC_BK, M_CONT> opx = {p.x, p.ldx, li0, p.in_f, t_end, (int64_t)(p.tokens - 1) * p.ldx + p.in_f};
+    GlobalOperand<DC_BO, DC_BK, M_CONT> opdy = {p.dy, p.lddy, lo0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
     gemm_mainloop<DC_BI, DC_BO, DC_BK>(acc, lds, opx, opdy, t_begin, (t_end - t_begin + DC_BK - 1) / DC_BK);
 
     long long ts1 = __builtin_readcyclecounter();
@@ -151,7 +151,7 @@ int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, co
     if (d->act_dtype != RDB_BF16 || d->coef_rows == 0) return RDB_E_UNSUPPORTED;
     if (d->in_f % 8 || d->out_f % 8 || ldx % 8 || lddy % 8 || ((uintptr_t)x & 15) || ((uintptr_t)dy & 15)) return RDB_E_UNSUPPORTED;
     if (d->tokens < 1 || d->tokens > (1 << 30) || d->out_f > (1 << 30) || d->in_f > (1 << 30) || d->out_f * d->in_f > (1ll << 31) ||
-        d->tokens * lddy >= (1ll << 31) || d->tokens * ldx >= (1ll << 31))
+        d->tokens * lddy >= (1ll << 30) || d->tokens * ldx >= (1ll << 30))
         return RDB_E_UNSUPPORTED;
     DcoefParams p;
     p.dy = (const bf16_t *)dy;

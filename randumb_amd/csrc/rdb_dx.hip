@@ -42,9 +42,9 @@ __global__ __launch_bounds__(256, 1) void dx_dyc_kernel(DyCParams p)
 #pragma unroll
         for (int ni = 0; ni < K1_BT / 64; ++ni) acc[mi][ni] = zero16();
     // "A": C[o][m], tile rows = m (contiguous in memory), contraction index = o
-    GlobalOperand<K1_BC, K1_BK, M_CONT> opc = {p.coef, (int64_t)p.k, m0, p.k, p.out_f};
+    GlobalOperand<K1_BC, K1_BK, M_CONT> opc = {p.coef, (int64_t)p.k, m0, p.k, p.out_f, (int64_t)p.out_f * p.k};
     // "B": dy[tok][o], contraction index contiguous
-    GlobalOperand<K1_BT, K1_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f};
+    GlobalOperand<K1_BT, K1_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
     gemm_mainloop<K1_BC, K1_BT, K1_BK>(acc, lds, opc, opdy, 0, (p.out_f + K1_BK - 1) / K1_BK);
     // acc[mi][ni][j]: m = m0 + wm*64 + mi*32 + 8*(j/4) + 4*g + j%4, tok = tok0 + wn*64 + ni*32 + r
 #pragma unroll
@@ -93,7 +93,7 @@ __global__ __launch_bounds__(256, 1) void dx_tn_kernel(TNParams p)
     // "A": 2^31 * noise(i, m), rows = i, contraction = m; values for m >= k meet zero rows of t
     NoiseOperandRowsAreElements<K2_BI, K2_BK> opn = {i0, p.seed};
     // "B": t[tok][m]
-    GlobalOperand<K2_BT, K2_BK, K_CONT> opt = {p.t, (int64_t)p.k, tok0, p.tokens, p.k};
+    GlobalOperand<K2_BT, K2_BK, K_CONT> opt = {p.t, (int64_t)p.k, tok0, p.tokens, p.k, (int64_t)p.tokens * p.k};
     gemm_mainloop<K2_BI, K2_BT, K2_BK>(acc, lds, opn, opt, 0, (p.k + K2_BK - 1) / K2_BK);
     // acc[mi][ni][j]: i = i0 + wm*96 + mi*32 + 8*(j/4) + 4*g + j%4, tok = tok0 + wn*64 + ni*32 + r
 #pragma unroll
@@ -119,7 +119,7 @@ static bool dx_factored_ok(const rdb_linear_desc *d)
 {
     return d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16 && d->coef_rows != 0 && d->k % 8 == 0 && d->in_f % 8 == 0 &&
            d->out_f % 8 == 0 && d->k > 0 && d->tokens > 0 && d->tokens < (1 << 30) && d->in_f < (1 << 30) && d->out_f < (1 << 30) &&
-           d->k < (1 << 24) && d->tokens * d->k < (1ll << 31) && d->out_f * d->k < (1ll << 31);
+           d->k < (1 << 24) && d->tokens * d->k < (1ll << 30) && d->out_f * d->k < (1ll << 30);
 }
 
 int64_t linear_dx_factored_workspace(const rdb_linear_desc *d)
@@ -134,7 +134,7 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
 {
     if (!dx_factored_ok(d) || scale_bias) return RDB_E_UNSUPPORTED;  // the random-bias term is not low rank
     if (!workspace || workspace_bytes < linear_dx_factored_workspace(d) || ((uintptr_t)workspace & 15)) return RDB_E_UNSUPPORTED;
-    if (d->tokens * lddy >= (1ll << 31)) return RDB_E_UNSUPPORTED;
+    if (d->tokens * lddy >= (1ll << 30)) return RDB_E_UNSUPPORTED;
     if (lddy % 8 || lddx % 4 || ((uintptr_t)dy & 15) || ((uintptr_t)coef & 15) || ((uintptr_t)dx & 7)) return RDB_E_UNSUPPORTED;
     // only worth it when the factored form is cheaper than forming the weight
     if (d->algo == RDB_ALGO_AUTO && d->k * (d->in_f + d->out_f) >= d->in_f * d->out_f) return RDB_E_UNSUPPORTED;

@@ -25,8 +25,11 @@ __device__ long long *rdb_profile_ptr;
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
-// 16 bytes of zeros in device memory: the load target of operand pieces that lie outside their matrix.
-__device__ __align__(16) const uint32_t rdb_zero_piece[4] = {0u, 0u, 0u, 0u};
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+// Byte offset that lies outside every buffer the tile engine reads (operands are smaller than 2^31 bytes): a buffer load
+// at this offset fails the hardware bounds check and returns zeros, without a branch and without touching memory.
+constexpr uint32_t BUFFER_OOB = 0x80000000u;
 
 enum OperandLayout { K_CONT = 0, M_CONT = 1 };
 
@@ -47,12 +50,11 @@ template <int ROWS, int BK, int LAYOUT> struct OperandTile {
     static constexpr int PER_THREAD = (PIECES + 255) / 256;
     static_assert(PIECES % 256 == 0, "operand stage must split evenly over 256 threads");
 
-    // Per-thread description of the pieces it copies from global memory: element offset of each piece at stage 0, and
-    // whether its tile row lies inside the matrix.  Built once, before the main loop.
+    // Per-thread description of the pieces it copies from global memory: byte offset of each piece at stage 0 (BUFFER_OOB
+    // when its tile row lies outside the matrix) and its contraction offset inside a stage.  Built once, before the loop.
     struct Pieces {
-        int off[PER_THREAD];
-        int kk[PER_THREAD];    // contraction offset of the piece inside a stage
-        bool rowok[PER_THREAD];
+        uint32_t off[PER_THREAD];
+        int kk[PER_THREAD];
     };
     __device__ static __forceinline__ Pieces pieces(int64_t ld, int row0, int nrows, int k_begin)
     {
@@ -69,35 +71,22 @@ template <int ROWS, int BK, int LAYOUT> struct OperandTile {
                 k = idx / (ROWS / 8);
                 row = row0 + (idx % (ROWS / 8)) * 8;
             }
-            q.rowok[p] = row < nrows;
-            const int rr = q.rowok[p] ? row : 0;
             q.kk[p] = k;
-            q.off[p] = (LAYOUT == K_CONT) ? (int)(rr * ld) + k_begin + k : (int)((k_begin + k) * ld) + rr;
+            const uint32_t elem = (LAYOUT == K_CONT) ? (uint32_t)(row * ld) + k_begin + k : (uint32_t)((k_begin + k) * ld) + row;
+            q.off[p] = row < nrows ? elem * 2u : BUFFER_OOB;
         }
         return q;
     }
 
-    // Global -> registers for the stage whose first contraction index is k0 = k_begin + stage*BK; `adv` is the element
-    // offset of that stage relative to stage 0 (stage*BK for K_CONT, stage*BK*ld for M_CONT).  Pieces outside the matrix
-    // (row >= nrows or k >= klim) are redirected to 16 bytes of zeros, so nothing downstream of the load has to wait for
-    // it; the host guarantees that the contiguous axis is a multiple of 8, so a piece is entirely inside or outside.
-    __device__ static __forceinline__ void load(f32x4 (&regs)[PER_THREAD], const bf16_t *__restrict__ src, const Pieces &q, int adv, int k0,
-                                                int klim)
-    {
-#pragma unroll
-        for (int p = 0; p < PER_THREAD; ++p) {
-            const bool ok = q.rowok[p] && (k0 + q.kk[p] < klim);
-            const bf16_t *ptr = ok ? src + (q.off[p] + adv) : reinterpret_cast<const bf16_t *>(rdb_zero_piece);
-            regs[p] = *reinterpret_cast<const f32x4 *>(ptr);
-        }
-    }
-
-    __device__ static __forceinline__ void load_piece(f32x4 &reg, const bf16_t *__restrict__ src, const Pieces &q, int p, int adv, int k0,
+    // Global -> register for piece p of the stage whose first contraction index is k0; `adv` is the byte offset of that
+    // stage relative to stage 0.  A buffer load: pieces outside the matrix (row >= nrows or k >= klim) carry an out-of-range
+    // offset and come back as zeros.  The host guarantees that the contiguous axis is a multiple of 8, so a 16-byte piece is
+    // entirely inside or outside.
+    __device__ static __forceinline__ void load_piece(f32x4 &reg, __amdgpu_buffer_rsrc_t rsrc, const Pieces &q, int p, uint32_t adv, int k0,
                                                       int klim)
     {
-        const bool ok = q.rowok[p] && (k0 + q.kk[p] < klim);
-        const bf16_t *ptr = ok ? src + (q.off[p] + adv) : reinterpret_cast<const bf16_t *>(rdb_zero_piece);
-        reg = *reinterpret_cast<const f32x4 *>(ptr);
+        const uint32_t o = (k0 + q.kk[p] < klim) ? q.off[p] + adv : BUFFER_OOB;
+        reg = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)o, 0, 0));
     }
 
     // Registers -> LDS stage.
@@ -182,23 +171,27 @@ inline int xcd_grid_size(int total) { return ((total + 7) / 8) * 8; }
 // ----------------------------------------------------------------------------------------------- operand providers
 // A provider fills the registers of one pipeline stage: load(regs, k0) with k0 the stage's first contraction index.
 
-// Operand read from global memory (offsets are 32-bit: the host checks that the matrix has fewer than 2^31 elements).
+// Operand read from global memory through a buffer resource (the operand must be smaller than 2^31 bytes).
+// extent: number of elements from `src` that may be read (last row's end).
 template <int ROWS, int BK, int LAYOUT> struct GlobalOperand {
     typedef OperandTile<ROWS, BK, LAYOUT> Tile;
     const bf16_t *src;
     int64_t ld;
     int row0, nrows, klim;  // klim: first contraction index that must read as zero
+    int64_t extent;
     typename Tile::Pieces q;
+    __amdgpu_buffer_rsrc_t rsrc;
     int k_begin;
     __device__ __forceinline__ void init(int kb)
     {
         k_begin = kb;
         q = Tile::pieces(ld, row0, nrows, kb);
+        rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(src), 0, (int)(extent * 2), 0x00020000);
     }
     __device__ __forceinline__ void load_piece(f32x4 &reg, int p, int stage) const
     {
-        const int adv = (LAYOUT == K_CONT) ? stage * BK : (int)(stage * BK * ld);
-        Tile::load_piece(reg, src, q, p, adv, k_begin + stage * BK, klim);
+        const uint32_t adv = (LAYOUT == K_CONT) ? (uint32_t)(stage * BK * 2) : (uint32_t)(stage * BK * ld * 2);
+        Tile::load_piece(reg, rsrc, q, p, adv, k_begin + stage * BK, klim);
     }
     __device__ __forceinline__ void load(f32x4 (&regs)[Tile::PER_THREAD], int stage) const
     {
