@@ -31,7 +31,6 @@ __global__ __launch_bounds__(256, 1) void dx_dyc_kernel(DyCParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
-    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
     // work item = (token tile, coefficient tile), coefficient tile fastest: neighbours share the dy tile
     const int w = xcd_work_item(blockIdx.x, p.tiles_c * p.tiles_t);
     if (w >= p.tiles_c * p.tiles_t) return;
@@ -46,21 +45,7 @@ __global__ __launch_bounds__(256, 1) void dx_dyc_kernel(DyCParams p)
     // "B": dy[tok][o], contraction index contiguous
     GlobalOperand<K1_BT, K1_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
     gemm_mainloop<K1_BC, K1_BT, K1_BK>(acc, lds, opc, opdy, 0, (p.out_f + K1_BK - 1) / K1_BK);
-    // acc[mi][ni][j]: m = m0 + wm*64 + mi*32 + 8*(j/4) + 4*g + j%4, tok = tok0 + wn*64 + ni*32 + r
-#pragma unroll
-    for (int ni = 0; ni < K1_BT / 64; ++ni) {
-        const int tok = tok0 + wn * 64 + ni * 32 + r;
-        if (tok >= p.tokens) continue;
-#pragma unroll
-        for (int mi = 0; mi < K1_BC / 64; ++mi)
-#pragma unroll
-            for (int jq = 0; jq < 4; ++jq) {
-                const int m = m0 + wm * 64 + mi * 32 + 8 * jq + 4 * g;
-                if (m < p.k)  // k % 8 == 0, so four consecutive coefficients are inside together
-                    store4<bf16_t>(p.t + (int64_t)tok * p.k + m, acc[mi][ni][jq * 4 + 0], acc[mi][ni][jq * 4 + 1],
-                                   acc[mi][ni][jq * 4 + 2], acc[mi][ni][jq * 4 + 3]);
-            }
-    }
+    store_tile_bf16<K1_BC, K1_BT>(acc, lds, p.t, p.k, m0, p.k, tok0, p.tokens, 1.0f, nullptr);
 }
 
 // ----------------------------------------------------------------------------------------------- kernel 2: dx = t . N
@@ -80,7 +65,6 @@ __global__ __launch_bounds__(256, 1) void dx_tn_kernel(TNParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
-    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
     // work item = (token tile, feature tile), feature tile fastest: neighbours share the t tile
     const int w = xcd_work_item(blockIdx.x, p.tiles_i * p.tiles_t);
     if (w >= p.tiles_i * p.tiles_t) return;
@@ -95,23 +79,7 @@ __global__ __launch_bounds__(256, 1) void dx_tn_kernel(TNParams p)
     // "B": t[tok][m]
     GlobalOperand<K2_BT, K2_BK, K_CONT> opt = {p.t, (int64_t)p.k, tok0, p.tokens, p.k, (int64_t)p.tokens * p.k};
     gemm_mainloop<K2_BI, K2_BT, K2_BK>(acc, lds, opn, opt, 0, (p.k + K2_BK - 1) / K2_BK);
-    // acc[mi][ni][j]: i = i0 + wm*96 + mi*32 + 8*(j/4) + 4*g + j%4, tok = tok0 + wn*64 + ni*32 + r
-#pragma unroll
-    for (int ni = 0; ni < K2_BT / 64; ++ni) {
-        const int tok = tok0 + wn * 64 + ni * 32 + r;
-        if (tok >= p.tokens) continue;
-#pragma unroll
-        for (int mi = 0; mi < K2_BI / 64; ++mi)
-#pragma unroll
-            for (int jq = 0; jq < 4; ++jq) {
-                const int i = i0 + wm * 96 + mi * 32 + 8 * jq + 4 * g;
-                if (i < p.in_f) {  // in_f % 8 == 0
-                    const float sc = 4.656612873077392578125e-10f;
-                    store4<bf16_t>(p.dx + (int64_t)tok * p.lddx + i, acc[mi][ni][jq * 4 + 0] * sc, acc[mi][ni][jq * 4 + 1] * sc,
-                                   acc[mi][ni][jq * 4 + 2] * sc, acc[mi][ni][jq * 4 + 3] * sc);
-                }
-            }
-    }
+    store_tile_bf16<K2_BI, K2_BT>(acc, lds, p.dx, p.lddx, i0, p.in_f, tok0, p.tokens, 4.656612873077392578125e-10f, nullptr);
 }
 
 // ----------------------------------------------------------------------------------------------- host side
@@ -135,7 +103,7 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
     if (!dx_factored_ok(d) || scale_bias) return RDB_E_UNSUPPORTED;  // the random-bias term is not low rank
     if (!workspace || workspace_bytes < linear_dx_factored_workspace(d) || ((uintptr_t)workspace & 15)) return RDB_E_UNSUPPORTED;
     if (d->tokens * lddy >= (1ll << 30)) return RDB_E_UNSUPPORTED;
-    if (lddy % 8 || lddx % 4 || ((uintptr_t)dy & 15) || ((uintptr_t)coef & 15) || ((uintptr_t)dx & 7)) return RDB_E_UNSUPPORTED;
+    if (lddy % 8 || lddx % 8 || ((uintptr_t)dy & 15) || ((uintptr_t)coef & 15) || ((uintptr_t)dx & 15)) return RDB_E_UNSUPPORTED;
     // only worth it when the factored form is cheaper than forming the weight
     if (d->algo == RDB_ALGO_AUTO && d->k * (d->in_f + d->out_f) >= d->in_f * d->out_f) return RDB_E_UNSUPPORTED;
 
@@ -150,7 +118,8 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
     {
         typedef OperandTile<K1_BC, K1_BK, M_CONT> TA;
         typedef OperandTile<K1_BT, K1_BK, K_CONT> TB;
-        const size_t smem = 2 * (TA::LDS_ELEMS + TB::LDS_ELEMS) * sizeof(bf16_t);
+        size_t smem = 2 * (TA::LDS_ELEMS + TB::LDS_ELEMS) * sizeof(bf16_t);
+        if (smem < (size_t)K1_BT * (K1_BC + 8) * sizeof(bf16_t)) smem = (size_t)K1_BT * (K1_BC + 8) * sizeof(bf16_t);
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(dx_dyc_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return set_error((int)e, "dx_dyc_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
         p1.tiles_c = (int)cdiv(d->k, K1_BC);
@@ -170,7 +139,8 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
     {
         typedef OperandTile<K2_BI, K2_BK, K_CONT> TA;
         typedef OperandTile<K2_BT, K2_BK, K_CONT> TB;
-        const size_t smem = 2 * (TA::LDS_ELEMS + TB::LDS_ELEMS) * sizeof(bf16_t);
+        size_t smem = 2 * (TA::LDS_ELEMS + TB::LDS_ELEMS) * sizeof(bf16_t);
+        if (smem < (size_t)K2_BT * (K2_BI + 8) * sizeof(bf16_t)) smem = (size_t)K2_BT * (K2_BI + 8) * sizeof(bf16_t);
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(dx_tn_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         if (e != hipSuccess) return set_error((int)e, "dx_tn_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
         p2.tiles_i = (int)cdiv(d->in_f, K2_BI);

@@ -16,6 +16,7 @@
 #endif
 
 #include "rdb_common.hpp"
+#include "rdb_tile.hpp"
 
 namespace rdb {
 
@@ -342,6 +343,45 @@ __device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / 64][BN / 64], b
         pipeline_stage<BK, MI, NI>(acc, lds, lds + STAGE, ra, rb, pa, pb, s + 2, wm, wn, lane);
         pipeline_stage<BK, MI, NI>(acc, lds + STAGE, lds, ra, rb, pa, pb, s + 3, wm, wn, lane);
     }
+}
+
+// Writes the block's BM x BN accumulator tile D[a][b] as bf16 to out[(b0 + b) * ld + a0 + a] (rows of `out` run along a),
+// v = acc * scale (+ bias[a0 + a]).  The tile is staged through LDS (BN x (BM + 8) elements) so that the global stores are
+// 16 bytes wide and contiguous along each row.  Needs a0, na, ld multiples of 8 and a 16-byte aligned `out`.
+// All 256 threads must call; `lds` must be free on entry (the main loop ends with a barrier) and is free again on return.
+template <int BM, int BN>
+__device__ __forceinline__ void store_tile_bf16(const f32x16 (&acc)[BM / 64][BN / 64], bf16_t *__restrict__ lds, bf16_t *__restrict__ out,
+                                                int64_t ld, int a0, int na, int b0, int nb, float scale, const bf16_t *__restrict__ bias)
+{
+    constexpr int MI = BM / 64, NI = BN / 64, LDS_LD = BM + 8;
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int jq = 0; jq < 4; ++jq) {
+            const int a = wm * MI * 32 + mi * 32 + 8 * jq + 4 * g;
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (bias) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) bv[e] = (a0 + a + e < na) ? bf16_to_f32(bias[a0 + a + e]) : 0.0f;
+            }
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) {
+                const int b = wn * NI * 32 + ni * 32 + r;
+                store4<bf16_t>(lds + b * LDS_LD + a, acc[mi][ni][jq * 4 + 0] * scale + bv[0], acc[mi][ni][jq * 4 + 1] * scale + bv[1],
+                               acc[mi][ni][jq * 4 + 2] * scale + bv[2], acc[mi][ni][jq * 4 + 3] * scale + bv[3]);
+            }
+        }
+    __syncthreads();
+    constexpr int PIECES = BM * BN / 8;
+#pragma unroll
+    for (int p = 0; p < PIECES / 256; ++p) {
+        const int idx = p * 256 + t;
+        const int b = idx / (BM / 8), a = (idx % (BM / 8)) * 8;
+        if (b0 + b < nb && a0 + a < na)
+            *reinterpret_cast<f32x4 *>(out + (int64_t)(b0 + b) * ld + a0 + a) = *reinterpret_cast<const f32x4 *>(lds + b * LDS_LD + a);
+    }
+    __syncthreads();
 }
 
 }  // namespace rdb

@@ -265,6 +265,13 @@ static int check_desc(const char *who, const rdb_linear_desc *d)
 int linear_fwd_strip(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
                      const rdb_linear_desc *d, int num_cus, hipStream_t s);
 
+// rdb_factored.hip
+int64_t linear_factored_workspace(const rdb_linear_desc *d);
+int linear_fwd_factored(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
+                        const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s);
+int linear_dcoef_factored(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus,
+                          void *workspace, int64_t workspace_bytes, hipStream_t s);
+
 // rdb_dx.hip
 int64_t linear_dx_factored_workspace(const rdb_linear_desc *d);
 int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias,
@@ -322,21 +329,34 @@ using namespace rdb;
 extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
 {
     if (!d) return 0;
-    if (op == RDB_OP_LINEAR_BWD_DX && d->algo != RDB_ALGO_TILE && d->algo != RDB_ALGO_STRIP) return linear_dx_factored_workspace(d);
+    if (d->algo == RDB_ALGO_TILE || d->algo == RDB_ALGO_STRIP) return 0;
+    if (op == RDB_OP_LINEAR_BWD_DX) return linear_dx_factored_workspace(d);
+    if (op == RDB_OP_LINEAR_FWD) return linear_factored_workspace(d);
+    if (op == RDB_OP_LINEAR_BWD_DCOEF) {  // reads no coefficients: their dtype does not matter
+        rdb_linear_desc dd = *d;
+        dd.coef_dtype = RDB_BF16;
+        return linear_factored_workspace(&dd);
+    }
     return 0;
 }
 
 extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias,
                               const void *bias, const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
 {
-    (void)workspace;
-    (void)workspace_bytes;
     int rc = check_desc("rdb_linear_fwd", d);
     if (rc) return rc;
     if (d->tokens == 0 || d->out_f == 0) return RDB_OK;
     if (!y || (!x && d->in_f > 0) || (!coef && d->k > 0)) return set_error(RDB_E_NULL, "rdb_linear_fwd: y, x or coef is NULL");
     if (ldy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_fwd: leading dimension smaller than the row");
     hipStream_t s = (hipStream_t)stream;
+    if (d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) {
+        rc = linear_fwd_factored(y, ldy, x, ldx, coef, scale_bias, bias, d, workspace, workspace_bytes, s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+        if (d->algo == RDB_ALGO_FACTORED)
+            return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd: the factored algorithm needs matrix-coef in bf16, bf16 activations, no "
+                                                "scale_bias, sizes that are multiples of 8, aligned rows and a workspace of "
+                                                "rdb_linear_workspace_bytes() bytes");
+    }
     if (d->algo != RDB_ALGO_TILE) {
         rc = linear_fwd_strip(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
@@ -401,8 +421,6 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
 extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const void *dy, int64_t lddy, const void *x, int64_t ldx,
                                     const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
 {
-    (void)workspace;
-    (void)workspace_bytes;
     int rc = check_desc("rdb_linear_bwd_dcoef", d);
     if (rc) return rc;
     const int64_t ncoef = (d->coef_rows ? d->coef_rows : 1) * d->k;
@@ -421,6 +439,14 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
     if (d->tokens == 0 || d->in_f == 0 || d->out_f == 0 || (ncoef == 0 && !d_scale_bias)) return RDB_OK;
     if (!dy || !x) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef: dy or x is NULL");
     if (lddy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dcoef: leading dimension smaller than the row");
+    if ((d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) && !d_scale_bias) {
+        rc = linear_dcoef_factored(dcoef, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
+    if (d->algo == RDB_ALGO_FACTORED)
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dcoef: the factored algorithm needs matrix-coef, bf16 activations, no scale_bias "
+                                            "gradient, sizes that are multiples of 8, aligned rows and a workspace of "
+                                            "rdb_linear_workspace_bytes() bytes");
     if (d->algo != RDB_ALGO_TILE) {
         rc = linear_dcoef_fast(dcoef, d_scale_bias, dy, lddy, x, ldx, d, num_compute_units(), s);
         if (rc != RDB_E_UNSUPPORTED) return rc;

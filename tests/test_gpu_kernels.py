@@ -304,7 +304,7 @@ BWD_SHAPES = [
 
 @pytest.mark.parametrize("T,in_f,out_f,k,seed", BWD_SHAPES)
 def test_linear_bwd_fast_kernels(hip, oracle, T, in_f, out_f, k, seed):
-    from randumb_amd._lib import RDB_ALGO_FACTORED, RDB_ALGO_TILE
+    from randumb_amd._lib import RDB_ALGO_FACTORED, RDB_ALGO_STRIP, RDB_ALGO_TILE
 
     print(f"case bwd fast T={T} in={in_f} out={out_f} k={k}", flush=True)
     x, dy, coef = _inputs(T, in_f, out_f, k, True, torch.bfloat16, seed)
@@ -319,6 +319,22 @@ def test_linear_bwd_fast_kernels(hip, oracle, T, in_f, out_f, k, seed):
     assert rel_l2(cpu(dc), want_dc) < BF16_TOL
     dc_ref, _ = hip.linear_bwd_dcoef(dyc, xc, k, out_f, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_TILE)
     assert rel_l2(cpu(dc), cpu(dc_ref)) < 1e-2
+    dc_f, _ = hip.linear_bwd_dcoef(dyc, xc, k, out_f, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    assert dc_f.shape == (out_f, k) and rel_l2(cpu(dc_f), want_dc) < BF16_TOL
+    dc_s, _ = hip.linear_bwd_dcoef(dyc, xc, k, out_f, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_STRIP)   # dW-tile kernel
+    assert rel_l2(cpu(dc_s), want_dc) < BF16_TOL
+    dc_a, _ = hip.linear_bwd_dcoef(dyc, xc, k, out_f, in_f, out_f, in_f, 1, seed)
+    assert rel_l2(cpu(dc_a), want_dc) < BF16_TOL
+    # forward: factored vs the oracle, vs the weight-forming kernel, with and without bias
+    want_y = oracle.linear_fwd(x.float().numpy(), coef.float().numpy(), in_f, out_f, seed)
+    y_f = hip.linear_fwd(xc, cc, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    assert y_f.shape == (T, out_f) and rel_l2(cpu(y_f), want_y) < BF16_TOL
+    y_t = hip.linear_fwd(xc, cc, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_TILE)
+    assert rel_l2(cpu(y_f), cpu(y_t)) < 1e-2
+    bias = torch.randn(out_f).bfloat16()
+    want_yb = oracle.linear_fwd(x.float().numpy(), coef.float().numpy(), in_f, out_f, seed, bias=bias.float().numpy())
+    assert rel_l2(cpu(hip.linear_fwd(xc, cc, in_f, out_f, in_f, 1, seed, bias=bias.cuda(), algo=RDB_ALGO_FACTORED)), want_yb) < BF16_TOL
+    assert rel_l2(cpu(hip.linear_fwd(xc, cc, in_f, out_f, in_f, 1, seed, bias=bias.cuda())), want_yb) < BF16_TOL
     want_ds = float(oracle.scale_bias_bwd(dW.astype(np.float32), seed)[0])
     assert abs(float(dsb) - want_ds) < 2e-2 * max(1.0, abs(want_ds), float(np.abs(dW).sum()) ** 0.5)
 
@@ -335,3 +351,12 @@ def test_factored_dx_needs_what_it_says(hip):
     with pytest.raises(RandumbHipError):
         hip.linear_bwd_dx(dy, C, 40, 48, 40, 1, 0, scale_bias=sb, algo=RDB_ALGO_FACTORED)
     assert hip.linear_bwd_dx(dy, C, 40, 48, 40, 1, 0, scale_bias=sb).shape == (64, 40)
+    x = torch.randn(64, 40, device="cuda").bfloat16()
+    with pytest.raises(RandumbHipError):
+        hip.linear_fwd(x, c, 40, 48, 40, 1, 0, algo=RDB_ALGO_FACTORED)
+    with pytest.raises(RandumbHipError):
+        hip.linear_fwd(x, C, 40, 48, 40, 1, 0, scale_bias=sb, algo=RDB_ALGO_FACTORED)
+    with pytest.raises(RandumbHipError):
+        hip.linear_bwd_dcoef(dy, x, 16, 0, 40, 48, 40, 1, 0, algo=RDB_ALGO_FACTORED)
+    with pytest.raises(RandumbHipError):
+        hip.linear_bwd_dcoef(dy, x, 16, 48, 40, 48, 40, 1, 0, want_scale_bias_grad=True, algo=RDB_ALGO_FACTORED)
