@@ -5,12 +5,18 @@ Workload (the configuration the headline metric is quoted on): one layer at the 
 shape, in = 768 -> out = 3072, coef dim k = 256 (matrix-coef, C is [3072 x 256]), 8192 tokens, bf16
 activations with fp32 accumulation, x ~ N(0,1), dy ~ N(0,1), C ~ N(0, 3*0.02^2/k), seed 0.  Synthetic data.
 
-A "step" is one pass of the hot path: y = x W^T, dx = dy W, dC = (dy^T x) N^T, all three through the C ABI of
-librandumb_hip.so with inputs already resident in HBM.  The printed JSON line reports
-  value        algorithmic TFLOP/s of the whole step, F = 6*T*in*out + 6*out*in*k
-  roofline     the slowest of the three kernels against the dense bf16 MFMA peak, from HIP-event timing
+A "step" is one pass of the hot path, y = x W^T, dx = dy W, dC = (dy^T x) N^T with W = C N never stored, through
+the C ABI of librandumb_hip.so with inputs already resident in HBM, the way a training step calls it:
+  forward   rdb_linear_project (z = x N^T, kept for the backward pass in place of x) + rdb_linear_fwd_projected
+  backward  rdb_linear_bwd_dx + rdb_linear_bwd_dcoef_projected (reuses z)
+The printed JSON line reports
+  value        algorithmic TFLOP/s of the whole step, F = 6*T*in*out + 6*out*in*k (three dense products plus the
+               weight generation per direction and the dC contraction).  The kernels use W = C N associatively and
+               execute fewer flops than F (config.executed_gflop_per_step); both figures are printed.
+  roofline     the slowest of forward / dx / dcoef against the dense bf16 MFMA peak, from HIP-event timing
   cpu_baseline the CPU restatement (materialise-then-matmul: oracle C + torch.matmul fp32) on the host cores
-  compare      the same products done as materialise-to-HBM + dense GEMM on the GPU, and a plain dense GEMM
+  compare      the one-call entry points (z recomputed in the backward pass), the kernels that do form W tiles on
+               chip, materialise-to-HBM + dense GEMM on the GPU, and a plain dense GEMM
 """
 import argparse
 import ctypes
@@ -27,16 +33,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 T, IN_F, OUT_F, K, SEED = 8192, 768, 3072, 256, 0
 
 
-def flops_fwd():
-    return 2.0 * T * IN_F * OUT_F + 2.0 * OUT_F * IN_F * K
-
-
-def flops_dx():
-    return 2.0 * T * IN_F * OUT_F + 2.0 * OUT_F * IN_F * K
-
-
-def flops_dcoef():
-    return 2.0 * T * IN_F * OUT_F + 2.0 * OUT_F * IN_F * K
+F_PER_PRODUCT = 2.0 * T * IN_F * OUT_F + 2.0 * OUT_F * IN_F * K      # one dense product + one W generation / dC contraction
+F_STEP = 3.0 * F_PER_PRODUCT
+# what the factored kernels execute: z, y, t, dx, dC products (z once per step)
+EXEC_STEP = 2.0 * T * K * (IN_F + OUT_F) + 2.0 * T * K * (OUT_F + IN_F) + 2.0 * T * K * OUT_F
 
 
 def main():
@@ -82,20 +82,48 @@ def main():
                                                                      _lib.RDB_OP_LINEAR_BWD_DCOEF))
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
     pws = vp(ws.data_ptr())
+    z_bytes = L.rdb_linear_projection_bytes(dref)
+    assert z_bytes == T * K * 2, "the projected form must apply to the headline workload"
+    z = torch.empty(T, K, dtype=torch.bfloat16, device=dev)
+    pz = vp(z.data_ptr())
 
-    def k_fwd():
-        _lib.check(L.rdb_linear_fwd(py, OUT_F, px, IN_F, pC, None, None, dref, pws, ws_bytes, stream), "rdb_linear_fwd")
+    def k_project():
+        _lib.check(L.rdb_linear_project(pz, px, IN_F, dref, stream), "rdb_linear_project")
+
+    def k_fwd_projected():
+        _lib.check(L.rdb_linear_fwd_projected(py, OUT_F, pz, pC, None, dref, stream), "rdb_linear_fwd_projected")
 
     def k_dx():
         _lib.check(L.rdb_linear_bwd_dx(pdx, IN_F, pdy, OUT_F, pC, None, dref, pws, ws_bytes, stream), "rdb_linear_bwd_dx")
 
-    def k_dcoef():
-        _lib.check(L.rdb_linear_bwd_dcoef(pdC, None, pdy, OUT_F, px, IN_F, dref, pws, ws_bytes, stream), "rdb_linear_bwd_dcoef")
+    def k_dcoef_projected():
+        _lib.check(L.rdb_linear_bwd_dcoef_projected(pdC, pdy, OUT_F, pz, dref, stream), "rdb_linear_bwd_dcoef_projected")
+
+    def k_fwd():
+        k_project()
+        k_fwd_projected()
 
     def step():
         k_fwd()
         k_dx()
-        k_dcoef()
+        k_dcoef_projected()
+
+    # the one-call entry points: the same kernels, z recomputed into the workspace by the coefficient gradient
+    def make_onecall(algo):
+        dd = _lib.LinearDesc.from_buffer_copy(d)
+        dd.algo = algo
+        r = ctypes.byref(dd)
+
+        def fwd():
+            _lib.check(L.rdb_linear_fwd(py, OUT_F, px, IN_F, pC, None, None, r, pws, ws_bytes, stream), "rdb_linear_fwd")
+
+        def dxf():
+            _lib.check(L.rdb_linear_bwd_dx(pdx, IN_F, pdy, OUT_F, pC, None, r, pws, ws_bytes, stream), "rdb_linear_bwd_dx")
+
+        def dcf():
+            _lib.check(L.rdb_linear_bwd_dcoef(pdC, None, pdy, OUT_F, px, IN_F, r, pws, ws_bytes, stream), "rdb_linear_bwd_dcoef")
+
+        return fwd, dxf, dcf, dd
 
     for _ in range(args.warmup):
         step()
@@ -106,10 +134,10 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
-    F = flops_fwd() + flops_dx() + flops_dcoef()
+    F = F_STEP
     value = F / (ms_per_step * 1e-3) / 1e12
 
-    # per-kernel durations from HIP events recorded on the stream the kernels are launched on
+    # per-call durations from HIP events recorded on the stream the kernels are launched on
     def event_ms(fn, iters):
         for _ in range(3):
             fn()
@@ -124,18 +152,25 @@ def main():
         return e0.elapsed_time(e1) / iters
 
     iters = max(10, min(args.steps, 50))
-    kern = {
-        "linear_fwd": (event_ms(k_fwd, iters), flops_fwd()),
-        "linear_bwd_dx": (event_ms(k_dx, iters), flops_dx()),
-        "linear_bwd_dcoef": (event_ms(k_dcoef, iters), flops_dcoef()),
+    calls = {
+        "rdb_linear_project": event_ms(k_project, iters),
+        "rdb_linear_fwd_projected": event_ms(k_fwd_projected, iters),
+        "rdb_linear_bwd_dx": event_ms(k_dx, iters),
+        "rdb_linear_bwd_dcoef_projected": event_ms(k_dcoef_projected, iters),
     }
-    dom = max(kern, key=lambda n: kern[n][0])
-    dom_ms, dom_flops = kern[dom]
-    achieved = dom_flops / (dom_ms * 1e-3) / 1e12
+    products = {   # each carries one third of F
+        "forward (factored_z_kernel + factored_y_kernel)": calls["rdb_linear_project"] + calls["rdb_linear_fwd_projected"],
+        "dx (dx_dyc_kernel + dx_tn_kernel)": calls["rdb_linear_bwd_dx"],
+        "dcoef (fill_zero_kernel + factored_dc_kernel)": calls["rdb_linear_bwd_dcoef_projected"],
+    }
+    dom = max(products, key=lambda n: products[n])
+    dom_ms = products[dom]
+    achieved = F_PER_PRODUCT / (dom_ms * 1e-3) / 1e12
     roofline = {
         "bound": "mfma", "kernel": dom, "achieved": round(achieved, 3), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 5), "traffic": None, "avg_kernel_ms": round(dom_ms, 5),
-        "kernels_ms": {n: round(v[0], 5) for n, v in kern.items()},
+        "algorithmic_gflop_per_launch": round(F_PER_PRODUCT / 1e9, 3),
+        "calls_ms": {n: round(v, 5) for n, v in calls.items()},
     }
 
     compare = None
@@ -155,7 +190,15 @@ def main():
         def dense_step():
             return x @ Wd.t(), dy @ Wd, dy.t() @ x
 
+        def onecall_ms(algo):
+            fwd, dxf, dcf, _keep = make_onecall(algo)
+            return {"fwd": round(event_ms(fwd, 20), 4), "dx": round(event_ms(dxf, 20 if algo != _lib.RDB_ALGO_TILE else 3), 4),
+                    "dcoef": round(event_ms(dcf, 20), 4)}
+
         compare = {
+            "one_call_entry_points_ms": onecall_ms(_lib.RDB_ALGO_AUTO),
+            "w_tiles_formed_on_chip_ms": {"fwd_strip": onecall_ms(_lib.RDB_ALGO_STRIP)["fwd"], "dcoef_dw_tile": onecall_ms(_lib.RDB_ALGO_STRIP)["dcoef"],
+                                          "dx_tile": onecall_ms(_lib.RDB_ALGO_TILE)["dx"]},
             "materialize_then_gemm_ms": round(event_ms(mat_gemm_step, 10), 4),
             "dense_gemm_only_ms": round(event_ms(dense_step, 20), 4),
         }
@@ -196,7 +239,9 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "single fused layer 768->3072, k=256 matrix-coef, 8192 tokens, bf16 act / fp32 accumulate, fwd+dx+dcoef",
-                   "tokens": T, "in": IN_F, "out": OUT_F, "k": K, "seed": SEED, "algorithmic_gflop_per_step": round(F / 1e9, 3)},
+                   "tokens": T, "in": IN_F, "out": OUT_F, "k": K, "seed": SEED, "algorithmic_gflop_per_step": round(F / 1e9, 3),
+                   "executed_gflop_per_step": round(EXEC_STEP / 1e9, 3), "executed_tflops": round(EXEC_STEP / (ms_per_step * 1e-3) / 1e12, 3),
+                   "algorithm": "factored: y=(x N^T) C^T, dx=(dy C) N, dC=dy^T (x N^T); z = x N^T computed once per step"},
         "frac_of_mfma_peak": round(value / MFMA_BF16_PEAK_TFLOPS, 5),
         "roofline": roofline, "cpu_baseline": cpu_baseline, "compare": compare,
     }

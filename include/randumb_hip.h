@@ -136,8 +136,10 @@ enum {
     RDB_ALGO_TILE = 1, /* regenerate W blocks in LDS per output block, contract with MFMA (any shape/dtype) */
     RDB_ALGO_STRIP = 2, /* forward only: build a whole strip W[strip, 0:in] in LDS once per workgroup, then stream the
                            tokens through it (matrix-coef, bf16, strip must fit LDS) */
-    RDB_ALGO_FACTORED = 3 /* matrix-coef only: use W = C.N associatively, e.g. dx = (dy.C).N, so that no weight tile is
-                             formed at all; the [tokens x k] intermediate lives in the caller's workspace */
+    RDB_ALGO_FACTORED = 3 /* matrix-coef, bf16 only: use W = C.N associatively so that no weight tile is formed at all:
+                             y = (x.N^T).C^T, dx = (dy.C).N, dcoef = dy^T.(x.N^T); the [tokens x k] intermediate lives
+                             in the caller's workspace.  With RDB_ALGO_STRIP the coefficient gradient runs the kernel
+                             that forms dW tiles and contracts them with regenerated noise on chip. */
 };
 
 enum { RDB_OP_LINEAR_FWD = 0, RDB_OP_LINEAR_BWD_DX = 1, RDB_OP_LINEAR_BWD_DCOEF = 2 };
@@ -168,6 +170,33 @@ int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t lddy, cons
 int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const void *dy, int64_t lddy, const void *x,
                          int64_t ldx, const rdb_linear_desc *desc, void *workspace, int64_t workspace_bytes,
                          void *stream);
+
+/* -------------------------------------------------------------------------- fused linear, projected form
+ * For matrix-coef layers with bf16 activations, z = x . N^T ([tokens x k], bf16: the activations projected onto the k
+ * noise directions of this layer's weight) is all that the forward product and the coefficient gradient need of x:
+ *   y = z . C^T (+ bias)        dcoef = dy^T . z
+ * rdb_linear_fwd and rdb_linear_bwd_dcoef compute z into their workspace on every call.  A training step can instead
+ * compute it once, keep it from the forward to the backward pass in place of x (it is k/in_f of the size of x) and
+ * call the two consumers below.  Replaces, like rdb_linear_fwd / rdb_linear_bwd_dcoef, materialize() + dense product
+ * (R.py:942-952) and MmBackward's dW followed by materialize_bwd (R.py:979-990, 304-359); the tensor autograd saves
+ * for the backward pass (there: x, with W re-materialised) becomes z.
+ * Needs: coef_rows == out_f, act_dtype RDB_BF16, tokens/in_f/out_f/k > 0, in_f, out_f, k multiples of 8,
+ * tokens*k < 2^30, 16-byte aligned pointers, leading dimensions multiples of 8; otherwise RDB_E_UNSUPPORTED. */
+
+/* Bytes of z for `desc` (tokens*k*2), or 0 when the projected form does not apply to it. */
+int64_t rdb_linear_projection_bytes(const rdb_linear_desc *desc);
+
+/* z[t, m] = sum_i x[t, i] * noise(PRIME*i + m), rounded to bf16 once. */
+int rdb_linear_project(void *z, const void *x, int64_t ldx, const rdb_linear_desc *desc, void *stream);
+
+/* y[t, o] = sum_m z[t, m] * coef[o, m] (+ bias[o]); coef must be bf16. */
+int rdb_linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, const void *bias,
+                             const rdb_linear_desc *desc, void *stream);
+
+/* dcoef[o, m] = sum_t dy[t, o] * z[t, m]; fp32 [out_f x k], OVERWRITTEN; partial sums over token ranges are combined
+ * with fp32 atomics. */
+int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *z,
+                                   const rdb_linear_desc *desc, void *stream);
 
 #ifdef __cplusplus
 }

@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256, 1) void linear_dcoef_fast_kernel(DcoefParams p
         for (int ni = 0; ni < DC_BO / 64; ++ni) acc[mi][ni] = zero16();
     GlobalOperand<DC_BI, DC_BK, M_CONT> opx = {p.x, p.ldx, li0, p.in_f, t_end, (int64_t)(p.tokens - 1) * p.ldx + p.in_f};
     GlobalOperand<DC_BO, DC_BK, M_CONT> opdy = {p.dy, p.lddy, lo0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
-    gemm_mainloop<DC_BI, DC_BO, DC_BK>(acc, lds, opx, opdy, t_begin, (t_end - t_begin + DC_BK - 1) / DC_BK);
+    gemm_mainloop<DC_BI, DC_BO, DC_BK, 1, 1>(acc, lds, opx, opdy, t_begin, (t_end - t_begin + DC_BK - 1) / DC_BK);
 
     long long ts1 = __builtin_readcyclecounter();
     // dW tile -> LDS as Ws[o][i] (bf16, i contiguous).  acc[mi][ni][j]: i = wm*96 + mi*32 + 8*(j/4) + 4*g + j%4, o = wn*96 + ni*32 + r

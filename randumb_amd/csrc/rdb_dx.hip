@@ -14,9 +14,12 @@
 
 namespace rdb {
 
+constexpr int X_BK = 64;
+
 // ----------------------------------------------------------------------------------------------- kernel 1: t = dy . C
-// tile: 128 coefficient columns (engine rows "m") x 128 tokens (engine rows "n"), contraction over out_f
-constexpr int K1_BC = 128, K1_BT = 128, K1_BK = 64;
+// tile: 128 coefficient columns (engine rows "a") x 64 tokens (engine rows "b"), contraction over out_f.  The output is
+// small (tokens x k), so the token tile is kept short to have a block for every compute unit; loads run two stages ahead.
+constexpr int K1_BC = 128, K1_BT = 64;
 
 struct DyCParams {
     const bf16_t *dy;
@@ -27,7 +30,7 @@ struct DyCParams {
     int tiles_c, tiles_t;
 };
 
-__global__ __launch_bounds__(256, 1) void dx_dyc_kernel(DyCParams p)
+__global__ __launch_bounds__(256, 2) void dx_dyc_kernel(DyCParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
@@ -41,16 +44,16 @@ __global__ __launch_bounds__(256, 1) void dx_dyc_kernel(DyCParams p)
 #pragma unroll
         for (int ni = 0; ni < K1_BT / 64; ++ni) acc[mi][ni] = zero16();
     // "A": C[o][m], tile rows = m (contiguous in memory), contraction index = o
-    GlobalOperand<K1_BC, K1_BK, M_CONT> opc = {p.coef, (int64_t)p.k, m0, p.k, p.out_f, (int64_t)p.out_f * p.k};
+    GlobalOperand<K1_BC, X_BK, M_CONT> opc = {p.coef, (int64_t)p.k, m0, p.k, p.out_f, (int64_t)p.out_f * p.k};
     // "B": dy[tok][o], contraction index contiguous
-    GlobalOperand<K1_BT, K1_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
-    gemm_mainloop<K1_BC, K1_BT, K1_BK>(acc, lds, opc, opdy, 0, (p.out_f + K1_BK - 1) / K1_BK);
+    GlobalOperand<K1_BT, X_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
+    gemm_mainloop<K1_BC, K1_BT, X_BK, 2, 2>(acc, lds, opc, opdy, 0, (p.out_f + X_BK - 1) / X_BK);
     store_tile_bf16<K1_BC, K1_BT>(acc, lds, p.t, p.k, m0, p.k, tok0, p.tokens, 1.0f, nullptr);
 }
 
 // ----------------------------------------------------------------------------------------------- kernel 2: dx = t . N
-// tile: 192 input features (engine rows "m", hashed operand) x 128 tokens (engine rows "n"), contraction over k
-constexpr int K2_BI = 192, K2_BT = 128, K2_BK = 64;
+// tile: 192 input features (engine rows "a", hashed operand) x 128 tokens (engine rows "b"), contraction over k
+constexpr int K2_BI = 192, K2_BT = 128;
 
 struct TNParams {
     const bf16_t *t;
@@ -75,10 +78,10 @@ __global__ __launch_bounds__(256, 1) void dx_tn_kernel(TNParams p)
 #pragma unroll
         for (int ni = 0; ni < K2_BT / 64; ++ni) acc[mi][ni] = zero16();
     // "A": 2^31 * noise(i, m), rows = i, contraction = m; values for m >= k meet zero rows of t
-    NoiseOperandRowsAreElements<K2_BI, K2_BK> opn = {i0, p.seed};
+    NoiseOperandRowsAreElements<K2_BI, X_BK> opn = {i0, p.seed};
     // "B": t[tok][m]
-    GlobalOperand<K2_BT, K2_BK, K_CONT> opt = {p.t, (int64_t)p.k, tok0, p.tokens, p.k, (int64_t)p.tokens * p.k};
-    gemm_mainloop<K2_BI, K2_BT, K2_BK>(acc, lds, opn, opt, 0, (p.k + K2_BK - 1) / K2_BK);
+    GlobalOperand<K2_BT, X_BK, K_CONT> opt = {p.t, (int64_t)p.k, tok0, p.tokens, p.k, (int64_t)p.tokens * p.k};
+    gemm_mainloop<K2_BI, K2_BT, X_BK, 1, 1>(acc, lds, opn, opt, 0, (p.k + X_BK - 1) / X_BK);
     store_tile_bf16<K2_BI, K2_BT>(acc, lds, p.dx, p.lddx, i0, p.in_f, tok0, p.tokens, 4.656612873077392578125e-10f, nullptr);
 }
 
@@ -115,19 +118,11 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
     p1.tokens = (int)d->tokens;
     p1.out_f = (int)d->out_f;
     p1.k = (int)d->k;
-    {
-        typedef OperandTile<K1_BC, K1_BK, M_CONT> TA;
-        typedef OperandTile<K1_BT, K1_BK, K_CONT> TB;
-        size_t smem = 2 * (TA::LDS_ELEMS + TB::LDS_ELEMS) * sizeof(bf16_t);
-        if (smem < (size_t)K1_BT * (K1_BC + 8) * sizeof(bf16_t)) smem = (size_t)K1_BT * (K1_BC + 8) * sizeof(bf16_t);
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(dx_dyc_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return set_error((int)e, "dx_dyc_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
-        p1.tiles_c = (int)cdiv(d->k, K1_BC);
-        p1.tiles_t = (int)cdiv(d->tokens, K1_BT);
-        dx_dyc_kernel<<<xcd_grid_size(p1.tiles_c * p1.tiles_t), 256, smem, s>>>(p1);
-        int rc = check_launch("dx_dyc_kernel");
-        if (rc) return rc;
-    }
+    p1.tiles_c = (int)cdiv(d->k, K1_BC);
+    p1.tiles_t = (int)cdiv(d->tokens, K1_BT);
+    int rc = launch_engine(dx_dyc_kernel, p1, p1.tiles_c * p1.tiles_t, engine_smem<K1_BC, K1_BT, X_BK, M_CONT, K_CONT>(), s, "dx_dyc_kernel");
+    if (rc) return rc;
+
     TNParams p2;
     p2.t = (const bf16_t *)workspace;
     p2.dx = (bf16_t *)dx;
@@ -136,18 +131,9 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
     p2.in_f = (int)d->in_f;
     p2.k = (int)d->k;
     p2.seed = d->seed;
-    {
-        typedef OperandTile<K2_BI, K2_BK, K_CONT> TA;
-        typedef OperandTile<K2_BT, K2_BK, K_CONT> TB;
-        size_t smem = 2 * (TA::LDS_ELEMS + TB::LDS_ELEMS) * sizeof(bf16_t);
-        if (smem < (size_t)K2_BT * (K2_BI + 8) * sizeof(bf16_t)) smem = (size_t)K2_BT * (K2_BI + 8) * sizeof(bf16_t);
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(dx_tn_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return set_error((int)e, "dx_tn_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
-        p2.tiles_i = (int)cdiv(d->in_f, K2_BI);
-        p2.tiles_t = (int)cdiv(d->tokens, K2_BT);
-        dx_tn_kernel<<<xcd_grid_size(p2.tiles_i * p2.tiles_t), 256, smem, s>>>(p2);
-        return check_launch("dx_tn_kernel");
-    }
+    p2.tiles_i = (int)cdiv(d->in_f, K2_BI);
+    p2.tiles_t = (int)cdiv(d->tokens, K2_BT);
+    return launch_engine(dx_tn_kernel, p2, p2.tiles_i * p2.tiles_t, engine_smem<K2_BI, K2_BT, X_BK, K_CONT, K_CONT>(), s, "dx_tn_kernel");
 }
 
 }  // namespace rdb

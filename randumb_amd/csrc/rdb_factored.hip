@@ -1,24 +1,26 @@
 // Forward and coefficient gradient of the fused linear layer, matrix-coef + bf16, "factored" algorithm.
 //
 // W = C . N has rank k, so with k < in*out/(in+out) it is cheaper never to form a weight tile:
-//   forward  y  = x . W^T   = (x . N^T) . C^T      z = x . N^T is [tokens x k]
+//   forward  y  = x . W^T   = (x . N^T) . C^T      z = x . N^T is [tokens x k], the "projection" of the activations
 //   dcoef    dC = dW . N^T  = dy^T . (x . N^T) = dy^T . z
 // Three kernels on the tile engine:
 //   z_kernel   z[tok, m]  = sum_i x[tok, i] * noise(PRIME*i + m)   noise hashed into the pipeline, interleaved with the MFMAs
 //   y_kernel   y[tok, o]  = sum_m z[tok, m] * C[o, m] (+ bias[o])  dense
 //   dc_kernel  dC[o, m]  += sum_tok dy[tok, o] * z[tok, m]         dense, token range split over blocks, fp32 atomics
-// z lives in the caller's workspace as bf16.  Replaces materialize() + dense product (src/rten_cpp/RandumbTensor.py:942-946)
-// and MmBackward's dW followed by materialize_bwd (RandumbTensor.py:979-990, 304-359).
+// z is bf16; it lives in the caller's workspace, or in a buffer the caller keeps from the forward to the backward pass (it
+// is all the backward pass needs of x, at k/in_f of its size).  Replaces materialize() + dense product
+// (src/rten_cpp/RandumbTensor.py:942-946) and MmBackward's dW followed by materialize_bwd (RandumbTensor.py:979-990, 304-359).
 #include "rdb_gemm.hpp"
 #include "rdb_tile.hpp"
 
 namespace rdb {
 
 constexpr float INV_2_31 = 4.656612873077392578125e-10f;
+constexpr int F_BK = 64;
 
 // ----------------------------------------------------------------------------------------------- z = x . N^T
-// tile: 64 coefficients (engine rows "a", hashed) x 256 tokens (engine rows "b"), contraction over in_f
-constexpr int KZ_BM = 64, KZ_BT = 256, KZ_BK = 64;
+// tile: 64 coefficients (engine rows "a", hashed) x 128 tokens (engine rows "b"), contraction over in_f; two blocks per CU
+constexpr int KZ_BM = 64, KZ_BT = 128;
 
 struct ZParams {
     const bf16_t *x;
@@ -29,7 +31,7 @@ struct ZParams {
     uint32_t seed;
 };
 
-__global__ __launch_bounds__(256, 1) void factored_z_kernel(ZParams p)
+__global__ __launch_bounds__(256, 2) void factored_z_kernel(ZParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
@@ -43,15 +45,16 @@ __global__ __launch_bounds__(256, 1) void factored_z_kernel(ZParams p)
 #pragma unroll
         for (int ni = 0; ni < KZ_BT / 64; ++ni) acc[mi][ni] = zero16();
     // "A": 2^31 * noise(i, m), rows = m, contraction = i; values for i >= in_f meet zero columns of x
-    NoiseOperandRowsAreCoefs<KZ_BM, KZ_BK> opn = {m0, p.seed};
-    GlobalOperand<KZ_BT, KZ_BK, K_CONT> opx = {p.x, p.ldx, tok0, p.tokens, p.in_f, (int64_t)(p.tokens - 1) * p.ldx + p.in_f};
-    gemm_mainloop<KZ_BM, KZ_BT, KZ_BK>(acc, lds, opn, opx, 0, (p.in_f + KZ_BK - 1) / KZ_BK);
+    NoiseOperandRowsAreCoefs<KZ_BM, F_BK> opn = {m0, p.seed};
+    GlobalOperand<KZ_BT, F_BK, K_CONT> opx = {p.x, p.ldx, tok0, p.tokens, p.in_f, (int64_t)(p.tokens - 1) * p.ldx + p.in_f};
+    gemm_mainloop<KZ_BM, KZ_BT, F_BK, 1, 1>(acc, lds, opn, opx, 0, (p.in_f + F_BK - 1) / F_BK);
     store_tile_bf16<KZ_BM, KZ_BT>(acc, lds, p.z, p.k, m0, p.k, tok0, p.tokens, INV_2_31, nullptr);
 }
 
 // ----------------------------------------------------------------------------------------------- y = z . C^T
-// tile: 192 output features (engine rows "a") x 256 tokens (engine rows "b"), contraction over k
-constexpr int KY_BO = 192, KY_BT = 256, KY_BK = 64;
+// tile: 128 output features (engine rows "a") x 128 tokens (engine rows "b"), contraction over k; two blocks per CU, so
+// one block's load latency and store phase overlap the other's matrix work (k is short: a block has few stages)
+constexpr int KY_BO = 128, KY_BT = 128;
 
 struct YParams {
     const bf16_t *z;
@@ -63,7 +66,7 @@ struct YParams {
     int tiles_o, tiles_t;
 };
 
-__global__ __launch_bounds__(256, 1) void factored_y_kernel(YParams p)
+__global__ __launch_bounds__(256, 2) void factored_y_kernel(YParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
@@ -76,15 +79,15 @@ __global__ __launch_bounds__(256, 1) void factored_y_kernel(YParams p)
     for (int mi = 0; mi < KY_BO / 64; ++mi)
 #pragma unroll
         for (int ni = 0; ni < KY_BT / 64; ++ni) acc[mi][ni] = zero16();
-    GlobalOperand<KY_BO, KY_BK, K_CONT> opc = {p.coef, (int64_t)p.k, o0, p.out_f, p.k, (int64_t)p.out_f * p.k};
-    GlobalOperand<KY_BT, KY_BK, K_CONT> opz = {p.z, (int64_t)p.k, tok0, p.tokens, p.k, (int64_t)p.tokens * p.k};
-    gemm_mainloop<KY_BO, KY_BT, KY_BK>(acc, lds, opc, opz, 0, (p.k + KY_BK - 1) / KY_BK);
+    GlobalOperand<KY_BO, F_BK, K_CONT> opc = {p.coef, (int64_t)p.k, o0, p.out_f, p.k, (int64_t)p.out_f * p.k};
+    GlobalOperand<KY_BT, F_BK, K_CONT> opz = {p.z, (int64_t)p.k, tok0, p.tokens, p.k, (int64_t)p.tokens * p.k};
+    gemm_mainloop<KY_BO, KY_BT, F_BK, 1, 1>(acc, lds, opc, opz, 0, (p.k + F_BK - 1) / F_BK);
     store_tile_bf16<KY_BO, KY_BT>(acc, lds, p.y, p.ldy, o0, p.out_f, tok0, p.tokens, 1.0f, p.bias);
 }
 
 // ----------------------------------------------------------------------------------------------- dC = dy^T . z
 // tile: 128 output features (engine rows "a") x 128 coefficients (engine rows "b"), contraction over a token range
-constexpr int KD_BO = 128, KD_BM = 128, KD_BK = 64;
+constexpr int KD_BO = 128, KD_BM = 128;
 
 struct DcParams {
     const bf16_t *dy;
@@ -112,9 +115,9 @@ __global__ __launch_bounds__(256, 1) void factored_dc_kernel(DcParams p)
     for (int mi = 0; mi < KD_BO / 64; ++mi)
 #pragma unroll
         for (int ni = 0; ni < KD_BM / 64; ++ni) acc[mi][ni] = zero16();
-    GlobalOperand<KD_BO, KD_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
-    GlobalOperand<KD_BM, KD_BK, M_CONT> opz = {p.z, (int64_t)p.k, m0, p.k, t_end, (int64_t)p.tokens * p.k};
-    gemm_mainloop<KD_BO, KD_BM, KD_BK>(acc, lds, opdy, opz, t_begin, (t_end - t_begin + KD_BK - 1) / KD_BK);
+    GlobalOperand<KD_BO, F_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
+    GlobalOperand<KD_BM, F_BK, M_CONT> opz = {p.z, (int64_t)p.k, m0, p.k, t_end, (int64_t)p.tokens * p.k};
+    gemm_mainloop<KD_BO, KD_BM, F_BK, 1, 1>(acc, lds, opdy, opz, t_begin, (t_end - t_begin + F_BK - 1) / F_BK);
     // acc[mi][ni][j]: o = o0 + wm*64 + mi*32 + 8*(j/4) + 4*g + j%4, m = m0 + wn*64 + ni*32 + r (32 consecutive m: coalesced)
 #pragma unroll
     for (int ni = 0; ni < KD_BM / 64; ++ni) {
@@ -131,37 +134,24 @@ __global__ __launch_bounds__(256, 1) void factored_dc_kernel(DcParams p)
 }
 
 // ----------------------------------------------------------------------------------------------- host side
-static bool factored_ok(const rdb_linear_desc *d)
+// What every factored kernel needs of the layer; coef_dtype is checked by the callers that read coefficients.
+static bool factored_shape_ok(const rdb_linear_desc *d)
 {
-    return d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16 && d->coef_rows != 0 && d->k % 8 == 0 && d->in_f % 8 == 0 &&
-           d->out_f % 8 == 0 && d->k > 0 && d->tokens > 0 && d->in_f > 0 && d->out_f > 0 && d->tokens * d->k < (1ll << 30) &&
-           d->out_f * d->k < (1ll << 30);
+    return d->act_dtype == RDB_BF16 && d->coef_rows != 0 && d->k % 8 == 0 && d->in_f % 8 == 0 && d->out_f % 8 == 0 && d->k > 0 &&
+           d->tokens > 0 && d->in_f > 0 && d->out_f > 0 && d->tokens * d->k < (1ll << 30) && d->out_f * d->k < (1ll << 30);
 }
 static bool cheaper_factored(const rdb_linear_desc *d) { return d->k * (d->in_f + d->out_f) < d->in_f * d->out_f; }
+static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
-int64_t linear_factored_workspace(const rdb_linear_desc *d)
+int64_t linear_projection_bytes(const rdb_linear_desc *d)
 {
-    if (!factored_ok(d)) return 0;
-    return d->tokens * d->k * (int64_t)sizeof(bf16_t);
+    return factored_shape_ok(d) ? d->tokens * d->k * (int64_t)sizeof(bf16_t) : 0;
 }
 
-template <class K, class P> static int launch_engine(K kernel, const P &p, int items, size_t smem, hipStream_t s, const char *name)
+// The three entry points below return RDB_E_UNSUPPORTED, without setting an error, when the request does not fit.
+int linear_project(void *z, const void *x, int64_t ldx, const rdb_linear_desc *d, hipStream_t s)
 {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return set_error((int)e, "%s: cannot reserve %zu bytes of LDS: %s", name, smem, hipGetErrorString(e));
-    kernel<<<xcd_grid_size(items), 256, smem, s>>>(p);
-    return check_launch(name);
-}
-
-template <int BM, int BN, int BK, int LA, int LB> static size_t engine_smem()
-{
-    const size_t stages = 2 * (OperandTile<BM, BK, LA>::LDS_ELEMS + OperandTile<BN, BK, LB>::LDS_ELEMS) * sizeof(bf16_t);
-    const size_t store = (size_t)BN * (BM + 8) * sizeof(bf16_t);
-    return stages > store ? stages : store;
-}
-
-static int launch_z(const void *x, int64_t ldx, void *z, const rdb_linear_desc *d, hipStream_t s)
-{
+    if (!factored_shape_ok(d) || d->tokens * ldx >= (1ll << 30) || ldx % 8 || !aligned16(x) || !aligned16(z)) return RDB_E_UNSUPPORTED;
     ZParams p;
     p.x = (const bf16_t *)x;
     p.z = (bf16_t *)z;
@@ -169,25 +159,18 @@ static int launch_z(const void *x, int64_t ldx, void *z, const rdb_linear_desc *
     p.tokens = (int)d->tokens;
     p.in_f = (int)d->in_f;
     p.k = (int)d->k;
+    p.seed = d->seed;
     p.tiles_m = (int)cdiv(d->k, KZ_BM);
     p.tiles_t = (int)cdiv(d->tokens, KZ_BT);
-    p.seed = d->seed;
-    return launch_engine(factored_z_kernel, p, p.tiles_m * p.tiles_t, engine_smem<KZ_BM, KZ_BT, KZ_BK, K_CONT, K_CONT>(), s, "factored_z_kernel");
+    return launch_engine(factored_z_kernel, p, p.tiles_m * p.tiles_t, engine_smem<KZ_BM, KZ_BT, F_BK, K_CONT, K_CONT>(), s, "factored_z_kernel");
 }
 
-// Returns RDB_E_UNSUPPORTED (without setting an error) when the request does not fit this algorithm.
-int linear_fwd_factored(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
-                        const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s)
+int linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, const void *bias, const rdb_linear_desc *d, hipStream_t s)
 {
-    if (!factored_ok(d) || scale_bias) return RDB_E_UNSUPPORTED;  // the random-bias term is not low rank
-    if (!workspace || workspace_bytes < linear_factored_workspace(d) || ((uintptr_t)workspace & 15)) return RDB_E_UNSUPPORTED;
-    if (d->tokens * ldx >= (1ll << 30) || ldx % 8 || ldy % 8 || ((uintptr_t)x & 15) || ((uintptr_t)coef & 15) || ((uintptr_t)y & 15))
+    if (!factored_shape_ok(d) || d->coef_dtype != RDB_BF16 || ldy % 8 || !aligned16(y) || !aligned16(z) || !aligned16(coef))
         return RDB_E_UNSUPPORTED;
-    if (d->algo == RDB_ALGO_AUTO && !cheaper_factored(d)) return RDB_E_UNSUPPORTED;
-    int rc = launch_z(x, ldx, workspace, d, s);
-    if (rc) return rc;
     YParams p;
-    p.z = (const bf16_t *)workspace;
+    p.z = (const bf16_t *)z;
     p.coef = (const bf16_t *)coef;
     p.bias = (const bf16_t *)bias;
     p.y = (bf16_t *)y;
@@ -197,26 +180,16 @@ int linear_fwd_factored(void *y, int64_t ldy, const void *x, int64_t ldx, const 
     p.k = (int)d->k;
     p.tiles_o = (int)cdiv(d->out_f, KY_BO);
     p.tiles_t = (int)cdiv(d->tokens, KY_BT);
-    return launch_engine(factored_y_kernel, p, p.tiles_o * p.tiles_t, engine_smem<KY_BO, KY_BT, KY_BK, K_CONT, K_CONT>(), s, "factored_y_kernel");
+    return launch_engine(factored_y_kernel, p, p.tiles_o * p.tiles_t, engine_smem<KY_BO, KY_BT, F_BK, K_CONT, K_CONT>(), s, "factored_y_kernel");
 }
 
-// dcoef must have been zeroed by the caller on the same stream.
-int linear_dcoef_factored(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus,
-                          void *workspace, int64_t workspace_bytes, hipStream_t s)
+// dcoef must have been zeroed on the same stream.
+int linear_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *z, const rdb_linear_desc *d, int num_cus, hipStream_t s)
 {
-    // coef_dtype does not matter here (no coefficients are read), but keep one eligibility rule for the whole family
-    rdb_linear_desc dd = *d;
-    dd.coef_dtype = RDB_BF16;
-    if (!factored_ok(&dd)) return RDB_E_UNSUPPORTED;
-    if (!workspace || workspace_bytes < linear_factored_workspace(&dd) || ((uintptr_t)workspace & 15)) return RDB_E_UNSUPPORTED;
-    if (d->tokens * ldx >= (1ll << 30) || d->tokens * lddy >= (1ll << 30) || ldx % 8 || lddy % 8 || ((uintptr_t)x & 15) || ((uintptr_t)dy & 15))
-        return RDB_E_UNSUPPORTED;
-    if (d->algo == RDB_ALGO_AUTO && !cheaper_factored(d)) return RDB_E_UNSUPPORTED;
-    int rc = launch_z(x, ldx, workspace, d, s);
-    if (rc) return rc;
+    if (!factored_shape_ok(d) || d->tokens * lddy >= (1ll << 30) || lddy % 8 || !aligned16(dy) || !aligned16(z)) return RDB_E_UNSUPPORTED;
     DcParams p;
     p.dy = (const bf16_t *)dy;
-    p.z = (const bf16_t *)workspace;
+    p.z = (const bf16_t *)z;
     p.dcoef = dcoef;
     p.lddy = lddy;
     p.tokens = (int)d->tokens;
@@ -224,14 +197,45 @@ int linear_dcoef_factored(float *dcoef, const void *dy, int64_t lddy, const void
     p.k = (int)d->k;
     p.tiles_o = (int)cdiv(d->out_f, KD_BO);
     p.tiles_m = (int)cdiv(d->k, KD_BM);
+    // split the token range so that tiles x splits is about one block per compute unit
     int splits = num_cus / (p.tiles_o * p.tiles_m);
     const int max_splits = (int)cdiv(d->tokens, 256);
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
-    p.tok_per_split = (int)(cdiv(cdiv(d->tokens, splits), KD_BK) * KD_BK);
+    p.tok_per_split = (int)(cdiv(cdiv(d->tokens, splits), F_BK) * F_BK);
     p.splits = (int)cdiv(d->tokens, p.tok_per_split);
-    return launch_engine(factored_dc_kernel, p, p.tiles_o * p.tiles_m * p.splits, engine_smem<KD_BO, KD_BM, KD_BK, M_CONT, M_CONT>(), s,
+    return launch_engine(factored_dc_kernel, p, p.tiles_o * p.tiles_m * p.splits, engine_smem<KD_BO, KD_BM, F_BK, M_CONT, M_CONT>(), s,
                          "factored_dc_kernel");
+}
+
+// y = (x . N^T) . C^T with the projection in the workspace.
+int linear_fwd_factored(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
+                        const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s)
+{
+    if (scale_bias || d->coef_dtype != RDB_BF16 || !factored_shape_ok(d)) return RDB_E_UNSUPPORTED;  // the random-bias term is not low rank
+    if (!workspace || workspace_bytes < linear_projection_bytes(d)) return RDB_E_UNSUPPORTED;
+    if (d->algo == RDB_ALGO_AUTO && !cheaper_factored(d)) return RDB_E_UNSUPPORTED;
+    // check everything before the first launch, so that a refusal leaves nothing half done
+    if (d->tokens * ldx >= (1ll << 30) || ldx % 8 || ldy % 8 || !aligned16(x) || !aligned16(coef) || !aligned16(y) || !aligned16(workspace))
+        return RDB_E_UNSUPPORTED;
+    int rc = linear_project(workspace, x, ldx, d, s);
+    if (rc) return rc;
+    return linear_fwd_projected(y, ldy, workspace, coef, bias, d, s);
+}
+
+// dC = dy^T . (x . N^T) with the projection in the workspace; dcoef must have been zeroed on the same stream.
+int linear_dcoef_factored(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus,
+                          void *workspace, int64_t workspace_bytes, hipStream_t s)
+{
+    if (!factored_shape_ok(d)) return RDB_E_UNSUPPORTED;
+    if (!workspace || workspace_bytes < linear_projection_bytes(d)) return RDB_E_UNSUPPORTED;
+    if (d->algo == RDB_ALGO_AUTO && !cheaper_factored(d)) return RDB_E_UNSUPPORTED;
+    if (d->tokens * ldx >= (1ll << 30) || d->tokens * lddy >= (1ll << 30) || ldx % 8 || lddy % 8 || !aligned16(x) || !aligned16(dy) ||
+        !aligned16(workspace))
+        return RDB_E_UNSUPPORTED;
+    int rc = linear_project(workspace, x, ldx, d, s);
+    if (rc) return rc;
+    return linear_dcoef_projected(dcoef, dy, lddy, workspace, d, num_cus, s);
 }
 
 }  // namespace rdb

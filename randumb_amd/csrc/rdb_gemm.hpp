@@ -8,21 +8,14 @@
 // fragments with two ds_read_b64_tr_b16 (the LDS transpose read of gfx950), which hands lane c of each 16-lane group
 // column c of a 4 (k) x 16 (row) patch, i.e. exactly the k-contiguous fragment the matrix core wants.
 //
-// Pipeline: global loads run two stages ahead in registers, one stage ahead in LDS (double buffer), one barrier per stage.
+// Pipeline: LDS is double buffered with one barrier per stage; global loads run DA (operand A) or DB (operand B) stages
+// further ahead in registers, so that enough bytes are in flight per compute unit to cover HBM latency.
 #pragma once
-
-#ifndef RDB_SCHED_FENCE
-#define RDB_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
-#endif
 
 #include "rdb_common.hpp"
 #include "rdb_tile.hpp"
 
 namespace rdb {
-
-#ifdef RDB_PROFILE_MAINLOOP
-__device__ long long *rdb_profile_ptr;
-#endif
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
@@ -43,7 +36,15 @@ union Frag8 {
 
 // One operand of the tile engine.  ROWS = tile rows (BM or BN), BK = contraction depth per stage.
 template <int ROWS, int BK, int LAYOUT> struct OperandTile {
-    static constexpr int PAD = 8;
+    // LDS layout, chosen so that the 16-byte copy stores and the fragment reads are both free of bank conflicts
+    // (64 banks of 4 bytes; a 128-bit access is served 16 lanes at a time, a 64-bit one 32 lanes at a time):
+    // K_CONT: rows of BK = 64 elements (128 bytes) without padding, 16-byte chunk c of row r stored at chunk position
+    //         c ^ ((r >> 1) & 7).  A store phase covers two whole rows (256 contiguous bytes); a read phase takes one
+    //         chunk from each of 16 consecutive rows, which the swizzle spreads over all 16 chunk positions of a row pair.
+    // M_CONT: rows (one per k) of ROWS elements plus 64 bytes of padding, so the 4 k-rows one ds_read_b64_tr_b16 phase
+    //         touches (64 bytes each) tile the 64 banks exactly.
+    static_assert(LAYOUT == M_CONT || BK == 64, "the swizzled K_CONT layout is laid out for 64-element rows");
+    static constexpr int PAD = (LAYOUT == K_CONT) ? 0 : 32;
     static constexpr int LAYOUT_ID = LAYOUT;
     static constexpr int LD = (LAYOUT == K_CONT) ? (BK + PAD) : (ROWS + PAD);     // LDS row stride, elements
     static constexpr int LDS_ELEMS = (LAYOUT == K_CONT) ? ROWS * LD : BK * LD;    // per stage
@@ -95,10 +96,12 @@ template <int ROWS, int BK, int LAYOUT> struct OperandTile {
     {
         const int idx = p * 256 + threadIdx.x;
         int off;
-        if (LAYOUT == K_CONT)
-            off = (idx / (BK / 8)) * LD + (idx % (BK / 8)) * 8;
-        else
+        if (LAYOUT == K_CONT) {
+            const int row = idx / (BK / 8), c = idx % (BK / 8);
+            off = row * LD + ((c ^ ((row >> 1) & 7)) * 8);
+        } else {
             off = (idx / (ROWS / 8)) * LD + (idx % (ROWS / 8)) * 8;
+        }
         *reinterpret_cast<f32x4 *>(lds + off) = reg;
     }
     __device__ static __forceinline__ void store(bf16_t *__restrict__ lds, const f32x4 (&regs)[PER_THREAD])
@@ -114,7 +117,8 @@ template <int ROWS, int BK, int LAYOUT> struct OperandTile {
         Frag8 f;
         const int r = lane & 31, g = lane >> 5;
         if (LAYOUT == K_CONT) {
-            f.v = *reinterpret_cast<const bf16x8 *>(lds + (rb + r) * LD + ks * 16 + g * 8);
+            // rb is a multiple of 32, so the swizzle depends on the lane only
+            f.v = *reinterpret_cast<const bf16x8 *>(lds + (rb + r) * LD + (((ks * 2 + g) ^ ((r >> 1) & 7)) * 8));
         } else {
             // 16-lane group q = (lane / 16) & 1 covers rows rb + 16q .. +15; source lane s of the group addresses
             // k = kb + s / 4, rows 4*(s % 4) .. +3; the result lane c receives rows' column c for k = kb .. kb+3.
@@ -127,35 +131,6 @@ template <int ROWS, int BK, int LAYOUT> struct OperandTile {
         return f.v;
     }
 };
-
-// Accumulates one LDS stage into the wave's (MI x NI) 32x32 blocks.  The fragments of k-step ks+1 are requested before the
-// MFMAs of k-step ks are issued, so LDS latency hides behind the matrix pipe.
-template <class TA, class TB, int BK, int MI, int NI>
-__device__ __forceinline__ void mma_stage(f32x16 (&acc)[MI][NI], const bf16_t *__restrict__ As, const bf16_t *__restrict__ Bs, int wm,
-                                          int wn, int lane)
-{
-    constexpr int KS = BK / 16;
-    bf16x8 fa[2][MI], fb[2][NI];
-#pragma unroll
-    for (int mi = 0; mi < MI; ++mi) fa[0][mi] = TA::frag(As, wm * MI * 32 + mi * 32, 0, lane);
-#pragma unroll
-    for (int ni = 0; ni < NI; ++ni) fb[0][ni] = TB::frag(Bs, wn * NI * 32 + ni * 32, 0, lane);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        const int cur = ks & 1, nxt = cur ^ 1;
-        if (ks + 1 < KS) {
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi) fa[nxt][mi] = TA::frag(As, wm * MI * 32 + mi * 32, ks + 1, lane);
-#pragma unroll
-            for (int ni = 0; ni < NI; ++ni) fb[nxt][ni] = TB::frag(Bs, wn * NI * 32 + ni * 32, ks + 1, lane);
-        }
-#pragma unroll
-        for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-            for (int ni = 0; ni < NI; ++ni)
-                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][mi], fb[cur][ni], acc[mi][ni], 0, 0, 0);
-    }
-}
 
 // ----------------------------------------------------------------------------------------------- work distribution
 // The 8 accelerator dies (XCDs) of the chip each have their own L2 and receive workgroups round-robin by linear block id.
@@ -257,13 +232,14 @@ template <int ROWS, int BK> struct NoiseOperandRowsAreCoefs {
 };
 
 // One pipeline stage: multiplies the LDS buffer `cur` into the accumulators while, slice by slice between the MFMAs, the
-// registers loaded during the previous stage go to the idle buffer `oth` and are refilled with stage `next_stage`.
-// The copy work and the next k-step's fragment reads are paced against the MFMAs with scheduling groups: every MFMA is
-// followed by a fixed number of memory instructions, so the vector-memory and LDS pipes run in the shadow of the matrix pipe.
+// registers `ra`/`rb` (holding the stage after this one) go to the idle buffer `oth` and are refilled with stages
+// next_a / next_b.  The copy work and the next k-step's fragment reads are paced against the MFMAs with scheduling
+// groups: every MFMA is followed by a fixed number of memory instructions, so the vector-memory and LDS pipes run in the
+// shadow of the matrix pipe.
 template <int BK, int MI, int NI, class PA, class PB>
 __device__ __forceinline__ void pipeline_stage(f32x16 (&acc)[MI][NI], const bf16_t *__restrict__ cur, bf16_t *__restrict__ oth,
                                                f32x4 (&ra)[PA::Tile::PER_THREAD], f32x4 (&rb)[PB::Tile::PER_THREAD], const PA &pa, const PB &pb,
-                                               int next_stage, int wm, int wn, int lane)
+                                               int next_a, int next_b, int wm, int wn, int lane)
 {
     typedef typename PA::Tile TA;
     typedef typename PB::Tile TB;
@@ -284,13 +260,13 @@ __device__ __forceinline__ void pipeline_stage(f32x16 (&acc)[MI][NI], const bf16
         for (int p = 0; p < TA::PER_THREAD; ++p)
             if (p % KS == ks) {
                 TA::store_piece(oth, ra[p], p);
-                pa.load_piece(ra[p], p, next_stage);
+                pa.load_piece(ra[p], p, next_a);
             }
 #pragma unroll
         for (int p = 0; p < TB::PER_THREAD; ++p)
             if ((p + TA::PER_THREAD) % KS == ks) {
                 TB::store_piece(oth + TA::LDS_ELEMS, rb[p], p);
-                pb.load_piece(rb[p], p, next_stage);
+                pb.load_piece(rb[p], p, next_b);
             }
         if (ks + 1 < KS) {
 #pragma unroll
@@ -313,35 +289,47 @@ __device__ __forceinline__ void pipeline_stage(f32x16 (&acc)[MI][NI], const bf16
 }
 
 // Main loop of the tile engine over `nstage` stages of BK starting at contraction index k_begin.
+// DA / DB (1, 2 or 4): how many stages ahead of the LDS copy the registers of operand A / B are loaded.
 // `lds` must hold 2 * (PA::Tile::LDS_ELEMS + PB::Tile::LDS_ELEMS) elements.  On return every wave has passed a barrier
-// after its last LDS read, so the caller may reuse `lds` at once.  An odd stage count is rounded up (the extra stage lies
-// past klim and reads as zeros), so the two-stage loop body has a single exit.
-template <int BM, int BN, int BK, class PA, class PB>
+// after its last LDS read, so the caller may reuse `lds` at once.  The stage count is rounded up to a multiple of the
+// unrolled trip (the extra stages lie past klim and read as zeros), so the loop body has a single exit.
+template <int BM, int BN, int BK, int DA, int DB, class PA, class PB>
 __device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / 64][BN / 64], bf16_t *__restrict__ lds, PA &pa, PB &pb, int k_begin,
                                               int nstage)
 {
     typedef typename PA::Tile TA;
     typedef typename PB::Tile TB;
+    static_assert((DA == 1 || DA == 2 || DA == 4) && (DB == 1 || DB == 2 || DB == 4), "prefetch depth must be 1, 2 or 4");
     constexpr int MI = BM / 64, NI = BN / 64;
     constexpr int STAGE = TA::LDS_ELEMS + TB::LDS_ELEMS;
+    constexpr int TRIP = (DA == 4 || DB == 4) ? 4 : 2;
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, wm = wave >> 1, wn = wave & 1;
     if (nstage <= 0) return;
     pa.init(k_begin);
     pb.init(k_begin);
 
-    f32x4 ra[TA::PER_THREAD], rb[TB::PER_THREAD];
-    pa.load(ra, 0);
-    pb.load(rb, 0);
-    TA::store(lds, ra);
-    TB::store(lds + TA::LDS_ELEMS, rb);
-    pa.load(ra, 1);
-    pb.load(rb, 1);
+    // registers of stage j live in slot j % D; stage 0 goes through a set of its own straight to LDS
+    f32x4 ra[DA][TA::PER_THREAD], rb[DB][TB::PER_THREAD];
+    {
+        f32x4 ra0[TA::PER_THREAD], rb0[TB::PER_THREAD];
+        pa.load(ra0, 0);
+        pb.load(rb0, 0);
+#pragma unroll
+        for (int j = 1; j <= DA; ++j) pa.load(ra[j % DA], j);
+#pragma unroll
+        for (int j = 1; j <= DB; ++j) pb.load(rb[j % DB], j);
+        TA::store(lds, ra0);
+        TB::store(lds + TA::LDS_ELEMS, rb0);
+    }
     __syncthreads();
 
-    for (int s = 0; s < nstage; s += 2) {
-        // stage s lives in buffer 0 and the registers hold stage s+1; then the roles of the buffers swap
-        pipeline_stage<BK, MI, NI>(acc, lds, lds + STAGE, ra, rb, pa, pb, s + 2, wm, wn, lane);
-        pipeline_stage<BK, MI, NI>(acc, lds + STAGE, lds, ra, rb, pa, pb, s + 3, wm, wn, lane);
+    for (int s = 0; s < nstage; s += TRIP) {
+#pragma unroll
+        for (int u = 0; u < TRIP; ++u) {
+            // stage s+u is in LDS buffer u % 2; slot (u+1) % D holds stage s+u+1 and is refilled with stage s+u+1+D
+            bf16_t *cur = lds + (u & 1) * STAGE, *oth = lds + ((u & 1) ^ 1) * STAGE;
+            pipeline_stage<BK, MI, NI>(acc, cur, oth, ra[(u + 1) % DA], rb[(u + 1) % DB], pa, pb, s + u + 1 + DA, s + u + 1 + DB, wm, wn, lane);
+        }
     }
 }
 
@@ -382,6 +370,24 @@ __device__ __forceinline__ void store_tile_bf16(const f32x16 (&acc)[BM / 64][BN 
             *reinterpret_cast<f32x4 *>(out + (int64_t)(b0 + b) * ld + a0 + a) = *reinterpret_cast<const f32x4 *>(lds + b * LDS_LD + a);
     }
     __syncthreads();
+}
+
+// ----------------------------------------------------------------------------------------------- host side helpers
+// Dynamic LDS of an engine kernel: the two pipeline stages, or the bf16 output staging tile if that is larger.
+template <int BM, int BN, int BK, int LA, int LB> inline size_t engine_smem()
+{
+    const size_t stages = 2 * (OperandTile<BM, BK, LA>::LDS_ELEMS + OperandTile<BN, BK, LB>::LDS_ELEMS) * sizeof(bf16_t);
+    const size_t store = (size_t)BN * (BM + 8) * sizeof(bf16_t);
+    return stages > store ? stages : store;
+}
+
+// Launches an engine kernel over `items` work items (one 256-thread block each, XCD-aware numbering).
+template <class K, class P> inline int launch_engine(K kernel, const P &p, int items, size_t smem, hipStream_t s, const char *name)
+{
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return set_error((int)e, "%s: cannot reserve %zu bytes of LDS: %s", name, smem, hipGetErrorString(e));
+    kernel<<<xcd_grid_size(items), 256, smem, s>>>(p);
+    return check_launch(name);
 }
 
 }  // namespace rdb

@@ -227,9 +227,24 @@ __global__ __launch_bounds__(TILE_THREADS) void linear_dcoef_kernel(LinParams p)
     }
 }
 
+// Clears n floats.  A fill kernel rather than hipMemsetAsync so that callers can capture the launch in a HIP graph.
+// 16-byte stores over the aligned middle, scalar stores on the ragged ends.
 __global__ __launch_bounds__(256) void fill_zero_kernel(float *p, int64_t n)
 {
-    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += (int64_t)gridDim.x * 256) p[e] = 0.0f;
+    const int64_t head = ((16 - ((uintptr_t)p & 15)) & 15) / 4 < n ? ((16 - ((uintptr_t)p & 15)) & 15) / 4 : n;
+    const int64_t nvec = (n - head) / 4, tail = head + nvec * 4;
+    const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x, nthr = (int64_t)gridDim.x * 256;
+    f32x4 *v = reinterpret_cast<f32x4 *>(p + head);
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int64_t e = tid; e < nvec; e += nthr) v[e] = zero;
+    if (tid < head) p[tid] = 0.0f;
+    if (tid < n - tail) p[tail + tid] = 0.0f;
+}
+static int fill_zero(float *p, int64_t n, hipStream_t s)
+{
+    const int64_t blocks = cdiv(cdiv(n, 4) + 8, 256);
+    fill_zero_kernel<<<(unsigned)(blocks < 2048 ? blocks : 2048), 256, 0, s>>>(p, n);
+    return check_launch("fill_zero_kernel");
 }
 
 // ----------------------------------------------------------------------------------------------- host side
@@ -266,7 +281,10 @@ int linear_fwd_strip(void *y, int64_t ldy, const void *x, int64_t ldx, const voi
                      const rdb_linear_desc *d, int num_cus, hipStream_t s);
 
 // rdb_factored.hip
-int64_t linear_factored_workspace(const rdb_linear_desc *d);
+int64_t linear_projection_bytes(const rdb_linear_desc *d);
+int linear_project(void *z, const void *x, int64_t ldx, const rdb_linear_desc *d, hipStream_t s);
+int linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, const void *bias, const rdb_linear_desc *d, hipStream_t s);
+int linear_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *z, const rdb_linear_desc *d, int num_cus, hipStream_t s);
 int linear_fwd_factored(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
                         const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s);
 int linear_dcoef_factored(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus,
@@ -331,12 +349,8 @@ extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
     if (!d) return 0;
     if (d->algo == RDB_ALGO_TILE || d->algo == RDB_ALGO_STRIP) return 0;
     if (op == RDB_OP_LINEAR_BWD_DX) return linear_dx_factored_workspace(d);
-    if (op == RDB_OP_LINEAR_FWD) return linear_factored_workspace(d);
-    if (op == RDB_OP_LINEAR_BWD_DCOEF) {  // reads no coefficients: their dtype does not matter
-        rdb_linear_desc dd = *d;
-        dd.coef_dtype = RDB_BF16;
-        return linear_factored_workspace(&dd);
-    }
+    if (op == RDB_OP_LINEAR_FWD) return d->coef_dtype == RDB_BF16 ? linear_projection_bytes(d) : 0;
+    if (op == RDB_OP_LINEAR_BWD_DCOEF) return linear_projection_bytes(d);  // reads no coefficients: their dtype does not matter
     return 0;
 }
 
@@ -427,13 +441,11 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
     if (ncoef > 0 && !dcoef) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef: dcoef is NULL");
     hipStream_t s = (hipStream_t)stream;
     if (ncoef > 0) {
-        fill_zero_kernel<<<(unsigned)(cdiv(ncoef, 256) < 1024 ? cdiv(ncoef, 256) : 1024), 256, 0, s>>>(dcoef, ncoef);
-        rc = check_launch("fill_zero_kernel");
+        rc = fill_zero(dcoef, ncoef, s);
         if (rc) return rc;
     }
     if (d_scale_bias) {
-        fill_zero_kernel<<<1, 256, 0, s>>>(d_scale_bias, 1);
-        rc = check_launch("fill_zero_kernel");
+        rc = fill_zero(d_scale_bias, 1, s);
         if (rc) return rc;
     }
     if (d->tokens == 0 || d->in_f == 0 || d->out_f == 0 || (ncoef == 0 && !d_scale_bias)) return RDB_OK;
@@ -470,4 +482,58 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
                    : launch(linear_dcoef_kernel<bf16_t, false>, grid, smem_dcoef<bf16_t>(), s, p, "linear_dcoef_kernel<bf16,vector>");
     return mat ? launch(linear_dcoef_kernel<float, true>, grid, smem_dcoef<float>(), s, p, "linear_dcoef_kernel<f32,matrix>")
                : launch(linear_dcoef_kernel<float, false>, grid, smem_dcoef<float>(), s, p, "linear_dcoef_kernel<f32,vector>");
+}
+
+// ----------------------------------------------------------------------------------------------- projected entry points
+static int check_projected(const char *who, const rdb_linear_desc *d)
+{
+    int rc = check_desc(who, d);
+    if (rc) return rc;
+    if (linear_projection_bytes(d) == 0)
+        return set_error(RDB_E_UNSUPPORTED, "%s: the projected form needs matrix-coef, bf16 activations, non-empty sizes that are "
+                                            "multiples of 8 and tokens*k < 2^30", who);
+    return RDB_OK;
+}
+
+extern "C" int64_t rdb_linear_projection_bytes(const rdb_linear_desc *d) { return d ? linear_projection_bytes(d) : 0; }
+
+extern "C" int rdb_linear_project(void *z, const void *x, int64_t ldx, const rdb_linear_desc *d, void *stream)
+{
+    int rc = check_projected("rdb_linear_project", d);
+    if (rc) return rc;
+    if (!z || !x) return set_error(RDB_E_NULL, "rdb_linear_project: z or x is NULL");
+    if (ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_project: leading dimension smaller than the row");
+    rc = linear_project(z, x, ldx, d, (hipStream_t)stream);
+    if (rc == RDB_E_UNSUPPORTED)
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_project: x and z must be 16-byte aligned, ldx a multiple of 8, tokens*ldx < 2^30");
+    return rc;
+}
+
+extern "C" int rdb_linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, const void *bias, const rdb_linear_desc *d,
+                                        void *stream)
+{
+    int rc = check_projected("rdb_linear_fwd_projected", d);
+    if (rc) return rc;
+    if (!y || !z || !coef) return set_error(RDB_E_NULL, "rdb_linear_fwd_projected: y, z or coef is NULL");
+    if (ldy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_fwd_projected: leading dimension smaller than the row");
+    rc = linear_fwd_projected(y, ldy, z, coef, bias, d, (hipStream_t)stream);
+    if (rc == RDB_E_UNSUPPORTED)
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd_projected: coefficients must be bf16; y, z and coef 16-byte aligned; ldy a "
+                                            "multiple of 8");
+    return rc;
+}
+
+extern "C" int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *z, const rdb_linear_desc *d, void *stream)
+{
+    int rc = check_projected("rdb_linear_bwd_dcoef_projected", d);
+    if (rc) return rc;
+    if (!dcoef || !dy || !z) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef_projected: dcoef, dy or z is NULL");
+    if (lddy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dcoef_projected: leading dimension smaller than the row");
+    if (lddy % 8 || !aligned16(dy) || !aligned16(z) || d->tokens * lddy >= (1ll << 30))
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dcoef_projected: dy and z must be 16-byte aligned, lddy a multiple of 8, "
+                                            "tokens*lddy < 2^30");
+    hipStream_t s = (hipStream_t)stream;
+    rc = fill_zero(dcoef, d->coef_rows * d->k, s);
+    if (rc) return rc;
+    return linear_dcoef_projected(dcoef, dy, lddy, z, d, num_compute_units(), s);
 }

@@ -254,3 +254,60 @@ def linear_bwd_dcoef(dy: torch.Tensor, x: torch.Tensor, k: int, coef_rows: int, 
                                     _stream(dy.device))
     _lib.check(rc, "rdb_linear_bwd_dcoef")
     return dcoef, dsb
+
+
+# ------------------------------------------------------------------------------------------------ fused linear, projected form
+def _proj_desc(tokens, in_f, out_f, k, seed, coef_dtype=torch.bfloat16) -> LinearDesc:
+    d = LinearDesc()
+    d.tokens, d.in_f, d.out_f, d.k, d.coef_rows = int(tokens), int(in_f), int(out_f), int(k), int(out_f)
+    d.sO, d.sI, d.seed = int(in_f), 1, _seed(seed)
+    d.act_dtype, d.coef_dtype, d.algo = RDB_BF16, _DT[coef_dtype], RDB_ALGO_AUTO
+    return d
+
+
+def linear_projection_supported(tokens: int, in_f: int, out_f: int, k: int) -> bool:
+    """Whether the projected form (matrix-coef, bf16) applies to a layer of these sizes."""
+    return _lib.load().rdb_linear_projection_bytes(ctypes.byref(_proj_desc(tokens, in_f, out_f, k, 0))) > 0
+
+
+def linear_project(x: torch.Tensor, k: int, out_f: int, seed: int) -> torch.Tensor:
+    """``z = x @ Noise.T`` (tokens, k) in bf16: all that the forward product and the coef gradient need of ``x``."""
+    _need_gpu("linear_project", x)
+    x = _act(x)
+    if x.dtype != torch.bfloat16:
+        raise ValueError("linear_project computes in bf16")
+    d = _proj_desc(x.shape[0], x.shape[1], out_f, k, seed)
+    z = torch.empty((x.shape[0], k), dtype=torch.bfloat16, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().rdb_linear_project(_p(z), _p(x), x.stride(0), ctypes.byref(d), _stream(x.device))
+    _lib.check(rc, "rdb_linear_project")
+    return z
+
+
+def linear_fwd_projected(z: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``y = z @ coef.T (+ bias)`` for matrix-coef ``coef`` (out_f, k) in bf16."""
+    _need_gpu("linear_fwd_projected", z, coef)
+    c = _native(coef)
+    z = z.contiguous()
+    out_f, k = c.shape
+    d = _proj_desc(z.shape[0], in_f, out_f, k, seed, c.dtype)
+    b = None if bias is None else bias.to(z.dtype).contiguous()
+    y = torch.empty((z.shape[0], out_f), dtype=z.dtype, device=z.device)
+    with torch.cuda.device(z.device):
+        rc = _lib.load().rdb_linear_fwd_projected(_p(y), y.stride(0), _p(z), _p(c), _p(b), ctypes.byref(d), _stream(z.device))
+    _lib.check(rc, "rdb_linear_fwd_projected")
+    return y
+
+
+def linear_bwd_dcoef_projected(dy: torch.Tensor, z: torch.Tensor, in_f: int, seed: int) -> torch.Tensor:
+    """``dcoef = dy.T @ z`` (out_f, k) in fp32."""
+    _need_gpu("linear_bwd_dcoef_projected", dy, z)
+    dy = _act(dy)
+    z = z.contiguous()
+    out_f, k = dy.shape[1], z.shape[1]
+    d = _proj_desc(dy.shape[0], in_f, out_f, k, seed)
+    dcoef = torch.empty((out_f, k), dtype=torch.float32, device=dy.device)
+    with torch.cuda.device(dy.device):
+        rc = _lib.load().rdb_linear_bwd_dcoef_projected(_p(dcoef), _p(dy), dy.stride(0), _p(z), ctypes.byref(d), _stream(dy.device))
+    _lib.check(rc, "rdb_linear_bwd_dcoef_projected")
+    return dcoef
