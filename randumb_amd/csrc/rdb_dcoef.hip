@@ -25,8 +25,6 @@ struct DcoefParams {
     int tokens, in_f, out_f, k;
     int tok_per_split, tiles_i, tiles_o, splits;
     uint32_t seed;
-    long long *dbgp;
-    int dbg;
 };
 
 __global__ __launch_bounds__(256, 1) void linear_dcoef_fast_kernel(DcoefParams p)
@@ -38,26 +36,19 @@ __global__ __launch_bounds__(256, 1) void linear_dcoef_fast_kernel(DcoefParams p
     const int w = xcd_work_item(blockIdx.x, p.tiles_i * p.tiles_o * p.splits);
     if (w >= p.tiles_i * p.tiles_o * p.splits) return;
     const int i0 = (w % p.tiles_i) * DC_BI, o0 = ((w / p.tiles_i) % p.tiles_o) * DC_BO, split = w / (p.tiles_i * p.tiles_o);
-    int t_begin = split * p.tok_per_split;
-    int t_end = (t_begin + p.tok_per_split < p.tokens) ? t_begin + p.tok_per_split : p.tokens;
-    int li0 = i0, lo0 = o0;
-    if (p.dbg & 1) { li0 = 0; lo0 = 0; t_end -= t_begin; t_begin = 0; }
+    const int t_begin = split * p.tok_per_split;
+    const int t_end = (t_begin + p.tok_per_split < p.tokens) ? t_begin + p.tok_per_split : p.tokens;
 
-#ifdef RDB_PROFILE_MAINLOOP
-    rdb_profile_ptr = p.dbgp;
-#endif
-    long long ts0 = __builtin_readcyclecounter();
     // main product: D[m = i][n = o] (x rows as the "A" tile, dy rows as the "B" tile), contraction over tokens
     f32x16 acc[DC_BI / 64][DC_BO / 64];
 #pragma unroll
     for (int mi = 0; mi < DC_BI / 64; ++mi)
 #pragma unroll
         for (int ni = 0; ni < DC_BO / 64; ++ni) acc[mi][ni] = zero16();
-    GlobalOperand<DC_BI, DC_BK, M_CONT> opx = {p.x, p.ldx, li0, p.in_f, t_end, (int64_t)(p.tokens - 1) * p.ldx + p.in_f};
-    GlobalOperand<DC_BO, DC_BK, M_CONT> opdy = {p.dy, p.lddy, lo0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
+    GlobalOperand<DC_BI, DC_BK, M_CONT> opx = {p.x, p.ldx, i0, p.in_f, t_end, (int64_t)(p.tokens - 1) * p.ldx + p.in_f};
+    GlobalOperand<DC_BO, DC_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
     gemm_mainloop<DC_BI, DC_BO, DC_BK, 1, 1>(acc, lds, opx, opdy, t_begin, (t_end - t_begin + DC_BK - 1) / DC_BK);
 
-    long long ts1 = __builtin_readcyclecounter();
     // dW tile -> LDS as Ws[o][i] (bf16, i contiguous).  acc[mi][ni][j]: i = wm*96 + mi*32 + 8*(j/4) + 4*g + j%4, o = wn*96 + ni*32 + r
     constexpr int LDW = DC_BI + 8;
     bf16_t *Ws = lds;                  // [DC_BO][LDW]
@@ -121,11 +112,6 @@ __global__ __launch_bounds__(256, 1) void linear_dcoef_fast_kernel(DcoefParams p
         __syncthreads();
     }
 
-    if (p.dbgp && t == 0 && blockIdx.x == 0) {
-        long long ts2 = __builtin_readcyclecounter();
-        p.dbgp[0] = ts1 - ts0;
-        p.dbgp[1] = ts2 - ts1;
-    }
     if (p.dsb) {  // d scale_bias += sum dW[o, i] * noise(o*in_f + i)
         float s = 0.0f;
         for (int e = t; e < DC_BO * DC_BI; e += 256) {
@@ -165,8 +151,6 @@ int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, co
     p.out_f = (int)d->out_f;
     p.k = (int)d->k;
     p.seed = d->seed;
-    p.dbg = getenv("RDB_DEBUG") ? atoi(getenv("RDB_DEBUG")) : 0;
-    p.dbgp = getenv("RDB_DBGP") ? (long long *)strtoull(getenv("RDB_DBGP"), nullptr, 0) : nullptr;
     const int ti = (int)cdiv(d->in_f, DC_BI), to = (int)cdiv(d->out_f, DC_BO);
     int splits = num_cus / (ti * to);
     const int max_splits = (int)cdiv(d->tokens, 256);

@@ -29,8 +29,6 @@ struct StripParams {
     int coef_dtype;
     int coef_vec;  // 16-byte loads of coef rows allowed
     uint32_t seed;
-    int dbg;
-    long long *dbgp;
 };
 
 union Pack8 {
@@ -111,8 +109,6 @@ __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
     const int in_pad = p.in_pad;
     const int nib = (in_pad - 8) / 32;  // 32-column blocks of the strip (in_f rounded up to 64)
 
-    long long ts[8];
-    ts[0] = __builtin_readcyclecounter();
     // ------------------------------------------------------------------ phase 1: W strip -> LDS
     {
         const float sb = p.scale_bias ? load_as_f32(p.scale_bias, p.coef_dtype, 0) : 0.0f;
@@ -134,7 +130,7 @@ __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
 #pragma unroll
                 for (int ob = 0; ob < OB; ++ob) ring[u][ob] = load_coef8<CMODE>(p, crow[ob], (u % ksteps) * 16 + g * 8);
         }
-        for (int ib = wave; ib < ((p.dbg & 4) ? 0 : nib); ib += 4) {
+        for (int ib = wave; ib < nib; ib += 4) {
             f32x16 acc[OB];
 #pragma unroll
             for (int ob = 0; ob < OB; ++ob) acc[ob] = zero16();
@@ -191,9 +187,7 @@ __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
             }
         }
     }
-    ts[1] = __builtin_readcyclecounter();
     __syncthreads();
-    ts[2] = __builtin_readcyclecounter();
 
     // ------------------------------------------------------------------ phase 2: stream tokens
     // token blocks of 32 rows: this block's range, then this wave's share of it
@@ -212,7 +206,6 @@ __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
         for (int mi = 0; mi < MI; ++mi) {
             int row = (rb + mi) * 32 + r;
             if (rb + mi >= w_hi || row >= p.tokens) row = p.tokens - 1;
-            if (p.dbg & 1) row = row & 7;
             xrow[mi] = p.x + (int64_t)row * p.ldx + g * 32;
         }
         f32x16 acc[MI][OB];
@@ -225,7 +218,6 @@ __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
         // so a lane's four fragments are 64 contiguous bytes of its row
         bf16x8 xa[2][MI][4];
         auto load_x = [&](int buf, int c) {  // chunk c lies entirely inside the row
-            if (p.dbg & 8) return;
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -283,7 +275,6 @@ __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
             compute(1, c);
         }
 
-        ts[3] = __builtin_readcyclecounter();
         // store: acc[mi][ob][j] = y[row = (rb+mi)*32 + 8*(j/4) + 4*g + j%4][o = o0 + ob*32 + r]
 #pragma unroll
         for (int ob = 0; ob < OB; ++ob) {
@@ -300,12 +291,6 @@ __global__ __launch_bounds__(256, 1) void linear_fwd_strip_kernel(StripParams p)
                 }
             }
         }
-        ts[4] = __builtin_readcyclecounter();
-        if (p.dbgp && lane == 0 && blockIdx.x < 8) {
-            long long *d = p.dbgp + (blockIdx.x * 4 + wave) * 16 + (rb == w_lo ? 0 : 8);
-            d[0] = ts[0]; d[1] = ts[1]; d[2] = ts[2]; d[3] = ts[3]; d[4] = ts[4]; d[5] = rb; d[6] = w_hi;
-        }
-        ts[2] = ts[4];
     }
 }
 
@@ -355,8 +340,6 @@ int linear_fwd_strip(void *y, int64_t ldy, const void *x, int64_t ldx, const voi
     const int ces = d->coef_dtype == RDB_BF16 ? 2 : 4;
     p.coef_vec = (((uintptr_t)coef & 15) == 0) && ((d->k * ces) % 16 == 0);
     p.seed = d->seed;
-    p.dbg = getenv("RDB_DEBUG") ? atoi(getenv("RDB_DEBUG")) : 0;
-    p.dbgp = getenv("RDB_DBGP") ? (long long *)strtoull(getenv("RDB_DBGP"), nullptr, 0) : nullptr;
     // widest strip that fits LDS; narrower strips when that leaves compute units idle
     int bo = 0;
     for (int cand : {96, 64, 32}) {
