@@ -30,6 +30,13 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+# HBM bytes per call of each product, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script scaled by what the same
+# counters read for a plain 256 MiB device copy (FETCH x2.000, WRITE x1.000): profiles/bench_c2_hbm_traffic.md
+HBM_TRAFFIC_BYTES = {
+    "forward (factored_z_kernel + factored_y_kernel)": 84.5e6,
+    "dx (dx_dyc_kernel + dx_tn_kernel)": 84.3e6,
+    "dcoef (fill_zero_kernel + factored_dc_kernel)": 79.4e6,
+}
 T, IN_F, OUT_F, K, SEED = 8192, 768, 3072, 256, 0
 
 
@@ -46,6 +53,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
     ap.add_argument("--no-compare", action="store_true", help="skip the materialise+GEMM comparison legs")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch plain device copies of 256 MiB (a known 256 MiB read + 256 MiB written per launch) so that "
+                         "hardware byte counters collected over this run can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -125,6 +135,14 @@ def main():
 
         return fwd, dxf, dcf, dd
 
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -168,7 +186,7 @@ def main():
     achieved = F_PER_PRODUCT / (dom_ms * 1e-3) / 1e12
     roofline = {
         "bound": "mfma", "kernel": dom, "achieved": round(achieved, 3), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-        "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 5), "traffic": None, "avg_kernel_ms": round(dom_ms, 5),
+        "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 5), "traffic": HBM_TRAFFIC_BYTES[dom], "avg_kernel_ms": round(dom_ms, 5),
         "algorithmic_gflop_per_launch": round(F_PER_PRODUCT / 1e9, 3),
         "calls_ms": {n: round(v, 5) for n, v in calls.items()},
     }
