@@ -170,7 +170,7 @@ class SillyLinear(SillyModuleMixin, nn.Module):
         if x2.dtype != w.dtype:
             x2 = x2.to(w.dtype)
         sb = w.scale_bias if w.fused_bias else None
-        y = ops.linear_fwd(x2, self.weight_coef, self.in_features, self.out_features, self.in_features, 1, w.seed, sb, self.bias)
+        y = ops.linear(x2, self.weight_coef, self.in_features, self.out_features, self.in_features, 1, w.seed, sb, self.bias)
         return y.reshape(*input.shape[:-1], self.out_features)
 
     def extra_repr(self) -> str:

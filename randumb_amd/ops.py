@@ -22,7 +22,8 @@ from . import hip
 
 __all__ = [
     "materialize_fwd", "materialize_bwd", "scale_bias_bwd", "embed_fwd", "embed_bwd",
-    "linear_fwd", "linear_bwd_dx", "linear_bwd_dcoef", "sq5_gen_2d", "sq5_gen_1d",
+    "linear_fwd", "linear_bwd_dx", "linear_bwd_dcoef", "linear", "linear_project", "linear_fwd_projected",
+    "linear_bwd_dcoef_projected", "sq5_gen_2d", "sq5_gen_1d",
 ]
 
 
@@ -196,6 +197,78 @@ def _lin_backward(ctx, dy):
 
 
 linear_fwd.register_autograd(_lin_backward, setup_context=_lin_setup_context)
+
+
+# ------------------------------------------------------------------------------------------------ projected form
+@custom_op("rten::linear_project", mutates_args=())
+def linear_project(x: Tensor, dcoefs_size: int, out_features: int, seed: int) -> Tensor:
+    """``z = x @ Noise.T`` (tokens, k): what the forward product and the coef gradient of a matrix-coef layer need of x."""
+    return hip.linear_project(x, dcoefs_size, out_features, seed)
+
+
+@linear_project.register_fake
+def _(x, dcoefs_size, out_features, seed):
+    return x.new_empty([x.shape[0], dcoefs_size])
+
+
+@custom_op("rten::linear_fwd_projected", mutates_args=())
+def linear_fwd_projected(z: Tensor, coefs: Tensor, in_features: int, seed: int, bias: Optional[Tensor]) -> Tensor:
+    return hip.linear_fwd_projected(z, coefs, in_features, seed, bias)
+
+
+@linear_fwd_projected.register_fake
+def _(z, coefs, in_features, seed, bias):
+    return z.new_empty([z.shape[0], coefs.shape[0]])
+
+
+@custom_op("rten::linear_bwd_dcoef_projected", mutates_args=())
+def linear_bwd_dcoef_projected(dy: Tensor, z: Tensor, in_features: int, seed: int) -> Tensor:
+    return hip.linear_bwd_dcoef_projected(dy, z, in_features, seed)
+
+
+@linear_bwd_dcoef_projected.register_fake
+def _(dy, z, in_features, seed):
+    return dy.new_empty([dy.shape[1], z.shape[1]], dtype=torch.float32)
+
+
+class _ProjectedLinear(torch.autograd.Function):
+    """``y = x @ W.T (+ bias)`` for a matrix-coef weight in bf16.  The forward pass computes ``z = x @ Noise.T`` once and
+    saves it for the backward pass in place of ``x`` (``k / in_features`` of its size); the reference's autograd saves
+    ``x`` and materialises ``W`` again (RandumbTensor.py:942-946, 979-990)."""
+
+    @staticmethod
+    def forward(ctx, x, coefs, in_features, out_features, seed, bias):
+        z = linear_project(x, coefs.shape[1], out_features, seed)
+        ctx.save_for_backward(z, coefs)
+        ctx.meta = (in_features, out_features, seed)
+        ctx.bias_dtype = None if bias is None else bias.dtype
+        return linear_fwd_projected(z, coefs, in_features, seed, bias)
+
+    @staticmethod
+    def backward(ctx, dy):
+        z, coefs = ctx.saved_tensors
+        in_f, out_f, seed = ctx.meta
+        dy = dy.contiguous()
+        dx = dcoefs = dbias = None
+        if ctx.needs_input_grad[0]:
+            dx = linear_bwd_dx(dy, coefs, in_f, out_f, in_f, 1, seed, None)
+        if ctx.needs_input_grad[1]:
+            dcoefs = linear_bwd_dcoef_projected(dy, z, in_f, seed).to(coefs.dtype)
+        if ctx.bias_dtype is not None and ctx.needs_input_grad[5]:
+            dbias = dy.sum(0).to(ctx.bias_dtype)
+        return dx, dcoefs, None, None, None, dbias
+
+
+def linear(x: Tensor, coefs: Tensor, in_features: int, out_features: int, stride_o: int, stride_i: int, seed: int,
+           scale_bias: Optional[Tensor], bias: Optional[Tensor]) -> Tensor:
+    """``x @ W.T (+ bias)`` with autograd, choosing the projected form when the layer qualifies (matrix-coef, bf16, no
+    fused random bias, sizes in multiples of 8) and ``rten::linear_fwd`` otherwise.  Same arguments as ``rten::linear_fwd``."""
+    if (scale_bias is None and coefs.dim() == 2 and coefs.shape[0] == out_features and stride_o == in_features and stride_i == 1
+            and x.is_cuda and x.dim() == 2 and x.dtype == torch.bfloat16 and coefs.dtype == torch.bfloat16
+            and (bias is None or bias.dtype == torch.bfloat16)
+            and hip.linear_projection_supported(x.shape[0], in_features, out_features, coefs.shape[1])):
+        return _ProjectedLinear.apply(x, coefs, in_features, out_features, seed, bias)
+    return linear_fwd(x, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias, bias)
 
 
 # ------------------------------------------------------------------------------------------------ rten_cpp::*
