@@ -236,7 +236,8 @@ template <int ROWS, int BK> struct NoiseOperandRowsAreCoefs {
 // next_a / next_b.  The copy work and the next k-step's fragment reads are paced against the MFMAs with scheduling
 // groups: every MFMA is followed by a fixed number of memory instructions, so the vector-memory and LDS pipes run in the
 // shadow of the matrix pipe.
-template <int BK, int MI, int NI, class PA, class PB>
+// STORE / RELOAD switch the copy work off for the stages at the end of the loop whose successors lie past the end.
+template <int BK, int MI, int NI, bool STORE, bool RELOAD, class PA, class PB>
 __device__ __forceinline__ void pipeline_stage(f32x16 (&acc)[MI][NI], const bf16_t *__restrict__ cur, bf16_t *__restrict__ oth,
                                                f32x4 (&ra)[PA::Tile::PER_THREAD], f32x4 (&rb)[PB::Tile::PER_THREAD], const PA &pa, const PB &pb,
                                                int next_a, int next_b, int wm, int wn, int lane)
@@ -245,7 +246,7 @@ __device__ __forceinline__ void pipeline_stage(f32x16 (&acc)[MI][NI], const bf16
     typedef typename PB::Tile TB;
     constexpr int KS = BK / 16;
     constexpr int FRAG_OPS = (MI * (TA::LAYOUT_ID == M_CONT ? 2 : 1)) + (NI * (TB::LAYOUT_ID == M_CONT ? 2 : 1));
-    constexpr int COPY_OPS = 2 * ((TA::PER_THREAD + TB::PER_THREAD + KS - 1) / KS);
+    constexpr int COPY_OPS = ((STORE ? 1 : 0) + (RELOAD ? 1 : 0)) * ((TA::PER_THREAD + TB::PER_THREAD + KS - 1) / KS);
     constexpr int MEM_PER_MFMA = (FRAG_OPS + COPY_OPS + MI * NI - 1) / (MI * NI);
     const bf16_t *As = cur, *Bs = cur + TA::LDS_ELEMS;
     bf16x8 fa[2][MI], fb[2][NI];
@@ -259,14 +260,14 @@ __device__ __forceinline__ void pipeline_stage(f32x16 (&acc)[MI][NI], const bf16
 #pragma unroll
         for (int p = 0; p < TA::PER_THREAD; ++p)
             if (p % KS == ks) {
-                TA::store_piece(oth, ra[p], p);
-                pa.load_piece(ra[p], p, next_a);
+                if (STORE) TA::store_piece(oth, ra[p], p);
+                if (RELOAD) pa.load_piece(ra[p], p, next_a);
             }
 #pragma unroll
         for (int p = 0; p < TB::PER_THREAD; ++p)
             if ((p + TA::PER_THREAD) % KS == ks) {
-                TB::store_piece(oth + TA::LDS_ELEMS, rb[p], p);
-                pb.load_piece(rb[p], p, next_b);
+                if (STORE) TB::store_piece(oth + TA::LDS_ELEMS, rb[p], p);
+                if (RELOAD) pb.load_piece(rb[p], p, next_b);
             }
         if (ks + 1 < KS) {
 #pragma unroll
@@ -292,7 +293,8 @@ __device__ __forceinline__ void pipeline_stage(f32x16 (&acc)[MI][NI], const bf16
 // DA / DB (1, 2 or 4): how many stages ahead of the LDS copy the registers of operand A / B are loaded.
 // `lds` must hold 2 * (PA::Tile::LDS_ELEMS + PB::Tile::LDS_ELEMS) elements.  On return every wave has passed a barrier
 // after its last LDS read, so the caller may reuse `lds` at once.  The stage count is rounded up to a multiple of the
-// unrolled trip (the extra stages lie past klim and read as zeros), so the loop body has a single exit.
+// unrolled trip (the extra stages lie past klim and read as zeros), so the loop body has a single exit; the last trip is
+// peeled and does no reloads.
 template <int BM, int BN, int BK, int DA, int DB, class PA, class PB>
 __device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / 64][BN / 64], bf16_t *__restrict__ lds, PA &pa, PB &pb, int k_begin,
                                               int nstage)
@@ -323,13 +325,26 @@ __device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / 64][BN / 64], b
     }
     __syncthreads();
 
-    for (int s = 0; s < nstage; s += TRIP) {
+    const int nround = (nstage + TRIP - 1) / TRIP * TRIP;
+    int s = 0;
+    for (; s + TRIP < nround; s += TRIP) {
 #pragma unroll
         for (int u = 0; u < TRIP; ++u) {
             // stage s+u is in LDS buffer u % 2; slot (u+1) % D holds stage s+u+1 and is refilled with stage s+u+1+D
             bf16_t *cur = lds + (u & 1) * STAGE, *oth = lds + ((u & 1) ^ 1) * STAGE;
-            pipeline_stage<BK, MI, NI>(acc, cur, oth, ra[(u + 1) % DA], rb[(u + 1) % DB], pa, pb, s + u + 1 + DA, s + u + 1 + DB, wm, wn, lane);
+            pipeline_stage<BK, MI, NI, true, true>(acc, cur, oth, ra[(u + 1) % DA], rb[(u + 1) % DB], pa, pb, s + u + 1 + DA, s + u + 1 + DB, wm,
+                                                   wn, lane);
         }
+    }
+    // last trip: everything it would reload lies past the end (a hashed operand would hash for nothing), and its last
+    // stage has nothing left to hand to LDS
+#pragma unroll
+    for (int u = 0; u < TRIP; ++u) {
+        bf16_t *cur = lds + (u & 1) * STAGE, *oth = lds + ((u & 1) ^ 1) * STAGE;
+        if (u + 1 < TRIP)
+            pipeline_stage<BK, MI, NI, true, false>(acc, cur, oth, ra[(u + 1) % DA], rb[(u + 1) % DB], pa, pb, 0, 0, wm, wn, lane);
+        else
+            pipeline_stage<BK, MI, NI, false, false>(acc, cur, oth, ra[(u + 1) % DA], rb[(u + 1) % DB], pa, pb, 0, 0, wm, wn, lane);
     }
 }
 
