@@ -181,7 +181,7 @@ int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const void *dy, int6
  * (R.py:942-952) and MmBackward's dW followed by materialize_bwd (R.py:979-990, 304-359); the tensor autograd saves
  * for the backward pass (there: x, with W re-materialised) becomes z.
  * Needs: coef_rows == out_f, act_dtype RDB_BF16, tokens/in_f/out_f/k > 0, in_f, out_f, k multiples of 8,
- * tokens*k < 2^30, 16-byte aligned pointers, leading dimensions multiples of 8; otherwise RDB_E_UNSUPPORTED. */
+ * tokens*k < 2^29, 16-byte aligned pointers, leading dimensions multiples of 8; otherwise RDB_E_UNSUPPORTED. */
 
 /* Bytes of z for `desc` (tokens*k*2), or 0 when the projected form does not apply to it. */
 int64_t rdb_linear_projection_bytes(const rdb_linear_desc *desc);

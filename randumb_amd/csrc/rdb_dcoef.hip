@@ -137,7 +137,7 @@ int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, co
     if (d->act_dtype != RDB_BF16 || d->coef_rows == 0) return RDB_E_UNSUPPORTED;
     if (d->in_f % 8 || d->out_f % 8 || ldx % 8 || lddy % 8 || ((uintptr_t)x & 15) || ((uintptr_t)dy & 15)) return RDB_E_UNSUPPORTED;
     if (d->tokens < 1 || d->tokens > (1 << 30) || d->out_f > (1 << 30) || d->in_f > (1 << 30) || d->out_f * d->in_f > (1ll << 31) ||
-        d->tokens * lddy >= (1ll << 30) || d->tokens * ldx >= (1ll << 30))
+        d->tokens * lddy >= (1ll << 29) || d->tokens * ldx >= (1ll << 29))
         return RDB_E_UNSUPPORTED;
     DcoefParams p;
     p.dy = (const bf16_t *)dy;

@@ -90,7 +90,7 @@ static bool dx_factored_ok(const rdb_linear_desc *d)
 {
     return d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16 && d->coef_rows != 0 && d->k % 8 == 0 && d->in_f % 8 == 0 &&
            d->out_f % 8 == 0 && d->k > 0 && d->tokens > 0 && d->tokens < (1 << 30) && d->in_f < (1 << 30) && d->out_f < (1 << 30) &&
-           d->k < (1 << 24) && d->tokens * d->k < (1ll << 30) && d->out_f * d->k < (1ll << 30);
+           d->k < (1 << 24) && d->tokens * d->k < (1ll << 29) && d->out_f * d->k < (1ll << 29);
 }
 
 int64_t linear_dx_factored_workspace(const rdb_linear_desc *d)
@@ -105,7 +105,7 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
 {
     if (!dx_factored_ok(d) || scale_bias) return RDB_E_UNSUPPORTED;  // the random-bias term is not low rank
     if (!workspace || workspace_bytes < linear_dx_factored_workspace(d) || ((uintptr_t)workspace & 15)) return RDB_E_UNSUPPORTED;
-    if (d->tokens * lddy >= (1ll << 30)) return RDB_E_UNSUPPORTED;
+    if (d->tokens * lddy >= (1ll << 29)) return RDB_E_UNSUPPORTED;
     if (lddy % 8 || lddx % 8 || ((uintptr_t)dy & 15) || ((uintptr_t)coef & 15) || ((uintptr_t)dx & 15)) return RDB_E_UNSUPPORTED;
     // only worth it when the factored form is cheaper than forming the weight
     if (d->algo == RDB_ALGO_AUTO && d->k * (d->in_f + d->out_f) >= d->in_f * d->out_f) return RDB_E_UNSUPPORTED;

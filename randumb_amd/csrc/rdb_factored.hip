@@ -138,7 +138,7 @@ __global__ __launch_bounds__(256, 1) void factored_dc_kernel(DcParams p)
 static bool factored_shape_ok(const rdb_linear_desc *d)
 {
     return d->act_dtype == RDB_BF16 && d->coef_rows != 0 && d->k % 8 == 0 && d->in_f % 8 == 0 && d->out_f % 8 == 0 && d->k > 0 &&
-           d->tokens > 0 && d->in_f > 0 && d->out_f > 0 && d->tokens * d->k < (1ll << 30) && d->out_f * d->k < (1ll << 30);
+           d->tokens > 0 && d->in_f > 0 && d->out_f > 0 && d->tokens * d->k < (1ll << 29) && d->out_f * d->k < (1ll << 29);
 }
 static bool cheaper_factored(const rdb_linear_desc *d) { return d->k * (d->in_f + d->out_f) < d->in_f * d->out_f; }
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
@@ -151,7 +151,7 @@ int64_t linear_projection_bytes(const rdb_linear_desc *d)
 // The three entry points below return RDB_E_UNSUPPORTED, without setting an error, when the request does not fit.
 int linear_project(void *z, const void *x, int64_t ldx, const rdb_linear_desc *d, hipStream_t s)
 {
-    if (!factored_shape_ok(d) || d->tokens * ldx >= (1ll << 30) || ldx % 8 || !aligned16(x) || !aligned16(z)) return RDB_E_UNSUPPORTED;
+    if (!factored_shape_ok(d) || d->tokens * ldx >= (1ll << 29) || ldx % 8 || !aligned16(x) || !aligned16(z)) return RDB_E_UNSUPPORTED;
     ZParams p;
     p.x = (const bf16_t *)x;
     p.z = (bf16_t *)z;
@@ -186,7 +186,7 @@ int linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, 
 // dcoef must have been zeroed on the same stream.
 int linear_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *z, const rdb_linear_desc *d, int num_cus, hipStream_t s)
 {
-    if (!factored_shape_ok(d) || d->tokens * lddy >= (1ll << 30) || lddy % 8 || !aligned16(dy) || !aligned16(z)) return RDB_E_UNSUPPORTED;
+    if (!factored_shape_ok(d) || d->tokens * lddy >= (1ll << 29) || lddy % 8 || !aligned16(dy) || !aligned16(z)) return RDB_E_UNSUPPORTED;
     DcParams p;
     p.dy = (const bf16_t *)dy;
     p.z = (const bf16_t *)z;
@@ -216,7 +216,7 @@ int linear_fwd_factored(void *y, int64_t ldy, const void *x, int64_t ldx, const 
     if (!workspace || workspace_bytes < linear_projection_bytes(d)) return RDB_E_UNSUPPORTED;
     if (d->algo == RDB_ALGO_AUTO && !cheaper_factored(d)) return RDB_E_UNSUPPORTED;
     // check everything before the first launch, so that a refusal leaves nothing half done
-    if (d->tokens * ldx >= (1ll << 30) || ldx % 8 || ldy % 8 || !aligned16(x) || !aligned16(coef) || !aligned16(y) || !aligned16(workspace))
+    if (d->tokens * ldx >= (1ll << 29) || ldx % 8 || ldy % 8 || !aligned16(x) || !aligned16(coef) || !aligned16(y) || !aligned16(workspace))
         return RDB_E_UNSUPPORTED;
     int rc = linear_project(workspace, x, ldx, d, s);
     if (rc) return rc;
@@ -230,7 +230,7 @@ int linear_dcoef_factored(float *dcoef, const void *dy, int64_t lddy, const void
     if (!factored_shape_ok(d)) return RDB_E_UNSUPPORTED;
     if (!workspace || workspace_bytes < linear_projection_bytes(d)) return RDB_E_UNSUPPORTED;
     if (d->algo == RDB_ALGO_AUTO && !cheaper_factored(d)) return RDB_E_UNSUPPORTED;
-    if (d->tokens * ldx >= (1ll << 30) || d->tokens * lddy >= (1ll << 30) || ldx % 8 || lddy % 8 || !aligned16(x) || !aligned16(dy) ||
+    if (d->tokens * ldx >= (1ll << 29) || d->tokens * lddy >= (1ll << 29) || ldx % 8 || lddy % 8 || !aligned16(x) || !aligned16(dy) ||
         !aligned16(workspace))
         return RDB_E_UNSUPPORTED;
     int rc = linear_project(workspace, x, ldx, d, s);

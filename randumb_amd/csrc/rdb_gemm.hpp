@@ -21,9 +21,10 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
-// Byte offset that lies outside every buffer the tile engine reads (operands are smaller than 2^31 bytes): a buffer load
-// at this offset fails the hardware bounds check and returns zeros, without a branch and without touching memory.
-constexpr uint32_t BUFFER_OOB = 0x80000000u;
+// Byte offset that lies outside every buffer the tile engine reads (operands are smaller than 2^30 bytes): a buffer load
+// at this offset fails the hardware bounds check and returns zeros, without a branch and without touching memory.  Two of
+// them, or one plus any in-range offset, still add up to an out-of-range offset below 2^32.
+constexpr uint32_t BUFFER_OOB = 0x40000000u;
 
 enum OperandLayout { K_CONT = 0, M_CONT = 1 };
 
@@ -52,12 +53,13 @@ template <int ROWS, int BK, int LAYOUT> struct OperandTile {
     static constexpr int PER_THREAD = (PIECES + 255) / 256;
     static_assert(PIECES % 256 == 0, "operand stage must split evenly over 256 threads");
 
-    // Per-thread description of the pieces it copies from global memory: byte offset of each piece at stage 0 (BUFFER_OOB
-    // when its tile row lies outside the matrix) and its contraction offset inside a stage.  Built once, before the loop.
+    // Per-thread description of the pieces it copies from global memory: byte offset of each piece at stage 0, BUFFER_OOB
+    // when its tile row lies outside the matrix.  Built once, before the loop.
     struct Pieces {
         uint32_t off[PER_THREAD];
-        int kk[PER_THREAD];
     };
+    // K_CONT: the contraction offset of a thread's pieces inside a stage is the same for all of them (256 % (BK/8) == 0).
+    __device__ static __forceinline__ int thread_kk() { return (threadIdx.x % (BK / 8)) * 8; }
     __device__ static __forceinline__ Pieces pieces(int64_t ld, int row0, int nrows, int k_begin)
     {
         Pieces q;
@@ -73,22 +75,18 @@ template <int ROWS, int BK, int LAYOUT> struct OperandTile {
                 k = idx / (ROWS / 8);
                 row = row0 + (idx % (ROWS / 8)) * 8;
             }
-            q.kk[p] = k;
             const uint32_t elem = (LAYOUT == K_CONT) ? (uint32_t)(row * ld) + k_begin + k : (uint32_t)((k_begin + k) * ld) + row;
             q.off[p] = row < nrows ? elem * 2u : BUFFER_OOB;
         }
         return q;
     }
 
-    // Global -> register for piece p of the stage whose first contraction index is k0; `adv` is the byte offset of that
-    // stage relative to stage 0.  A buffer load: pieces outside the matrix (row >= nrows or k >= klim) carry an out-of-range
-    // offset and come back as zeros.  The host guarantees that the contiguous axis is a multiple of 8, so a 16-byte piece is
-    // entirely inside or outside.
-    __device__ static __forceinline__ void load_piece(f32x4 &reg, __amdgpu_buffer_rsrc_t rsrc, const Pieces &q, int p, uint32_t adv, int k0,
-                                                      int klim)
+    // Global -> register for piece p; `adv` is the byte offset of the stage relative to stage 0, or BUFFER_OOB.  A buffer
+    // load: pieces outside the matrix carry an out-of-range offset and come back as zeros.  The host guarantees that the
+    // contiguous axis is a multiple of 8, so a 16-byte piece is entirely inside or outside.
+    __device__ static __forceinline__ void load_piece(f32x4 &reg, __amdgpu_buffer_rsrc_t rsrc, const Pieces &q, int p, uint32_t adv)
     {
-        const uint32_t o = (k0 + q.kk[p] < klim) ? q.off[p] + adv : BUFFER_OOB;
-        reg = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)o, 0, 0));
+        reg = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(q.off[p] + adv), 0, 0));
     }
 
     // Registers -> LDS stage.
@@ -157,17 +155,27 @@ template <int ROWS, int BK, int LAYOUT> struct GlobalOperand {
     int64_t extent;
     typename Tile::Pieces q;
     __amdgpu_buffer_rsrc_t rsrc;
-    int k_begin;
+    int k_begin, kk;
     __device__ __forceinline__ void init(int kb)
     {
         k_begin = kb;
+        kk = Tile::thread_kk();
         q = Tile::pieces(ld, row0, nrows, kb);
-        rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(src), 0, (int)(extent * 2), 0x00020000);
+        // M_CONT: contraction indices are rows of the source, so clipping the buffer at row klim makes the hardware bounds
+        // check zero everything from klim on.  K_CONT clips per thread in load_piece().
+        int64_t bytes = extent * 2;
+        if (LAYOUT == M_CONT && (int64_t)klim * ld * 2 < bytes) bytes = (int64_t)klim * ld * 2;
+        rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(src), 0, (int)bytes, 0x00020000);
     }
     __device__ __forceinline__ void load_piece(f32x4 &reg, int p, int stage) const
     {
-        const uint32_t adv = (LAYOUT == K_CONT) ? (uint32_t)(stage * BK * 2) : (uint32_t)(stage * BK * ld * 2);
-        Tile::load_piece(reg, rsrc, q, p, adv, k_begin + stage * BK, klim);
+        // one offset per stage (the same expression for every piece: computed once), one add per piece
+        uint32_t adv;
+        if (LAYOUT == K_CONT)
+            adv = (k_begin + stage * BK + kk < klim) ? (uint32_t)(stage * BK * 2) : BUFFER_OOB;
+        else
+            adv = (uint32_t)stage * (uint32_t)(BK * 2) * (uint32_t)ld;
+        Tile::load_piece(reg, rsrc, q, p, adv);
     }
     __device__ __forceinline__ void load(f32x4 (&regs)[Tile::PER_THREAD], int stage) const
     {

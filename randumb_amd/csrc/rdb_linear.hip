@@ -491,7 +491,7 @@ static int check_projected(const char *who, const rdb_linear_desc *d)
     if (rc) return rc;
     if (linear_projection_bytes(d) == 0)
         return set_error(RDB_E_UNSUPPORTED, "%s: the projected form needs matrix-coef, bf16 activations, non-empty sizes that are "
-                                            "multiples of 8 and tokens*k < 2^30", who);
+                                            "multiples of 8 and tokens*k < 2^29", who);
     return RDB_OK;
 }
 
@@ -505,7 +505,7 @@ extern "C" int rdb_linear_project(void *z, const void *x, int64_t ldx, const rdb
     if (ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_project: leading dimension smaller than the row");
     rc = linear_project(z, x, ldx, d, (hipStream_t)stream);
     if (rc == RDB_E_UNSUPPORTED)
-        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_project: x and z must be 16-byte aligned, ldx a multiple of 8, tokens*ldx < 2^30");
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_project: x and z must be 16-byte aligned, ldx a multiple of 8, tokens*ldx < 2^29");
     return rc;
 }
 
@@ -529,9 +529,9 @@ extern "C" int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int6
     if (rc) return rc;
     if (!dcoef || !dy || !z) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef_projected: dcoef, dy or z is NULL");
     if (lddy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dcoef_projected: leading dimension smaller than the row");
-    if (lddy % 8 || !aligned16(dy) || !aligned16(z) || d->tokens * lddy >= (1ll << 30))
+    if (lddy % 8 || !aligned16(dy) || !aligned16(z) || d->tokens * lddy >= (1ll << 29))
         return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dcoef_projected: dy and z must be 16-byte aligned, lddy a multiple of 8, "
-                                            "tokens*lddy < 2^30");
+                                            "tokens*lddy < 2^29");
     hipStream_t s = (hipStream_t)stream;
     rc = fill_zero(dcoef, d->coef_rows * d->k, s);
     if (rc) return rc;
