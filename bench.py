@@ -8,12 +8,12 @@ activations with fp32 accumulation, x ~ N(0,1), dy ~ N(0,1), C ~ N(0, 3*0.02^2/k
 A "step" is one pass of the hot path, y = x W^T, dx = dy W, dC = (dy^T x) N^T with W = C N never stored, through
 the C ABI of librandumb_hip.so with inputs already resident in HBM, the way a training step calls it:
   forward   rdb_linear_project (z = x N^T, kept for the backward pass in place of x) + rdb_linear_fwd_projected
-  backward  rdb_linear_bwd_dx + rdb_linear_bwd_dcoef_projected (reuses z)
+  backward  rdb_linear_bwd_projected (dx and dC from dy, z, C in two launches)
 The printed JSON line reports
   value        algorithmic TFLOP/s of the whole step, F = 6*T*in*out + 6*out*in*k (three dense products plus the
                weight generation per direction and the dC contraction).  The kernels use W = C N associatively and
                execute fewer flops than F (config.executed_gflop_per_step); both figures are printed.
-  roofline     the slowest of forward / dx / dcoef against the dense bf16 MFMA peak, from HIP-event timing
+  roofline     the backward call (two thirds of F, the slowest call) against the dense bf16 MFMA peak, from HIP events
   cpu_baseline the CPU restatement (materialise-then-matmul: oracle C + torch.matmul fp32) on the host cores
   compare      the one-call entry points (z recomputed in the backward pass), the kernels that do form W tiles on
                chip, materialise-to-HBM + dense GEMM on the GPU, and a plain dense GEMM
@@ -34,8 +34,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # counters read for a plain 256 MiB device copy (FETCH x2.000, WRITE x1.000): profiles/bench_c2_hbm_traffic.md
 HBM_TRAFFIC_BYTES = {
     "forward (factored_z_kernel + factored_y_kernel)": 84.5e6,
-    "dx (dx_dyc_kernel + dx_tn_kernel)": 84.3e6,
-    "dcoef (fill_zero_kernel + factored_dc_kernel)": 79.4e6,
+    "backward (dx_dyc_kernel + bwd_dc_tn_kernel)": 84.3e6 + 76.3e6,
 }
 T, IN_F, OUT_F, K, SEED = 8192, 768, 3072, 256, 0
 
@@ -113,10 +112,12 @@ def main():
         k_project()
         k_fwd_projected()
 
+    def k_bwd():
+        _lib.check(L.rdb_linear_bwd_projected(pdx, IN_F, pdC, pdy, OUT_F, pz, pC, dref, pws, ws_bytes, stream), "rdb_linear_bwd_projected")
+
     def step():
         k_fwd()
-        k_dx()
-        k_dcoef_projected()
+        k_bwd()
 
     # the one-call entry points: the same kernels, z recomputed into the workspace by the coefficient gradient
     def make_onecall(algo):
@@ -173,21 +174,21 @@ def main():
     calls = {
         "rdb_linear_project": event_ms(k_project, iters),
         "rdb_linear_fwd_projected": event_ms(k_fwd_projected, iters),
-        "rdb_linear_bwd_dx": event_ms(k_dx, iters),
-        "rdb_linear_bwd_dcoef_projected": event_ms(k_dcoef_projected, iters),
+        "rdb_linear_bwd_projected": event_ms(k_bwd, iters),
+        "rdb_linear_bwd_dx (separate call)": event_ms(k_dx, iters),
+        "rdb_linear_bwd_dcoef_projected (separate call)": event_ms(k_dcoef_projected, iters),
     }
-    products = {   # each carries one third of F
-        "forward (factored_z_kernel + factored_y_kernel)": calls["rdb_linear_project"] + calls["rdb_linear_fwd_projected"],
-        "dx (dx_dyc_kernel + dx_tn_kernel)": calls["rdb_linear_bwd_dx"],
-        "dcoef (fill_zero_kernel + factored_dc_kernel)": calls["rdb_linear_bwd_dcoef_projected"],
+    products = {   # share of F: forward one third, backward (dx and dC) two thirds
+        "forward (factored_z_kernel + factored_y_kernel)": (calls["rdb_linear_project"] + calls["rdb_linear_fwd_projected"], F_PER_PRODUCT),
+        "backward (dx_dyc_kernel + bwd_dc_tn_kernel)": (calls["rdb_linear_bwd_projected"], 2 * F_PER_PRODUCT),
     }
-    dom = max(products, key=lambda n: products[n])
-    dom_ms = products[dom]
-    achieved = F_PER_PRODUCT / (dom_ms * 1e-3) / 1e12
+    dom = max(products, key=lambda n: products[n][0])
+    dom_ms, dom_flops = products[dom]
+    achieved = dom_flops / (dom_ms * 1e-3) / 1e12
     roofline = {
         "bound": "mfma", "kernel": dom, "achieved": round(achieved, 3), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 5), "traffic": HBM_TRAFFIC_BYTES[dom], "avg_kernel_ms": round(dom_ms, 5),
-        "algorithmic_gflop_per_launch": round(F_PER_PRODUCT / 1e9, 3),
+        "algorithmic_gflop_per_launch": round(dom_flops / 1e9, 3),
         "calls_ms": {n: round(v, 5) for n, v in calls.items()},
     }
 

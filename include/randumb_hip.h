@@ -198,6 +198,16 @@ int rdb_linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *co
 int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *z,
                                    const rdb_linear_desc *desc, void *stream);
 
+/* Whole backward pass of the layer from the saved projection, in two kernel launches instead of five:
+ * dx[t, i] = sum_o dy[t, o] * W[o, i] (act dtype) and dcoef = dy^T . z (fp32, OVERWRITTEN).  The first launch computes
+ * dy . C and clears dcoef on the side; the second runs the dcoef blocks and the (dy.C).N blocks side by side, which lean on
+ * different units of a compute unit (LDS + matrix cores against the integer hash on the vector ALU).
+ * workspace: rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX, desc) bytes.  Same requirements as the other projected
+ * entry points, coef in bf16; dcoef 16-byte aligned. */
+int rdb_linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z,
+                             const void *coef, const rdb_linear_desc *desc, void *workspace,
+                             int64_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

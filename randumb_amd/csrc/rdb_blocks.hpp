@@ -1,0 +1,127 @@
+// Block bodies shared by more than one kernel: the coefficient-gradient block (dC = dy^T . z) and the second block of the
+// input gradient (dx = t . N) run as kernels of their own and side by side in one launch of the merged backward kernel.
+#pragma once
+#include "rdb_gemm.hpp"
+#include "rdb_tile.hpp"
+
+namespace rdb {
+
+constexpr int B_BK = 64;
+
+// ----------------------------------------------------------------------------------------------- dC = dy^T . z
+// tile: 128 output features (engine rows "a") x 128 coefficients (engine rows "b"), contraction over a token range
+constexpr int KD_BO = 128, KD_BM = 128;
+
+struct DcParams {
+    const bf16_t *dy;
+    const bf16_t *z;
+    float *dcoef;
+    int64_t lddy;
+    int tokens, out_f, k;
+    int tiles_o, tiles_m, splits, tok_per_split;
+};
+
+// `block`: index of this block among the blocks that run this body.
+__device__ __forceinline__ void dc_block(const DcParams &p, bf16_t *lds, int block)
+{
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
+    // work item = (token split, output tile, coefficient tile), coefficient tile fastest: neighbours share the dy stream
+    const int total = p.tiles_o * p.tiles_m * p.splits;
+    const int w = xcd_work_item(block, total);
+    if (w >= total) return;
+    const int m0 = (w % p.tiles_m) * KD_BM, o0 = ((w / p.tiles_m) % p.tiles_o) * KD_BO, split = w / (p.tiles_m * p.tiles_o);
+    const int t_begin = split * p.tok_per_split;
+    const int t_end = (t_begin + p.tok_per_split < p.tokens) ? t_begin + p.tok_per_split : p.tokens;
+    f32x16 acc[KD_BO / 64][KD_BM / 64];
+#pragma unroll
+    for (int mi = 0; mi < KD_BO / 64; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < KD_BM / 64; ++ni) acc[mi][ni] = zero16();
+    GlobalOperand<KD_BO, B_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
+    GlobalOperand<KD_BM, B_BK, M_CONT> opz = {p.z, (int64_t)p.k, m0, p.k, t_end, (int64_t)p.tokens * p.k};
+    gemm_mainloop<KD_BO, KD_BM, B_BK, 1, 1>(acc, lds, opdy, opz, t_begin, (t_end - t_begin + B_BK - 1) / B_BK);
+    // acc[mi][ni][j]: o = o0 + wm*64 + mi*32 + 8*(j/4) + 4*g + j%4, m = m0 + wn*64 + ni*32 + r (32 consecutive m: coalesced)
+#pragma unroll
+    for (int ni = 0; ni < KD_BM / 64; ++ni) {
+        const int m = m0 + wn * 64 + ni * 32 + r;
+        if (m >= p.k) continue;
+#pragma unroll
+        for (int mi = 0; mi < KD_BO / 64; ++mi)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int o = o0 + wm * 64 + mi * 32 + 8 * (j / 4) + 4 * g + (j % 4);
+                if (o < p.out_f) unsafeAtomicAdd(p.dcoef + (int64_t)o * p.k + m, acc[mi][ni][j]);
+            }
+    }
+}
+
+// ----------------------------------------------------------------------------------------------- kernel 2: dx = t . N
+// tile: 192 input features (engine rows "a", hashed operand) x 128 tokens (engine rows "b"), contraction over k
+constexpr int K2_BI = 192, K2_BT = 128;
+
+struct TNParams {
+    const bf16_t *t;
+    bf16_t *dx;
+    int64_t lddx;
+    int tokens, in_f, k;
+    int tiles_i, tiles_t;
+    uint32_t seed;
+};
+
+__device__ __forceinline__ void tn_block(const TNParams &p, bf16_t *lds, int block)
+{
+    // work item = (token tile, feature tile), feature tile fastest: neighbours share the t tile
+    const int w = xcd_work_item(block, p.tiles_i * p.tiles_t);
+    if (w >= p.tiles_i * p.tiles_t) return;
+    const int i0 = (w % p.tiles_i) * K2_BI, tok0 = (w / p.tiles_i) * K2_BT;
+    f32x16 acc[K2_BI / 64][K2_BT / 64];
+#pragma unroll
+    for (int mi = 0; mi < K2_BI / 64; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < K2_BT / 64; ++ni) acc[mi][ni] = zero16();
+    // "A": 2^31 * noise(i, m), rows = i, contraction = m; values for m >= k meet zero rows of t
+    NoiseOperandRowsAreElements<K2_BI, B_BK> opn = {i0, p.seed};
+    // "B": t[tok][m]
+    GlobalOperand<K2_BT, B_BK, K_CONT> opt = {p.t, (int64_t)p.k, tok0, p.tokens, p.k, (int64_t)p.tokens * p.k};
+    gemm_mainloop<K2_BI, K2_BT, B_BK, 1, 1>(acc, lds, opn, opt, 0, (p.k + B_BK - 1) / B_BK);
+    store_tile_bf16<K2_BI, K2_BT>(acc, lds, p.dx, p.lddx, i0, p.in_f, tok0, p.tokens, 4.656612873077392578125e-10f, nullptr);
+}
+
+// ----------------------------------------------------------------------------------------------- host side
+// Parameters of the coefficient-gradient blocks for layer d; the token range is split so that tiles x splits is about one
+// block per compute unit.  Returns the number of work items.
+inline int make_dc_params(DcParams &p, float *dcoef, const void *dy, int64_t lddy, const void *z, const rdb_linear_desc *d, int num_cus)
+{
+    p.dy = (const bf16_t *)dy;
+    p.z = (const bf16_t *)z;
+    p.dcoef = dcoef;
+    p.lddy = lddy;
+    p.tokens = (int)d->tokens;
+    p.out_f = (int)d->out_f;
+    p.k = (int)d->k;
+    p.tiles_o = (int)cdiv(d->out_f, KD_BO);
+    p.tiles_m = (int)cdiv(d->k, KD_BM);
+    int splits = num_cus / (p.tiles_o * p.tiles_m);
+    const int max_splits = (int)cdiv(d->tokens, 256);
+    if (splits > max_splits) splits = max_splits;
+    if (splits < 1) splits = 1;
+    p.tok_per_split = (int)(cdiv(cdiv(d->tokens, splits), B_BK) * B_BK);
+    p.splits = (int)cdiv(d->tokens, p.tok_per_split);
+    return p.tiles_o * p.tiles_m * p.splits;
+}
+
+inline int make_tn_params(TNParams &p, void *dx, int64_t lddx, const void *t, const rdb_linear_desc *d)
+{
+    p.t = (const bf16_t *)t;
+    p.dx = (bf16_t *)dx;
+    p.lddx = lddx;
+    p.tokens = (int)d->tokens;
+    p.in_f = (int)d->in_f;
+    p.k = (int)d->k;
+    p.seed = d->seed;
+    p.tiles_i = (int)cdiv(d->in_f, K2_BI);
+    p.tiles_t = (int)cdiv(d->tokens, K2_BT);
+    return p.tiles_i * p.tiles_t;
+}
+
+}  // namespace rdb

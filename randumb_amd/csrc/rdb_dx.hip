@@ -9,8 +9,7 @@
 //                                                          registers, stage by stage, interleaved with the MFMAs)
 // Replaces autograd's MmBackward on the re-materialised weight (materialize() + dense product,
 // src/rten_cpp/RandumbTensor.py:942-946).
-#include "rdb_gemm.hpp"
-#include "rdb_tile.hpp"
+#include "rdb_blocks.hpp"
 
 namespace rdb {
 
@@ -25,6 +24,8 @@ struct DyCParams {
     const bf16_t *dy;
     const bf16_t *coef;
     bf16_t *t;
+    float *zero;     // NULL, or an array this launch clears on the side (16-byte aligned, zero_n a multiple of 4)
+    int64_t zero_n;
     int64_t lddy;
     int tokens, out_f, k;
     int tiles_c, tiles_t;
@@ -34,6 +35,11 @@ __global__ __launch_bounds__(256, 2) void dx_dyc_kernel(DyCParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
+    if (p.zero) {  // a kernel later in the stream accumulates into this array with atomics
+        const f32x4 z4 = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < p.zero_n / 4; e += (int64_t)gridDim.x * 256)
+            reinterpret_cast<f32x4 *>(p.zero)[e] = z4;
+    }
     // work item = (token tile, coefficient tile), coefficient tile fastest: neighbours share the dy tile
     const int w = xcd_work_item(blockIdx.x, p.tiles_c * p.tiles_t);
     if (w >= p.tiles_c * p.tiles_t) return;
@@ -52,37 +58,31 @@ __global__ __launch_bounds__(256, 2) void dx_dyc_kernel(DyCParams p)
 }
 
 // ----------------------------------------------------------------------------------------------- kernel 2: dx = t . N
-// tile: 192 input features (engine rows "a", hashed operand) x 128 tokens (engine rows "b"), contraction over k
-constexpr int K2_BI = 192, K2_BT = 128;
-
-struct TNParams {
-    const bf16_t *t;
-    bf16_t *dx;
-    int64_t lddx;
-    int tokens, in_f, k;
-    int tiles_i, tiles_t;
-    uint32_t seed;
-};
-
+// body in rdb_blocks.hpp (tn_block)
 __global__ __launch_bounds__(256, 1) void dx_tn_kernel(TNParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
+    tn_block(p, reinterpret_cast<bf16_t *>(smem_raw), blockIdx.x);
+}
+
+// ----------------------------------------------------------------------------------------------- dC and dx = t . N in one launch
+// The coefficient-gradient blocks (LDS- and matrix-core-bound) and the dx = t.N blocks (bound by the integer hash on the
+// vector ALU) are independent once t, z and a zeroed dcoef exist, and lean on different units: launched as one grid, two
+// blocks per compute unit, they overlap instead of queueing.  Both bodies use exactly 80 KB of LDS.
+struct BwdParams {
+    DcParams dc;
+    TNParams tn;
+    int dc_blocks;  // multiple of 8, so both parts keep their die assignment
+};
+
+__global__ __launch_bounds__(256, 2) void bwd_dc_tn_kernel(BwdParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
-    // work item = (token tile, feature tile), feature tile fastest: neighbours share the t tile
-    const int w = xcd_work_item(blockIdx.x, p.tiles_i * p.tiles_t);
-    if (w >= p.tiles_i * p.tiles_t) return;
-    const int i0 = (w % p.tiles_i) * K2_BI, tok0 = (w / p.tiles_i) * K2_BT;
-    f32x16 acc[K2_BI / 64][K2_BT / 64];
-#pragma unroll
-    for (int mi = 0; mi < K2_BI / 64; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < K2_BT / 64; ++ni) acc[mi][ni] = zero16();
-    // "A": 2^31 * noise(i, m), rows = i, contraction = m; values for m >= k meet zero rows of t
-    NoiseOperandRowsAreElements<K2_BI, X_BK> opn = {i0, p.seed};
-    // "B": t[tok][m]
-    GlobalOperand<K2_BT, X_BK, K_CONT> opt = {p.t, (int64_t)p.k, tok0, p.tokens, p.k, (int64_t)p.tokens * p.k};
-    gemm_mainloop<K2_BI, K2_BT, X_BK, 1, 1>(acc, lds, opn, opt, 0, (p.k + X_BK - 1) / X_BK);
-    store_tile_bf16<K2_BI, K2_BT>(acc, lds, p.dx, p.lddx, i0, p.in_f, tok0, p.tokens, 4.656612873077392578125e-10f, nullptr);
+    if ((int)blockIdx.x < p.dc_blocks)
+        dc_block(p.dc, lds, blockIdx.x);
+    else
+        tn_block(p.tn, lds, blockIdx.x - p.dc_blocks);
 }
 
 // ----------------------------------------------------------------------------------------------- host side
@@ -99,6 +99,21 @@ int64_t linear_dx_factored_workspace(const rdb_linear_desc *d)
     return d->tokens * d->k * (int64_t)sizeof(bf16_t);
 }
 
+static void make_dyc_params(DyCParams &p1, const void *dy, int64_t lddy, const void *coef, void *t, const rdb_linear_desc *d)
+{
+    p1.dy = (const bf16_t *)dy;
+    p1.coef = (const bf16_t *)coef;
+    p1.t = (bf16_t *)t;
+    p1.zero = nullptr;
+    p1.zero_n = 0;
+    p1.lddy = lddy;
+    p1.tokens = (int)d->tokens;
+    p1.out_f = (int)d->out_f;
+    p1.k = (int)d->k;
+    p1.tiles_c = (int)cdiv(d->k, K1_BC);
+    p1.tiles_t = (int)cdiv(d->tokens, K1_BT);
+}
+
 // Returns RDB_E_UNSUPPORTED (without setting an error) when the request does not fit this algorithm.
 int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias,
                        const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s)
@@ -111,29 +126,40 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
     if (d->algo == RDB_ALGO_AUTO && d->k * (d->in_f + d->out_f) >= d->in_f * d->out_f) return RDB_E_UNSUPPORTED;
 
     DyCParams p1;
-    p1.dy = (const bf16_t *)dy;
-    p1.coef = (const bf16_t *)coef;
-    p1.t = (bf16_t *)workspace;
-    p1.lddy = lddy;
-    p1.tokens = (int)d->tokens;
-    p1.out_f = (int)d->out_f;
-    p1.k = (int)d->k;
-    p1.tiles_c = (int)cdiv(d->k, K1_BC);
-    p1.tiles_t = (int)cdiv(d->tokens, K1_BT);
+    make_dyc_params(p1, dy, lddy, coef, workspace, d);
     int rc = launch_engine(dx_dyc_kernel, p1, p1.tiles_c * p1.tiles_t, engine_smem<K1_BC, K1_BT, X_BK, M_CONT, K_CONT>(), s, "dx_dyc_kernel");
     if (rc) return rc;
-
     TNParams p2;
-    p2.t = (const bf16_t *)workspace;
-    p2.dx = (bf16_t *)dx;
-    p2.lddx = lddx;
-    p2.tokens = (int)d->tokens;
-    p2.in_f = (int)d->in_f;
-    p2.k = (int)d->k;
-    p2.seed = d->seed;
-    p2.tiles_i = (int)cdiv(d->in_f, K2_BI);
-    p2.tiles_t = (int)cdiv(d->tokens, K2_BT);
-    return launch_engine(dx_tn_kernel, p2, p2.tiles_i * p2.tiles_t, engine_smem<K2_BI, K2_BT, X_BK, K_CONT, K_CONT>(), s, "dx_tn_kernel");
+    const int items = make_tn_params(p2, dx, lddx, workspace, d);
+    return launch_engine(dx_tn_kernel, p2, items, engine_smem<K2_BI, K2_BT, X_BK, K_CONT, K_CONT>(), s, "dx_tn_kernel");
+}
+
+// Whole backward pass of the layer from the saved projection z: dx = (dy.C).N and dcoef = dy^T.z in two launches.
+// Returns RDB_E_UNSUPPORTED (without setting an error) when the request does not fit.
+int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z, const void *coef,
+                         const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s)
+{
+    if (!dx_factored_ok(d)) return RDB_E_UNSUPPORTED;
+    if (!workspace || workspace_bytes < linear_dx_factored_workspace(d) || ((uintptr_t)workspace & 15)) return RDB_E_UNSUPPORTED;
+    if (d->tokens * lddy >= (1ll << 29) || lddy % 8 || lddx % 8) return RDB_E_UNSUPPORTED;
+    if (((uintptr_t)dy & 15) || ((uintptr_t)coef & 15) || ((uintptr_t)dx & 15) || ((uintptr_t)z & 15) || ((uintptr_t)dcoef & 15))
+        return RDB_E_UNSUPPORTED;
+    DyCParams p1;
+    make_dyc_params(p1, dy, lddy, coef, workspace, d);
+    p1.zero = dcoef;  // cleared here, accumulated into by the next launch
+    p1.zero_n = d->out_f * d->k;
+    int rc = launch_engine(dx_dyc_kernel, p1, p1.tiles_c * p1.tiles_t, engine_smem<K1_BC, K1_BT, X_BK, M_CONT, K_CONT>(), s, "dx_dyc_kernel");
+    if (rc) return rc;
+    BwdParams p;
+    const int dc_items = make_dc_params(p.dc, dcoef, dy, lddy, z, d, num_cus);
+    const int tn_items = make_tn_params(p.tn, dx, lddx, workspace, d);
+    p.dc_blocks = xcd_grid_size(dc_items);
+    size_t smem = engine_smem<KD_BO, KD_BM, X_BK, M_CONT, M_CONT>();
+    if (smem < engine_smem<K2_BI, K2_BT, X_BK, K_CONT, K_CONT>()) smem = engine_smem<K2_BI, K2_BT, X_BK, K_CONT, K_CONT>();
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dc_tn_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return set_error((int)e, "bwd_dc_tn_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+    bwd_dc_tn_kernel<<<p.dc_blocks + xcd_grid_size(tn_items), 256, smem, s>>>(p);
+    return check_launch("bwd_dc_tn_kernel");
 }
 
 }  // namespace rdb

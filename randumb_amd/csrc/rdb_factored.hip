@@ -10,8 +10,7 @@
 // z is bf16; it lives in the caller's workspace, or in a buffer the caller keeps from the forward to the backward pass (it
 // is all the backward pass needs of x, at k/in_f of its size).  Replaces materialize() + dense product
 // (src/rten_cpp/RandumbTensor.py:942-946) and MmBackward's dW followed by materialize_bwd (RandumbTensor.py:979-990, 304-359).
-#include "rdb_gemm.hpp"
-#include "rdb_tile.hpp"
+#include "rdb_blocks.hpp"
 
 namespace rdb {
 
@@ -86,51 +85,11 @@ __global__ __launch_bounds__(256, 2) void factored_y_kernel(YParams p)
 }
 
 // ----------------------------------------------------------------------------------------------- dC = dy^T . z
-// tile: 128 output features (engine rows "a") x 128 coefficients (engine rows "b"), contraction over a token range
-constexpr int KD_BO = 128, KD_BM = 128;
-
-struct DcParams {
-    const bf16_t *dy;
-    const bf16_t *z;
-    float *dcoef;
-    int64_t lddy;
-    int tokens, out_f, k;
-    int tiles_o, tiles_m, splits, tok_per_split;
-};
-
+// body in rdb_blocks.hpp (dc_block)
 __global__ __launch_bounds__(256, 1) void factored_dc_kernel(DcParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
-    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
-    // work item = (token split, output tile, coefficient tile), coefficient tile fastest: neighbours share the dy stream
-    const int total = p.tiles_o * p.tiles_m * p.splits;
-    const int w = xcd_work_item(blockIdx.x, total);
-    if (w >= total) return;
-    const int m0 = (w % p.tiles_m) * KD_BM, o0 = ((w / p.tiles_m) % p.tiles_o) * KD_BO, split = w / (p.tiles_m * p.tiles_o);
-    const int t_begin = split * p.tok_per_split;
-    const int t_end = (t_begin + p.tok_per_split < p.tokens) ? t_begin + p.tok_per_split : p.tokens;
-    f32x16 acc[KD_BO / 64][KD_BM / 64];
-#pragma unroll
-    for (int mi = 0; mi < KD_BO / 64; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < KD_BM / 64; ++ni) acc[mi][ni] = zero16();
-    GlobalOperand<KD_BO, F_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
-    GlobalOperand<KD_BM, F_BK, M_CONT> opz = {p.z, (int64_t)p.k, m0, p.k, t_end, (int64_t)p.tokens * p.k};
-    gemm_mainloop<KD_BO, KD_BM, F_BK, 1, 1>(acc, lds, opdy, opz, t_begin, (t_end - t_begin + F_BK - 1) / F_BK);
-    // acc[mi][ni][j]: o = o0 + wm*64 + mi*32 + 8*(j/4) + 4*g + j%4, m = m0 + wn*64 + ni*32 + r (32 consecutive m: coalesced)
-#pragma unroll
-    for (int ni = 0; ni < KD_BM / 64; ++ni) {
-        const int m = m0 + wn * 64 + ni * 32 + r;
-        if (m >= p.k) continue;
-#pragma unroll
-        for (int mi = 0; mi < KD_BO / 64; ++mi)
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const int o = o0 + wm * 64 + mi * 32 + 8 * (j / 4) + 4 * g + (j % 4);
-                if (o < p.out_f) unsafeAtomicAdd(p.dcoef + (int64_t)o * p.k + m, acc[mi][ni][j]);
-            }
-    }
+    dc_block(p, reinterpret_cast<bf16_t *>(smem_raw), blockIdx.x);
 }
 
 // ----------------------------------------------------------------------------------------------- host side
@@ -188,23 +147,8 @@ int linear_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const voi
 {
     if (!factored_shape_ok(d) || d->tokens * lddy >= (1ll << 29) || lddy % 8 || !aligned16(dy) || !aligned16(z)) return RDB_E_UNSUPPORTED;
     DcParams p;
-    p.dy = (const bf16_t *)dy;
-    p.z = (const bf16_t *)z;
-    p.dcoef = dcoef;
-    p.lddy = lddy;
-    p.tokens = (int)d->tokens;
-    p.out_f = (int)d->out_f;
-    p.k = (int)d->k;
-    p.tiles_o = (int)cdiv(d->out_f, KD_BO);
-    p.tiles_m = (int)cdiv(d->k, KD_BM);
-    // split the token range so that tiles x splits is about one block per compute unit
-    int splits = num_cus / (p.tiles_o * p.tiles_m);
-    const int max_splits = (int)cdiv(d->tokens, 256);
-    if (splits > max_splits) splits = max_splits;
-    if (splits < 1) splits = 1;
-    p.tok_per_split = (int)(cdiv(cdiv(d->tokens, splits), F_BK) * F_BK);
-    p.splits = (int)cdiv(d->tokens, p.tok_per_split);
-    return launch_engine(factored_dc_kernel, p, p.tiles_o * p.tiles_m * p.splits, engine_smem<KD_BO, KD_BM, F_BK, M_CONT, M_CONT>(), s,
+    const int items = make_dc_params(p, dcoef, dy, lddy, z, d, num_cus);
+    return launch_engine(factored_dc_kernel, p, items, engine_smem<KD_BO, KD_BM, F_BK, M_CONT, M_CONT>(), s,
                          "factored_dc_kernel");
 }
 

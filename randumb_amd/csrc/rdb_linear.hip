@@ -291,6 +291,8 @@ int linear_dcoef_factored(float *dcoef, const void *dy, int64_t lddy, const void
                           void *workspace, int64_t workspace_bytes, hipStream_t s);
 
 // rdb_dx.hip
+int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z, const void *coef,
+                         const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
 int64_t linear_dx_factored_workspace(const rdb_linear_desc *d);
 int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias,
                        const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s);
@@ -536,4 +538,19 @@ extern "C" int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int6
     rc = fill_zero(dcoef, d->coef_rows * d->k, s);
     if (rc) return rc;
     return linear_dcoef_projected(dcoef, dy, lddy, z, d, num_compute_units(), s);
+}
+
+extern "C" int rdb_linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z, const void *coef,
+                                        const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    int rc = check_projected("rdb_linear_bwd_projected", d);
+    if (rc) return rc;
+    if (!dx || !dcoef || !dy || !z || !coef) return set_error(RDB_E_NULL, "rdb_linear_bwd_projected: dx, dcoef, dy, z or coef is NULL");
+    if (lddy < d->out_f || lddx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_projected: leading dimension smaller than the row");
+    rc = linear_bwd_projected(dx, lddx, dcoef, dy, lddy, z, coef, d, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
+    if (rc == RDB_E_UNSUPPORTED)
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_projected: coefficients must be bf16; all pointers 16-byte aligned; lddy, lddx "
+                                            "multiples of 8; tokens*lddy < 2^29; workspace of rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX) "
+                                            "bytes");
+    return rc;
 }

@@ -311,3 +311,24 @@ def linear_bwd_dcoef_projected(dy: torch.Tensor, z: torch.Tensor, in_f: int, see
         rc = _lib.load().rdb_linear_bwd_dcoef_projected(_p(dcoef), _p(dy), dy.stride(0), _p(z), ctypes.byref(d), _stream(dy.device))
     _lib.check(rc, "rdb_linear_bwd_dcoef_projected")
     return dcoef
+
+
+def linear_bwd_projected(dy: torch.Tensor, z: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int):
+    """Whole backward pass of a matrix-coef bf16 layer from the saved projection: ``(dx, dcoef)`` with ``dx = dy @ W`` in
+    bf16 and ``dcoef = dy.T @ z`` in fp32, in two kernel launches."""
+    _need_gpu("linear_bwd_projected", dy, z, coef)
+    dy = _act(dy)
+    z = z.contiguous()
+    c = _native(coef)
+    out_f, k = c.shape
+    d = _proj_desc(dy.shape[0], in_f, out_f, k, seed, c.dtype)
+    dx = torch.empty((dy.shape[0], in_f), dtype=dy.dtype, device=dy.device)
+    dcoef = torch.empty((out_f, k), dtype=torch.float32, device=dy.device)
+    L = _lib.load()
+    ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX, ctypes.byref(d))
+    ws = _workspace(ws_bytes, dy.device)
+    with torch.cuda.device(dy.device):
+        rc = L.rdb_linear_bwd_projected(_p(dx), dx.stride(0), _p(dcoef), _p(dy), dy.stride(0), _p(z), _p(c), ctypes.byref(d), _p(ws),
+                                        ws_bytes, _stream(dy.device))
+    _lib.check(rc, "rdb_linear_bwd_projected")
+    return dx, dcoef

@@ -23,7 +23,7 @@ from . import hip
 __all__ = [
     "materialize_fwd", "materialize_bwd", "scale_bias_bwd", "embed_fwd", "embed_bwd",
     "linear_fwd", "linear_bwd_dx", "linear_bwd_dcoef", "linear", "linear_project", "linear_fwd_projected",
-    "linear_bwd_dcoef_projected", "sq5_gen_2d", "sq5_gen_1d",
+    "linear_bwd_dcoef_projected", "linear_bwd_projected", "sq5_gen_2d", "sq5_gen_1d",
 ]
 
 
@@ -231,6 +231,18 @@ def _(dy, z, in_features, seed):
     return dy.new_empty([dy.shape[1], z.shape[1]], dtype=torch.float32)
 
 
+@custom_op("rten::linear_bwd_projected", mutates_args=())
+def linear_bwd_projected(dy: Tensor, z: Tensor, coefs: Tensor, in_features: int, seed: int) -> List[Tensor]:
+    """``[dx, dcoef]`` of a matrix-coef bf16 layer from the saved projection, in one call."""
+    dx, dcoef = hip.linear_bwd_projected(dy, z, coefs, in_features, seed)
+    return [dx, dcoef]
+
+
+@linear_bwd_projected.register_fake
+def _(dy, z, coefs, in_features, seed):
+    return [dy.new_empty([dy.shape[0], in_features]), dy.new_empty([coefs.shape[0], coefs.shape[1]], dtype=torch.float32)]
+
+
 class _ProjectedLinear(torch.autograd.Function):
     """``y = x @ W.T (+ bias)`` for a matrix-coef weight in bf16.  The forward pass computes ``z = x @ Noise.T`` once and
     saves it for the backward pass in place of ``x`` (``k / in_features`` of its size); the reference's autograd saves
@@ -250,9 +262,12 @@ class _ProjectedLinear(torch.autograd.Function):
         in_f, out_f, seed = ctx.meta
         dy = dy.contiguous()
         dx = dcoefs = dbias = None
-        if ctx.needs_input_grad[0]:
+        if ctx.needs_input_grad[0] and ctx.needs_input_grad[1]:
+            dx, dc = linear_bwd_projected(dy, z, coefs, in_f, seed)
+            dcoefs = dc.to(coefs.dtype)
+        elif ctx.needs_input_grad[0]:
             dx = linear_bwd_dx(dy, coefs, in_f, out_f, in_f, 1, seed, None)
-        if ctx.needs_input_grad[1]:
+        elif ctx.needs_input_grad[1]:
             dcoefs = linear_bwd_dcoef_projected(dy, z, in_f, seed).to(coefs.dtype)
         if ctx.bias_dtype is not None and ctx.needs_input_grad[5]:
             dbias = dy.sum(0).to(ctx.bias_dtype)

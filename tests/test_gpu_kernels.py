@@ -364,6 +364,22 @@ def test_linear_projected_form(hip, oracle, T, in_f, out_f, k, seed):
     assert rel_l2(cpu(dc1), cpu(dc)) < 1e-5
 
 
+@pytest.mark.parametrize("T,in_f,out_f,k,seed", BWD_SHAPES)
+def test_linear_bwd_projected_one_call(hip, oracle, T, in_f, out_f, k, seed):
+    """dx and dcoef from one call (two launches, dcoef blocks and dx blocks side by side) against the oracle and against
+    the separate entry points."""
+    print(f"case bwd projected T={T} in={in_f} out={out_f} k={k}", flush=True)
+    x, dy, coef = _inputs(T, in_f, out_f, k, True, torch.bfloat16, seed)
+    want_dx, want_dc, _ = oracle.linear_bwd(x.float().numpy(), dy.float().numpy(), coef.float().numpy(), in_f, out_f, seed)
+    z = hip.linear_project(x.cuda(), k, out_f, seed)
+    for _ in range(2):   # the second call finds dcoef's buffer dirty in the allocator: it must be cleared by the call
+        dx, dc = hip.linear_bwd_projected(dy.cuda(), z, coef.cuda(), in_f, seed)
+        assert dx.shape == (T, in_f) and rel_l2(cpu(dx), want_dx) < BF16_TOL
+        assert dc.shape == (out_f, k) and rel_l2(cpu(dc), want_dc) < BF16_TOL
+    assert torch.equal(dx, hip.linear_bwd_dx(dy.cuda(), coef.cuda(), in_f, out_f, in_f, 1, seed, algo=3))
+    assert rel_l2(cpu(dc), cpu(hip.linear_bwd_dcoef_projected(dy.cuda(), z, in_f, seed))) < 1e-5
+
+
 def test_projected_form_rejects_what_it_cannot_do(hip):
     from randumb_amd._lib import RandumbHipError
 
