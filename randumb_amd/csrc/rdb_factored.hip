@@ -18,8 +18,10 @@ constexpr float INV_2_31 = 4.656612873077392578125e-10f;
 constexpr int F_BK = 64;
 
 // ----------------------------------------------------------------------------------------------- z = x . N^T
-// tile: 64 coefficients (engine rows "a", hashed) x 128 tokens (engine rows "b"), contraction over in_f; two blocks per CU
-constexpr int KZ_BM = 64, KZ_BT = 128;
+// tile: 32 coefficients (engine rows "a", hashed) x 256 tokens (engine rows "b"), 4 waves side by side along the tokens,
+// contraction over in_f; two blocks per CU.  The noise tile is hashed once per block, so the hash work of the kernel is
+// (tokens / 256) * in_f * k: the token tile is as long as the accumulators allow and the coefficient tile as short.
+constexpr int KZ_BM = 32, KZ_BT = 256, KZ_WM = 1;
 
 struct ZParams {
     const bf16_t *x;
@@ -38,16 +40,17 @@ __global__ __launch_bounds__(256, 2) void factored_z_kernel(ZParams p)
     const int w = xcd_work_item(blockIdx.x, p.tiles_m * p.tiles_t);
     if (w >= p.tiles_m * p.tiles_t) return;
     const int m0 = (w % p.tiles_m) * KZ_BM, tok0 = (w / p.tiles_m) * KZ_BT;
-    f32x16 acc[KZ_BM / 64][KZ_BT / 64];
+    constexpr int MI = KZ_BM / (32 * KZ_WM), NI = KZ_BT / (128 / KZ_WM);
+    f32x16 acc[MI][NI];
 #pragma unroll
-    for (int mi = 0; mi < KZ_BM / 64; ++mi)
+    for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < KZ_BT / 64; ++ni) acc[mi][ni] = zero16();
+        for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = zero16();
     // "A": 2^31 * noise(i, m), rows = m, contraction = i; values for i >= in_f meet zero columns of x
     NoiseOperandRowsAreCoefs<KZ_BM, F_BK> opn = {m0, p.seed};
     GlobalOperand<KZ_BT, F_BK, K_CONT> opx = {p.x, p.ldx, tok0, p.tokens, p.in_f, (int64_t)(p.tokens - 1) * p.ldx + p.in_f};
-    gemm_mainloop<KZ_BM, KZ_BT, F_BK, 1, 1>(acc, lds, opn, opx, 0, (p.in_f + F_BK - 1) / F_BK);
-    store_tile_bf16<KZ_BM, KZ_BT>(acc, lds, p.z, p.k, m0, p.k, tok0, p.tokens, INV_2_31, nullptr);
+    gemm_mainloop<KZ_BM, KZ_BT, F_BK, 1, 1, KZ_WM>(acc, lds, opn, opx, 0, (p.in_f + F_BK - 1) / F_BK);
+    store_tile_bf16<KZ_BM, KZ_BT, KZ_WM>(acc, lds, p.z, p.k, m0, p.k, tok0, p.tokens, INV_2_31, nullptr);
 }
 
 // ----------------------------------------------------------------------------------------------- y = z . C^T

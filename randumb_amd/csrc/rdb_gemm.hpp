@@ -303,17 +303,20 @@ __device__ __forceinline__ void pipeline_stage(f32x16 (&acc)[MI][NI], const bf16
 // after its last LDS read, so the caller may reuse `lds` at once.  The stage count is rounded up to a multiple of the
 // unrolled trip (the extra stages lie past klim and read as zeros), so the loop body has a single exit; the last trip is
 // peeled and does no reloads.
-template <int BM, int BN, int BK, int DA, int DB, class PA, class PB>
-__device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / 64][BN / 64], bf16_t *__restrict__ lds, PA &pa, PB &pb, int k_begin,
-                                              int nstage)
+// WM: waves along the A rows (2: 2 x 2 waves, 1: 1 x 4, 4: 4 x 1); a wave owns (BM / WM) x (BN / (4 / WM)) of the tile.
+template <int BM, int BN, int BK, int DA, int DB, int WM = 2, class PA, class PB>
+__device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / (32 * WM)][BN / (128 / WM)], bf16_t *__restrict__ lds, PA &pa, PB &pb,
+                                              int k_begin, int nstage)
 {
     typedef typename PA::Tile TA;
     typedef typename PB::Tile TB;
     static_assert((DA == 1 || DA == 2 || DA == 4) && (DB == 1 || DB == 2 || DB == 4), "prefetch depth must be 1, 2 or 4");
-    constexpr int MI = BM / 64, NI = BN / 64;
+    static_assert(WM == 1 || WM == 2 || WM == 4, "4 waves as 1x4, 2x2 or 4x1");
+    constexpr int WN = 4 / WM, MI = BM / (32 * WM), NI = BN / (32 * WN);
+    static_assert(MI * 32 * WM == BM && NI * 32 * WN == BN, "tile must split into 32-row blocks per wave");
     constexpr int STAGE = TA::LDS_ELEMS + TB::LDS_ELEMS;
     constexpr int TRIP = (DA == 4 || DB == 4) ? 4 : 2;
-    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, wm = wave >> 1, wn = wave & 1;
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, wm = wave / WN, wn = wave % WN;
     if (nstage <= 0) return;
     pa.init(k_begin);
     pb.init(k_begin);
@@ -360,12 +363,13 @@ __device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / 64][BN / 64], b
 // v = acc * scale (+ bias[a0 + a]).  The tile is staged through LDS (BN x (BM + 8) elements) so that the global stores are
 // 16 bytes wide and contiguous along each row.  Needs a0, na, ld multiples of 8 and a 16-byte aligned `out`.
 // All 256 threads must call; `lds` must be free on entry (the main loop ends with a barrier) and is free again on return.
-template <int BM, int BN>
-__device__ __forceinline__ void store_tile_bf16(const f32x16 (&acc)[BM / 64][BN / 64], bf16_t *__restrict__ lds, bf16_t *__restrict__ out,
-                                                int64_t ld, int a0, int na, int b0, int nb, float scale, const bf16_t *__restrict__ bias)
+template <int BM, int BN, int WM = 2>
+__device__ __forceinline__ void store_tile_bf16(const f32x16 (&acc)[BM / (32 * WM)][BN / (128 / WM)], bf16_t *__restrict__ lds,
+                                                bf16_t *__restrict__ out, int64_t ld, int a0, int na, int b0, int nb, float scale,
+                                                const bf16_t *__restrict__ bias)
 {
-    constexpr int MI = BM / 64, NI = BN / 64, LDS_LD = BM + 8;
-    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
+    constexpr int WN = 4 / WM, MI = BM / (32 * WM), NI = BN / (32 * WN), LDS_LD = BM + 8;
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave / WN, wn = wave % WN;
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
