@@ -42,6 +42,10 @@ T, IN_F, OUT_F, K, SEED = 8192, 768, 3072, 256, 0
 F_PER_PRODUCT = 2.0 * T * IN_F * OUT_F + 2.0 * OUT_F * IN_F * K      # one dense product + one W generation / dC contraction
 F_STEP = 3.0 * F_PER_PRODUCT
 # what the factored kernels execute: z, y, t, dx, dC products (z once per step)
+EXEC = {
+    "forward (factored_z_kernel + factored_y_kernel)": 2.0 * T * K * (IN_F + OUT_F),
+    "backward (dx_dyc_kernel + bwd_dc_tn_kernel)": 2.0 * T * K * (OUT_F + IN_F) + 2.0 * T * K * OUT_F,
+}
 EXEC_STEP = 2.0 * T * K * (IN_F + OUT_F) + 2.0 * T * K * (OUT_F + IN_F) + 2.0 * T * K * OUT_F
 
 
@@ -189,6 +193,7 @@ def main():
         "bound": "mfma", "kernel": dom, "achieved": round(achieved, 3), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 5), "traffic": HBM_TRAFFIC_BYTES[dom], "avg_kernel_ms": round(dom_ms, 5),
         "algorithmic_gflop_per_launch": round(dom_flops / 1e9, 3),
+        "executed_gflop_per_launch": round(EXEC[dom] / 1e9, 3), "executed_frac": round(EXEC[dom] / (dom_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 5),
         "calls_ms": {n: round(v, 5) for n, v in calls.items()},
     }
 

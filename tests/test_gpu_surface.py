@@ -221,3 +221,37 @@ def test_rt_mm_and_cpp_ops(ra, oracle):
     w = torch.ops.rten.materialize_fwd(c.requires_grad_(), [P, Q], [Q, 1], seed, None, False)
     w.sum().backward()
     assert rel_l2(cpu(c.grad), oracle.materialize_bwd(np.ones(P * Q, np.float32), k, seed)) < F32_TOL
+
+
+def test_step_is_graph_capturable(ra):
+    """The forward and backward calls of a layer record into a HIP graph (no allocation, no memset node: the library clears
+    with a fill kernel) and every replay, with eager work in between, gives the eager result."""
+    print("case graph capture", flush=True)
+    from randumb_amd import hip
+
+    T, in_f, out_f, k, seed = 512, 256, 384, 64, 5
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(T, in_f, generator=g).bfloat16().cuda()
+    dy = torch.randn(T, out_f, generator=g).bfloat16().cuda()
+    C = (torch.randn(out_f, k, generator=g) * 0.05).bfloat16().cuda()
+
+    def step():
+        z = hip.linear_project(x, k, out_f, seed)
+        y = hip.linear_fwd_projected(z, C, in_f, seed)
+        dx, dc = hip.linear_bwd_projected(dy, z, C, in_f, seed)
+        return y, dx, dc
+
+    want = [t.clone() for t in step()]
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        got = step()
+    for i in range(4):
+        for t in got:
+            t.fill_(3.0)
+        _ = step()                      # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1]), f"replay {i}"
+        assert float((got[2] - want[2]).abs().max()) <= 1e-5 * float(want[2].abs().max()), f"replay {i}"
