@@ -49,6 +49,46 @@ EXEC = {
 EXEC_STEP = 2.0 * T * K * (IN_F + OUT_F) + 2.0 * T * K * (OUT_F + IN_F) + 2.0 * T * K * OUT_F
 
 
+def other_configs(event_ms):
+    """The other two single-layer configurations, timed for the record (they are parity-test cases, not the metric)."""
+    import torch
+
+    from randumb_amd import hip
+
+    out = {}
+    # small-k fp32 regime: 4096 -> 4096, k = 16, forward at batch 1 / 16 / 256.  "effective" = the bytes a stored-W product
+    # would move (4*(out*in + B*in + B*out)) over the time; the fused kernel itself reads 4*(B*in + out*k) and writes 4*B*out.
+    in_f = out_f = 4096
+    g = torch.Generator().manual_seed(0)
+    C = (torch.randn(out_f, 16, generator=g) / 64.0).cuda()
+    small = {}
+    for B in (1, 16, 256):
+        x = torch.randn(B, in_f, generator=g).cuda()
+        ms = event_ms(lambda: hip.linear_fwd(x, C, in_f, out_f, in_f, 1, 0), 20)
+        stored = 4.0 * (out_f * in_f + B * in_f + B * out_f)
+        actual = 4.0 * (B * in_f + out_f * 16 + B * out_f)
+        small[f"batch_{B}"] = {"fwd_ms": round(ms, 4), "effective_GBps_vs_stored_W": round(stored / ms / 1e6, 1),
+                               "actual_HBM_GBps": round(actual / ms / 1e6, 2)}
+    out["in4096_out4096_k16_fp32_matrix_coef"] = small
+    # LLM-sized layer: 4096 -> 14336, k = 1024, 4096 tokens, bf16, forward + backward through the projected entry points
+    T, in_f, out_f, k = 4096, 4096, 14336, 1024
+    x = torch.randn(T, in_f, generator=g).bfloat16().cuda()
+    dy = torch.randn(T, out_f, generator=g).bfloat16().cuda()
+    C = (torch.randn(out_f, k, generator=g) / 64.0 * (3.0 / k) ** 0.5).bfloat16().cuda()
+
+    def step():
+        z = hip.linear_project(x, k, out_f, 0)
+        hip.linear_fwd_projected(z, C, in_f, 0)
+        hip.linear_bwd_projected(dy, z, C, in_f, 0)
+
+    ms = event_ms(step, 10)
+    F = 6.0 * T * in_f * out_f + 6.0 * out_f * in_f * k
+    out["in4096_out14336_k1024_T4096_bf16"] = {"fwd_bwd_ms": round(ms, 4), "algorithmic_TFLOPs": round(F / ms / 1e9, 1),
+                                               "frac_of_mfma_peak": round(F / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                               "note": "includes torch allocation of outputs and workspace per call"}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -227,6 +267,10 @@ def main():
             "dense_gemm_only_ms": round(event_ms(dense_step, 20), 4),
         }
 
+    other = None
+    if not args.no_compare:
+        other = other_configs(event_ms)
+
     cpu_baseline = None
     if not args.no_cpu_baseline:
         from oracle import oracle
@@ -267,7 +311,7 @@ def main():
                    "executed_gflop_per_step": round(EXEC_STEP / 1e9, 3), "executed_tflops": round(EXEC_STEP / (ms_per_step * 1e-3) / 1e12, 3),
                    "algorithm": "factored: y=(x N^T) C^T, dx=(dy C) N, dC=dy^T (x N^T); z = x N^T computed once per step"},
         "frac_of_mfma_peak": round(value / MFMA_BF16_PEAK_TFLOPS, 5),
-        "roofline": roofline, "cpu_baseline": cpu_baseline, "compare": compare,
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "compare": compare, "other_configs": other,
     }
     print(json.dumps(out))
 
