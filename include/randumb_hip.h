@@ -136,9 +136,10 @@ enum {
     RDB_ALGO_TILE = 1, /* regenerate W blocks in LDS per output block, contract with MFMA (any shape/dtype) */
     RDB_ALGO_STRIP = 2, /* forward only: build a whole strip W[strip, 0:in] in LDS once per workgroup, then stream the
                            tokens through it (matrix-coef, bf16, strip must fit LDS) */
-    RDB_ALGO_FACTORED = 3 /* matrix-coef, bf16 only: use W = C.N associatively so that no weight tile is formed at all:
+    RDB_ALGO_FACTORED = 3 /* matrix-coef only: use W = C.N associatively so that no weight tile is formed at all:
                              y = (x.N^T).C^T, dx = (dy.C).N, dcoef = dy^T.(x.N^T); the [tokens x k] intermediate lives
-                             in the caller's workspace.  With RDB_ALGO_STRIP the coefficient gradient runs the kernel
+                             in the caller's workspace.  bf16 activations and coef: matrix-core kernels; fp32 with
+                             k <= 64 and tokens <= 4096 (the GEMV-like regime): vector-ALU kernels, bit-reproducible.  With RDB_ALGO_STRIP the coefficient gradient runs the kernel
                              that forms dW tiles and contracts them with regenerated noise on chip. */
 };
 

@@ -290,6 +290,15 @@ int linear_fwd_factored(void *y, int64_t ldy, const void *x, int64_t ldx, const 
 int linear_dcoef_factored(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus,
                           void *workspace, int64_t workspace_bytes, hipStream_t s);
 
+// rdb_smallk.hip
+int64_t linear_smallk_workspace(const rdb_linear_desc *d);
+int linear_fwd_smallk(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
+                      const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s);
+int linear_dx_smallk(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias, const rdb_linear_desc *d,
+                     void *workspace, int64_t workspace_bytes, hipStream_t s);
+int linear_dcoef_smallk(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, void *workspace,
+                        int64_t workspace_bytes, hipStream_t s);
+
 // rdb_dx.hip
 int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z, const void *coef,
                          const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
@@ -350,6 +359,11 @@ extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
 {
     if (!d) return 0;
     if (d->algo == RDB_ALGO_TILE || d->algo == RDB_ALGO_STRIP) return 0;
+    if (d->act_dtype == RDB_F32) {  // fp32: the small-k kernels, whose scratch is one [tokens x k] fp32 matrix
+        rdb_linear_desc dd = *d;
+        if (op == RDB_OP_LINEAR_BWD_DCOEF) dd.coef_dtype = RDB_F32;
+        return (op == RDB_OP_LINEAR_FWD || op == RDB_OP_LINEAR_BWD_DX || op == RDB_OP_LINEAR_BWD_DCOEF) ? linear_smallk_workspace(&dd) : 0;
+    }
     if (op == RDB_OP_LINEAR_BWD_DX) return linear_dx_factored_workspace(d);
     if (op == RDB_OP_LINEAR_FWD) return d->coef_dtype == RDB_BF16 ? linear_projection_bytes(d) : 0;
     if (op == RDB_OP_LINEAR_BWD_DCOEF) return linear_projection_bytes(d);  // reads no coefficients: their dtype does not matter
@@ -368,10 +382,12 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
     if (d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) {
         rc = linear_fwd_factored(y, ldy, x, ldx, coef, scale_bias, bias, d, workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
+        rc = linear_fwd_smallk(y, ldy, x, ldx, coef, scale_bias, bias, d, workspace, workspace_bytes, s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
         if (d->algo == RDB_ALGO_FACTORED)
-            return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd: the factored algorithm needs matrix-coef in bf16, bf16 activations, no "
-                                                "scale_bias, sizes that are multiples of 8, aligned rows and a workspace of "
-                                                "rdb_linear_workspace_bytes() bytes");
+            return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd: the factored algorithm needs matrix-coef, no scale_bias, a workspace of "
+                                                "rdb_linear_workspace_bytes() bytes and either bf16 (activations and coef; sizes that are "
+                                                "multiples of 8; aligned rows) or fp32 with k <= 64 and tokens <= 4096");
     }
     if (d->algo != RDB_ALGO_TILE) {
         rc = linear_fwd_strip(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), s);
@@ -410,10 +426,12 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
     if (d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) {
         rc = linear_dx_factored(dx, lddx, dy, lddy, coef, scale_bias, d, workspace, workspace_bytes, (hipStream_t)stream);
         if (rc != RDB_E_UNSUPPORTED) return rc;
+        rc = linear_dx_smallk(dx, lddx, dy, lddy, coef, scale_bias, d, workspace, workspace_bytes, (hipStream_t)stream);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
         if (d->algo == RDB_ALGO_FACTORED)
-            return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dx: the factored algorithm needs matrix-coef in bf16, bf16 activations, no "
-                                                "scale_bias, sizes that are multiples of 8, aligned rows and a workspace of "
-                                                "rdb_linear_workspace_bytes() bytes");
+            return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dx: the factored algorithm needs matrix-coef, no scale_bias, a workspace of "
+                                                "rdb_linear_workspace_bytes() bytes and either bf16 (activations and coef; sizes that are "
+                                                "multiples of 8; aligned rows) or fp32 with k <= 64 and tokens <= 4096");
     }
     const int es = d->act_dtype == RDB_BF16 ? 2 : 4;
     LinParams p = {};
@@ -456,11 +474,13 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
     if ((d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) && !d_scale_bias) {
         rc = linear_dcoef_factored(dcoef, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
+        rc = linear_dcoef_smallk(dcoef, dy, lddy, x, ldx, d, workspace, workspace_bytes, s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
     }
     if (d->algo == RDB_ALGO_FACTORED)
-        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dcoef: the factored algorithm needs matrix-coef, bf16 activations, no scale_bias "
-                                            "gradient, sizes that are multiples of 8, aligned rows and a workspace of "
-                                            "rdb_linear_workspace_bytes() bytes");
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dcoef: the factored algorithm needs matrix-coef, no scale_bias gradient, a "
+                                            "workspace of rdb_linear_workspace_bytes() bytes and either bf16 activations (sizes that are "
+                                            "multiples of 8; aligned rows) or fp32 with k <= 64 and tokens <= 4096");
     if (d->algo != RDB_ALGO_TILE) {
         rc = linear_dcoef_fast(dcoef, d_scale_bias, dy, lddy, x, ldx, d, num_compute_units(), s);
         if (rc != RDB_E_UNSUPPORTED) return rc;

@@ -1,0 +1,279 @@
+// Fused linear layer, matrix-coef + fp32, small coefficient dimension and few tokens (the GEMV-like regime): factored
+// algorithm on the vector ALU.
+//
+// With k <= 64 and a handful of tokens the layer moves almost no data (x, C, y) and does almost no arithmetic once W = C . N
+// is used associatively; what remains is the hash of N, in_f * k values per token tile:
+//   forward  z = x . N^T [T x k],  y = z . C^T (+ bias)
+//   dx       t = dy . C  [T x k],  dx = t . N
+//   dcoef    z as above,           dC = dy^T . z
+// Everything is fp32 FMA with partial sums combined in a fixed order (no atomics): results are bit-reproducible.
+// Replaces materialize() + dense product (src/rten_cpp/RandumbTensor.py:942-946) and MmBackward's dW followed by
+// materialize_bwd (RandumbTensor.py:979-990, 304-359) in the regime where a stored-W product would be bound by reading W.
+#include "rdb_common.hpp"
+
+namespace rdb {
+
+constexpr int SK_TT = 8;    // tokens per block of the contracting kernel
+constexpr int SK_ET = 16;   // tokens per block of the expanding kernel
+constexpr int SK_MAX_K = 64;
+
+// sum over the partial matrices p[ch][idx], ch = 0 .. nchunk-1, in chunk order; loads issued eight at a time
+__device__ __forceinline__ float sum_partials(const float *__restrict__ p, int64_t stride, int nchunk)
+{
+    float v = 0.0f;
+    for (int c0 = 0; c0 < nchunk; c0 += 8) {
+        float l[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) l[u] = p[(int64_t)((c0 + u < nchunk) ? c0 + u : nchunk - 1) * stride];  // always a valid address
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v += (c0 + u < nchunk) ? l[u] : 0.0f;
+    }
+    return v;
+}
+
+// out[t, m] = sum_j src[t, j] * B(j, m),  B(j, m) = noise(PRIME*j + m) (HASH) or coef[j, m]; j runs over J = in_f or out_f.
+// Block = 8 tokens x one chunk of 256 values of j (blockIdx.y), so that even a single token spreads the hash over many
+// compute units; thread = (m % 16, one of 16 interleaved slices of the chunk); the source rows go through LDS (coalesced
+// loads, broadcast reads); slices meet in LDS in slice order.  The block writes a partial result, out[chunk][t][m]; the
+// expanding kernel adds the chunks up in chunk order while it loads them.
+template <bool HASH>
+__global__ __launch_bounds__(256) void smallk_contract_kernel(float *__restrict__ out, const float *__restrict__ src, int64_t lds_src,
+                                                              const float *__restrict__ coef, int T, int J, int k, uint32_t seed)
+{
+    constexpr int JC = 256, MC = SK_MAX_K / 16;
+    __shared__ float xs[SK_TT][JC];
+    __shared__ float red[16][SK_TT][16];
+    const int tid = threadIdx.x, m16 = tid & 15, slice = tid >> 4;
+    const int t0 = blockIdx.x * SK_TT;
+    float acc[MC][SK_TT];
+#pragma unroll
+    for (int c = 0; c < MC; ++c)
+#pragma unroll
+        for (int tt = 0; tt < SK_TT; ++tt) acc[c][tt] = 0.0f;
+    {
+        const int jc = blockIdx.y * JC;
+#pragma unroll
+        for (int tt = 0; tt < SK_TT; ++tt) xs[tt][tid] = (t0 + tt < T && jc + tid < J) ? src[(int64_t)(t0 + tt) * lds_src + jc + tid] : 0.0f;
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < MC; ++c) {
+            const int m = c * 16 + m16;
+            if (c * 16 < k) {  // uniform
+                uint32_t first = sq5_first((uint32_t)(jc + slice), (uint32_t)m, seed);
+                for (int jj = 0; jj < JC / 16; ++jj, first += 16u * PN1) {
+                    const int j = jc + slice + 16 * jj;
+                    // no branches in here: out-of-range (j, m) read a valid address and are zeroed by a select
+                    float b = HASH ? sq5_unit(sq5_tail(first)) : coef[(int64_t)(j < J ? j : J - 1) * k + (m < k ? m : k - 1)];
+                    b = (m < k && j < J) ? b : 0.0f;
+#pragma unroll
+                    for (int tt = 0; tt < SK_TT; ++tt) acc[c][tt] = fmaf(xs[tt][slice + 16 * jj], b, acc[c][tt]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int c = 0; c < MC; ++c) {
+        if (c * 16 >= k) break;
+#pragma unroll
+        for (int tt = 0; tt < SK_TT; ++tt) red[slice][tt][m16] = acc[c][tt];
+        __syncthreads();
+        if (tid < SK_TT * 16) {
+            const int tt = tid >> 4, m = c * 16 + m16;
+            float s = 0.0f;
+#pragma unroll
+            for (int sl = 0; sl < 16; ++sl) s += red[sl][tt][m16];
+            if (t0 + tt < T && m < k) out[((int64_t)blockIdx.y * T + t0 + tt) * k + m] = s;
+        }
+        __syncthreads();
+    }
+}
+
+// out[t, c] = sum_m src[t, m] * B(c, m) (+ bias[c]),  B(c, m) = noise(PRIME*c + m) (HASH) or coef[c, m]; c runs over the
+// cols = in_f or out_f.  Block = 256 columns x 16 tokens; a thread owns one column and keeps its 16 B values in registers.
+// src holds `nchunk` partial matrices [T x k] (from the contracting kernel), added up here in chunk order.
+template <bool HASH>
+__global__ __launch_bounds__(256) void smallk_expand_kernel(float *__restrict__ out, int64_t ld_out, const float *__restrict__ src, int nchunk,
+                                                            const float *__restrict__ coef, const float *__restrict__ bias, int T, int cols,
+                                                            int k, uint32_t seed)
+{
+    __shared__ __align__(16) float s[SK_ET][SK_MAX_K];
+    const int tid = threadIdx.x;
+    const int c = blockIdx.x * 256 + tid, t0 = blockIdx.y * SK_ET;
+    // s = sum of the partial matrices in chunk order; columns from k on take part as zeros.  A thread owns up to 4 entries
+    // and keeps the loads of 8 chunks of all of them in flight at once: the kernel is a chain of memory latencies otherwise.
+    {
+        constexpr int PER = SK_ET * SK_MAX_K / 256;
+        float v[PER];
+        const float *ptr[PER];
+        bool ok[PER];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int e = tid + 256 * i, tt = e / k, m = e % k;   // entries e < SK_ET * k, row-major over (tt, m < k)
+            v[i] = 0.0f;
+            ok[i] = e < SK_ET * k && t0 + tt < T;
+            ptr[i] = ok[i] ? src + (int64_t)(t0 + tt) * k + m : src;   // always a valid address
+        }
+        const int64_t stride = (int64_t)T * k;
+        for (int c0 = 0; c0 < nchunk; c0 += 8) {
+            float l[PER][8];
+#pragma unroll
+            for (int i = 0; i < PER; ++i)
+#pragma unroll
+                for (int u = 0; u < 8; ++u) l[i][u] = ptr[i][(int64_t)((c0 + u < nchunk) ? c0 + u : nchunk - 1) * stride];
+#pragma unroll
+            for (int i = 0; i < PER; ++i)
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[i] += (ok[i] && c0 + u < nchunk) ? l[i][u] : 0.0f;
+        }
+        for (int e = tid; e < SK_ET * SK_MAX_K; e += 256) s[e / SK_MAX_K][e % SK_MAX_K] = 0.0f;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int e = tid + 256 * i;
+            if (e < SK_ET * k) s[e / k][e % k] = v[i];
+        }
+    }
+    __syncthreads();
+    if (c >= cols) return;
+    float acc[SK_ET];
+#pragma unroll
+    for (int tt = 0; tt < SK_ET; ++tt) acc[tt] = 0.0f;
+    for (int mc = 0; mc < k; mc += 16) {
+        float b[16];
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {  // branch-free: a column from k on reads a valid address and becomes 0
+            const float v = HASH ? sq5_unit(sq5_tail(sq5_first((uint32_t)c, (uint32_t)(mc + m), seed)))
+                                 : coef[(int64_t)c * k + ((mc + m < k) ? mc + m : k - 1)];
+            b[m] = (mc + m < k) ? v : 0.0f;
+        }
+        // mc <= 48 and m <= 15: always inside the 64 columns of s
+#pragma unroll
+        for (int tt = 0; tt < SK_ET; ++tt) {
+            const f32x4 *row = reinterpret_cast<const f32x4 *>(&s[tt][mc]);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const f32x4 sv = row[q];
+                acc[tt] = fmaf(sv[0], b[4 * q], acc[tt]);
+                acc[tt] = fmaf(sv[1], b[4 * q + 1], acc[tt]);
+                acc[tt] = fmaf(sv[2], b[4 * q + 2], acc[tt]);
+                acc[tt] = fmaf(sv[3], b[4 * q + 3], acc[tt]);
+            }
+        }
+    }
+    const float bv = bias ? bias[c] : 0.0f;
+#pragma unroll
+    for (int tt = 0; tt < SK_ET; ++tt)
+        if (t0 + tt < T) out[(int64_t)(t0 + tt) * ld_out + c] = acc[tt] + bv;
+}
+
+// dC[o, m] = sum_t dy[t, o] * z[t, m].  Block = 256 output rows x one chunk of 16 coefficients; z goes through LDS in tiles
+// of 64 tokens; a thread owns one output row and walks the tokens in order.
+__global__ __launch_bounds__(256) void smallk_dcoef_kernel(float *__restrict__ dcoef, const float *__restrict__ dy, int64_t lddy,
+                                                           const float *__restrict__ z, int nchunk, int T, int out_f, int k)
+{
+    __shared__ __align__(16) float zs[64][16];
+    const int tid = threadIdx.x;
+    const int o = blockIdx.x * 256 + tid, mc = blockIdx.y * 16;
+    float acc[16];
+#pragma unroll
+    for (int m = 0; m < 16; ++m) acc[m] = 0.0f;
+    for (int t0 = 0; t0 < T; t0 += 64) {
+        for (int e = tid; e < 64 * 16; e += 256) {
+            const int tt = e >> 4, m = e & 15;
+            zs[tt][m] = (t0 + tt < T && mc + m < k) ? sum_partials(z + (int64_t)(t0 + tt) * k + mc + m, (int64_t)T * k, nchunk) : 0.0f;
+        }
+        __syncthreads();
+        if (o < out_f) {
+            const int n = (T - t0 < 64) ? T - t0 : 64;
+            for (int tt = 0; tt < n; ++tt) {
+                const float g = dy[(int64_t)(t0 + tt) * lddy + o];
+#pragma unroll
+                for (int m = 0; m < 16; ++m) acc[m] = fmaf(g, zs[tt][m], acc[m]);
+            }
+        }
+        __syncthreads();
+    }
+    if (o < out_f) {
+#pragma unroll
+        for (int m = 0; m < 16; ++m)
+            if (mc + m < k) dcoef[(int64_t)o * k + mc + m] = acc[m];
+    }
+}
+
+// ----------------------------------------------------------------------------------------------- host side
+// The regime this file is for; AUTO additionally wants it to be the cheaper way.
+static bool smallk_ok(const rdb_linear_desc *d)
+{
+    return d->act_dtype == RDB_F32 && d->coef_dtype == RDB_F32 && d->coef_rows != 0 && d->k > 0 && d->k <= SK_MAX_K && d->tokens > 0 &&
+           d->tokens <= 4096 && d->in_f > 0 && d->out_f > 0 && d->in_f < (1 << 30) && d->out_f < (1 << 30);
+}
+static bool smallk_wanted(const rdb_linear_desc *d)
+{
+    return d->algo == RDB_ALGO_FACTORED || (d->tokens <= 1024 && d->k * (d->in_f + d->out_f) < d->in_f * d->out_f);
+}
+
+// scratch: one partial [tokens x k] fp32 matrix per 256-chunk of the longer of in_f and out_f
+int64_t linear_smallk_workspace(const rdb_linear_desc *d)
+{
+    if (!smallk_ok(d)) return 0;
+    const int64_t longer = d->in_f > d->out_f ? d->in_f : d->out_f;
+    return cdiv(longer, 256) * d->tokens * d->k * (int64_t)sizeof(float);
+}
+
+static bool ws_ok(const rdb_linear_desc *d, const void *ws, int64_t bytes) { return ws && bytes >= linear_smallk_workspace(d) && ((uintptr_t)ws & 3) == 0; }
+
+// The three entry points return RDB_E_UNSUPPORTED, without setting an error, when the request does not fit.
+int linear_fwd_smallk(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
+                      const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s)
+{
+    if (!smallk_ok(d) || scale_bias || !smallk_wanted(d) || !ws_ok(d, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    const int T = (int)d->tokens, k = (int)d->k;
+    float *z = (float *)workspace;
+    const int nchunk = (int)cdiv(d->in_f, 256);
+    smallk_contract_kernel<true><<<dim3((unsigned)cdiv(T, SK_TT), nchunk), 256, 0, s>>>(z, (const float *)x, ldx, nullptr, T, (int)d->in_f, k,
+                                                                                        d->seed);
+    int rc = check_launch("smallk_contract_kernel<hash>");
+    if (rc) return rc;
+    dim3 grid((unsigned)cdiv(d->out_f, 256), (unsigned)cdiv(T, SK_ET));
+    smallk_expand_kernel<false><<<grid, 256, 0, s>>>((float *)y, ldy, z, nchunk, (const float *)coef, (const float *)bias, T, (int)d->out_f, k,
+                                                     d->seed);
+    return check_launch("smallk_expand_kernel<coef>");
+}
+
+int linear_dx_smallk(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias, const rdb_linear_desc *d,
+                     void *workspace, int64_t workspace_bytes, hipStream_t s)
+{
+    if (!smallk_ok(d) || scale_bias || !smallk_wanted(d) || !ws_ok(d, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    const int T = (int)d->tokens, k = (int)d->k;
+    float *t = (float *)workspace;
+    const int nchunk = (int)cdiv(d->out_f, 256);
+    smallk_contract_kernel<false><<<dim3((unsigned)cdiv(T, SK_TT), nchunk), 256, 0, s>>>(t, (const float *)dy, lddy, (const float *)coef, T,
+                                                                                         (int)d->out_f, k, d->seed);
+    int rc = check_launch("smallk_contract_kernel<coef>");
+    if (rc) return rc;
+    dim3 grid((unsigned)cdiv(d->in_f, 256), (unsigned)cdiv(T, SK_ET));
+    smallk_expand_kernel<true><<<grid, 256, 0, s>>>((float *)dx, lddx, t, nchunk, nullptr, nullptr, T, (int)d->in_f, k, d->seed);
+    return check_launch("smallk_expand_kernel<hash>");
+}
+
+// dcoef is overwritten (no zero fill needed).
+int linear_dcoef_smallk(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, void *workspace,
+                        int64_t workspace_bytes, hipStream_t s)
+{
+    rdb_linear_desc dd = *d;
+    dd.coef_dtype = RDB_F32;  // no coefficients are read here
+    if (!smallk_ok(&dd) || !smallk_wanted(&dd) || !ws_ok(&dd, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    const int T = (int)d->tokens, k = (int)d->k;
+    float *z = (float *)workspace;
+    const int nchunk = (int)cdiv(d->in_f, 256);
+    smallk_contract_kernel<true><<<dim3((unsigned)cdiv(T, SK_TT), nchunk), 256, 0, s>>>(z, (const float *)x, ldx, nullptr, T, (int)d->in_f, k,
+                                                                                        d->seed);
+    int rc = check_launch("smallk_contract_kernel<hash>");
+    if (rc) return rc;
+    dim3 grid((unsigned)cdiv(d->out_f, 256), (unsigned)cdiv(k, 16));
+    smallk_dcoef_kernel<<<grid, 256, 0, s>>>(dcoef, (const float *)dy, lddy, z, nchunk, T, (int)d->out_f, k);
+    return check_launch("smallk_dcoef_kernel");
+}
+
+}  // namespace rdb

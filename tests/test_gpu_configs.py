@@ -115,6 +115,35 @@ def test_small_k_fp32_regime(hip, oracle, batch, matrix):
     assert rel_l2(cpu(y), want_y) < F32_TOL
     assert rel_l2(cpu(dx), want_dx) < F32_TOL
     assert rel_l2(cpu(dC), want_dC) < F32_TOL
+    if matrix:
+        # AUTO takes the factored small-k kernels here; the kernels that form W tiles must agree, and so must a bias
+        from randumb_amd._lib import RDB_ALGO_FACTORED, RDB_ALGO_TILE
+
+        bias = torch.randn(out_f, generator=g)
+        for algo in (RDB_ALGO_FACTORED, RDB_ALGO_TILE):
+            yb = hip.linear_fwd(x.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, bias=bias.cuda(), algo=algo)
+            assert rel_l2(cpu(yb), want_y + bias.numpy()) < F32_TOL, algo
+            assert rel_l2(cpu(hip.linear_bwd_dx(dy.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, algo=algo)), want_dx) < F32_TOL, algo
+            assert rel_l2(cpu(hip.linear_bwd_dcoef(dy.cuda(), x.cuda(), k, out_f, in_f, out_f, in_f, 1, seed, algo=algo)[0]), want_dC) < F32_TOL
+        y2 = hip.linear_fwd(x.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+        assert torch.equal(y2, hip.linear_fwd(x.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED))  # reproducible
+
+
+def test_small_k_fp32_ragged_shapes(hip, oracle):
+    """The fp32 small-k kernels on sizes that divide nothing: 5 tokens, 77 -> 130, k = 23, with bias."""
+    from randumb_amd._lib import RDB_ALGO_FACTORED
+
+    print("case small-k ragged", flush=True)
+    T, in_f, out_f, k, seed = 5, 77, 130, 23, 9
+    g = torch.Generator().manual_seed(4)
+    x, dy = torch.randn(T, in_f, generator=g), torch.randn(T, out_f, generator=g)
+    C, bias = torch.randn(out_f, k, generator=g) * 0.1, torch.randn(out_f, generator=g)
+    y = hip.linear_fwd(x.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, bias=bias.cuda(), algo=RDB_ALGO_FACTORED)
+    dx = hip.linear_bwd_dx(dy.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    dC, _ = hip.linear_bwd_dcoef(dy.cuda(), x.cuda(), k, out_f, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    want_dx, want_dC, _ = oracle.linear_bwd(x.numpy(), dy.numpy(), C.numpy(), in_f, out_f, seed)
+    assert rel_l2(cpu(y), oracle.linear_fwd(x.numpy(), C.numpy(), in_f, out_f, seed, bias=bias.numpy())) < F32_TOL
+    assert rel_l2(cpu(dx), want_dx) < F32_TOL and rel_l2(cpu(dC), want_dC) < F32_TOL
 
 
 GPT2_SHAPES = [("qkv", 768, 2304), ("proj", 768, 768), ("fc", 768, 3072), ("mlp_proj", 3072, 768)]
