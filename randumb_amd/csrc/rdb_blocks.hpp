@@ -56,8 +56,9 @@ __device__ __forceinline__ void dc_block(const DcParams &p, bf16_t *lds, int blo
 }
 
 // ----------------------------------------------------------------------------------------------- kernel 2: dx = t . N
-// tile: 192 input features (engine rows "a", hashed operand) x 128 tokens (engine rows "b"), contraction over k
-constexpr int K2_BI = 192, K2_BT = 128;
+// tile: 64 input features (engine rows "a", hashed operand) x 256 tokens (engine rows "b"), 4 waves side by side along the
+// tokens, contraction over k.  The noise tile is hashed once per block: a long token tile halves the hash work of a 128-token one.
+constexpr int K2_BI = 64, K2_BT = 256, K2_WM = 1;
 
 struct TNParams {
     const bf16_t *t;
@@ -74,17 +75,18 @@ __device__ __forceinline__ void tn_block(const TNParams &p, bf16_t *lds, int blo
     const int w = xcd_work_item(block, p.tiles_i * p.tiles_t);
     if (w >= p.tiles_i * p.tiles_t) return;
     const int i0 = (w % p.tiles_i) * K2_BI, tok0 = (w / p.tiles_i) * K2_BT;
-    f32x16 acc[K2_BI / 64][K2_BT / 64];
+    constexpr int MI = K2_BI / (32 * K2_WM), NI = K2_BT / (128 / K2_WM);
+    f32x16 acc[MI][NI];
 #pragma unroll
-    for (int mi = 0; mi < K2_BI / 64; ++mi)
+    for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < K2_BT / 64; ++ni) acc[mi][ni] = zero16();
+        for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = zero16();
     // "A": 2^31 * noise(i, m), rows = i, contraction = m; values for m >= k meet zero rows of t
     NoiseOperandRowsAreElements<K2_BI, B_BK> opn = {i0, p.seed};
     // "B": t[tok][m]
     GlobalOperand<K2_BT, B_BK, K_CONT> opt = {p.t, (int64_t)p.k, tok0, p.tokens, p.k, (int64_t)p.tokens * p.k};
-    gemm_mainloop<K2_BI, K2_BT, B_BK, 1, 1>(acc, lds, opn, opt, 0, (p.k + B_BK - 1) / B_BK);
-    store_tile_bf16<K2_BI, K2_BT>(acc, lds, p.dx, p.lddx, i0, p.in_f, tok0, p.tokens, 4.656612873077392578125e-10f, nullptr);
+    gemm_mainloop<K2_BI, K2_BT, B_BK, 1, 1, K2_WM>(acc, lds, opn, opt, 0, (p.k + B_BK - 1) / B_BK);
+    store_tile_bf16<K2_BI, K2_BT, K2_WM>(acc, lds, p.dx, p.lddx, i0, p.in_f, tok0, p.tokens, 4.656612873077392578125e-10f, nullptr);
 }
 
 // ----------------------------------------------------------------------------------------------- host side
