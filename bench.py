@@ -101,6 +101,25 @@ def other_configs(event_ms):
     out["in4096_out14336_k1024_T4096_bf16"] = {"fwd_bwd_ms": round(ms, 4), "algorithmic_TFLOPs": round(F / ms / 1e9, 1),
                                                "frac_of_mfma_peak": round(F / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
                                                "note": "includes torch allocation of outputs and workspace per call"}
+    # GPT-2 small with random-backed linears: 12 layers, d = 768, 12 heads, vocab 50304, k = 256, seeds 0..47, bf16,
+    # batch 8 x 1024 random token ids; one training step (forward + backward).  Attention, norms, embedding, head and loss
+    # are stock PyTorch; the 48 linears run the projected kernels.
+    from randumb_amd.SillyLayers import listgen, stepgen
+    from randumb_amd.gpt import RT_GPT, RT_GPTConfig
+
+    torch.manual_seed(0)
+    model = RT_GPT(RT_GPTConfig(int_dim_gen=listgen([256] * 48), seed_gen=stepgen(0, 1))).to(torch.bfloat16).cuda()
+    idx = torch.randint(0, 50304, (8, 1024), generator=g).cuda()
+    tgt = torch.randint(0, 50304, (8, 1024), generator=g).cuda()
+
+    def gpt_step():
+        model.zero_grad(set_to_none=True)
+        model(idx, tgt).backward()
+
+    ms = event_ms(gpt_step, 5)
+    out["gpt2_small_12L_k256_seeds0to47_bf16_8x1024"] = {"fwd_bwd_ms": round(ms, 2), "tokens_per_s": round(8192 / ms * 1e3, 0),
+                                                        "note": "random-backed qkv/proj/fc/mlp-proj; attention, norms, embedding, "
+                                                                "head and loss are stock PyTorch"}
     return out
 
 

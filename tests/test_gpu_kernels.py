@@ -346,21 +346,22 @@ def test_linear_projected_form(hip, oracle, T, in_f, out_f, k, seed):
     x, dy, coef = _inputs(T, in_f, out_f, k, True, torch.bfloat16, seed)
     xn, dyn, cn = x.float().numpy(), dy.float().numpy(), coef.float().numpy()
     assert hip.linear_projection_supported(T, in_f, out_f, k)
-    z = hip.linear_project(x.cuda(), k, out_f, seed)
+    xg, dyg, cg = x.cuda(), dy.cuda(), coef.cuda()
+    z = hip.linear_project(xg, k, out_f, seed)
     noise = oracle.noise_2d(in_f, k, seed).astype(np.float64)          # noise[i, m] = noise(PRIME*i + m)
     want_z = xn.astype(np.float64) @ noise
     assert z.shape == (T, k) and z.dtype == torch.bfloat16 and rel_l2(cpu(z), want_z) < 5e-3  # one bf16 rounding of z
     bias = torch.randn(out_f).bfloat16()
-    y = hip.linear_fwd_projected(z, coef.cuda(), in_f, seed, bias=bias.cuda())
+    y = hip.linear_fwd_projected(z, cg, in_f, seed, bias=bias.cuda())
     want_y = oracle.linear_fwd(xn, cn, in_f, out_f, seed, bias=bias.float().numpy())
     assert y.shape == (T, out_f) and rel_l2(cpu(y), want_y) < BF16_TOL
-    dc = hip.linear_bwd_dcoef_projected(dy.cuda(), z, in_f, seed)
+    dc = hip.linear_bwd_dcoef_projected(dyg, z, in_f, seed)
     _, want_dc, _ = oracle.linear_bwd(xn, dyn, cn, in_f, out_f, seed)
     assert dc.shape == (out_f, k) and rel_l2(cpu(dc), want_dc) < BF16_TOL
     # the one-call entry points do the same arithmetic: equal up to the order of the fp32 atomics
-    y1 = hip.linear_fwd(x.cuda(), coef.cuda(), in_f, out_f, in_f, 1, seed, bias=bias.cuda(), algo=3)
+    y1 = hip.linear_fwd(xg, cg, in_f, out_f, in_f, 1, seed, bias=bias.cuda(), algo=3)
     assert torch.equal(y1, y)
-    dc1, _ = hip.linear_bwd_dcoef(dy.cuda(), x.cuda(), k, out_f, in_f, out_f, in_f, 1, seed, algo=3)
+    dc1, _ = hip.linear_bwd_dcoef(dyg, xg, k, out_f, in_f, out_f, in_f, 1, seed, algo=3)
     assert rel_l2(cpu(dc1), cpu(dc)) < 1e-5
 
 
