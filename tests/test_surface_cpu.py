@@ -46,6 +46,49 @@ def test_argument_errors_come_back_as_codes_without_a_gpu():
     assert L.rdb_materialize_bwd_workspace_bytes(3072, 256, 768, 2359296) == 0
 
 
+def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
+    """Host logic of the fused-linear entry points: scratch sizes, which layers qualify for the projected form, and argument
+    errors that must come back before anything touches a GPU."""
+    from randumb_amd import _lib
+
+    L = _lib.load()
+
+    def desc(tokens, in_f, out_f, k, act=_lib.RDB_BF16, coef=_lib.RDB_BF16, rows=None, algo=_lib.RDB_ALGO_AUTO):
+        d = _lib.LinearDesc()
+        d.tokens, d.in_f, d.out_f, d.k, d.coef_rows, d.sO, d.sI = tokens, in_f, out_f, k, out_f if rows is None else rows, in_f, 1
+        d.act_dtype, d.coef_dtype, d.algo = act, coef, algo
+        return d
+
+    d = desc(8192, 768, 3072, 256)
+    r = ctypes.byref(d)
+    zbytes = 8192 * 256 * 2
+    assert L.rdb_linear_projection_bytes(r) == zbytes
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, r) == zbytes
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, r) == zbytes
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DCOEF, r) == zbytes
+    # kernels that form W tiles need no scratch; neither does a layer the factored form does not apply to
+    for algo in (_lib.RDB_ALGO_TILE, _lib.RDB_ALGO_STRIP):
+        assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(8192, 768, 3072, 256, algo=algo))) == 0
+    assert L.rdb_linear_projection_bytes(ctypes.byref(desc(64, 100, 32, 16))) == 0                     # in_f % 8
+    assert L.rdb_linear_projection_bytes(ctypes.byref(desc(64, 96, 32, 16, rows=0))) == 0              # vector-coef
+    assert L.rdb_linear_projection_bytes(ctypes.byref(desc(64, 96, 32, 16, act=_lib.RDB_F32))) == 0    # fp32 activations
+    assert L.rdb_linear_projection_bytes(None) == 0
+    # fp32, small k: one partial [tokens x k] matrix per 256 values of the longer side
+    f32 = desc(16, 4096, 4096, 16, act=_lib.RDB_F32, coef=_lib.RDB_F32)
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(f32)) == 16 * 16 * 16 * 4
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(16, 4096, 4096, 128, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 0
+
+    bad = ctypes.byref(desc(64, 100, 32, 16))
+    assert L.rdb_linear_project(None, None, 100, bad, None) == -5  # RDB_E_UNSUPPORTED
+    assert b"projected form" in L.rdb_last_error_string()
+    assert L.rdb_linear_project(None, None, 768, r, None) == -1                                          # NULL pointers
+    assert L.rdb_linear_fwd_projected(None, 3072, None, None, None, r, None) == -1
+    assert L.rdb_linear_bwd_dcoef_projected(None, None, 3072, None, r, None) == -1
+    assert L.rdb_linear_bwd_projected(None, 768, None, None, 3072, None, None, r, None, 0, None) == -1
+    assert L.rdb_linear_fwd_projected(ctypes.c_void_p(16), 8, ctypes.c_void_p(16), ctypes.c_void_p(16), None, r, None) == -2  # ldy < out_f
+    assert L.rdb_linear_project(None, None, 768, None, None) == -1
+
+
 def test_view_ops_stay_lazy_and_only_change_shape_and_stride():
     c = torch.nn.Parameter(torch.randn(18))
     rt = CreateRandumbTensor(c, 1337, (3, 6))
