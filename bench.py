@@ -98,8 +98,10 @@ def other_configs(event_ms):
 
     ms = event_ms(step, 10)
     F = 6.0 * T * in_f * out_f + 6.0 * out_f * in_f * k
+    executed = 4.0 * T * k * (in_f + out_f) + 2.0 * T * k * out_f
     out["in4096_out14336_k1024_T4096_bf16"] = {"fwd_bwd_ms": round(ms, 4), "algorithmic_TFLOPs": round(F / ms / 1e9, 1),
                                                "frac_of_mfma_peak": round(F / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                               "executed_TFLOPs": round(executed / ms / 1e9, 1),
                                                "note": "includes torch allocation of outputs and workspace per call"}
     # GPT-2 small with random-backed linears: 12 layers, d = 768, 12 heads, vocab 50304, k = 256, seeds 0..47, bf16,
     # batch 8 x 1024 random token ids; one training step (forward + backward).  Attention, norms, embedding, head and loss
@@ -288,6 +290,17 @@ def main():
         def dense_step():
             return x @ Wd.t(), dy @ Wd, dy.t() @ x
 
+        def vendor_skinny():
+            # the three dense products of the factored algorithm given to the vendor GEMM (torch.matmul), for reference
+            # against factored_y_kernel / dx_dyc_kernel / factored_dc_kernel in profiles/bench_c2_kernel_trace.md
+            zz = torch.randn(T, K, device=dev).bfloat16()
+            yy = torch.empty(T, OUT_F, device=dev, dtype=torch.bfloat16)
+            tt = torch.empty(T, K, device=dev, dtype=torch.bfloat16)
+            cc = torch.empty(OUT_F, K, device=dev, dtype=torch.bfloat16)
+            return {"y = z.C^T": round(event_ms(lambda: torch.matmul(zz, C.t(), out=yy), 30), 4),
+                    "t = dy.C": round(event_ms(lambda: torch.matmul(dy, C, out=tt), 30), 4),
+                    "dC = dy^T.z": round(event_ms(lambda: torch.matmul(dy.t(), zz, out=cc), 30), 4)}
+
         def onecall_ms(algo):
             fwd, dxf, dcf, _keep = make_onecall(algo)
             return {"fwd": round(event_ms(fwd, 20), 4), "dx": round(event_ms(dxf, 20 if algo != _lib.RDB_ALGO_TILE else 3), 4),
@@ -297,6 +310,7 @@ def main():
             "one_call_entry_points_ms": onecall_ms(_lib.RDB_ALGO_AUTO),
             "w_tiles_formed_on_chip_ms": {"fwd_strip": onecall_ms(_lib.RDB_ALGO_STRIP)["fwd"], "dcoef_dw_tile": onecall_ms(_lib.RDB_ALGO_STRIP)["dcoef"],
                                           "dx_tile": onecall_ms(_lib.RDB_ALGO_TILE)["dx"]},
+            "vendor_gemm_on_the_factored_shapes_ms": vendor_skinny(),
             "materialize_then_gemm_ms": round(event_ms(mat_gemm_step, 10), 4),
             "dense_gemm_only_ms": round(event_ms(dense_step, 20), 4),
         }
