@@ -415,3 +415,23 @@ def test_factored_dx_needs_what_it_says(hip):
         hip.linear_bwd_dcoef(dy, x, 16, 0, 40, 48, 40, 1, 0, algo=RDB_ALGO_FACTORED)
     with pytest.raises(RandumbHipError):
         hip.linear_bwd_dcoef(dy, x, 16, 48, 40, 48, 40, 1, 0, want_scale_bias_grad=True, algo=RDB_ALGO_FACTORED)
+
+
+def test_projected_path_random_shapes(hip, oracle):
+    """Twenty random layer shapes (multiples of 8, ragged against every tile size) through the projected entry points."""
+    rng = np.random.default_rng(2024)
+    for case in range(20):
+        T = int(rng.integers(1, 90)) * 8 - int(rng.integers(0, 8))          # tokens need not be a multiple of anything
+        in_f, out_f, k = (int(rng.integers(1, 66)) * 8 for _ in range(3))
+        seed = int(rng.integers(0, 2**32))
+        print(f"case random projected {case}: T={T} in={in_f} out={out_f} k={k} seed={seed}", flush=True)
+        x, dy, coef = _inputs(T, in_f, out_f, k, True, torch.bfloat16, case)
+        xn, dyn, cn = x.float().numpy(), dy.float().numpy(), coef.float().numpy()
+        xg, dyg, cg = x.cuda(), dy.cuda(), coef.cuda()
+        z = hip.linear_project(xg, k, out_f, seed)
+        y = hip.linear_fwd_projected(z, cg, in_f, seed)
+        dx, dc = hip.linear_bwd_projected(dyg, z, cg, in_f, seed)
+        want_dx, want_dc, _ = oracle.linear_bwd(xn, dyn, cn, in_f, out_f, seed)
+        assert rel_l2(cpu(y), oracle.linear_fwd(xn, cn, in_f, out_f, seed)) < BF16_TOL, case
+        assert rel_l2(cpu(dx), want_dx) < BF16_TOL, case
+        assert rel_l2(cpu(dc), want_dc) < BF16_TOL, case
