@@ -73,6 +73,9 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     assert L.rdb_linear_projection_bytes(ctypes.byref(desc(64, 96, 32, 16, rows=0))) == 0              # vector-coef
     assert L.rdb_linear_projection_bytes(ctypes.byref(desc(64, 96, 32, 16, act=_lib.RDB_F32))) == 0    # fp32 activations
     assert L.rdb_linear_projection_bytes(None) == 0
+    # operands of 2^29 elements or more are outside the engine's 32-bit buffer addressing: no projected form
+    assert L.rdb_linear_projection_bytes(ctypes.byref(desc(1 << 21, 768, 3072, 256))) == 0          # tokens*k = 2^29
+    assert L.rdb_linear_projection_bytes(ctypes.byref(desc((1 << 21) - 8, 768, 3072, 256))) == ((1 << 21) - 8) * 256 * 2
     # fp32, small k: one partial [tokens x k] matrix per 256 values of the longer side
     f32 = desc(16, 4096, 4096, 16, act=_lib.RDB_F32, coef=_lib.RDB_F32)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(f32)) == 16 * 16 * 16 * 4
