@@ -134,13 +134,15 @@ typedef struct rdb_linear_desc {
 enum {
     RDB_ALGO_AUTO = 0, /* fastest kernel the request qualifies for */
     RDB_ALGO_TILE = 1, /* regenerate W blocks in LDS per output block, contract with MFMA (any shape/dtype) */
-    RDB_ALGO_STRIP = 2, /* forward only: build a whole strip W[strip, 0:in] in LDS once per workgroup, then stream the
-                           tokens through it (matrix-coef, bf16, strip must fit LDS) */
+    RDB_ALGO_STRIP = 2, /* form W on chip with the noise hashed once per workgroup (matrix-coef, bf16 activations).
+                           forward: a whole strip W[strip, 0:in] is built in LDS, then the tokens stream through it (the
+                           strip must fit LDS).  dx: the workgroup keeps the noise columns of its 128 input features in
+                           LDS and re-forms W in chunks of 64 output rows on the matrix cores (bf16 coef, k <= 256, no
+                           scale_bias).  dcoef: dW tiles are formed and contracted with regenerated noise on chip. */
     RDB_ALGO_FACTORED = 3 /* matrix-coef only: use W = C.N associatively so that no weight tile is formed at all:
                              y = (x.N^T).C^T, dx = (dy.C).N, dcoef = dy^T.(x.N^T); the [tokens x k] intermediate lives
                              in the caller's workspace.  bf16 activations and coef: matrix-core kernels; fp32 with
-                             k <= 64 and tokens <= 4096 (the GEMV-like regime): vector-ALU kernels, bit-reproducible.  With RDB_ALGO_STRIP the coefficient gradient runs the kernel
-                             that forms dW tiles and contracts them with regenerated noise on chip. */
+                             k <= 64 and tokens <= 4096 (the GEMV-like regime): vector-ALU kernels, bit-reproducible. */
 };
 
 enum { RDB_OP_LINEAR_FWD = 0, RDB_OP_LINEAR_BWD_DX = 1, RDB_OP_LINEAR_BWD_DCOEF = 2 };

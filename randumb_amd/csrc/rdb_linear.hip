@@ -290,6 +290,10 @@ int linear_fwd_factored(void *y, int64_t ldy, const void *x, int64_t ldx, const 
 int linear_dcoef_factored(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus,
                           void *workspace, int64_t workspace_bytes, hipStream_t s);
 
+// rdb_dxstrip.hip
+int linear_dx_nstrip(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias, const rdb_linear_desc *d,
+                     hipStream_t s);
+
 // rdb_smallk.hip
 int64_t linear_smallk_workspace(const rdb_linear_desc *d);
 int linear_fwd_smallk(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
@@ -432,6 +436,13 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
             return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dx: the factored algorithm needs matrix-coef, no scale_bias, a workspace of "
                                                 "rdb_linear_workspace_bytes() bytes and either bf16 (activations and coef; sizes that are "
                                                 "multiples of 8; aligned rows) or fp32 with k <= 64 and tokens <= 4096");
+    }
+    if (d->algo != RDB_ALGO_TILE) {  // forms W chunks on chip, with the block's noise columns hashed once
+        rc = linear_dx_nstrip(dx, lddx, dy, lddy, coef, scale_bias, d, (hipStream_t)stream);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+        if (d->algo == RDB_ALGO_STRIP)
+            return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dx: the strip algorithm needs matrix-coef in bf16 with k <= 256, bf16 "
+                                                "activations, no scale_bias, sizes that are multiples of 8 and aligned rows");
     }
     const int es = d->act_dtype == RDB_BF16 ? 2 : 4;
     LinParams p = {};

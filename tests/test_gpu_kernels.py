@@ -298,13 +298,14 @@ BWD_SHAPES = [
     (2048, 768, 3072, 256, 0),   # a quarter of the headline workload
     (1000, 200, 328, 72, 3),     # ragged against every tile size (multiples of 8 only)
     (64, 8, 8, 8, 5),
+    (520, 136, 200, 248, 11),    # k = 8 mod 16, a partial chunk of output rows, three token tiles
     (300, 1024, 96, 512, 9),     # k larger than in*out/(in+out): the factored form is not cheaper, still exact when forced
 ]
 
 
 @pytest.mark.parametrize("T,in_f,out_f,k,seed", BWD_SHAPES)
 def test_linear_bwd_fast_kernels(hip, oracle, T, in_f, out_f, k, seed):
-    from randumb_amd._lib import RDB_ALGO_FACTORED, RDB_ALGO_STRIP, RDB_ALGO_TILE
+    from randumb_amd._lib import RandumbHipError, RDB_ALGO_FACTORED, RDB_ALGO_STRIP, RDB_ALGO_TILE
 
     print(f"case bwd fast T={T} in={in_f} out={out_f} k={k}", flush=True)
     x, dy, coef = _inputs(T, in_f, out_f, k, True, torch.bfloat16, seed)
@@ -315,6 +316,13 @@ def test_linear_bwd_fast_kernels(hip, oracle, T, in_f, out_f, k, seed):
     dx_ref = hip.linear_bwd_dx(dyc, cc, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_TILE)
     assert rel_l2(cpu(dx), cpu(dx_ref)) < 1e-2
     assert rel_l2(cpu(hip.linear_bwd_dx(dyc, cc, in_f, out_f, in_f, 1, seed)), want_dx) < BF16_TOL  # whatever AUTO picks
+    if k <= 256:   # the kernel that forms W chunks on chip from a noise strip kept in LDS
+        dx_s = hip.linear_bwd_dx(dyc, cc, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_STRIP)
+        assert dx_s.shape == (T, in_f) and rel_l2(cpu(dx_s), want_dx) < BF16_TOL
+        assert rel_l2(cpu(dx_s), cpu(dx_ref)) < 1e-2
+    else:
+        with pytest.raises(RandumbHipError, match="strip algorithm"):
+            hip.linear_bwd_dx(dyc, cc, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_STRIP)
     dc, dsb = hip.linear_bwd_dcoef(dyc, xc, k, out_f, in_f, out_f, in_f, 1, seed, want_scale_bias_grad=True)
     assert rel_l2(cpu(dc), want_dc) < BF16_TOL
     dc_ref, _ = hip.linear_bwd_dcoef(dyc, xc, k, out_f, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_TILE)
