@@ -283,10 +283,11 @@ int linear_fwd_strip(void *y, int64_t ldy, const void *x, int64_t ldx, const voi
 // rdb_factored.hip
 int64_t linear_projection_bytes(const rdb_linear_desc *d);
 int linear_project(void *z, const void *x, int64_t ldx, const rdb_linear_desc *d, hipStream_t s);
-int linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, const void *bias, const rdb_linear_desc *d, hipStream_t s);
+int linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, const void *bias, const rdb_linear_desc *d, int num_cus,
+                         hipStream_t s);
 int linear_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *z, const rdb_linear_desc *d, int num_cus, hipStream_t s);
 int linear_fwd_factored(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
-                        const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s);
+                        const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
 int linear_dcoef_factored(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus,
                           void *workspace, int64_t workspace_bytes, hipStream_t s);
 
@@ -384,7 +385,7 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
     if (ldy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_fwd: leading dimension smaller than the row");
     hipStream_t s = (hipStream_t)stream;
     if (d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) {
-        rc = linear_fwd_factored(y, ldy, x, ldx, coef, scale_bias, bias, d, workspace, workspace_bytes, s);
+        rc = linear_fwd_factored(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
         rc = linear_fwd_smallk(y, ldy, x, ldx, coef, scale_bias, bias, d, workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
@@ -549,7 +550,7 @@ extern "C" int rdb_linear_fwd_projected(void *y, int64_t ldy, const void *z, con
     if (rc) return rc;
     if (!y || !z || !coef) return set_error(RDB_E_NULL, "rdb_linear_fwd_projected: y, z or coef is NULL");
     if (ldy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_fwd_projected: leading dimension smaller than the row");
-    rc = linear_fwd_projected(y, ldy, z, coef, bias, d, (hipStream_t)stream);
+    rc = linear_fwd_projected(y, ldy, z, coef, bias, d, num_compute_units(), (hipStream_t)stream);
     if (rc == RDB_E_UNSUPPORTED)
         return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd_projected: coefficients must be bf16; y, z and coef 16-byte aligned; ldy a "
                                             "multiple of 8");
