@@ -168,7 +168,7 @@ def main():
 
     # caller-owned scratch, sized by the library (nothing is allocated inside the timed region)
     ws_bytes = max(L.rdb_linear_workspace_bytes(op, dref) for op in (_lib.RDB_OP_LINEAR_FWD, _lib.RDB_OP_LINEAR_BWD_DX,
-                                                                     _lib.RDB_OP_LINEAR_BWD_DCOEF))
+                                                                     _lib.RDB_OP_LINEAR_BWD_DCOEF, _lib.RDB_OP_LINEAR_BWD_PROJECTED))
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
     pws = vp(ws.data_ptr())
     z_bytes = L.rdb_linear_projection_bytes(dref)

@@ -145,7 +145,7 @@ enum {
                              k <= 64 and tokens <= 4096 (the GEMV-like regime): vector-ALU kernels, bit-reproducible. */
 };
 
-enum { RDB_OP_LINEAR_FWD = 0, RDB_OP_LINEAR_BWD_DX = 1, RDB_OP_LINEAR_BWD_DCOEF = 2 };
+enum { RDB_OP_LINEAR_FWD = 0, RDB_OP_LINEAR_BWD_DX = 1, RDB_OP_LINEAR_BWD_DCOEF = 2, RDB_OP_LINEAR_BWD_PROJECTED = 3 };
 
 /* Device scratch (bytes) that entry point `op` can use for `desc`; 0 when it has no use for any.  A NULL or too small
  * workspace is never an error with RDB_ALGO_AUTO: the library then runs a kernel that needs none. */
@@ -202,11 +202,13 @@ int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, c
                                    const rdb_linear_desc *desc, void *stream);
 
 /* Whole backward pass of the layer from the saved projection, in two kernel launches instead of five:
- * dx[t, i] = sum_o dy[t, o] * W[o, i] (act dtype) and dcoef = dy^T . z (fp32, OVERWRITTEN).  The first launch computes
- * dy . C and clears dcoef on the side; the second runs the dcoef blocks and the (dy.C).N blocks side by side, which lean on
- * different units of a compute unit (LDS + matrix cores against the integer hash on the vector ALU).
- * workspace: rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX, desc) bytes.  Same requirements as the other projected
- * entry points, coef in bf16; dcoef 16-byte aligned. */
+ * dx[t, i] = sum_o dy[t, o] * W[o, i] (act dtype) and dcoef = dy^T . z (fp32, OVERWRITTEN).
+ * workspace: rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_PROJECTED, desc) bytes holds dy.C and the partial sums of dcoef
+ * over token ranges.  Then the first launch runs the two long contractions over dy (dy.C and the dcoef partial sums) side by
+ * side, and the second the (dy.C).N blocks beside blocks that add the partial sums in a fixed order: no atomics, the
+ * result is the same bit for bit from run to run.  With the RDB_OP_LINEAR_BWD_DX amount only (room for dy.C) the first
+ * launch computes dy.C and clears dcoef, and the second combines the dcoef blocks with fp32 atomics beside (dy.C).N.
+ * Same requirements as the other projected entry points, coef in bf16; dcoef 16-byte aligned. */
 int rdb_linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z,
                              const void *coef, const rdb_linear_desc *desc, void *workspace,
                              int64_t workspace_bytes, void *stream);

@@ -14,7 +14,7 @@ SO_PATH = os.path.join(_HERE, "librandumb_hip.so")
 
 RDB_F32, RDB_BF16 = 0, 1
 RDB_ALGO_AUTO, RDB_ALGO_TILE, RDB_ALGO_STRIP, RDB_ALGO_FACTORED = 0, 1, 2, 3
-RDB_OP_LINEAR_FWD, RDB_OP_LINEAR_BWD_DX, RDB_OP_LINEAR_BWD_DCOEF = 0, 1, 2
+RDB_OP_LINEAR_FWD, RDB_OP_LINEAR_BWD_DX, RDB_OP_LINEAR_BWD_DCOEF, RDB_OP_LINEAR_BWD_PROJECTED = 0, 1, 2, 3
 
 # every exported entry point, in header order; tests check the list against the built library
 EXPORTS = [

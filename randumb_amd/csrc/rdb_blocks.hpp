@@ -1,5 +1,6 @@
-// Block bodies shared by more than one kernel: the coefficient-gradient block (dC = dy^T . z) and the second block of the
-// input gradient (dx = t . N) run as kernels of their own and side by side in one launch of the merged backward kernel.
+// Block bodies shared by more than one kernel: the coefficient-gradient block (dC = dy^T . z), the reduction of its partial
+// sums and the second block of the input gradient (dx = t . N) run as kernels of their own and side by side in the merged
+// backward kernels.
 #pragma once
 #include "rdb_gemm.hpp"
 #include "rdb_tile.hpp"
@@ -16,6 +17,8 @@ struct DcParams {
     const bf16_t *dy;
     const bf16_t *z;
     float *dcoef;
+    float *partial;  // NULL: the token splits add into dcoef (zeroed beforehand) with atomics; else split s stores its sums
+                     // into partial[s][out_f][k] and a reduction pass (red_block) writes dcoef
     int64_t lddy;
     int tokens, out_f, k;
     int tiles_o, tiles_m, splits, tok_per_split;
@@ -41,6 +44,7 @@ __device__ __forceinline__ void dc_block(const DcParams &p, bf16_t *lds, int blo
     GlobalOperand<KD_BM, B_BK, M_CONT> opz = {p.z, (int64_t)p.k, m0, p.k, t_end, (int64_t)p.tokens * p.k};
     gemm_mainloop<KD_BO, KD_BM, B_BK, 1, 1>(acc, lds, opdy, opz, t_begin, (t_end - t_begin + B_BK - 1) / B_BK);
     // acc[mi][ni][j]: o = o0 + wm*64 + mi*32 + 8*(j/4) + 4*g + j%4, m = m0 + wn*64 + ni*32 + r (32 consecutive m: coalesced)
+    float *out = p.partial ? p.partial + (int64_t)split * p.out_f * p.k : p.dcoef;
 #pragma unroll
     for (int ni = 0; ni < KD_BM / 64; ++ni) {
         const int m = m0 + wn * 64 + ni * 32 + r;
@@ -50,8 +54,38 @@ __device__ __forceinline__ void dc_block(const DcParams &p, bf16_t *lds, int blo
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
                 const int o = o0 + wm * 64 + mi * 32 + 8 * (j / 4) + 4 * g + (j % 4);
-                if (o < p.out_f) unsafeAtomicAdd(p.dcoef + (int64_t)o * p.k + m, acc[mi][ni][j]);
+                if (o < p.out_f) {
+                    if (p.partial)
+                        out[(int64_t)o * p.k + m] = acc[mi][ni][j];
+                    else
+                        unsafeAtomicAdd(out + (int64_t)o * p.k + m, acc[mi][ni][j]);
+                }
             }
+    }
+}
+
+// ----------------------------------------------------------------------------------------------- dC = sum of the splits' partial sums
+// Added in split order, so the result does not depend on how the blocks were scheduled.
+struct RedParams {
+    const float *partial;  // [splits][n]
+    float *out;            // [n]
+    int64_t n;             // multiple of 4
+    int splits;
+};
+
+__device__ __forceinline__ void red_block(const RedParams &p, int block, int nblocks)
+{
+    const int64_t n4 = p.n / 4;
+    for (int64_t e = (int64_t)block * 256 + threadIdx.x; e < n4; e += (int64_t)nblocks * 256) {
+        f32x4 v = reinterpret_cast<const f32x4 *>(p.partial)[e];
+        for (int sidx = 1; sidx < p.splits; ++sidx) {
+            const f32x4 u = reinterpret_cast<const f32x4 *>(p.partial + (int64_t)sidx * p.n)[e];
+            v[0] += u[0];
+            v[1] += u[1];
+            v[2] += u[2];
+            v[3] += u[3];
+        }
+        reinterpret_cast<f32x4 *>(p.out)[e] = v;
     }
 }
 
@@ -97,6 +131,7 @@ inline int make_dc_params(DcParams &p, float *dcoef, const void *dy, int64_t ldd
     p.dy = (const bf16_t *)dy;
     p.z = (const bf16_t *)z;
     p.dcoef = dcoef;
+    p.partial = nullptr;
     p.lddy = lddy;
     p.tokens = (int)d->tokens;
     p.out_f = (int)d->out_f;

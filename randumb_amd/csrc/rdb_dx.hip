@@ -31,17 +31,11 @@ struct DyCParams {
     int tiles_c, tiles_t;
 };
 
-__global__ __launch_bounds__(256, 2) void dx_dyc_kernel(DyCParams p)
+// `block`: index of this block among the blocks that run this body.
+__device__ __forceinline__ void dyc_block(const DyCParams &p, bf16_t *lds, int block)
 {
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
-    if (p.zero) {  // a kernel later in the stream accumulates into this array with atomics
-        const f32x4 z4 = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < p.zero_n / 4; e += (int64_t)gridDim.x * 256)
-            reinterpret_cast<f32x4 *>(p.zero)[e] = z4;
-    }
     // work item = (token tile, coefficient tile), coefficient tile fastest: neighbours share the dy tile
-    const int w = xcd_work_item(blockIdx.x, p.tiles_c * p.tiles_t);
+    const int w = xcd_work_item(block, p.tiles_c * p.tiles_t);
     if (w >= p.tiles_c * p.tiles_t) return;
     const int m0 = (w % p.tiles_c) * K1_BC, tok0 = (w / p.tiles_c) * K1_BT;
     f32x16 acc[K1_BC / 64][K1_BT / 64];
@@ -55,6 +49,17 @@ __global__ __launch_bounds__(256, 2) void dx_dyc_kernel(DyCParams p)
     GlobalOperand<K1_BT, X_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
     gemm_mainloop<K1_BC, K1_BT, X_BK, 2, 2>(acc, lds, opc, opdy, 0, (p.out_f + X_BK - 1) / X_BK);
     store_tile_bf16<K1_BC, K1_BT>(acc, lds, p.t, p.k, m0, p.k, tok0, p.tokens, 1.0f, nullptr);
+}
+
+__global__ __launch_bounds__(256, 2) void dx_dyc_kernel(DyCParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    if (p.zero) {  // a kernel later in the stream accumulates into this array with atomics
+        const f32x4 z4 = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < p.zero_n / 4; e += (int64_t)gridDim.x * 256)
+            reinterpret_cast<f32x4 *>(p.zero)[e] = z4;
+    }
+    dyc_block(p, reinterpret_cast<bf16_t *>(smem_raw), blockIdx.x);
 }
 
 // ----------------------------------------------------------------------------------------------- kernel 2: dx = t . N
@@ -85,6 +90,42 @@ __global__ __launch_bounds__(256, 2) void bwd_dc_tn_kernel(BwdParams p)
         tn_block(p.tn, lds, blockIdx.x - p.dc_blocks);
 }
 
+// ----------------------------------------------------------------------------------------------- the backward pass regrouped
+// With room for the coefficient gradient's partial sums in the workspace nothing has to be zeroed first, so the two long
+// contractions over dy, t = dy.C and dC = dy^T.z, can share a launch: both run the tile engine with four waves a block and
+// wait on memory much of the time, and two blocks per compute unit fill each other's gaps (they also read the same dy).
+// The second launch runs the dx = t.N blocks and, beside them, the blocks that add the partial sums up in split order.
+struct BwdAParams {
+    DcParams dc;
+    DyCParams dyc;
+    int dc_blocks;  // multiple of 8, so both parts keep their die assignment
+};
+
+__global__ __launch_bounds__(256, 2) void bwd_dc_dyc_kernel(BwdAParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
+    if ((int)blockIdx.x < p.dc_blocks)
+        dc_block(p.dc, lds, blockIdx.x);
+    else
+        dyc_block(p.dyc, lds, blockIdx.x - p.dc_blocks);
+}
+
+struct BwdBParams {
+    TNParams tn;
+    RedParams red;
+    int tn_blocks;
+};
+
+__global__ __launch_bounds__(256, 2) void bwd_tn_red_kernel(BwdBParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    if ((int)blockIdx.x < p.tn_blocks)
+        tn_block(p.tn, reinterpret_cast<bf16_t *>(smem_raw), blockIdx.x);
+    else
+        red_block(p.red, blockIdx.x - p.tn_blocks, gridDim.x - p.tn_blocks);
+}
+
 // ----------------------------------------------------------------------------------------------- host side
 static bool dx_factored_ok(const rdb_linear_desc *d)
 {
@@ -97,6 +138,17 @@ int64_t linear_dx_factored_workspace(const rdb_linear_desc *d)
 {
     if (!dx_factored_ok(d)) return 0;
     return d->tokens * d->k * (int64_t)sizeof(bf16_t);
+}
+
+static int64_t align256(int64_t n) { return (n + 255) / 256 * 256; }
+
+// Workspace of the regrouped backward pass: t, then the partial sums of the coefficient gradient.
+int64_t linear_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus)
+{
+    if (!dx_factored_ok(d)) return 0;
+    DcParams dc;
+    make_dc_params(dc, nullptr, nullptr, d->out_f, nullptr, d, num_cus);
+    return align256(linear_dx_factored_workspace(d)) + (int64_t)dc.splits * d->out_f * d->k * (int64_t)sizeof(float);
 }
 
 static void make_dyc_params(DyCParams &p1, const void *dy, int64_t lddy, const void *coef, void *t, const rdb_linear_desc *d)
@@ -146,16 +198,45 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
         return RDB_E_UNSUPPORTED;
     DyCParams p1;
     make_dyc_params(p1, dy, lddy, coef, workspace, d);
-    p1.zero = dcoef;  // cleared here, accumulated into by the next launch
+    const size_t smem_dc = engine_smem<KD_BO, KD_BM, X_BK, M_CONT, M_CONT>(), smem_tn = engine_smem<K2_BI, K2_BT, X_BK, K_CONT, K_CONT>();
+    const size_t smem_dyc = engine_smem<K1_BC, K1_BT, X_BK, M_CONT, K_CONT>();
+    if (workspace_bytes >= linear_bwd_projected_workspace(d, num_cus)) {
+        BwdAParams a;
+        const int dc_items = make_dc_params(a.dc, dcoef, dy, lddy, z, d, num_cus);
+        a.dc.partial = reinterpret_cast<float *>(static_cast<char *>(workspace) + align256(linear_dx_factored_workspace(d)));
+        a.dyc = p1;
+        a.dc_blocks = xcd_grid_size(dc_items);
+        size_t smem = smem_dc > smem_dyc ? smem_dc : smem_dyc;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dc_dyc_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return set_error((int)e, "bwd_dc_dyc_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+        bwd_dc_dyc_kernel<<<a.dc_blocks + xcd_grid_size(p1.tiles_c * p1.tiles_t), 256, smem, s>>>(a);
+        int rc = check_launch("bwd_dc_dyc_kernel");
+        if (rc) return rc;
+        BwdBParams b;
+        const int tn_items = make_tn_params(b.tn, dx, lddx, workspace, d);
+        b.tn_blocks = xcd_grid_size(tn_items);
+        b.red.partial = a.dc.partial;
+        b.red.out = dcoef;
+        b.red.n = d->out_f * d->k;
+        b.red.splits = a.dc.splits;
+        int red_blocks = (int)cdiv(b.red.n / 4, 256 * 8);
+        if (red_blocks > num_cus / 2) red_blocks = num_cus / 2;
+        if (red_blocks < 1) red_blocks = 1;
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_tn_red_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_tn);
+        if (e != hipSuccess) return set_error((int)e, "bwd_tn_red_kernel: cannot reserve %zu bytes of LDS: %s", smem_tn, hipGetErrorString(e));
+        bwd_tn_red_kernel<<<b.tn_blocks + red_blocks, 256, smem_tn, s>>>(b);
+        return check_launch("bwd_tn_red_kernel");
+    }
+    // workspace for t only: dy.C first (clearing dcoef on the side), then the coefficient gradient with atomics beside t.N
+    p1.zero = dcoef;
     p1.zero_n = d->out_f * d->k;
-    int rc = launch_engine(dx_dyc_kernel, p1, p1.tiles_c * p1.tiles_t, engine_smem<K1_BC, K1_BT, X_BK, M_CONT, K_CONT>(), s, "dx_dyc_kernel");
+    int rc = launch_engine(dx_dyc_kernel, p1, p1.tiles_c * p1.tiles_t, smem_dyc, s, "dx_dyc_kernel");
     if (rc) return rc;
     BwdParams p;
     const int dc_items = make_dc_params(p.dc, dcoef, dy, lddy, z, d, num_cus);
     const int tn_items = make_tn_params(p.tn, dx, lddx, workspace, d);
     p.dc_blocks = xcd_grid_size(dc_items);
-    size_t smem = engine_smem<KD_BO, KD_BM, X_BK, M_CONT, M_CONT>();
-    if (smem < engine_smem<K2_BI, K2_BT, X_BK, K_CONT, K_CONT>()) smem = engine_smem<K2_BI, K2_BT, X_BK, K_CONT, K_CONT>();
+    const size_t smem = smem_dc > smem_tn ? smem_dc : smem_tn;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dc_tn_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return set_error((int)e, "bwd_dc_tn_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
     bwd_dc_tn_kernel<<<p.dc_blocks + xcd_grid_size(tn_items), 256, smem, s>>>(p);

@@ -308,6 +308,7 @@ int linear_dcoef_smallk(float *dcoef, const void *dy, int64_t lddy, const void *
 int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z, const void *coef,
                          const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
 int64_t linear_dx_factored_workspace(const rdb_linear_desc *d);
+int64_t linear_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus);
 int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias,
                        const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s);
 
@@ -370,6 +371,7 @@ extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
         return (op == RDB_OP_LINEAR_FWD || op == RDB_OP_LINEAR_BWD_DX || op == RDB_OP_LINEAR_BWD_DCOEF) ? linear_smallk_workspace(&dd) : 0;
     }
     if (op == RDB_OP_LINEAR_BWD_DX) return linear_dx_factored_workspace(d);
+    if (op == RDB_OP_LINEAR_BWD_PROJECTED) return linear_bwd_projected_workspace(d, num_compute_units());
     if (op == RDB_OP_LINEAR_FWD) return d->coef_dtype == RDB_BF16 ? linear_projection_bytes(d) : 0;
     if (op == RDB_OP_LINEAR_BWD_DCOEF) return linear_projection_bytes(d);  // reads no coefficients: their dtype does not matter
     return 0;

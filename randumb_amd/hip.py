@@ -11,7 +11,7 @@ import torch
 
 from . import _lib
 from ._lib import (LinearDesc, RDB_ALGO_AUTO, RDB_BF16, RDB_F32, RDB_OP_LINEAR_BWD_DCOEF, RDB_OP_LINEAR_BWD_DX,
-                   RDB_OP_LINEAR_FWD)
+                   RDB_OP_LINEAR_BWD_PROJECTED, RDB_OP_LINEAR_FWD)
 
 _DT = {torch.float32: RDB_F32, torch.bfloat16: RDB_BF16}
 
@@ -313,9 +313,10 @@ def linear_bwd_dcoef_projected(dy: torch.Tensor, z: torch.Tensor, in_f: int, see
     return dcoef
 
 
-def linear_bwd_projected(dy: torch.Tensor, z: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int):
+def linear_bwd_projected(dy: torch.Tensor, z: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int, ordered_sums: bool = True):
     """Whole backward pass of a matrix-coef bf16 layer from the saved projection: ``(dx, dcoef)`` with ``dx = dy @ W`` in
-    bf16 and ``dcoef = dy.T @ z`` in fp32, in two kernel launches."""
+    bf16 and ``dcoef = dy.T @ z`` in fp32, in two kernel launches.  ``ordered_sums`` gives the library room for the partial
+    sums of ``dcoef`` (added in a fixed order: bit-reproducible); without it they are combined with fp32 atomics."""
     _need_gpu("linear_bwd_projected", dy, z, coef)
     dy = _act(dy)
     z = z.contiguous()
@@ -325,7 +326,7 @@ def linear_bwd_projected(dy: torch.Tensor, z: torch.Tensor, coef: torch.Tensor, 
     dx = torch.empty((dy.shape[0], in_f), dtype=dy.dtype, device=dy.device)
     dcoef = torch.empty((out_f, k), dtype=torch.float32, device=dy.device)
     L = _lib.load()
-    ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX, ctypes.byref(d))
+    ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_PROJECTED if ordered_sums else RDB_OP_LINEAR_BWD_DX, ctypes.byref(d))
     ws = _workspace(ws_bytes, dy.device)
     with torch.cuda.device(dy.device):
         rc = L.rdb_linear_bwd_projected(_p(dx), dx.stride(0), _p(dcoef), _p(dy), dy.stride(0), _p(z), _p(c), ctypes.byref(d), _p(ws),

@@ -381,12 +381,20 @@ def test_linear_bwd_projected_one_call(hip, oracle, T, in_f, out_f, k, seed):
     x, dy, coef = _inputs(T, in_f, out_f, k, True, torch.bfloat16, seed)
     want_dx, want_dc, _ = oracle.linear_bwd(x.float().numpy(), dy.float().numpy(), coef.float().numpy(), in_f, out_f, seed)
     z = hip.linear_project(x.cuda(), k, out_f, seed)
-    for _ in range(2):   # the second call finds dcoef's buffer dirty in the allocator: it must be cleared by the call
-        dx, dc = hip.linear_bwd_projected(dy.cuda(), z, coef.cuda(), in_f, seed)
-        assert dx.shape == (T, in_f) and rel_l2(cpu(dx), want_dx) < BF16_TOL
-        assert dc.shape == (out_f, k) and rel_l2(cpu(dc), want_dc) < BF16_TOL
-    assert torch.equal(dx, hip.linear_bwd_dx(dy.cuda(), coef.cuda(), in_f, out_f, in_f, 1, seed, algo=3))
-    assert rel_l2(cpu(dc), cpu(hip.linear_bwd_dcoef_projected(dy.cuda(), z, in_f, seed))) < 1e-5
+    dyc, cc = dy.cuda(), coef.cuda()
+    dx_sep = hip.linear_bwd_dx(dyc, cc, in_f, out_f, in_f, 1, seed, algo=3)
+    dc_sep = hip.linear_bwd_dcoef_projected(dyc, z, in_f, seed)
+    for ordered in (True, False):   # partial sums added in order (bigger workspace) / combined with atomics
+        runs = []
+        for _ in range(2):   # the second call finds dcoef's buffer dirty in the allocator: it must be overwritten by the call
+            dx, dc = hip.linear_bwd_projected(dyc, z, cc, in_f, seed, ordered_sums=ordered)
+            assert dx.shape == (T, in_f) and rel_l2(cpu(dx), want_dx) < BF16_TOL
+            assert dc.shape == (out_f, k) and rel_l2(cpu(dc), want_dc) < BF16_TOL
+            runs.append(dc)
+        assert torch.equal(dx, dx_sep)
+        assert rel_l2(cpu(dc), cpu(dc_sep)) < 1e-5
+        if ordered:
+            assert torch.equal(runs[0], runs[1])   # no atomics on this path: the same bits every time
 
 
 def test_projected_form_rejects_what_it_cannot_do(hip):
