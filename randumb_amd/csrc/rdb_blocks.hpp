@@ -76,7 +76,7 @@ struct RedParams {
 __device__ __forceinline__ void red_block(const RedParams &p, int block, int nblocks)
 {
     const int64_t n4 = p.n / 4;
-    for (int64_t e = (int64_t)block * 256 + threadIdx.x; e < n4; e += (int64_t)nblocks * 256) {
+    for (int64_t e = (int64_t)block * blockDim.x + threadIdx.x; e < n4; e += (int64_t)nblocks * blockDim.x) {
         f32x4 v = reinterpret_cast<const f32x4 *>(p.partial)[e];
         for (int sidx = 1; sidx < p.splits; ++sidx) {
             const f32x4 u = reinterpret_cast<const f32x4 *>(p.partial + (int64_t)sidx * p.n)[e];

@@ -10,6 +10,7 @@
 // Replaces autograd's MmBackward on the re-materialised weight (materialize() + dense product,
 // src/rten_cpp/RandumbTensor.py:942-946).
 #include "rdb_blocks.hpp"
+#include "rdb_stationary.hpp"
 
 namespace rdb {
 
@@ -126,6 +127,28 @@ __global__ __launch_bounds__(256, 2) void bwd_tn_red_kernel(BwdBParams p)
         red_block(p.red, blockIdx.x - p.tn_blocks, gridDim.x - p.tn_blocks);
 }
 
+// dx = t . N for k <= 256 with t held in registers (rdb_stationary.hpp), alone and beside the reduction blocks.
+template <int KG> __global__ __launch_bounds__(ST_THREADS, 1) void dx_tns_kernel(StParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    stationary_block<KG, false, true>(p, smem_raw, blockIdx.x);
+}
+
+struct BwdBsParams {
+    StParams tn;
+    RedParams red;
+    int tn_blocks;
+};
+
+template <int KG> __global__ __launch_bounds__(ST_THREADS, 1) void bwd_tns_red_kernel(BwdBsParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    if ((int)blockIdx.x < p.tn_blocks)
+        stationary_block<KG, false, true>(p.tn, smem_raw, blockIdx.x);
+    else
+        red_block(p.red, blockIdx.x - p.tn_blocks, gridDim.x - p.tn_blocks);
+}
+
 // ----------------------------------------------------------------------------------------------- host side
 static bool dx_factored_ok(const rdb_linear_desc *d)
 {
@@ -166,9 +189,24 @@ static void make_dyc_params(DyCParams &p1, const void *dy, int64_t lddy, const v
     p1.tiles_t = (int)cdiv(d->tokens, K1_BT);
 }
 
+// t . N with t in registers applies when k is short enough and dx fits a buffer descriptor.
+static bool tn_stationary_ok(const rdb_linear_desc *d, int64_t lddx) { return d->k <= ST_KMAX && d->tokens * lddx < (1ll << 29); }
+
+static int make_tns_params(StParams &q, void *dx, int64_t lddx, const void *t, const rdb_linear_desc *d, int num_cus)
+{
+    q.z = (const bf16_t *)t;
+    q.coef = nullptr;
+    q.bias = nullptr;
+    q.y = (bf16_t *)dx;
+    q.ldy = lddx;
+    q.k = (int)d->k;
+    q.seed = d->seed;
+    return make_stationary_grid(q, d->tokens, d->in_f, num_cus);
+}
+
 // Returns RDB_E_UNSUPPORTED (without setting an error) when the request does not fit this algorithm.
 int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias,
-                       const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s)
+                       const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
     if (!dx_factored_ok(d) || scale_bias) return RDB_E_UNSUPPORTED;  // the random-bias term is not low rank
     if (!workspace || workspace_bytes < linear_dx_factored_workspace(d) || ((uintptr_t)workspace & 15)) return RDB_E_UNSUPPORTED;
@@ -181,6 +219,17 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
     make_dyc_params(p1, dy, lddy, coef, workspace, d);
     int rc = launch_engine(dx_dyc_kernel, p1, p1.tiles_c * p1.tiles_t, engine_smem<K1_BC, K1_BT, X_BK, M_CONT, K_CONT>(), s, "dx_dyc_kernel");
     if (rc) return rc;
+    if (tn_stationary_ok(d, lddx)) {
+        StParams q;
+        const int items = make_tns_params(q, dx, lddx, workspace, d, num_cus);
+        const int kg = (int)cdiv(d->k, 64);
+        switch (kg) {
+        case 1: return launch_stationary(dx_tns_kernel<1>, q, items, stationary_smem(kg), s, "dx_tns_kernel<1>");
+        case 2: return launch_stationary(dx_tns_kernel<2>, q, items, stationary_smem(kg), s, "dx_tns_kernel<2>");
+        case 3: return launch_stationary(dx_tns_kernel<3>, q, items, stationary_smem(kg), s, "dx_tns_kernel<3>");
+        default: return launch_stationary(dx_tns_kernel<4>, q, items, stationary_smem(kg), s, "dx_tns_kernel<4>");
+        }
+    }
     TNParams p2;
     const int items = make_tn_params(p2, dx, lddx, workspace, d);
     return launch_engine(dx_tn_kernel, p2, items, engine_smem<K2_BI, K2_BT, X_BK, K_CONT, K_CONT>(), s, "dx_tn_kernel");
@@ -212,13 +261,38 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
         bwd_dc_dyc_kernel<<<a.dc_blocks + xcd_grid_size(p1.tiles_c * p1.tiles_t), 256, smem, s>>>(a);
         int rc = check_launch("bwd_dc_dyc_kernel");
         if (rc) return rc;
+        RedParams red;
+        red.partial = a.dc.partial;
+        red.out = dcoef;
+        red.n = d->out_f * d->k;
+        red.splits = a.dc.splits;
+        if (tn_stationary_ok(d, lddx)) {
+            BwdBsParams bs;
+            const int items = make_tns_params(bs.tn, dx, lddx, workspace, d, num_cus);
+            bs.red = red;
+            bs.tn_blocks = xcd_grid_size(items);
+            int rblocks = (int)cdiv(red.n / 4, ST_THREADS * 8);
+            if (rblocks > num_cus / 4) rblocks = num_cus / 4;
+            if (rblocks < 1) rblocks = 1;
+            const int kg = (int)cdiv(d->k, 64);
+            const size_t smem_s = stationary_smem(kg);
+            const void *fn = kg == 1 ? (const void *)bwd_tns_red_kernel<1> : kg == 2 ? (const void *)bwd_tns_red_kernel<2>
+                           : kg == 3 ? (const void *)bwd_tns_red_kernel<3> : (const void *)bwd_tns_red_kernel<4>;
+            e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_s);
+            if (e != hipSuccess) return set_error((int)e, "bwd_tns_red_kernel: cannot reserve %zu bytes of LDS: %s", smem_s, hipGetErrorString(e));
+            const dim3 grid(bs.tn_blocks + rblocks), block(ST_THREADS);
+            switch (kg) {
+            case 1: bwd_tns_red_kernel<1><<<grid, block, smem_s, s>>>(bs); break;
+            case 2: bwd_tns_red_kernel<2><<<grid, block, smem_s, s>>>(bs); break;
+            case 3: bwd_tns_red_kernel<3><<<grid, block, smem_s, s>>>(bs); break;
+            default: bwd_tns_red_kernel<4><<<grid, block, smem_s, s>>>(bs); break;
+            }
+            return check_launch("bwd_tns_red_kernel");
+        }
         BwdBParams b;
         const int tn_items = make_tn_params(b.tn, dx, lddx, workspace, d);
         b.tn_blocks = xcd_grid_size(tn_items);
-        b.red.partial = a.dc.partial;
-        b.red.out = dcoef;
-        b.red.n = d->out_f * d->k;
-        b.red.splits = a.dc.splits;
+        b.red = red;
         int red_blocks = (int)cdiv(b.red.n / 4, 256 * 8);
         if (red_blocks > num_cus / 2) red_blocks = num_cus / 2;
         if (red_blocks < 1) red_blocks = 1;
