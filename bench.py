@@ -33,8 +33,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # HBM bytes per call of each product, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script scaled by what the same
 # counters read for a plain 256 MiB device copy (FETCH x2.000, WRITE x1.000): profiles/bench_c2_hbm_traffic.md
 HBM_TRAFFIC_BYTES = {
-    "forward (factored_z_kernel + factored_y_kernel)": 84.5e6,
-    "backward (dx_dyc_kernel + bwd_dc_tn_kernel)": 84.3e6 + 76.3e6,
+    "forward (factored_z_kernel + factored_ys_kernel)": 84.5e6,
+    "backward (bwd_dc_dyc_kernel + bwd_tns_red_kernel)": 84.3e6 + 76.3e6,
 }
 T, IN_F, OUT_F, K, SEED = 8192, 768, 3072, 256, 0
 
@@ -43,8 +43,8 @@ F_PER_PRODUCT = 2.0 * T * IN_F * OUT_F + 2.0 * OUT_F * IN_F * K      # one dense
 F_STEP = 3.0 * F_PER_PRODUCT
 # what the factored kernels execute: z, y, t, dx, dC products (z once per step)
 EXEC = {
-    "forward (factored_z_kernel + factored_y_kernel)": 2.0 * T * K * (IN_F + OUT_F),
-    "backward (dx_dyc_kernel + bwd_dc_tn_kernel)": 2.0 * T * K * (OUT_F + IN_F) + 2.0 * T * K * OUT_F,
+    "forward (factored_z_kernel + factored_ys_kernel)": 2.0 * T * K * (IN_F + OUT_F),
+    "backward (bwd_dc_dyc_kernel + bwd_tns_red_kernel)": 2.0 * T * K * (OUT_F + IN_F) + 2.0 * T * K * OUT_F,
 }
 EXEC_STEP = 2.0 * T * K * (IN_F + OUT_F) + 2.0 * T * K * (OUT_F + IN_F) + 2.0 * T * K * OUT_F
 
@@ -259,8 +259,8 @@ def main():
         "rdb_linear_bwd_dcoef_projected (separate call)": event_ms(k_dcoef_projected, iters),
     }
     products = {   # share of F: forward one third, backward (dx and dC) two thirds
-        "forward (factored_z_kernel + factored_y_kernel)": (calls["rdb_linear_project"] + calls["rdb_linear_fwd_projected"], F_PER_PRODUCT),
-        "backward (dx_dyc_kernel + bwd_dc_tn_kernel)": (calls["rdb_linear_bwd_projected"], 2 * F_PER_PRODUCT),
+        "forward (factored_z_kernel + factored_ys_kernel)": (calls["rdb_linear_project"] + calls["rdb_linear_fwd_projected"], F_PER_PRODUCT),
+        "backward (bwd_dc_dyc_kernel + bwd_tns_red_kernel)": (calls["rdb_linear_bwd_projected"], 2 * F_PER_PRODUCT),
     }
     dom = max(products, key=lambda n: products[n][0])
     dom_ms, dom_flops = products[dom]
@@ -292,7 +292,7 @@ def main():
 
         def vendor_skinny():
             # the three dense products of the factored algorithm given to the vendor GEMM (torch.matmul), for reference
-            # against factored_y_kernel / dx_dyc_kernel / factored_dc_kernel in profiles/bench_c2_kernel_trace.md
+            # against factored_ys_kernel / dx_dyc_kernel / factored_dc_kernel in profiles/bench_c2_kernel_trace.md
             zz = torch.randn(T, K, device=dev).bfloat16()
             yy = torch.empty(T, OUT_F, device=dev, dtype=torch.bfloat16)
             tt = torch.empty(T, K, device=dev, dtype=torch.bfloat16)
