@@ -33,8 +33,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # HBM bytes per call of each product, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this script scaled by what the same
 # counters read for a plain 256 MiB device copy (FETCH x2.000, WRITE x1.000): profiles/bench_c2_hbm_traffic.md
 HBM_TRAFFIC_BYTES = {
-    "forward (factored_z_kernel + factored_ys_kernel)": 84.5e6,
-    "backward (bwd_dc_dyc_kernel + bwd_tns_red_kernel)": 84.3e6 + 76.3e6,
+    "forward (factored_z_kernel + factored_ys_kernel)": 84.2e6,
+    "backward (bwd_dc_dyc_kernel + bwd_tns_red_kernel)": 143.3e6 + 35.9e6,
 }
 T, IN_F, OUT_F, K, SEED = 8192, 768, 3072, 256, 0
 
