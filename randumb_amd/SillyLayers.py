@@ -177,6 +177,44 @@ class SillyLinear(SillyModuleMixin, nn.Module):
         return (f"in_features={self.in_features}, out_features={self.out_features}, int_dim={self.int_dim}, seeds={self.seed}, "
                 f"bias={self.bias is not None}, matrix_coef={self.matrix_coef}, fused={self.fused}")
 
+class SillyConv2d(SillyModuleMixin, nn.Conv2d):
+    """``nn.Conv2d`` whose kernel (and bias) are vector-coef pseudorandom tensors.  Same constructor as the reference
+    (SillyLayers.py:230-297): ``int_dim`` and ``seed`` are lists or generators yielding two values (weight, bias).
+
+    The kernel is a 4-D pseudorandom tensor ``(out_channels, in_channels / groups, kh, kw)``: element ``a`` of its contiguous
+    storage is ``sum_m noise(PRIME*a + m) * coef[m]``.  The convolution itself is the stock one: the tensor materialises for
+    the duration of ``aten.convolution`` and the kernel's gradient reaches the coefficients through
+    :class:`RandumbTensorConstructor`.  (The reference passes the 4-D size and strides into a kernel that takes two of each,
+    SillyLayers.py:282-287 with RandumbTensor.py:375-380; here N-D shapes materialise through their storage extent.)
+    """
+
+    num_seeds = 2
+
+    def __init__(self, in_channels: int, out_channels: int, int_dim: Union[list, GeneratorType], seed: Union[list, GeneratorType],
+                 kernel_size, stride=1, padding=0, dilation=1, groups: int = 1, bias: bool = True, rt_bias: bool = False,
+                 padding_mode: str = "zeros", device=None, dtype=None) -> None:
+        self.int_dim = _take(int_dim, self.num_seeds)
+        self.seed = _take(seed, self.num_seeds)
+        self.rt_bias = rt_bias
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, groups, bias, padding_mode,
+                         device=device, dtype=dtype)
+
+    def reset_parameters(self) -> None:
+        # nn.Conv2d.__init__ has made dense parameters; keep their shapes, replace them (SillyLayers.py:280-294)
+        w = self.weight
+        self.weight_coef = nn.Parameter(torch.empty(self.int_dim[0], dtype=w.dtype, device=w.device), requires_grad=True)
+        del self.weight
+        self.register_buffer("weight", CreateRandumbTensor(self.weight_coef, self.seed[0], tuple(w.shape), fused_bias=self.rt_bias))
+        if self.bias is not None:
+            b = self.bias
+            self.bias_coef = nn.Parameter(torch.empty(self.int_dim[1], dtype=b.dtype, device=b.device), requires_grad=True)
+            del self.bias
+            self.register_buffer("bias", CreateRandumbTensor(self.bias_coef, self.seed[1], tuple(b.shape), fused_bias=self.rt_bias))
+        self.init_zero_coef_uniform_bias()
+
+    def extra_repr(self) -> str:
+        return f"{super().extra_repr()}, int_dim={self.int_dim}, seeds={self.seed}"
+
 
 class SillyEmbedding(SillyModuleMixin, nn.Module):
     """Embedding whose table is a vector-coef pseudorandom tensor; only the requested rows are ever generated

@@ -194,6 +194,49 @@ def test_bf16_layer_matches_oracle(ra, oracle):
     assert l.weight_coef.grad.dtype == torch.bfloat16 and rel_l2(cpu(l.weight_coef.grad), dC) < BF16_TOL
 
 
+def test_conv2d_layers_match_a_dense_autograd_graph(ra, oracle):
+    """Two convolution layers with pseudorandom kernels (the front of the reference's MNIST net, mnist.py:55-84) against the
+    same convolutions on dense kernels built from the oracle, in fp64 on the CPU: output, input gradient, and the gradient
+    of every coefficient vector and scale."""
+    print("case conv2d", flush=True)
+    g = torch.Generator().manual_seed(5)
+    ints, seeds = ra.stepgen(48, 0), ra.stepgen(77, 1)
+    c1 = ra.SillyConv2d(1, 8, int_dim=ints, seed=seeds, kernel_size=3, stride=1, rt_bias=True)
+    c2 = ra.SillyConv2d(8, 16, int_dim=ints, seed=seeds, kernel_size=3, stride=2, padding=1, rt_bias=True)
+    with torch.no_grad():
+        for c in (c1, c2):
+            c.weight_coef.copy_(torch.randn(48, generator=g) * 0.1)
+            c.bias_coef.copy_(torch.randn(48, generator=g) * 0.1)
+    c1, c2 = c1.cuda(), c2.cuda()
+    x = torch.rand(4, 1, 12, 12, generator=g)
+    xg = x.cuda().requires_grad_()
+    y = c2(F.relu(c1(xg)))
+    assert y.shape == (4, 16, 5, 5) and c1.weight._tensor is None
+    y.square().sum().backward()
+
+    # dense twin: W_flat = Noise(seed) @ coef + scale * noise1d(seed), element index = offset in the contiguous kernel
+    leaves, kernels = {}, {}
+    for name, c, seed_w, seed_b in (("c1", c1, 77, 78), ("c2", c2, 79, 80)):
+        for kind, rt, seed in (("weight", c.weight, seed_w), ("bias", c.bias, seed_b)):
+            n = rt.numel()
+            coef = torch.tensor(cpu(getattr(c, kind + "_coef")), dtype=torch.float64, requires_grad=True)
+            sb = torch.tensor(cpu(getattr(c, kind + "_scale_bias")), dtype=torch.float64, requires_grad=True)
+            noise = torch.tensor(oracle.noise_2d(n, 48, seed), dtype=torch.float64)
+            bias = torch.tensor(oracle.noise_1d(n, seed), dtype=torch.float64)
+            kernels[name, kind] = (noise @ coef + sb * bias).reshape(tuple(rt.shape))
+            leaves[name, kind] = (coef, sb)
+    xd = x.double().requires_grad_()
+    yd = F.conv2d(F.relu(F.conv2d(xd, kernels["c1", "weight"], kernels["c1", "bias"])), kernels["c2", "weight"], kernels["c2", "bias"],
+                  stride=2, padding=1)
+    yd.square().sum().backward()
+    assert rel_l2(cpu(y), yd.detach().numpy()) < 1e-5
+    assert rel_l2(cpu(xg.grad), xd.grad.numpy()) < 1e-4
+    for (name, kind), (coef, sb) in leaves.items():
+        c = c1 if name == "c1" else c2
+        assert rel_l2(cpu(getattr(c, kind + "_coef").grad), coef.grad.numpy()) < 1e-4, (name, kind)
+        assert rel_l2(cpu(getattr(c, kind + "_scale_bias").grad), sb.grad.numpy()) < 1e-4, (name, kind)
+
+
 def test_embedding_layer(ra, oracle):
     print("case embedding", flush=True)
     e = ra.SillyEmbedding(1000, 48, [32], [9], device="cuda")

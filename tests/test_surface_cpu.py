@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import randumb_amd as ra
-from randumb_amd import CreateRandumbTensor, RandumbTensor, SillyLinear, listgen, stepgen
+from randumb_amd import CreateRandumbTensor, RandumbTensor, SillyConv2d, SillyLinear, listgen, stepgen
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -151,6 +151,26 @@ def test_silly_linear_surface():
     assert l1.weight.scale_bias is l1.weight_scale_bias and l1.weight._coef is l1.weight_coef
     m = SillyLinear(12, 5, [8, 8], [1, 2], matrix_coef=True)
     assert m.weight_coef.shape == (5, 8) and m.fused and m.weight.coef_rows == 5
+
+
+def test_silly_conv2d_surface():
+    """Constructor, parameter and buffer names, shapes and default init of the convolution layer (SillyLayers.py:230-297)."""
+    ints, seeds = stepgen(64, 0), stepgen(1337, 1)
+    c1 = SillyConv2d(1, 32, int_dim=ints, seed=seeds, kernel_size=3, stride=1, rt_bias=True)
+    c2 = SillyConv2d(32, 64, int_dim=ints, seed=seeds, kernel_size=3, stride=1, rt_bias=True, bias=False)
+    assert c1.seed == [1337, 1338] and c2.seed == [1339, 1340] and c1.int_dim == [64, 64]
+    assert sorted(n for n, _ in c1.named_parameters()) == ["bias_coef", "bias_scale_bias", "weight_coef", "weight_scale_bias"]
+    assert sorted(n for n, _ in c1.named_buffers()) == ["bias", "weight"]
+    assert isinstance(c1.weight, RandumbTensor) and c1.weight.shape == (32, 1, 3, 3) and c1.weight.stride() == (9, 9, 3, 1)
+    assert c1.bias.shape == (32,) and c1.weight_coef.shape == (64,) and c1.weight.fused_bias
+    assert c2.bias is None and c2.weight.shape == (64, 32, 3, 3) and c2.weight.noise_matrix_shape == (64 * 32 * 9, 64)
+    # default init: zero coefficients, scale_bias = sqrt(3) * gain / sqrt(fan_in) with fan_in = in_channels * kh * kw
+    assert not c2.weight_coef.any()
+    want = math.sqrt(3.0) * math.sqrt(1.0 / 3.0) / math.sqrt(32 * 9)
+    assert abs(float(c2.weight_scale_bias) - want) < 1e-7
+    c2 = c2.to(torch.bfloat16)
+    assert c2.weight.dtype == torch.bfloat16 and c2.weight._coef is c2.weight_coef and c2.weight.shape == (64, 32, 3, 3)
+    assert "int_dim=[64, 64]" in repr(c2)
 
 
 def test_apply_rebuilds_tensors_on_the_converted_parameters():
