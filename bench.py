@@ -250,6 +250,17 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / iters
 
+    # spread of single steps, each between its own pair of events (as triton's do_bench reports: median, 20th, 80th percentile)
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    evs[0].record()
+    for i in range(args.steps):
+        step()
+        evs[i + 1].record()
+    torch.cuda.synchronize()
+    per_step = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(args.steps))
+    pct = lambda q: per_step[min(len(per_step) - 1, int(q * len(per_step)))]
+    step_spread = {"p20": round(pct(0.2), 5), "p50": round(pct(0.5), 5), "p80": round(pct(0.8), 5)}
+
     iters = max(10, min(args.steps, 50))
     calls = {
         "rdb_linear_project": event_ms(k_project, iters),
@@ -364,6 +375,7 @@ def main():
                    "executed_gflop_per_step": round(EXEC_STEP / 1e9, 3), "executed_tflops": round(EXEC_STEP / (ms_per_step * 1e-3) / 1e12, 3),
                    "algorithm": "factored: y=(x N^T) C^T, dx=(dy C) N, dC=dy^T (x N^T); z = x N^T computed once per step"},
         "frac_of_mfma_peak": round(value / MFMA_BF16_PEAK_TFLOPS, 5),
+        "ms_per_step_events": step_spread,
         "roofline": roofline, "cpu_baseline": cpu_baseline, "compare": compare, "other_configs": other,
     }
     print(json.dumps(out))
