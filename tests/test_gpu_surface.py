@@ -237,6 +237,44 @@ def test_conv2d_layers_match_a_dense_autograd_graph(ra, oracle):
         assert rel_l2(cpu(getattr(c, kind + "_scale_bias").grad), sb.grad.numpy()) < 1e-4, (name, kind)
 
 
+def test_mnist_conv_net_trains(ra):
+    """The reference's MNIST net (mnist/mnist.py:55-84: two pseudorandom convolutions, two pseudorandom linears) on a fixed
+    synthetic batch: every parameter gets a finite gradient and a few SGD steps lower the loss."""
+    print("case conv net", flush=True)
+    torch.manual_seed(0)
+    ints, seeds = ra.stepgen(64, 0), ra.stepgen(1337, 1)
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv1 = ra.SillyConv2d(1, 32, int_dim=ints, seed=seeds, kernel_size=3, stride=1, rt_bias=True)
+            self.conv2 = ra.SillyConv2d(32, 64, int_dim=ints, seed=seeds, kernel_size=3, stride=1, rt_bias=True)
+            self.fc1 = ra.SillyLinear(9216, 128, ints, seeds, bias=False, rt_bias=True)
+            self.fc2 = ra.SillyLinear(128, 10, ints, seeds, bias=False, rt_bias=True)
+
+        def forward(self, x):
+            x = F.max_pool2d(F.relu(self.conv2(F.relu(self.conv1(x)))), 2)
+            return F.log_softmax(self.fc2(F.relu(self.fc1(torch.flatten(x, 1)))), dim=1)
+
+    net = Net().cuda()
+    assert [l.seed for l in (net.conv1, net.conv2, net.fc1, net.fc2)] == [[1337, 1338], [1339, 1340], [1341, 1342], [1343, 1344]]
+    x, target = torch.rand(16, 1, 28, 28).cuda(), torch.randint(0, 10, (16,)).cuda()
+    # a coefficient moves every weight that shares it, so its gradient is large: steps of fixed length along the gradient
+    params, losses = list(net.parameters()), []
+    for _ in range(6):
+        net.zero_grad()
+        loss = F.nll_loss(net(x), target)
+        loss.backward()
+        for name, p in net.named_parameters():
+            assert p.grad is not None and torch.isfinite(p.grad).all(), name
+        norm = torch.sqrt(sum((p.grad.double() ** 2).sum() for p in params)).item()
+        with torch.no_grad():
+            for p in params:
+                p -= (0.02 / norm) * p.grad
+        losses.append(float(loss.detach()))
+    assert losses[-1] < losses[0], losses
+
+
 def test_embedding_layer(ra, oracle):
     print("case embedding", flush=True)
     e = ra.SillyEmbedding(1000, 48, [32], [9], device="cuda")
