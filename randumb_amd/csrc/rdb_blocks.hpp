@@ -77,13 +77,20 @@ __device__ __forceinline__ void red_block(const RedParams &p, int block, int nbl
 {
     const int64_t n4 = p.n / 4;
     for (int64_t e = (int64_t)block * blockDim.x + threadIdx.x; e < n4; e += (int64_t)nblocks * blockDim.x) {
-        f32x4 v = reinterpret_cast<const f32x4 *>(p.partial)[e];
-        for (int sidx = 1; sidx < p.splits; ++sidx) {
-            const f32x4 u = reinterpret_cast<const f32x4 *>(p.partial + (int64_t)sidx * p.n)[e];
-            v[0] += u[0];
-            v[1] += u[1];
-            v[2] += u[2];
-            v[3] += u[3];
+        const f32x4 *src = reinterpret_cast<const f32x4 *>(p.partial) + e;
+        f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+        // eight loads in flight at a time (a loop of single loads would wait out the memory latency once per split);
+        // the additions stay in split order
+        for (int s0 = 0; s0 < p.splits; s0 += 8) {
+            f32x4 u[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int sidx = s0 + j < p.splits ? s0 + j : p.splits - 1;   // clamped: loaded, not added
+                u[j] = src[(int64_t)sidx * n4];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (s0 + j < p.splits) v += u[j];
         }
         reinterpret_cast<f32x4 *>(p.out)[e] = v;
     }

@@ -271,8 +271,8 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
             const int items = make_tns_params(bs.tn, dx, lddx, workspace, d, num_cus);
             bs.red = red;
             bs.tn_blocks = xcd_grid_size(items);
-            int rblocks = (int)cdiv(red.n / 4, ST_THREADS * 8);
-            if (rblocks > num_cus / 4) rblocks = num_cus / 4;
+            int rblocks = (int)cdiv(red.n / 4 * red.splits, ST_THREADS * 16);   // about 16 loads of 16 bytes a thread
+            if (rblocks > num_cus / 2) rblocks = num_cus / 2;
             if (rblocks < 1) rblocks = 1;
             const int kg = (int)cdiv(d->k, 64);
             const size_t smem_s = stationary_smem(kg);
@@ -293,8 +293,8 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
         const int tn_items = make_tn_params(b.tn, dx, lddx, workspace, d);
         b.tn_blocks = xcd_grid_size(tn_items);
         b.red = red;
-        int red_blocks = (int)cdiv(b.red.n / 4, 256 * 8);
-        if (red_blocks > num_cus / 2) red_blocks = num_cus / 2;
+        int red_blocks = (int)cdiv(b.red.n / 4 * b.red.splits, 256 * 16);
+        if (red_blocks > num_cus) red_blocks = num_cus;
         if (red_blocks < 1) red_blocks = 1;
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_tn_red_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_tn);
         if (e != hipSuccess) return set_error((int)e, "bwd_tn_red_kernel: cannot reserve %zu bytes of LDS: %s", smem_tn, hipGetErrorString(e));
