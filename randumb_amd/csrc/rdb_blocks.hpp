@@ -18,7 +18,7 @@ struct DcParams {
     const bf16_t *z;
     float *dcoef;
     float *partial;  // NULL: the token splits add into dcoef (zeroed beforehand) with atomics; else split s stores its sums
-                     // into partial[s][out_f][k] and a reduction pass (red_block) writes dcoef
+                     // into partial[s][out_f][k] and a reduction pass (red_block) writes dcoef (a single split: partial = dcoef)
     int64_t lddy;
     int tokens, out_f, k;
     int tiles_o, tiles_m, splits, tok_per_split;

@@ -252,7 +252,9 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
     if (workspace_bytes >= linear_bwd_projected_workspace(d, num_cus)) {
         BwdAParams a;
         const int dc_items = make_dc_params(a.dc, dcoef, dy, lddy, z, d, num_cus);
-        a.dc.partial = reinterpret_cast<float *>(static_cast<char *>(workspace) + align256(linear_dx_factored_workspace(d)));
+        // one token range only: its sums are the result, stored straight into dcoef, and nothing is left to add up
+        const bool direct = a.dc.splits == 1;
+        a.dc.partial = direct ? dcoef : reinterpret_cast<float *>(static_cast<char *>(workspace) + align256(linear_dx_factored_workspace(d)));
         a.dyc = p1;
         a.dc_blocks = xcd_grid_size(dc_items);
         size_t smem = smem_dc > smem_dyc ? smem_dc : smem_dyc;
@@ -274,6 +276,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
             int rblocks = (int)cdiv(red.n / 4 * red.splits, ST_THREADS * 16);   // about 16 loads of 16 bytes a thread
             if (rblocks > num_cus / 2) rblocks = num_cus / 2;
             if (rblocks < 1) rblocks = 1;
+            if (direct) rblocks = 0;
             const int kg = (int)cdiv(d->k, 64);
             const size_t smem_s = stationary_smem(kg);
             const void *fn = kg == 1 ? (const void *)bwd_tns_red_kernel<1> : kg == 2 ? (const void *)bwd_tns_red_kernel<2>
@@ -296,6 +299,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
         int red_blocks = (int)cdiv(b.red.n / 4 * b.red.splits, 256 * 16);
         if (red_blocks > num_cus) red_blocks = num_cus;
         if (red_blocks < 1) red_blocks = 1;
+        if (direct) red_blocks = 0;
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_tn_red_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_tn);
         if (e != hipSuccess) return set_error((int)e, "bwd_tn_red_kernel: cannot reserve %zu bytes of LDS: %s", smem_tn, hipGetErrorString(e));
         bwd_tn_red_kernel<<<b.tn_blocks + red_blocks, 256, smem_tn, s>>>(b);
