@@ -30,6 +30,8 @@ struct DyCParams {
     int64_t lddy;
     int tokens, out_f, k;
     int tiles_c, tiles_t;
+    int frag_ksteps;  // 0: t row-major [tokens x k]; else t in fragment order with this many k-steps per 32 tokens and scaled
+                      // by 2^-31, for the kernel that keeps it in registers (rdb_stationary.hpp)
 };
 
 // `block`: index of this block among the blocks that run this body.
@@ -49,7 +51,11 @@ __device__ __forceinline__ void dyc_block(const DyCParams &p, bf16_t *lds, int b
     // "B": dy[tok][o], contraction index contiguous
     GlobalOperand<K1_BT, X_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
     gemm_mainloop<K1_BC, K1_BT, X_BK, 2, 2>(acc, lds, opc, opdy, 0, (p.out_f + X_BK - 1) / X_BK);
-    store_tile_bf16<K1_BC, K1_BT>(acc, lds, p.t, p.k, m0, p.k, tok0, p.tokens, 1.0f, nullptr);
+    if (p.frag_ksteps)
+        store_tile_bf16_frag<K1_BC, K1_BT>(acc, lds, p.t, p.frag_ksteps, m0, p.frag_ksteps * 16, tok0, (p.tokens + 31) / 32 * 32,
+                                           4.656612873077392578125e-10f);
+    else
+        store_tile_bf16<K1_BC, K1_BT>(acc, lds, p.t, p.k, m0, p.k, tok0, p.tokens, 1.0f, nullptr);
 }
 
 __global__ __launch_bounds__(256, 2) void dx_dyc_kernel(DyCParams p)
@@ -131,7 +137,7 @@ __global__ __launch_bounds__(256, 2) void bwd_tn_red_kernel(BwdBParams p)
 template <int KG> __global__ __launch_bounds__(ST_THREADS, 1) void dx_tns_kernel(StParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    stationary_block<KG, false, true>(p, smem_raw, blockIdx.x);
+    stationary_block<KG, false, true, true>(p, smem_raw, blockIdx.x);
 }
 
 struct BwdBsParams {
@@ -144,7 +150,7 @@ template <int KG> __global__ __launch_bounds__(ST_THREADS, 1) void bwd_tns_red_k
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     if ((int)blockIdx.x < p.tn_blocks)
-        stationary_block<KG, false, true>(p.tn, smem_raw, blockIdx.x);
+        stationary_block<KG, false, true, true>(p.tn, smem_raw, blockIdx.x);
     else
         red_block(p.red, blockIdx.x - p.tn_blocks, gridDim.x - p.tn_blocks);
 }
@@ -157,9 +163,11 @@ static bool dx_factored_ok(const rdb_linear_desc *d)
            d->k < (1 << 24) && d->tokens * d->k < (1ll << 29) && d->out_f * d->k < (1ll << 29);
 }
 
+// t = dy.C: [tokens x k] bf16, or, for the kernel that keeps t in registers, tokens padded to 32 and k to 64
 int64_t linear_dx_factored_workspace(const rdb_linear_desc *d)
 {
     if (!dx_factored_ok(d)) return 0;
+    if (d->k <= ST_KMAX) return cdiv(d->tokens, 32) * 32 * cdiv(d->k, 64) * 64 * (int64_t)sizeof(bf16_t);
     return d->tokens * d->k * (int64_t)sizeof(bf16_t);
 }
 
@@ -187,6 +195,7 @@ static void make_dyc_params(DyCParams &p1, const void *dy, int64_t lddy, const v
     p1.k = (int)d->k;
     p1.tiles_c = (int)cdiv(d->k, K1_BC);
     p1.tiles_t = (int)cdiv(d->tokens, K1_BT);
+    p1.frag_ksteps = 0;
 }
 
 // t . N with t in registers applies when k is short enough and dx fits a buffer descriptor.
@@ -217,17 +226,20 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
 
     DyCParams p1;
     make_dyc_params(p1, dy, lddy, coef, workspace, d);
+    const bool stationary = tn_stationary_ok(d, lddx);
+    const int kg = (int)cdiv(d->k, 64);
+    if (stationary) p1.frag_ksteps = kg * 4;
     int rc = launch_engine(dx_dyc_kernel, p1, p1.tiles_c * p1.tiles_t, engine_smem<K1_BC, K1_BT, X_BK, M_CONT, K_CONT>(), s, "dx_dyc_kernel");
     if (rc) return rc;
-    if (tn_stationary_ok(d, lddx)) {
+    if (stationary) {
         StParams q;
         const int items = make_tns_params(q, dx, lddx, workspace, d, num_cus);
-        const int kg = (int)cdiv(d->k, 64);
+        const size_t smem = stationary_smem(kg, true);
         switch (kg) {
-        case 1: return launch_stationary(dx_tns_kernel<1>, q, items, stationary_smem(kg), s, "dx_tns_kernel<1>");
-        case 2: return launch_stationary(dx_tns_kernel<2>, q, items, stationary_smem(kg), s, "dx_tns_kernel<2>");
-        case 3: return launch_stationary(dx_tns_kernel<3>, q, items, stationary_smem(kg), s, "dx_tns_kernel<3>");
-        default: return launch_stationary(dx_tns_kernel<4>, q, items, stationary_smem(kg), s, "dx_tns_kernel<4>");
+        case 1: return launch_stationary(dx_tns_kernel<1>, q, items, smem, s, "dx_tns_kernel<1>");
+        case 2: return launch_stationary(dx_tns_kernel<2>, q, items, smem, s, "dx_tns_kernel<2>");
+        case 3: return launch_stationary(dx_tns_kernel<3>, q, items, smem, s, "dx_tns_kernel<3>");
+        default: return launch_stationary(dx_tns_kernel<4>, q, items, smem, s, "dx_tns_kernel<4>");
         }
     }
     TNParams p2;
@@ -256,6 +268,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
         const bool direct = a.dc.splits == 1;
         a.dc.partial = direct ? dcoef : reinterpret_cast<float *>(static_cast<char *>(workspace) + align256(linear_dx_factored_workspace(d)));
         a.dyc = p1;
+        if (tn_stationary_ok(d, lddx)) a.dyc.frag_ksteps = (int)cdiv(d->k, 64) * 4;   // the t.N kernel below keeps t in registers
         a.dc_blocks = xcd_grid_size(dc_items);
         size_t smem = smem_dc > smem_dyc ? smem_dc : smem_dyc;
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dc_dyc_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -278,7 +291,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
             if (rblocks < 1) rblocks = 1;
             if (direct) rblocks = 0;
             const int kg = (int)cdiv(d->k, 64);
-            const size_t smem_s = stationary_smem(kg);
+            const size_t smem_s = stationary_smem(kg, true);
             const void *fn = kg == 1 ? (const void *)bwd_tns_red_kernel<1> : kg == 2 ? (const void *)bwd_tns_red_kernel<2>
                            : kg == 3 ? (const void *)bwd_tns_red_kernel<3> : (const void *)bwd_tns_red_kernel<4>;
             e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_s);

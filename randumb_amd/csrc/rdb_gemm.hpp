@@ -399,6 +399,43 @@ __device__ __forceinline__ void store_tile_bf16(const f32x16 (&acc)[BM / (32 * W
     __syncthreads();
 }
 
+// Accumulators -> bf16 in MFMA-fragment order, for a consumer that keeps this matrix in registers as the "b" operand
+// (rdb_stationary.hpp): 32 rows b by 16 columns a form one k-step of 1024 bytes, lane (b % 32, half) holding 8 columns:
+//   element (b, a) -> ((b / 32) * ksteps + a / 16) * 512 + ((a / 8) % 2 * 32 + b % 32) * 8 + a % 8.
+// Columns up to na and rows up to nb are written (pass them rounded up to the padding the consumer reads: the accumulators
+// there are zeros).  Needs a0 a multiple of 8 and b0 of 32; `out` 16-byte aligned.
+template <int BM, int BN, int WM = 2>
+__device__ __forceinline__ void store_tile_bf16_frag(const f32x16 (&acc)[BM / (32 * WM)][BN / (128 / WM)], bf16_t *__restrict__ lds,
+                                                     bf16_t *__restrict__ out, int ksteps, int a0, int na, int b0, int nb, float scale)
+{
+    constexpr int WN = 4 / WM, MI = BM / (32 * WM), NI = BN / (32 * WN), LDS_LD = BM + 8;
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave / WN, wn = wave % WN;
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int jq = 0; jq < 4; ++jq) {
+            const int a = wm * MI * 32 + mi * 32 + 8 * jq + 4 * g;
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) {
+                const int b = wn * NI * 32 + ni * 32 + r;
+                store4<bf16_t>(lds + b * LDS_LD + a, acc[mi][ni][jq * 4 + 0] * scale, acc[mi][ni][jq * 4 + 1] * scale,
+                               acc[mi][ni][jq * 4 + 2] * scale, acc[mi][ni][jq * 4 + 3] * scale);
+            }
+        }
+    __syncthreads();
+    constexpr int PIECES = BM * BN / 8;
+#pragma unroll
+    for (int p = 0; p < PIECES / 256; ++p) {
+        const int idx = p * 256 + t;
+        const int b = idx % BN, a = (idx / BN) * 8;   // neighbouring lanes: neighbouring rows of one 8-column piece, 16 bytes apart in `out`
+        const int gb = b0 + b, ga = a0 + a;
+        if (gb < nb && ga < na)
+            *reinterpret_cast<f32x4 *>(out + ((int64_t)(gb >> 5) * ksteps + (ga >> 4)) * 512 + (((ga >> 3) & 1) * 32 + (gb & 31)) * 8) =
+                *reinterpret_cast<const f32x4 *>(lds + b * LDS_LD + a);
+    }
+    __syncthreads();
+}
+
 // ----------------------------------------------------------------------------------------------- host side helpers
 // Dynamic LDS of an engine kernel: the two pipeline stages, or the bf16 output staging tile if that is larger.
 template <int BM, int BN, int BK, int LA, int LB> inline size_t engine_smem()

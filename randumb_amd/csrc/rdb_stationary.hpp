@@ -19,7 +19,8 @@ constexpr int ST_BT = 256, ST_BO = 64, ST_STG_LD = ST_BO + 8, ST_WAVES = 8, ST_T
 constexpr int ST_KMAX = 256;
 
 struct StParams {
-    const bf16_t *z;     // left operand [tokens x k], row-major
+    const bf16_t *z;     // left operand [tokens x k]: row-major, or (ZFRAG) in fragment order as store_tile_bf16_frag writes it,
+                         // tokens padded to 32 and k to KG * 64, the noise flavour's 2^-31 already applied
     const bf16_t *coef;  // right operand [out_f x k] (not used when the right operand is noise)
     const bf16_t *bias;  // [out_f] or NULL
     bf16_t *y;           // [tokens x out_f], leading dimension ldy
@@ -184,7 +185,8 @@ template <int KG, bool BIAS, bool NOISE> struct StBlock {
 };
 
 // `block`: index of this block among the blocks that run this body; all ST_THREADS threads of the block must call.
-template <int KG, bool BIAS, bool NOISE> __device__ __forceinline__ void stationary_block(const StParams &p, unsigned char *smem_raw, int block)
+template <int KG, bool BIAS, bool NOISE, bool ZFRAG = false>
+__device__ __forceinline__ void stationary_block(const StParams &p, unsigned char *smem_raw, int block)
 {
     typedef StBlock<KG, BIAS, NOISE> B;
     const int t = threadIdx.x, wave = t >> 6;
@@ -204,46 +206,61 @@ template <int KG, bool BIAS, bool NOISE> __device__ __forceinline__ void station
     b.rs_c = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.coef), 0, NOISE ? 0 : (int)((int64_t)p.out_f * p.k * 2), 0x00020000);
     b.rs_y = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, (int)(((int64_t)(p.tokens - 1) * p.ldy + p.out_f) * 2), 0x00020000);
     b.rs_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.bias), 0, p.bias ? p.out_f * 2 : 0, 0x00020000);  // no bias: zeros
-    const __amdgpu_buffer_rsrc_t rs_z =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.z), 0, (int)((int64_t)p.tokens * p.k * 2), 0x00020000);
     b.t = t;
-    if (!NOISE) b.issue(b.unit0);
-    // Left operand's fragments: operand "b" of the MFMA (rows = tokens); tokens past the end and coefficients past k read as
-    // zeros.  A lane's fragment pieces lie 16 bytes here, 16 bytes there; read straight from global memory that costs a cache
-    // line per lane and instruction, so the tile goes through LDS first: whole rows in, fragments out.
-    {
-        constexpr int ZQ = ST_BT * B::cpr / ST_THREADS;
-        bf16_t *zs = b.Cs;   // [256 tok][ldk]: larger than the two tile buffers and the patches, the launch reserves for it
-        const int btok0 = (w / p.splits) * ST_BT;
-        f32x4 zr[ZQ];
+    if (ZFRAG) {
+        // the fragments lie ready in memory, a k-step of a wave's 32 tokens in 1024 consecutive bytes: no staging, no barrier
+        const int64_t padded = (int64_t)((p.tokens + 31) / 32) * 32 * B::kpad;
+        const __amdgpu_buffer_rsrc_t rs_z = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.z), 0, (int)(padded * 2), 0x00020000);
+        if (!NOISE) b.issue(b.unit0);
+        const int tile = tok0 >> 5;
 #pragma unroll
-        for (int q = 0; q < ZQ; ++q) {
-            const int idx = q * ST_THREADS + t, row = idx / B::cpr, cm = (idx % B::cpr) * 8, tok = btok0 + row;
-            const uint32_t a = (tok < p.tokens && cm < p.k) ? (uint32_t)(((int64_t)tok * p.k + cm) * 2) : BUFFER_OOB;
-            zr[q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)a, 0, 0));
+        for (int ks = 0; ks < KG * 4; ++ks) {
+            const uint32_t a = tok0 < p.tokens ? (uint32_t)(((tile * (KG * 4) + ks) * 512 + b.lane * 8) * 2) : BUFFER_OOB;
+            b.zf[ks] = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)a, 0, 0));
         }
         if (NOISE) b.hash_piece_all(b.unit0);   // the first noise tile is hashed while the loads are in flight
-#pragma unroll
-        for (int q = 0; q < ZQ; ++q) {
-            const int idx = q * ST_THREADS + t;
-            f32x4 v = zr[q];
-            if (NOISE) {   // 2^-31 of the noise scale: a power of two, exact in bf16
-                Frag8 f;
-                f.f4 = v;
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    f.u[e] = f32x2_to_bf16x2(__uint_as_float(f.u[e] << 16) * 4.656612873077392578125e-10f,
-                                             __uint_as_float(f.u[e] & 0xffff0000u) * 4.656612873077392578125e-10f);
-                v = f.f4;
+        b.commit(b.Cs);                          // first tile of the right operand; the barrier at the top of step 0 publishes it
+    } else {
+        const __amdgpu_buffer_rsrc_t rs_z =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.z), 0, (int)((int64_t)p.tokens * p.k * 2), 0x00020000);
+        if (!NOISE) b.issue(b.unit0);
+        // Left operand's fragments: operand "b" of the MFMA (rows = tokens); tokens past the end and coefficients past k read as
+        // zeros.  A lane's fragment pieces lie 16 bytes here, 16 bytes there; read straight from global memory that costs a cache
+        // line per lane and instruction, so the tile goes through LDS first: whole rows in, fragments out.
+        {
+            constexpr int ZQ = ST_BT * B::cpr / ST_THREADS;
+            bf16_t *zs = b.Cs;   // [256 tok][ldk]: larger than the two tile buffers and the patches, the launch reserves for it
+            const int btok0 = (w / p.splits) * ST_BT;
+            f32x4 zr[ZQ];
+    #pragma unroll
+            for (int q = 0; q < ZQ; ++q) {
+                const int idx = q * ST_THREADS + t, row = idx / B::cpr, cm = (idx % B::cpr) * 8, tok = btok0 + row;
+                const uint32_t a = (tok < p.tokens && cm < p.k) ? (uint32_t)(((int64_t)tok * p.k + cm) * 2) : BUFFER_OOB;
+                zr[q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)a, 0, 0));
             }
-            *reinterpret_cast<f32x4 *>(zs + (idx / B::cpr) * B::ldk + (idx % B::cpr) * 8) = v;
+            if (NOISE) b.hash_piece_all(b.unit0);   // the first noise tile is hashed while the loads are in flight
+    #pragma unroll
+            for (int q = 0; q < ZQ; ++q) {
+                const int idx = q * ST_THREADS + t;
+                f32x4 v = zr[q];
+                if (NOISE) {   // 2^-31 of the noise scale: a power of two, exact in bf16
+                    Frag8 f;
+                    f.f4 = v;
+    #pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        f.u[e] = f32x2_to_bf16x2(__uint_as_float(f.u[e] << 16) * 4.656612873077392578125e-10f,
+                                                 __uint_as_float(f.u[e] & 0xffff0000u) * 4.656612873077392578125e-10f);
+                    v = f.f4;
+                }
+                *reinterpret_cast<f32x4 *>(zs + (idx / B::cpr) * B::ldk + (idx % B::cpr) * 8) = v;
+            }
+            __syncthreads();
+    #pragma unroll
+            for (int ks = 0; ks < KG * 4; ++ks)
+                b.zf[ks] = *reinterpret_cast<const bf16x8 *>(zs + (wave * ST_TW + b.r) * B::ldk + ks * 16 + b.g * 8);
+            __syncthreads();
+            b.commit(zs);   // first tile of the right operand; the barrier at the top of step 0 publishes it
         }
-        __syncthreads();
-#pragma unroll
-        for (int ks = 0; ks < KG * 4; ++ks)
-            b.zf[ks] = *reinterpret_cast<const bf16x8 *>(zs + (wave * ST_TW + b.r) * B::ldk + ks * 16 + b.g * 8);
-        __syncthreads();
-        b.commit(zs);   // first tile of the right operand; the barrier at the top of step 0 publishes it
     }
     b.tok_y = tok0 + (b.lane >> 3);
     b.off_y = (uint32_t)(((int64_t)b.tok_y * p.ldy + (b.lane & 7) * 8) * 2);  // only used when the token exists: below 2^30
@@ -266,11 +283,11 @@ template <int KG, bool BIAS, bool NOISE> __device__ __forceinline__ void station
 }
 
 // ----------------------------------------------------------------------------------------------- host side
-inline size_t stationary_smem(int kg)
+inline size_t stationary_smem(int kg, bool zfrag = false)
 {
     const size_t steady = ((size_t)2 * ST_BO * (kg * 64 + 8) + ST_BT * ST_STG_LD) * sizeof(bf16_t);  // two tiles + the waves' patches
     const size_t staging = (size_t)ST_BT * (kg * 64 + 8) * sizeof(bf16_t);                              // the left operand's tile, once
-    return steady > staging ? steady : staging;
+    return steady > staging || zfrag ? steady : staging;
 }
 
 // Grid of the stationary kernels for [tokens x out_f]: about one block per compute unit.  Returns the number of work items.
