@@ -34,7 +34,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 # counters read for a plain 256 MiB device copy (FETCH x2.000, WRITE x1.000): profiles/bench_c2_hbm_traffic.md
 HBM_TRAFFIC_BYTES = {
     "forward (factored_z_kernel + factored_ys_kernel)": 84.2e6,
-    "backward (bwd_dc_dyc_kernel + bwd_tns_red_kernel)": 143.3e6 + 35.9e6,
+    "backward (bwd_dc_dyc_kernel + bwd_tns_red_kernel)": 144.1e6 + 35.8e6,
 }
 T, IN_F, OUT_F, K, SEED = 8192, 768, 3072, 256, 0
 
