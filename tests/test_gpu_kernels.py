@@ -434,7 +434,8 @@ def test_factored_dx_needs_what_it_says(hip):
 
 
 def test_projected_path_random_shapes(hip, oracle):
-    """Twenty random layer shapes (multiples of 8, ragged against every tile size) through the projected entry points."""
+    """Twenty random layer shapes (multiples of 8, ragged against every tile size) through the projected entry points, with
+    and without bias, with the workspace for ordered sums and with the smaller one."""
     rng = np.random.default_rng(2024)
     for case in range(20):
         T = int(rng.integers(1, 90)) * 8 - int(rng.integers(0, 8))          # tokens need not be a multiple of anything
@@ -444,10 +445,12 @@ def test_projected_path_random_shapes(hip, oracle):
         x, dy, coef = _inputs(T, in_f, out_f, k, True, torch.bfloat16, case)
         xn, dyn, cn = x.float().numpy(), dy.float().numpy(), coef.float().numpy()
         xg, dyg, cg = x.cuda(), dy.cuda(), coef.cuda()
+        bias = torch.randn(out_f).bfloat16() if case % 2 == 0 else None
         z = hip.linear_project(xg, k, out_f, seed)
-        y = hip.linear_fwd_projected(z, cg, in_f, seed)
-        dx, dc = hip.linear_bwd_projected(dyg, z, cg, in_f, seed)
+        y = hip.linear_fwd_projected(z, cg, in_f, seed, bias=None if bias is None else bias.cuda())
+        dx, dc = hip.linear_bwd_projected(dyg, z, cg, in_f, seed, ordered_sums=case % 3 != 0)
         want_dx, want_dc, _ = oracle.linear_bwd(xn, dyn, cn, in_f, out_f, seed)
-        assert rel_l2(cpu(y), oracle.linear_fwd(xn, cn, in_f, out_f, seed)) < BF16_TOL, case
+        want_y = oracle.linear_fwd(xn, cn, in_f, out_f, seed, bias=None if bias is None else bias.float().numpy())
+        assert rel_l2(cpu(y), want_y) < BF16_TOL, case
         assert rel_l2(cpu(dx), want_dx) < BF16_TOL, case
         assert rel_l2(cpu(dc), want_dc) < BF16_TOL, case
