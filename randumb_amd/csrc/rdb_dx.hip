@@ -234,7 +234,7 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
     if (stationary) {
         StParams q;
         const int items = make_tns_params(q, dx, lddx, workspace, d, num_cus);
-        const size_t smem = stationary_smem(kg, true);
+        const size_t smem = stationary_smem(kg);
         switch (kg) {
         case 1: return launch_stationary(dx_tns_kernel<1>, q, items, smem, s, "dx_tns_kernel<1>");
         case 2: return launch_stationary(dx_tns_kernel<2>, q, items, smem, s, "dx_tns_kernel<2>");
@@ -291,7 +291,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
             if (rblocks < 1) rblocks = 1;
             if (direct) rblocks = 0;
             const int kg = (int)cdiv(d->k, 64);
-            const size_t smem_s = stationary_smem(kg, true);
+            const size_t smem_s = stationary_smem(kg);
             const void *fn = kg == 1 ? (const void *)bwd_tns_red_kernel<1> : kg == 2 ? (const void *)bwd_tns_red_kernel<2>
                            : kg == 3 ? (const void *)bwd_tns_red_kernel<3> : (const void *)bwd_tns_red_kernel<4>;
             e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_s);

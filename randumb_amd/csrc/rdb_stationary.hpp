@@ -225,41 +225,48 @@ __device__ __forceinline__ void stationary_block(const StParams &p, unsigned cha
             __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.z), 0, (int)((int64_t)p.tokens * p.k * 2), 0x00020000);
         if (!NOISE) b.issue(b.unit0);
         // Left operand's fragments: operand "b" of the MFMA (rows = tokens); tokens past the end and coefficients past k read as
-        // zeros.  A lane's fragment pieces lie 16 bytes here, 16 bytes there; read straight from global memory that costs a cache
-        // line per lane and instruction, so the tile goes through LDS first: whole rows in, fragments out.
+        // zeros.  A lane's fragment pieces lie 16 bytes here, 16 bytes there; read straight from global memory that costs a
+        // cache line per lane and instruction, so a wave passes its 32 tokens through a patch of LDS of its own: whole rows in,
+        // fragments out, half of the coefficients at a time, with no block-wide barrier.  The patches lie in the second tile
+        // buffer and the epilogue patches, which nobody writes before the barrier of step 0.
         {
-            constexpr int ZQ = ST_BT * B::cpr / ST_THREADS;
-            bf16_t *zs = b.Cs;   // [256 tok][ldk]: larger than the two tile buffers and the patches, the launch reserves for it
-            const int btok0 = (w / p.splits) * ST_BT;
-            f32x4 zr[ZQ];
-    #pragma unroll
-            for (int q = 0; q < ZQ; ++q) {
-                const int idx = q * ST_THREADS + t, row = idx / B::cpr, cm = (idx % B::cpr) * 8, tok = btok0 + row;
-                const uint32_t a = (tok < p.tokens && cm < p.k) ? (uint32_t)(((int64_t)tok * p.k + cm) * 2) : BUFFER_OOB;
-                zr[q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)a, 0, 0));
-            }
-            if (NOISE) b.hash_piece_all(b.unit0);   // the first noise tile is hashed while the loads are in flight
-    #pragma unroll
-            for (int q = 0; q < ZQ; ++q) {
-                const int idx = q * ST_THREADS + t;
-                f32x4 v = zr[q];
-                if (NOISE) {   // 2^-31 of the noise scale: a power of two, exact in bf16
-                    Frag8 f;
-                    f.f4 = v;
-    #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        f.u[e] = f32x2_to_bf16x2(__uint_as_float(f.u[e] << 16) * 4.656612873077392578125e-10f,
-                                                 __uint_as_float(f.u[e] & 0xffff0000u) * 4.656612873077392578125e-10f);
-                    v = f.f4;
+            constexpr int HK = B::kpad / 2, HLD = HK + 8, HQ = 32 * (HK / 8) / 64;   // half a row: HK coefficients; pieces per lane
+            static_assert(ST_WAVES * 32 * HLD <= ST_BO * B::ldk + ST_BT * ST_STG_LD, "the waves' patches fit beside the first tile buffer");
+            bf16_t *zs = b.Cs + ST_BO * B::ldk + wave * 32 * HLD;
+            f32x4 zr[2][HQ];
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int q = 0; q < HQ; ++q) {
+                    const int idx = q * 64 + b.lane, row = idx / (HK / 8), cm = h * HK + (idx % (HK / 8)) * 8, tok = tok0 + row;
+                    const uint32_t a = (tok < p.tokens && cm < p.k) ? (uint32_t)(((int64_t)tok * p.k + cm) * 2) : BUFFER_OOB;
+                    zr[h][q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)a, 0, 0));
                 }
-                *reinterpret_cast<f32x4 *>(zs + (idx / B::cpr) * B::ldk + (idx % B::cpr) * 8) = v;
+            if (NOISE) b.hash_piece_all(b.unit0);   // the first noise tile is hashed while the loads are in flight
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                for (int q = 0; q < HQ; ++q) {
+                    const int idx = q * 64 + b.lane;
+                    f32x4 v = zr[h][q];
+                    if (NOISE) {   // 2^-31 of the noise scale: a power of two, exact in bf16
+                        Frag8 f;
+                        f.f4 = v;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            f.u[e] = f32x2_to_bf16x2(__uint_as_float(f.u[e] << 16) * 4.656612873077392578125e-10f,
+                                                     __uint_as_float(f.u[e] & 0xffff0000u) * 4.656612873077392578125e-10f);
+                        v = f.f4;
+                    }
+                    *reinterpret_cast<f32x4 *>(zs + (idx / (HK / 8)) * HLD + (idx % (HK / 8)) * 8) = v;
+                }
+                __builtin_amdgcn_wave_barrier();   // LDS serves a wave's instructions in order: the reads below see these writes
+#pragma unroll
+                for (int ks = 0; ks < KG * 2; ++ks)
+                    b.zf[h * KG * 2 + ks] = *reinterpret_cast<const bf16x8 *>(zs + b.r * HLD + ks * 16 + b.g * 8);
+                __builtin_amdgcn_wave_barrier();
             }
-            __syncthreads();
-    #pragma unroll
-            for (int ks = 0; ks < KG * 4; ++ks)
-                b.zf[ks] = *reinterpret_cast<const bf16x8 *>(zs + (wave * ST_TW + b.r) * B::ldk + ks * 16 + b.g * 8);
-            __syncthreads();
-            b.commit(zs);   // first tile of the right operand; the barrier at the top of step 0 publishes it
+            b.commit(b.Cs);   // first tile of the right operand; the barrier at the top of step 0 publishes it
         }
     }
     b.tok_y = tok0 + (b.lane >> 3);
@@ -283,11 +290,9 @@ __device__ __forceinline__ void stationary_block(const StParams &p, unsigned cha
 }
 
 // ----------------------------------------------------------------------------------------------- host side
-inline size_t stationary_smem(int kg, bool zfrag = false)
+inline size_t stationary_smem(int kg)
 {
-    const size_t steady = ((size_t)2 * ST_BO * (kg * 64 + 8) + ST_BT * ST_STG_LD) * sizeof(bf16_t);  // two tiles + the waves' patches
-    const size_t staging = (size_t)ST_BT * (kg * 64 + 8) * sizeof(bf16_t);                              // the left operand's tile, once
-    return steady > staging || zfrag ? steady : staging;
+    return ((size_t)2 * ST_BO * (kg * 64 + 8) + ST_BT * ST_STG_LD) * sizeof(bf16_t);  // two tiles + the waves' patches
 }
 
 // Grid of the stationary kernels for [tokens x out_f]: about one block per compute unit.  Returns the number of work items.
