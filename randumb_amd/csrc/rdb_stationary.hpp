@@ -31,7 +31,8 @@ struct StParams {
 };
 
 // KG: k rounded up to groups of 64 (compile time: the k loop is one straight line of code).  NOISE: the right operand's
-// rows are 2^31 * noise(PRIME*row + m), hashed into the tile, and the left operand is scaled by 2^-31 once (exact in bf16).
+// rows are 2^31 * noise(PRIME*row + m), hashed into the tile; the producer of the left operand has scaled it by 2^-31
+// (exact in bf16).
 template <int KG, bool BIAS, bool NOISE> struct StBlock {
     static constexpr int kpad = KG * 64, ldk = kpad + 8, cpr = kpad / 8, ncp = ST_BO * cpr, NQ = ncp / ST_THREADS;
     const StParams &p;
@@ -207,7 +208,7 @@ __device__ __forceinline__ void stationary_block(const StParams &p, unsigned cha
     b.rs_y = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, (int)(((int64_t)(p.tokens - 1) * p.ldy + p.out_f) * 2), 0x00020000);
     b.rs_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.bias), 0, p.bias ? p.out_f * 2 : 0, 0x00020000);  // no bias: zeros
     b.t = t;
-    if (ZFRAG) {
+    if constexpr (ZFRAG) {
         // the fragments lie ready in memory, a k-step of a wave's 32 tokens in 1024 consecutive bytes: no staging, no barrier
         const int64_t padded = (int64_t)((p.tokens + 31) / 32) * 32 * B::kpad;
         const __amdgpu_buffer_rsrc_t rs_z = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.z), 0, (int)(padded * 2), 0x00020000);
@@ -221,9 +222,10 @@ __device__ __forceinline__ void stationary_block(const StParams &p, unsigned cha
         if (NOISE) b.hash_piece_all(b.unit0);   // the first noise tile is hashed while the loads are in flight
         b.commit(b.Cs);                          // first tile of the right operand; the barrier at the top of step 0 publishes it
     } else {
+        static_assert(!NOISE, "the noise flavour takes its left operand in fragment order");
         const __amdgpu_buffer_rsrc_t rs_z =
             __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.z), 0, (int)((int64_t)p.tokens * p.k * 2), 0x00020000);
-        if (!NOISE) b.issue(b.unit0);
+        b.issue(b.unit0);
         // Left operand's fragments: operand "b" of the MFMA (rows = tokens); tokens past the end and coefficients past k read as
         // zeros.  A lane's fragment pieces lie 16 bytes here, 16 bytes there; read straight from global memory that costs a
         // cache line per lane and instruction, so a wave passes its 32 tokens through a patch of LDS of its own: whole rows in,
@@ -242,22 +244,12 @@ __device__ __forceinline__ void stationary_block(const StParams &p, unsigned cha
                     const uint32_t a = (tok < p.tokens && cm < p.k) ? (uint32_t)(((int64_t)tok * p.k + cm) * 2) : BUFFER_OOB;
                     zr[h][q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)a, 0, 0));
                 }
-            if (NOISE) b.hash_piece_all(b.unit0);   // the first noise tile is hashed while the loads are in flight
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
 #pragma unroll
                 for (int q = 0; q < HQ; ++q) {
                     const int idx = q * 64 + b.lane;
-                    f32x4 v = zr[h][q];
-                    if (NOISE) {   // 2^-31 of the noise scale: a power of two, exact in bf16
-                        Frag8 f;
-                        f.f4 = v;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            f.u[e] = f32x2_to_bf16x2(__uint_as_float(f.u[e] << 16) * 4.656612873077392578125e-10f,
-                                                     __uint_as_float(f.u[e] & 0xffff0000u) * 4.656612873077392578125e-10f);
-                        v = f.f4;
-                    }
+                    const f32x4 v = zr[h][q];
                     *reinterpret_cast<f32x4 *>(zs + (idx / (HK / 8)) * HLD + (idx % (HK / 8)) * 8) = v;
                 }
                 __builtin_amdgcn_wave_barrier();   // LDS serves a wave's instructions in order: the reads below see these writes
