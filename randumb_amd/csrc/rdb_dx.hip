@@ -167,7 +167,8 @@ static bool dx_factored_ok(const rdb_linear_desc *d)
 int64_t linear_dx_factored_workspace(const rdb_linear_desc *d)
 {
     if (!dx_factored_ok(d)) return 0;
-    if (d->k <= ST_KMAX) return cdiv(d->tokens, 32) * 32 * cdiv(d->k, 64) * 64 * (int64_t)sizeof(bf16_t);
+    if (d->k <= ST_KMAX && cdiv(d->tokens, 32) * 32 * cdiv(d->k, 64) * 64 < (1ll << 29))
+        return cdiv(d->tokens, 32) * 32 * cdiv(d->k, 64) * 64 * (int64_t)sizeof(bf16_t);
     return d->tokens * d->k * (int64_t)sizeof(bf16_t);
 }
 
@@ -199,7 +200,10 @@ static void make_dyc_params(DyCParams &p1, const void *dy, int64_t lddy, const v
 }
 
 // t . N with t in registers applies when k is short enough and dx fits a buffer descriptor.
-static bool tn_stationary_ok(const rdb_linear_desc *d, int64_t lddx) { return d->k <= ST_KMAX && d->tokens * lddx < (1ll << 29); }
+static bool tn_stationary_ok(const rdb_linear_desc *d, int64_t lddx)
+{   // dx and the padded, fragment-ordered t must each fit a buffer descriptor
+    return d->k <= ST_KMAX && d->tokens * lddx < (1ll << 29) && cdiv(d->tokens, 32) * 32 * cdiv(d->k, 64) * 64 < (1ll << 29);
+}
 
 static int make_tns_params(StParams &q, void *dx, int64_t lddx, const void *t, const rdb_linear_desc *d, int num_cus)
 {

@@ -69,6 +69,10 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     # whole backward pass: dy.C plus the partial sums of the coefficient gradient, one [out x k] fp32 matrix per token split
     extra = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_PROJECTED, r) - zbytes
     assert extra > 0 and extra % (3072 * 256 * 4) == 0
+    # dy.C is kept padded (tokens to 32, k to 64) for the kernel that holds it in registers, unless that would pass the
+    # operand size limit: then it stays [tokens x k]
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(desc(1000, 200, 328, 72))) == 1024 * 128 * 2
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(desc((1 << 26) - 8, 768, 3072, 8))) == ((1 << 26) - 8) * 8 * 2
     # kernels that form W tiles need no scratch; neither does a layer the factored form does not apply to
     for algo in (_lib.RDB_ALGO_TILE, _lib.RDB_ALGO_STRIP):
         assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(8192, 768, 3072, 256, algo=algo))) == 0
