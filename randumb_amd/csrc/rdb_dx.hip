@@ -180,6 +180,7 @@ int64_t linear_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus)
     if (!dx_factored_ok(d)) return 0;
     DcParams dc;
     make_dc_params(dc, nullptr, nullptr, d->out_f, nullptr, d, num_cus);
+    if (dc.splits == 1) return linear_dx_factored_workspace(d);   // a single token range is stored straight into dcoef
     return align256(linear_dx_factored_workspace(d)) + (int64_t)dc.splits * d->out_f * d->k * (int64_t)sizeof(float);
 }
 
