@@ -62,6 +62,7 @@ __device__ __forceinline__ void dc_block(const DcParams &p, bf16_t *lds, int blo
                 }
             }
     }
+    RDB_STAMP(3);
 }
 
 // ----------------------------------------------------------------------------------------------- dC = sum of the splits' partial sums
@@ -76,6 +77,7 @@ struct RedParams {
 __device__ __forceinline__ void red_block(const RedParams &p, int block, int nblocks)
 {
     const int64_t n4 = p.n / 4;
+    RDB_STAMP(0);
     for (int64_t e = (int64_t)block * blockDim.x + threadIdx.x; e < n4; e += (int64_t)nblocks * blockDim.x) {
         const f32x4 *src = reinterpret_cast<const f32x4 *>(p.partial) + e;
         f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -94,6 +96,7 @@ __device__ __forceinline__ void red_block(const RedParams &p, int block, int nbl
         }
         reinterpret_cast<f32x4 *>(p.out)[e] = v;
     }
+    RDB_STAMP(3);
 }
 
 // ----------------------------------------------------------------------------------------------- kernel 2: dx = t . N
@@ -128,6 +131,7 @@ __device__ __forceinline__ void tn_block(const TNParams &p, bf16_t *lds, int blo
     GlobalOperand<K2_BT, B_BK, K_CONT> opt = {p.t, (int64_t)p.k, tok0, p.tokens, p.k, (int64_t)p.tokens * p.k};
     gemm_mainloop<K2_BI, K2_BT, B_BK, 1, 1, K2_WM>(acc, lds, opn, opt, 0, (p.k + B_BK - 1) / B_BK);
     store_tile_bf16<K2_BI, K2_BT, K2_WM>(acc, lds, p.dx, p.lddx, i0, p.in_f, tok0, p.tokens, 4.656612873077392578125e-10f, nullptr);
+    RDB_STAMP(3);
 }
 
 // ----------------------------------------------------------------------------------------------- host side

@@ -94,4 +94,21 @@ __device__ __forceinline__ float load_as_f32(const void *p, int dtype, int64_t i
 
 inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// ----------------------------------------------------------------------------------------------- timeline stamps
+// RDB_STAMP(slot) records when thread 0 of a block passes a point of a kernel.  Compiled out of the library; a timing
+// harness defines RDB_STAMPS, a __device__ pointer rdb_stamp_buf and a __device__ int rdb_stamp_threads (0, or the block size
+// of the one kernel to record when a call launches several) before including the kernel sources and then finds, per block,
+// 16 slots of two counters: the constant-rate wall clock (comparable across compute units) and the shader clock.
+#ifdef RDB_STAMPS
+#define RDB_STAMP(slot)                                                                                                  \
+    do {                                                                                                                 \
+        if (threadIdx.x == 0 && rdb_stamp_buf && (rdb_stamp_threads == 0 || rdb_stamp_threads == (int)blockDim.x)) {                                                                         \
+            rdb_stamp_buf[((size_t)blockIdx.x * 16 + (slot)) * 2] = wall_clock64();                                      \
+            rdb_stamp_buf[((size_t)blockIdx.x * 16 + (slot)) * 2 + 1] = clock64();                                       \
+        }                                                                                                                \
+    } while (0)
+#else
+#define RDB_STAMP(slot) ((void)0)
+#endif
+
 }  // namespace rdb

@@ -56,6 +56,7 @@ __device__ __forceinline__ void dyc_block(const DyCParams &p, bf16_t *lds, int b
                                            4.656612873077392578125e-10f);
     else
         store_tile_bf16<K1_BC, K1_BT>(acc, lds, p.t, p.k, m0, p.k, tok0, p.tokens, 1.0f, nullptr);
+    RDB_STAMP(3);
 }
 
 __global__ __launch_bounds__(256, 2) void dx_dyc_kernel(DyCParams p)

@@ -52,6 +52,7 @@ __global__ __launch_bounds__(256, 2) void factored_z_kernel(ZParams p)
     GlobalOperand<KZ_BT, F_BK, K_CONT> opx = {p.x, p.ldx, tok0, p.tokens, p.in_f, (int64_t)(p.tokens - 1) * p.ldx + p.in_f};
     gemm_mainloop<KZ_BM, KZ_BT, F_BK, 1, 1, KZ_WM>(acc, lds, opn, opx, 0, (p.in_f + F_BK - 1) / F_BK);
     store_tile_bf16<KZ_BM, KZ_BT, KZ_WM>(acc, lds, p.z, p.k, m0, p.k, tok0, p.tokens, INV_2_31, nullptr);
+    RDB_STAMP(3);
 }
 
 // ----------------------------------------------------------------------------------------------- y = z . C^T

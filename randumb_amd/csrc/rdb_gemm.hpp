@@ -318,6 +318,7 @@ __device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / (32 * WM)][BN /
     constexpr int TRIP = (DA == 4 || DB == 4) ? 4 : 2;
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, wm = wave / WN, wn = wave % WN;
     if (nstage <= 0) return;
+    RDB_STAMP(0);
     pa.init(k_begin);
     pb.init(k_begin);
 
@@ -335,6 +336,7 @@ __device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / (32 * WM)][BN /
         TB::store(lds + TA::LDS_ELEMS, rb0);
     }
     __syncthreads();
+    RDB_STAMP(1);
 
     const int nround = (nstage + TRIP - 1) / TRIP * TRIP;
     int s = 0;
@@ -357,6 +359,7 @@ __device__ __forceinline__ void gemm_mainloop(f32x16 (&acc)[BM / (32 * WM)][BN /
         else
             pipeline_stage<BK, MI, NI, false, false>(acc, cur, oth, ra[(u + 1) % DA], rb[(u + 1) % DB], pa, pb, 0, 0, wm, wn, lane);
     }
+    RDB_STAMP(2);
 }
 
 // Writes the block's BM x BN accumulator tile D[a][b] as bf16 to out[(b0 + b) * ld + a0 + a] (rows of `out` run along a),

@@ -204,6 +204,7 @@ __device__ __forceinline__ void stationary_block(const StParams &p, unsigned cha
     b.unit0 = (w % p.splits) * p.units_per_split;
     b.nunits = min(p.units_per_split, (p.out_f + ST_BO - 1) / ST_BO - b.unit0);
     if (b.nunits <= 0) return;
+    RDB_STAMP(0);
     b.rs_c = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.coef), 0, NOISE ? 0 : (int)((int64_t)p.out_f * p.k * 2), 0x00020000);
     b.rs_y = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, (int)(((int64_t)(p.tokens - 1) * p.ldy + p.out_f) * 2), 0x00020000);
     b.rs_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.bias), 0, p.bias ? p.out_f * 2 : 0, 0x00020000);  // no bias: zeros
@@ -267,7 +268,9 @@ __device__ __forceinline__ void stationary_block(const StParams &p, unsigned cha
     // step s: MFMAs of unit s (while there is one) and the epilogue of unit s - 1; even steps accumulate in A, odd ones in B
     f32x16 accA[2], accB[2];
     const int n = b.nunits;
+    RDB_STAMP(1);
     b.template step<true, false>(accA, accB, 0);
+    RDB_STAMP(2);
     int s = 1;
     for (; s + 1 < n; s += 2) {
         b.template step<true, true>(accB, accA, s);
@@ -279,6 +282,7 @@ __device__ __forceinline__ void stationary_block(const StParams &p, unsigned cha
     } else {       // s == n, odd
         b.template step<false, true>(accB, accA, s);
     }
+    RDB_STAMP(3);
 }
 
 // ----------------------------------------------------------------------------------------------- host side
