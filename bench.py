@@ -92,7 +92,7 @@ def other_configs(event_ms):
     C = (torch.randn(out_f, k, generator=g) / 64.0 * (3.0 / k) ** 0.5).bfloat16().cuda()
 
     def step():
-        z = hip.linear_project(x, k, out_f, 0)
+        z = hip.linear_project(x, k, out_f, 0, coef=C)
         hip.linear_fwd_projected(z, C, in_f, 0)
         hip.linear_bwd_projected(dy, z, C, in_f, 0)
 
@@ -172,12 +172,12 @@ def main():
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
     pws = vp(ws.data_ptr())
     z_bytes = L.rdb_linear_projection_bytes(dref)
-    assert z_bytes == T * K * 2, "the projected form must apply to the headline workload"
-    z = torch.empty(T, K, dtype=torch.bfloat16, device=dev)
+    assert z_bytes > 0, "the projected form must apply to the headline workload"
+    z = torch.empty(z_bytes, dtype=torch.uint8, device=dev)   # the projection state: z in two orders and C transposed
     pz = vp(z.data_ptr())
 
     def k_project():
-        _lib.check(L.rdb_linear_project(pz, px, IN_F, dref, stream), "rdb_linear_project")
+        _lib.check(L.rdb_linear_project(pz, px, IN_F, pC, dref, stream), "rdb_linear_project")
 
     def k_fwd_projected():
         _lib.check(L.rdb_linear_fwd_projected(py, OUT_F, pz, pC, None, dref, stream), "rdb_linear_fwd_projected")

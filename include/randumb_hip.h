@@ -179,29 +179,51 @@ int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const void *dy, int6
  * noise directions of this layer's weight) is all that the forward product and the coefficient gradient need of x:
  *   y = z . C^T (+ bias)        dcoef = dy^T . z
  * rdb_linear_fwd and rdb_linear_bwd_dcoef compute z into their workspace on every call.  A training step can instead
- * compute it once, keep it from the forward to the backward pass in place of x (it is k/in_f of the size of x) and
- * call the two consumers below.  Replaces, like rdb_linear_fwd / rdb_linear_bwd_dcoef, materialize() + dense product
- * (R.py:942-952) and MmBackward's dW followed by materialize_bwd (R.py:979-990, 304-359); the tensor autograd saves
- * for the backward pass (there: x, with W re-materialised) becomes z.
- * Needs: coef_rows == out_f, act_dtype RDB_BF16, tokens/in_f/out_f/k > 0, in_f, out_f, k multiples of 8,
- * tokens*k < 2^29, 16-byte aligned pointers, leading dimensions multiples of 8; otherwise RDB_E_UNSUPPORTED. */
+ * compute it once, keep it from the forward to the backward pass in place of x and call the consumers below.  Replaces,
+ * like rdb_linear_fwd / rdb_linear_bwd_dcoef, materialize() + dense product (R.py:942-952) and MmBackward's dW followed by
+ * materialize_bwd (R.py:979-990, 304-359); the tensor autograd saves for the backward pass (there: x, with W
+ * re-materialised) becomes the projection state.
+ *
+ * The projection STATE is an opaque caller-owned device buffer of rdb_linear_projection_bytes(desc) bytes, 16-byte aligned,
+ * written by rdb_linear_project and read by the other three.  It holds z in the element orders its consumers' matrix
+ * instructions take their operands in (z for the forward product, z transposed for the coefficient gradient; about
+ * 2 * tokens * k * 2 bytes with k rounded up to 64) and, if rdb_linear_project was given the coefficients, C transposed for
+ * the input gradient (out_f * k * 2 bytes): the kernels then fetch these small operands straight into registers and only
+ * the large operand (dy) is staged through on-chip memory.  Needs: coef_rows == out_f, act_dtype RDB_BF16,
+ * tokens/in_f/out_f/k > 0, in_f, out_f, k multiples of 8, tokens*k and out_f*k (k rounded up to 64, tokens and out_f to
+ * 64) below 2^29, 16-byte aligned pointers, leading dimensions multiples of 8; otherwise RDB_E_UNSUPPORTED. */
 
-/* Bytes of z for `desc` (tokens*k*2), or 0 when the projected form does not apply to it. */
+/* Bytes of the projection state for `desc`, or 0 when the projected form does not apply to it. */
 int64_t rdb_linear_projection_bytes(const rdb_linear_desc *desc);
 
-/* z[t, m] = sum_i x[t, i] * noise(PRIME*i + m), rounded to bf16 once. */
-int rdb_linear_project(void *z, const void *x, int64_t ldx, const rdb_linear_desc *desc, void *stream);
+/* Where the pieces lie inside the state, for tools and tests that want to look at z (no reference counterpart: the
+ * reference keeps x).  Returns 0 and fills info[0..7], or RDB_E_UNSUPPORTED:
+ *   info[0] byte offset of z for the forward product    info[1] 1: fragment order, rows = tokens; 0: row-major [tokens x k]
+ *   info[2] byte offset of z transposed (fragment order, rows = coefficients)
+ *   info[3] byte offset of C transposed (fragment order, rows = coefficients); valid when the state's first 32-bit word is 1
+ *   info[4] k rounded up to 64   info[5] tokens rounded up to 32   info[6] tokens rounded up to 64   info[7] out_f rounded up to 64
+ * Fragment order of a matrix M[row][kk] with `ksteps` = (padded kk extent) / 16 k-steps per block of 32 rows:
+ *   element (row, kk) at ((row/32)*ksteps + kk/16)*512 + ((kk/8)%2*32 + row%32)*8 + kk%8   (in elements). */
+int rdb_linear_projection_layout(const rdb_linear_desc *desc, int64_t *info);
+
+/* state <- z[t, m] = sum_i x[t, i] * noise(PRIME*i + m), rounded to bf16 once.  coef: NULL, or the layer's bf16
+ * coefficients [out_f x k], whose transposed copy then goes into the state for rdb_linear_bwd_projected; the values the
+ * backward pass is later given as `coef` must be the same (as they are between the forward and the backward pass of one
+ * training step).  A state written with coef == NULL serves every consumer too (rdb_linear_bwd_projected then reads the
+ * coefficients through on-chip memory). */
+int rdb_linear_project(void *state, const void *x, int64_t ldx, const void *coef, const rdb_linear_desc *desc,
+                       void *stream);
 
 /* y[t, o] = sum_m z[t, m] * coef[o, m] (+ bias[o]); coef must be bf16. */
-int rdb_linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, const void *bias,
+int rdb_linear_fwd_projected(void *y, int64_t ldy, const void *state, const void *coef, const void *bias,
                              const rdb_linear_desc *desc, void *stream);
 
 /* dcoef[o, m] = sum_t dy[t, o] * z[t, m]; fp32 [out_f x k], OVERWRITTEN; partial sums over token ranges are combined
  * with fp32 atomics. */
-int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *z,
+int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *state,
                                    const rdb_linear_desc *desc, void *stream);
 
-/* Whole backward pass of the layer from the saved projection, in two kernel launches instead of five:
+/* Whole backward pass of the layer from the projection state, in two kernel launches instead of five:
  * dx[t, i] = sum_o dy[t, o] * W[o, i] (act dtype) and dcoef = dy^T . z (fp32, OVERWRITTEN).
  * workspace: rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_PROJECTED, desc) bytes holds dy.C and the partial sums of dcoef
  * over token ranges.  Then the first launch runs the two long contractions over dy (dy.C and the dcoef partial sums) side by
@@ -209,7 +231,7 @@ int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, c
  * result is the same bit for bit from run to run.  With the RDB_OP_LINEAR_BWD_DX amount only (room for dy.C) the first
  * launch computes dy.C and clears dcoef, and the second combines the dcoef blocks with fp32 atomics beside (dy.C).N.
  * Same requirements as the other projected entry points, coef in bf16; dcoef 16-byte aligned. */
-int rdb_linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z,
+int rdb_linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *state,
                              const void *coef, const rdb_linear_desc *desc, void *workspace,
                              int64_t workspace_bytes, void *stream);
 

@@ -2,6 +2,7 @@
 // sums and the second block of the input gradient (dx = t . N) run as kernels of their own and side by side in the merged
 // backward kernels.
 #pragma once
+#include "rdb_direct.hpp"
 #include "rdb_gemm.hpp"
 #include "rdb_tile.hpp"
 
@@ -15,7 +16,9 @@ constexpr int KD_BO = 128, KD_BM = 128;
 
 struct DcParams {
     const bf16_t *dy;
-    const bf16_t *z;
+    const bf16_t *z;     // row-major [tokens x k] (dc_block) ...
+    const bf16_t *ztf;   // ... or transposed in fragment order, rows = coefficients (dc_block_direct)
+    int tsteps, kpad;    // of ztf: token k-steps per row block (tokens rounded up to 64, / 16), k rounded up to 64
     float *dcoef;
     float *partial;  // NULL: the token splits add into dcoef (zeroed beforehand) with atomics; else split s stores its sums
                      // into partial[s][out_f][k] and a reduction pass (red_block) writes dcoef (a single split: partial = dcoef)
@@ -24,26 +27,11 @@ struct DcParams {
     int tiles_o, tiles_m, splits, tok_per_split;
 };
 
-// `block`: index of this block among the blocks that run this body.
-__device__ __forceinline__ void dc_block(const DcParams &p, bf16_t *lds, int block)
+// Stores (or adds) a block's 128 x 128 sums: acc[mi][ni][j] is o = o0 + wm*64 + mi*32 + 8*(j/4) + 4*g + j%4,
+// m = m0 + wn*64 + ni*32 + r (32 consecutive m per store: coalesced).
+__device__ __forceinline__ void dc_store(const DcParams &p, const f32x16 (&acc)[KD_BO / 64][KD_BM / 64], int o0, int m0, int split)
 {
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
-    // work item = (token split, output tile, coefficient tile), coefficient tile fastest: neighbours share the dy stream
-    const int total = p.tiles_o * p.tiles_m * p.splits;
-    const int w = xcd_work_item(block, total);
-    if (w >= total) return;
-    const int m0 = (w % p.tiles_m) * KD_BM, o0 = ((w / p.tiles_m) % p.tiles_o) * KD_BO, split = w / (p.tiles_m * p.tiles_o);
-    const int t_begin = split * p.tok_per_split;
-    const int t_end = (t_begin + p.tok_per_split < p.tokens) ? t_begin + p.tok_per_split : p.tokens;
-    f32x16 acc[KD_BO / 64][KD_BM / 64];
-#pragma unroll
-    for (int mi = 0; mi < KD_BO / 64; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < KD_BM / 64; ++ni) acc[mi][ni] = zero16();
-    GlobalOperand<KD_BO, B_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
-    GlobalOperand<KD_BM, B_BK, M_CONT> opz = {p.z, (int64_t)p.k, m0, p.k, t_end, (int64_t)p.tokens * p.k};
-    gemm_mainloop<KD_BO, KD_BM, B_BK, 1, 1>(acc, lds, opdy, opz, t_begin, (t_end - t_begin + B_BK - 1) / B_BK);
-    // acc[mi][ni][j]: o = o0 + wm*64 + mi*32 + 8*(j/4) + 4*g + j%4, m = m0 + wn*64 + ni*32 + r (32 consecutive m: coalesced)
     float *out = p.partial ? p.partial + (int64_t)split * p.out_f * p.k : p.dcoef;
 #pragma unroll
     for (int ni = 0; ni < KD_BM / 64; ++ni) {
@@ -62,6 +50,52 @@ __device__ __forceinline__ void dc_block(const DcParams &p, bf16_t *lds, int blo
                 }
             }
     }
+}
+
+// `block`: index of this block among the blocks that run this body.
+__device__ __forceinline__ void dc_block(const DcParams &p, bf16_t *lds, int block)
+{
+    // work item = (token split, output tile, coefficient tile), coefficient tile fastest: neighbours share the dy stream
+    const int total = p.tiles_o * p.tiles_m * p.splits;
+    const int w = xcd_work_item(block, total);
+    if (w >= total) return;
+    const int m0 = (w % p.tiles_m) * KD_BM, o0 = ((w / p.tiles_m) % p.tiles_o) * KD_BO, split = w / (p.tiles_m * p.tiles_o);
+    const int t_begin = split * p.tok_per_split;
+    const int t_end = (t_begin + p.tok_per_split < p.tokens) ? t_begin + p.tok_per_split : p.tokens;
+    f32x16 acc[KD_BO / 64][KD_BM / 64];
+#pragma unroll
+    for (int mi = 0; mi < KD_BO / 64; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < KD_BM / 64; ++ni) acc[mi][ni] = zero16();
+    GlobalOperand<KD_BO, B_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
+    GlobalOperand<KD_BM, B_BK, M_CONT> opz = {p.z, (int64_t)p.k, m0, p.k, t_end, (int64_t)p.tokens * p.k};
+    gemm_mainloop<KD_BO, KD_BM, B_BK, 1, 1>(acc, lds, opdy, opz, t_begin, (t_end - t_begin + B_BK - 1) / B_BK);
+    dc_store(p, acc, o0, m0, split);
+    RDB_STAMP(3);
+}
+
+// The same block with z taken from its transposed, fragment-ordered copy: only dy passes through LDS.
+__device__ __forceinline__ void dc_block_direct(const DcParams &p, bf16_t *lds, int block)
+{
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, wm = wave >> 1, wn = wave & 1;
+    const int total = p.tiles_o * p.tiles_m * p.splits;
+    const int w = xcd_work_item(block, total);
+    if (w >= total) return;
+    const int m0 = (w % p.tiles_m) * KD_BM, o0 = ((w / p.tiles_m) % p.tiles_o) * KD_BO, split = w / (p.tiles_m * p.tiles_o);
+    const int t_begin = split * p.tok_per_split;
+    const int t_end = (t_begin + p.tok_per_split < p.tokens) ? t_begin + p.tok_per_split : p.tokens;
+    f32x16 acc[KD_BO / 64][KD_BM / 64];
+#pragma unroll
+    for (int mi = 0; mi < KD_BO / 64; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < KD_BM / 64; ++ni) acc[mi][ni] = zero16();
+    // staged "A": dy[tok][o], tile rows = o (contiguous in memory), contraction = tokens
+    GlobalOperand<KD_BO, B_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
+    // direct "B": z^T fragments of this wave's 64 coefficients
+    FragSource fz;
+    fz.init(p.ztf, (int64_t)p.kpad * p.tsteps * 16, p.tsteps, (m0 + wn * 64) >> 5, lane);
+    direct_mainloop<KD_BO / 64, KD_BM / 64, true, 2, 2>(acc, lds, opdy, fz, t_begin, (t_end - t_begin + B_BK - 1) / B_BK, wm * 64, lane);
+    dc_store(p, acc, o0, m0, split);
     RDB_STAMP(3);
 }
 
@@ -141,6 +175,9 @@ inline int make_dc_params(DcParams &p, float *dcoef, const void *dy, int64_t ldd
 {
     p.dy = (const bf16_t *)dy;
     p.z = (const bf16_t *)z;
+    p.ztf = nullptr;
+    p.tsteps = 0;
+    p.kpad = 0;
     p.dcoef = dcoef;
     p.partial = nullptr;
     p.lddy = lddy;

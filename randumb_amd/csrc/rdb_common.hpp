@@ -95,16 +95,21 @@ __device__ __forceinline__ float load_as_f32(const void *p, int dtype, int64_t i
 inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // ----------------------------------------------------------------------------------------------- timeline stamps
-// RDB_STAMP(slot) records when thread 0 of a block passes a point of a kernel.  Compiled out of the library; a timing
-// harness defines RDB_STAMPS, a __device__ pointer rdb_stamp_buf and a __device__ int rdb_stamp_threads (0, or the block size
-// of the one kernel to record when a call launches several) before including the kernel sources and then finds, per block,
-// 16 slots of two counters: the constant-rate wall clock (comparable across compute units) and the shader clock.
+// RDB_STAMP(slot), slot 0..3, records when thread 0 of a block passes a point of a kernel.  Compiled out of the library.  A
+// timing harness defines RDB_STAMPS and a __device__ pointer rdb_stamp_buf before including the kernel sources and then
+// finds, per block, 4 kernels x 4 slots of two counters: the constant-rate wall clock (comparable across compute units) and
+// the shader clock.  Which of the 4 kernels a launch is, the harness says with an expression RDB_STAMP_KERNEL_ID over the
+// launch geometry (no extra registers or LDS in the kernels, so their occupancy is that of the library's build).
 #ifdef RDB_STAMPS
+#ifndef RDB_STAMP_KERNEL_ID
+#define RDB_STAMP_KERNEL_ID 0
+#endif
 #define RDB_STAMP(slot)                                                                                                  \
     do {                                                                                                                 \
-        if (threadIdx.x == 0 && rdb_stamp_buf && (rdb_stamp_threads == 0 || rdb_stamp_threads == (int)blockDim.x)) {                                                                         \
-            rdb_stamp_buf[((size_t)blockIdx.x * 16 + (slot)) * 2] = wall_clock64();                                      \
-            rdb_stamp_buf[((size_t)blockIdx.x * 16 + (slot)) * 2 + 1] = clock64();                                       \
+        if (threadIdx.x == 0 && rdb_stamp_buf) {                                                                         \
+            const size_t at_ = ((size_t)blockIdx.x * 16 + (RDB_STAMP_KERNEL_ID) * 4 + (slot)) * 2;                       \
+            rdb_stamp_buf[at_] = wall_clock64();                                                                         \
+            rdb_stamp_buf[at_ + 1] = clock64();                                                                          \
         }                                                                                                                \
     } while (0)
 #else

@@ -24,6 +24,9 @@ constexpr int K1_BC = 128, K1_BT = 64;
 struct DyCParams {
     const bf16_t *dy;
     const bf16_t *coef;
+    const bf16_t *ctf;      // NULL, or C transposed in fragment order (rows = coefficients), valid when *ctf_flag != 0
+    const uint32_t *ctf_flag;
+    int osteps, kpad;       // of ctf: k-steps per row block (out_f rounded up to 64, / 16), k rounded up to 64
     bf16_t *t;
     float *zero;     // NULL, or an array this launch clears on the side (16-byte aligned, zero_n a multiple of 4)
     int64_t zero_n;
@@ -56,6 +59,29 @@ __device__ __forceinline__ void dyc_block(const DyCParams &p, bf16_t *lds, int b
                                            4.656612873077392578125e-10f);
     else
         store_tile_bf16<K1_BC, K1_BT>(acc, lds, p.t, p.k, m0, p.k, tok0, p.tokens, 1.0f, nullptr);
+    RDB_STAMP(3);
+}
+
+// The same block with C taken from its transposed, fragment-ordered copy: only dy passes through LDS.  The four waves split
+// the coefficient rows (one 32-row block each, no fragment loaded twice) and share the 64 tokens.
+__device__ __forceinline__ void dyc_block_direct(const DyCParams &p, bf16_t *lds, int block)
+{
+    const int w = xcd_work_item(block, p.tiles_c * p.tiles_t);
+    if (w >= p.tiles_c * p.tiles_t) return;
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
+    const int m0 = (w % p.tiles_c) * K1_BC, tok0 = (w / p.tiles_c) * K1_BT;
+    f32x16 acc[1][K1_BT / 32];
+#pragma unroll
+    for (int ni = 0; ni < K1_BT / 32; ++ni) acc[0][ni] = zero16();
+    GlobalOperand<K1_BT, X_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
+    FragSource fc;
+    fc.init(p.ctf, (int64_t)p.kpad * p.osteps * 16, p.osteps, (m0 >> 5) + wave, lane);
+    direct_mainloop<K1_BT / 32, 1, false, 2, 2>(acc, lds, opdy, fc, 0, (p.out_f + X_BK - 1) / X_BK, 0, lane);
+    if (p.frag_ksteps)
+        store_tile_bf16_frag<K1_BC, K1_BT, 4>(acc, lds, p.t, p.frag_ksteps, m0, p.frag_ksteps * 16, tok0, (p.tokens + 31) / 32 * 32,
+                                              4.656612873077392578125e-10f);
+    else
+        store_tile_bf16<K1_BC, K1_BT, 4>(acc, lds, p.t, p.k, m0, p.k, tok0, p.tokens, 1.0f, nullptr);
     RDB_STAMP(3);
 }
 
@@ -93,7 +119,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dc_tn_kernel(BwdParams p)
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
     if ((int)blockIdx.x < p.dc_blocks)
-        dc_block(p.dc, lds, blockIdx.x);
+        dc_block_direct(p.dc, lds, blockIdx.x);
     else
         tn_block(p.tn, lds, blockIdx.x - p.dc_blocks);
 }
@@ -113,10 +139,17 @@ __global__ __launch_bounds__(256, 2) void bwd_dc_dyc_kernel(BwdAParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
-    if ((int)blockIdx.x < p.dc_blocks)
-        dc_block(p.dc, lds, blockIdx.x);
-    else
-        dyc_block(p.dyc, lds, blockIdx.x - p.dc_blocks);
+    if ((int)blockIdx.x < p.dc_blocks) {
+        if (p.dc.ztf)
+            dc_block_direct(p.dc, lds, blockIdx.x);
+        else
+            dc_block(p.dc, lds, blockIdx.x);
+    } else {
+        if (p.dyc.ctf && *p.dyc.ctf_flag)   // the forward pass left the transposed coefficients in the state
+            dyc_block_direct(p.dyc, lds, blockIdx.x - p.dc_blocks);
+        else
+            dyc_block(p.dyc, lds, blockIdx.x - p.dc_blocks);
+    }
 }
 
 struct BwdBParams {
@@ -157,6 +190,8 @@ template <int KG> __global__ __launch_bounds__(ST_THREADS, 1) void bwd_tns_red_k
 }
 
 // ----------------------------------------------------------------------------------------------- host side
+void dc_params_from_state(DcParams &p, const void *state, const rdb_linear_desc *d);   // rdb_factored.hip
+
 static bool dx_factored_ok(const rdb_linear_desc *d)
 {
     return d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16 && d->coef_rows != 0 && d->k % 8 == 0 && d->in_f % 8 == 0 &&
@@ -189,6 +224,10 @@ static void make_dyc_params(DyCParams &p1, const void *dy, int64_t lddy, const v
 {
     p1.dy = (const bf16_t *)dy;
     p1.coef = (const bf16_t *)coef;
+    p1.ctf = nullptr;
+    p1.ctf_flag = nullptr;
+    p1.osteps = 0;
+    p1.kpad = 0;
     p1.t = (bf16_t *)t;
     p1.zero = nullptr;
     p1.zero_n = 0;
@@ -269,11 +308,19 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
     const size_t smem_dyc = engine_smem<K1_BC, K1_BT, X_BK, M_CONT, K_CONT>();
     if (workspace_bytes >= linear_bwd_projected_workspace(d, num_cus)) {
         BwdAParams a;
-        const int dc_items = make_dc_params(a.dc, dcoef, dy, lddy, z, d, num_cus);
+        const int dc_items = make_dc_params(a.dc, dcoef, dy, lddy, nullptr, d, num_cus);
+        dc_params_from_state(a.dc, z, d);
         // one token range only: its sums are the result, stored straight into dcoef, and nothing is left to add up
         const bool direct = a.dc.splits == 1;
         a.dc.partial = direct ? dcoef : reinterpret_cast<float *>(static_cast<char *>(workspace) + align256(linear_dx_factored_workspace(d)));
         a.dyc = p1;
+        {   // the transposed coefficients, if the forward pass left them in the state (its header says so)
+            const ProjLayout L = proj_layout(d);
+            a.dyc.ctf = reinterpret_cast<const bf16_t *>(static_cast<const char *>(z) + L.ctf_off);
+            a.dyc.ctf_flag = static_cast<const uint32_t *>(z);
+            a.dyc.osteps = (int)(L.out64 / 16);
+            a.dyc.kpad = L.kpad;
+        }
         if (tn_stationary_ok(d, lddx)) a.dyc.frag_ksteps = (int)cdiv(d->k, 64) * 4;   // the t.N kernel below keeps t in registers
         a.dc_blocks = xcd_grid_size(dc_items);
         size_t smem = smem_dc > smem_dyc ? smem_dc : smem_dyc;
@@ -330,7 +377,8 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
     int rc = launch_engine(dx_dyc_kernel, p1, p1.tiles_c * p1.tiles_t, smem_dyc, s, "dx_dyc_kernel");
     if (rc) return rc;
     BwdParams p;
-    const int dc_items = make_dc_params(p.dc, dcoef, dy, lddy, z, d, num_cus);
+    const int dc_items = make_dc_params(p.dc, dcoef, dy, lddy, nullptr, d, num_cus);
+    dc_params_from_state(p.dc, z, d);
     const int tn_items = make_tn_params(p.tn, dx, lddx, workspace, d);
     p.dc_blocks = xcd_grid_size(dc_items);
     const size_t smem = smem_dc > smem_tn ? smem_dc : smem_tn;

@@ -26,9 +26,14 @@ constexpr int KZ_BM = 32, KZ_BT = 256, KZ_WM = 1;
 
 struct ZParams {
     const bf16_t *x;
-    bf16_t *z;
+    const bf16_t *coef;  // NULL, or C [out_f x k] to transpose into ctf on the side
+    bf16_t *zf;          // z for the forward product: fragment order (frag_fwd) or row-major [tokens x k]
+    bf16_t *ztf;         // z transposed in fragment order, rows = coefficients
+    bf16_t *ctf;         // C transposed in fragment order, rows = coefficients
+    uint32_t *flag;      // header word 0 of the state: 1 when ctf has been written by this launch
     int64_t ldx;
-    int tokens, in_f, k;
+    int tokens, in_f, out_f, k;
+    int kpad, tok32, tok64, out64, frag_fwd;
     int tiles_m, tiles_t;
     uint32_t seed;
 };
@@ -37,6 +42,26 @@ __global__ __launch_bounds__(256, 2) void factored_z_kernel(ZParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
+    if (blockIdx.x == 0 && t == 0) *p.flag = p.coef ? 1u : 0u;
+    if (p.coef) {
+        // C transposed into fragment order, a 1 KB unit (32 coefficients x 16 output features) per wave and turn: lane (r, g)
+        // gathers C[o0 + 8 g + j][m0 + r], j = 0..7 (32 lanes read 64 consecutive bytes of a row) and stores its 16 bytes
+        const int osteps = p.out64 >> 4, units = (p.kpad >> 5) * osteps, r = lane & 31, g = lane >> 5;
+        for (int u = blockIdx.x * 4 + wave; u < units; u += gridDim.x * 4) {
+            const int mb = u / osteps, os = u % osteps, m = mb * 32 + r;
+            uint32_t w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int o = os * 16 + g * 8 + 2 * j;   // out_f is even: o and o + 1 exist together
+                const bool in = m < p.k && o < p.out_f;
+                const uint32_t lo = in ? p.coef[(int64_t)o * p.k + m] : 0u, hi = in ? p.coef[(int64_t)(o + 1) * p.k + m] : 0u;
+                w[j] = lo | (hi << 16);
+            }
+            const i32x4 v = {(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+            *reinterpret_cast<i32x4 *>(p.ctf + (int64_t)u * 512 + lane * 8) = v;
+        }
+    }
     // work item = (token tile, coefficient tile), coefficient tile fastest: neighbours share the x tile
     const int w = xcd_work_item(blockIdx.x, p.tiles_m * p.tiles_t);
     if (w >= p.tiles_m * p.tiles_t) return;
@@ -51,7 +76,57 @@ __global__ __launch_bounds__(256, 2) void factored_z_kernel(ZParams p)
     NoiseOperandRowsAreCoefs<KZ_BM, F_BK> opn = {m0, p.seed};
     GlobalOperand<KZ_BT, F_BK, K_CONT> opx = {p.x, p.ldx, tok0, p.tokens, p.in_f, (int64_t)(p.tokens - 1) * p.ldx + p.in_f};
     gemm_mainloop<KZ_BM, KZ_BT, F_BK, 1, 1, KZ_WM>(acc, lds, opn, opx, 0, (p.in_f + F_BK - 1) / F_BK);
-    store_tile_bf16<KZ_BM, KZ_BT, KZ_WM>(acc, lds, p.z, p.k, m0, p.k, tok0, p.tokens, INV_2_31, nullptr);
+    // The tile D[a = coefficient][b = token] goes to LDS once, as bf16 rows of tokens (LD elements apart), and leaves in
+    // up to two orders.  Rows of tokens past the end and coefficients past k hold zeros or finite values: every byte of the
+    // state's z pieces is written, so that their consumers may multiply padding with zeros.
+    static_assert(MI == 1 && KZ_WM == 1, "the epilogue below is written for one 32-coefficient row block per wave");
+    constexpr int LD = KZ_BM + 8;
+    {
+        const int r = lane & 31, g = lane >> 5;
+#pragma unroll
+        for (int jq = 0; jq < 4; ++jq)
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) {
+                const int b = wave * NI * 32 + ni * 32 + r;
+                store4<bf16_t>(lds + b * LD + 8 * jq + 4 * g, acc[0][ni][jq * 4 + 0] * INV_2_31, acc[0][ni][jq * 4 + 1] * INV_2_31,
+                               acc[0][ni][jq * 4 + 2] * INV_2_31, acc[0][ni][jq * 4 + 3] * INV_2_31);
+            }
+    }
+    __syncthreads();
+    constexpr int PIECES = KZ_BM * KZ_BT / 8;
+    if (p.frag_fwd) {
+        // rows = tokens, k = coefficients: a piece is 8 coefficients of one token, neighbouring lanes take neighbouring tokens
+        const int ksteps = p.kpad >> 4;
+#pragma unroll
+        for (int q = 0; q < PIECES / 256; ++q) {
+            const int idx = q * 256 + t, b = idx % KZ_BT, a = (idx / KZ_BT) * 8;
+            const int gb = tok0 + b, ga = m0 + a;
+            if (gb < p.tok32)
+                *reinterpret_cast<f32x4 *>(p.zf + ((int64_t)(gb >> 5) * ksteps + (ga >> 4)) * 512 + (((ga >> 3) & 1) * 32 + (gb & 31)) * 8) =
+                    *reinterpret_cast<const f32x4 *>(lds + b * LD + a);
+        }
+    } else {
+#pragma unroll
+        for (int q = 0; q < PIECES / 256; ++q) {
+            const int idx = q * 256 + t, b = idx / (KZ_BM / 8), a = (idx % (KZ_BM / 8)) * 8;
+            if (tok0 + b < p.tokens && m0 + a < p.k)
+                *reinterpret_cast<f32x4 *>(p.zf + (int64_t)(tok0 + b) * p.k + m0 + a) = *reinterpret_cast<const f32x4 *>(lds + b * LD + a);
+        }
+    }
+    {
+        // rows = coefficients, k = tokens: the LDS transpose read turns 16 token rows x 32 coefficients into the fragment
+        const int tsteps = p.tok64 >> 4, s = lane & 15, qq = (lane >> 4) & 1, g = lane >> 5;
+#pragma unroll
+        for (int q = 0; q < KZ_BT / 16 / 4; ++q) {
+            const int ks = wave * (KZ_BT / 16 / 4) + q;   // token k-step inside the tile
+            if (tok0 + ks * 16 >= p.tok64) continue;
+            const bf16_t *src = lds + (ks * 16 + g * 8 + (s >> 2)) * LD + qq * 16 + (s & 3) * 4;
+            Frag8 f;
+            f.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(src));
+            f.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(src + 4 * LD));
+            *reinterpret_cast<f32x4 *>(p.ztf + ((int64_t)(m0 >> 5) * tsteps + (tok0 >> 4) + ks) * 512 + lane * 8) = f.f4;
+        }
+    }
     RDB_STAMP(3);
 }
 
@@ -90,11 +165,12 @@ __global__ __launch_bounds__(256, 2) void factored_y_kernel(YParams p)
 }
 
 // ----------------------------------------------------------------------------------------------- y = z . C^T, k <= 256
-// body in rdb_stationary.hpp: the projection of a token stays in registers, the rows of C stream through LDS
+// body in rdb_stationary.hpp: the projection of a token stays in registers (read in fragment order, as factored_z_kernel
+// leaves it), the rows of C stream through LDS
 template <int KG, bool BIAS> __global__ __launch_bounds__(ST_THREADS, 1) void factored_ys_kernel(StParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    stationary_block<KG, BIAS, false>(p, smem_raw, blockIdx.x);
+    stationary_block<KG, BIAS, false, true>(p, smem_raw, blockIdx.x);
 }
 
 // ----------------------------------------------------------------------------------------------- dC = dy^T . z
@@ -102,49 +178,73 @@ template <int KG, bool BIAS> __global__ __launch_bounds__(ST_THREADS, 1) void fa
 __global__ __launch_bounds__(256, 1) void factored_dc_kernel(DcParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    dc_block(p, reinterpret_cast<bf16_t *>(smem_raw), blockIdx.x);
+    if (p.ztf)
+        dc_block_direct(p, reinterpret_cast<bf16_t *>(smem_raw), blockIdx.x);
+    else
+        dc_block(p, reinterpret_cast<bf16_t *>(smem_raw), blockIdx.x);
 }
 
 // ----------------------------------------------------------------------------------------------- host side
 // What every factored kernel needs of the layer; coef_dtype is checked by the callers that read coefficients.
-static bool factored_shape_ok(const rdb_linear_desc *d)
-{
-    return d->act_dtype == RDB_BF16 && d->coef_rows != 0 && d->k % 8 == 0 && d->in_f % 8 == 0 && d->out_f % 8 == 0 && d->k > 0 &&
-           d->tokens > 0 && d->in_f > 0 && d->out_f > 0 && d->tokens * d->k < (1ll << 29) && d->out_f * d->k < (1ll << 29);
-}
+static bool factored_shape_ok(const rdb_linear_desc *d) { return proj_layout(d).ok; }
 static bool cheaper_factored(const rdb_linear_desc *d) { return d->k * (d->in_f + d->out_f) < d->in_f * d->out_f; }
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
-int64_t linear_projection_bytes(const rdb_linear_desc *d)
+int64_t linear_projection_bytes(const rdb_linear_desc *d) { return proj_layout(d).bytes; }
+
+static bf16_t *state_piece(const void *state, int64_t off) { return reinterpret_cast<bf16_t *>(static_cast<char *>(const_cast<void *>(state)) + off); }
+
+// Fills the coefficient-gradient parameters that name the projection state's pieces.
+void dc_params_from_state(DcParams &p, const void *state, const rdb_linear_desc *d)
 {
-    return factored_shape_ok(d) ? d->tokens * d->k * (int64_t)sizeof(bf16_t) : 0;
+    const ProjLayout L = proj_layout(d);
+    p.z = nullptr;
+    p.ztf = state_piece(state, L.ztf_off);
+    p.tsteps = (int)(L.tok64 / 16);
+    p.kpad = L.kpad;
 }
 
-// The three entry points below return RDB_E_UNSUPPORTED, without setting an error, when the request does not fit.
-int linear_project(void *z, const void *x, int64_t ldx, const rdb_linear_desc *d, hipStream_t s)
+// The entry points below return RDB_E_UNSUPPORTED, without setting an error, when the request does not fit.
+// state <- projection of x (z for the forward product, z transposed for the coefficient gradient) and, when coef is given,
+// the transposed coefficients for the input gradient.
+int linear_project(void *state, const void *x, int64_t ldx, const void *coef, const rdb_linear_desc *d, hipStream_t s)
 {
-    if (!factored_shape_ok(d) || d->tokens * ldx >= (1ll << 29) || ldx % 8 || !aligned16(x) || !aligned16(z)) return RDB_E_UNSUPPORTED;
+    const ProjLayout L = proj_layout(d);
+    if (!L.ok || d->tokens * ldx >= (1ll << 29) || ldx % 8 || !aligned16(x) || !aligned16(state)) return RDB_E_UNSUPPORTED;
+    if (coef && d->coef_dtype != RDB_BF16) coef = nullptr;   // the transposed copy is an operand of the bf16 kernels only
     ZParams p;
     p.x = (const bf16_t *)x;
-    p.z = (bf16_t *)z;
+    p.coef = (const bf16_t *)coef;
+    p.zf = state_piece(state, L.zf_off);
+    p.ztf = state_piece(state, L.ztf_off);
+    p.ctf = state_piece(state, L.ctf_off);
+    p.flag = reinterpret_cast<uint32_t *>(state);
     p.ldx = ldx;
     p.tokens = (int)d->tokens;
     p.in_f = (int)d->in_f;
+    p.out_f = (int)d->out_f;
     p.k = (int)d->k;
+    p.kpad = L.kpad;
+    p.tok32 = (int)L.tok32;
+    p.tok64 = (int)L.tok64;
+    p.out64 = (int)L.out64;
+    p.frag_fwd = L.frag_fwd ? 1 : 0;
     p.seed = d->seed;
-    p.tiles_m = (int)cdiv(d->k, KZ_BM);
+    p.tiles_m = L.kpad / KZ_BM;   // every coefficient row block of the padded pieces is written
     p.tiles_t = (int)cdiv(d->tokens, KZ_BT);
     return launch_engine(factored_z_kernel, p, p.tiles_m * p.tiles_t, engine_smem<KZ_BM, KZ_BT, F_BK, K_CONT, K_CONT>(), s, "factored_z_kernel");
 }
 
-int linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, const void *bias, const rdb_linear_desc *d, int num_cus,
+int linear_fwd_projected(void *y, int64_t ldy, const void *state, const void *coef, const void *bias, const rdb_linear_desc *d, int num_cus,
                          hipStream_t s)
 {
-    if (!factored_shape_ok(d) || d->coef_dtype != RDB_BF16 || ldy % 8 || !aligned16(y) || !aligned16(z) || !aligned16(coef))
-        return RDB_E_UNSUPPORTED;
-    if (d->k <= ST_KMAX && ((uintptr_t)bias & 7) == 0 && d->tokens * ldy < (1ll << 29)) {  // the contraction of a token fits in registers
+    const ProjLayout L = proj_layout(d);
+    if (!L.ok || d->coef_dtype != RDB_BF16 || ldy % 8 || !aligned16(y) || !aligned16(state) || !aligned16(coef)) return RDB_E_UNSUPPORTED;
+    const bf16_t *zf = state_piece(state, L.zf_off);
+    if (L.frag_fwd) {   // the contraction of a token fits in registers; z lies in fragment order
+        if (((uintptr_t)bias & 7) || d->tokens * ldy >= (1ll << 29)) return RDB_E_UNSUPPORTED;
         StParams q;
-        q.z = (const bf16_t *)z;
+        q.z = zf;
         q.coef = (const bf16_t *)coef;
         q.bias = (const bf16_t *)bias;
         q.y = (bf16_t *)y;
@@ -170,7 +270,7 @@ int linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, 
         }
     }
     YParams p;
-    p.z = (const bf16_t *)z;
+    p.z = zf;
     p.coef = (const bf16_t *)coef;
     p.bias = (const bf16_t *)bias;
     p.y = (bf16_t *)y;
@@ -184,16 +284,17 @@ int linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, 
 }
 
 // dcoef must have been zeroed on the same stream.
-int linear_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *z, const rdb_linear_desc *d, int num_cus, hipStream_t s)
+int linear_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *state, const rdb_linear_desc *d, int num_cus, hipStream_t s)
 {
-    if (!factored_shape_ok(d) || d->tokens * lddy >= (1ll << 29) || lddy % 8 || !aligned16(dy) || !aligned16(z)) return RDB_E_UNSUPPORTED;
+    if (!factored_shape_ok(d) || d->tokens * lddy >= (1ll << 29) || lddy % 8 || !aligned16(dy) || !aligned16(state)) return RDB_E_UNSUPPORTED;
     DcParams p;
-    const int items = make_dc_params(p, dcoef, dy, lddy, z, d, num_cus);
+    const int items = make_dc_params(p, dcoef, dy, lddy, nullptr, d, num_cus);
+    dc_params_from_state(p, state, d);
     return launch_engine(factored_dc_kernel, p, items, engine_smem<KD_BO, KD_BM, F_BK, M_CONT, M_CONT>(), s,
                          "factored_dc_kernel");
 }
 
-// y = (x . N^T) . C^T with the projection in the workspace.
+// y = (x . N^T) . C^T with the projection state in the workspace.
 int linear_fwd_factored(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
                         const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
@@ -203,12 +304,13 @@ int linear_fwd_factored(void *y, int64_t ldy, const void *x, int64_t ldx, const 
     // check everything before the first launch, so that a refusal leaves nothing half done
     if (d->tokens * ldx >= (1ll << 29) || ldx % 8 || ldy % 8 || !aligned16(x) || !aligned16(coef) || !aligned16(y) || !aligned16(workspace))
         return RDB_E_UNSUPPORTED;
-    int rc = linear_project(workspace, x, ldx, d, s);
+    if (proj_layout(d).frag_fwd && (((uintptr_t)bias & 7) || d->tokens * ldy >= (1ll << 29))) return RDB_E_UNSUPPORTED;
+    int rc = linear_project(workspace, x, ldx, nullptr, d, s);
     if (rc) return rc;
     return linear_fwd_projected(y, ldy, workspace, coef, bias, d, num_cus, s);
 }
 
-// dC = dy^T . (x . N^T) with the projection in the workspace; dcoef must have been zeroed on the same stream.
+// dC = dy^T . (x . N^T) with the projection state in the workspace; dcoef must have been zeroed on the same stream.
 int linear_dcoef_factored(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus,
                           void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
@@ -218,7 +320,7 @@ int linear_dcoef_factored(float *dcoef, const void *dy, int64_t lddy, const void
     if (d->tokens * ldx >= (1ll << 29) || d->tokens * lddy >= (1ll << 29) || ldx % 8 || lddy % 8 || !aligned16(x) || !aligned16(dy) ||
         !aligned16(workspace))
         return RDB_E_UNSUPPORTED;
-    int rc = linear_project(workspace, x, ldx, d, s);
+    int rc = linear_project(workspace, x, ldx, nullptr, d, s);
     if (rc) return rc;
     return linear_dcoef_projected(dcoef, dy, lddy, workspace, d, num_cus, s);
 }

@@ -9,6 +9,7 @@
 // contraction in steps of 32.  Reference behaviour replaced: materialize() + dense product per aten.mm
 // (src/rten_cpp/RandumbTensor.py:942-952, 771-791), autograd's MmBackward on the dense weight, and
 // RandumbTensorConstructor.backward -> materialize_bwd / scale_bias_bwd (RandumbTensor.py:979-990).
+#include "rdb_direct.hpp"
 #include "rdb_tile.hpp"
 
 namespace rdb {
@@ -282,7 +283,7 @@ int linear_fwd_strip(void *y, int64_t ldy, const void *x, int64_t ldx, const voi
 
 // rdb_factored.hip
 int64_t linear_projection_bytes(const rdb_linear_desc *d);
-int linear_project(void *z, const void *x, int64_t ldx, const rdb_linear_desc *d, hipStream_t s);
+int linear_project(void *state, const void *x, int64_t ldx, const void *coef, const rdb_linear_desc *d, hipStream_t s);
 int linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, const void *bias, const rdb_linear_desc *d, int num_cus,
                          hipStream_t s);
 int linear_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *z, const rdb_linear_desc *d, int num_cus, hipStream_t s);
@@ -527,21 +528,39 @@ static int check_projected(const char *who, const rdb_linear_desc *d)
     if (rc) return rc;
     if (linear_projection_bytes(d) == 0)
         return set_error(RDB_E_UNSUPPORTED, "%s: the projected form needs matrix-coef, bf16 activations, non-empty sizes that are "
-                                            "multiples of 8 and tokens*k < 2^29", who);
+                                            "multiples of 8, and tokens*k and out_f*k (k rounded up to 64) below 2^29", who);
     return RDB_OK;
 }
 
 extern "C" int64_t rdb_linear_projection_bytes(const rdb_linear_desc *d) { return d ? linear_projection_bytes(d) : 0; }
 
-extern "C" int rdb_linear_project(void *z, const void *x, int64_t ldx, const rdb_linear_desc *d, void *stream)
+extern "C" int rdb_linear_projection_layout(const rdb_linear_desc *d, int64_t *info)
+{
+    int rc = check_projected("rdb_linear_projection_layout", d);
+    if (rc) return rc;
+    if (!info) return set_error(RDB_E_NULL, "rdb_linear_projection_layout: info is NULL");
+    const ProjLayout L = proj_layout(d);
+    info[0] = L.zf_off;
+    info[1] = L.frag_fwd ? 1 : 0;
+    info[2] = L.ztf_off;
+    info[3] = L.ctf_off;
+    info[4] = L.kpad;
+    info[5] = L.tok32;
+    info[6] = L.tok64;
+    info[7] = L.out64;
+    return RDB_OK;
+}
+
+extern "C" int rdb_linear_project(void *state, const void *x, int64_t ldx, const void *coef, const rdb_linear_desc *d, void *stream)
 {
     int rc = check_projected("rdb_linear_project", d);
     if (rc) return rc;
-    if (!z || !x) return set_error(RDB_E_NULL, "rdb_linear_project: z or x is NULL");
+    if (!state || !x) return set_error(RDB_E_NULL, "rdb_linear_project: state or x is NULL");
     if (ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_project: leading dimension smaller than the row");
-    rc = linear_project(z, x, ldx, d, (hipStream_t)stream);
+    if (coef && !aligned16(coef)) return set_error(RDB_E_ALIGN, "rdb_linear_project: coef must be 16-byte aligned");
+    rc = linear_project(state, x, ldx, coef, d, (hipStream_t)stream);
     if (rc == RDB_E_UNSUPPORTED)
-        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_project: x and z must be 16-byte aligned, ldx a multiple of 8, tokens*ldx < 2^29");
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_project: x and state must be 16-byte aligned, ldx a multiple of 8, tokens*ldx < 2^29");
     return rc;
 }
 
@@ -554,8 +573,8 @@ extern "C" int rdb_linear_fwd_projected(void *y, int64_t ldy, const void *z, con
     if (ldy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_fwd_projected: leading dimension smaller than the row");
     rc = linear_fwd_projected(y, ldy, z, coef, bias, d, num_compute_units(), (hipStream_t)stream);
     if (rc == RDB_E_UNSUPPORTED)
-        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd_projected: coefficients must be bf16; y, z and coef 16-byte aligned; ldy a "
-                                            "multiple of 8");
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd_projected: coefficients must be bf16; y, state and coef 16-byte aligned; ldy "
+                                            "a multiple of 8; with k <= 256 also bias 8-byte aligned and tokens*ldy < 2^29");
     return rc;
 }
 

@@ -15,6 +15,11 @@
 
 namespace rdb {
 
+#ifndef RDB_Y_STORE_AUX
+#define RDB_Y_STORE_AUX 2   // cache policy of the output row stores: non-temporal (y and dx are not read again by this library, and
+                           // lines that do not linger in L2 need no write-back when the kernel ends: the next launch starts sooner)
+#endif
+
 constexpr int ST_BT = 256, ST_BO = 64, ST_STG_LD = ST_BO + 8, ST_WAVES = 8, ST_THREADS = ST_WAVES * 64, ST_TW = ST_BT / ST_WAVES;
 constexpr int ST_KMAX = 256;
 
@@ -135,7 +140,7 @@ template <int KG, bool BIAS, bool NOISE> struct StBlock {
                     const int qq = h * 2 + q;
                     const uint32_t a = (o0 + (lane & 7) * 8 < p.out_f && tok_y + qq * 8 < p.tokens)
                                            ? off_y + (uint32_t)(qq * 8 * (int)p.ldy * 2 + o0 * 2) : BUFFER_OOB;
-                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v[q]), rs_y, (int)a, 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v[q]), rs_y, (int)a, 0, RDB_Y_STORE_AUX);
                 }
                 if (op == 9) __builtin_amdgcn_wave_barrier();
             }

@@ -265,64 +265,132 @@ def _proj_desc(tokens, in_f, out_f, k, seed, coef_dtype=torch.bfloat16) -> Linea
     return d
 
 
+def linear_projection_bytes(tokens: int, in_f: int, out_f: int, k: int) -> int:
+    """Size of the projection state of a layer of these sizes; 0 when the projected form (matrix-coef, bf16) does not apply."""
+    return int(_lib.load().rdb_linear_projection_bytes(ctypes.byref(_proj_desc(tokens, in_f, out_f, k, 0))))
+
+
 def linear_projection_supported(tokens: int, in_f: int, out_f: int, k: int) -> bool:
-    """Whether the projected form (matrix-coef, bf16) applies to a layer of these sizes."""
-    return _lib.load().rdb_linear_projection_bytes(ctypes.byref(_proj_desc(tokens, in_f, out_f, k, 0))) > 0
+    """Whether the projected entry points run a layer of these sizes: matrix-coef bf16, sizes in multiples of 8, and
+    activations and gradients inside the kernels' 32-bit addressing (tokens*in_f, tokens*out_f < 2^29)."""
+    if tokens * in_f >= 2**29 or tokens * out_f >= 2**29:
+        return False
+    return linear_projection_bytes(tokens, in_f, out_f, k) > 0
 
 
-def linear_project(x: torch.Tensor, k: int, out_f: int, seed: int) -> torch.Tensor:
-    """``z = x @ Noise.T`` (tokens, k) in bf16: all that the forward product and the coef gradient need of ``x``."""
-    _need_gpu("linear_project", x)
+def linear_projection_preferred(tokens: int, in_f: int, out_f: int, k: int) -> bool:
+    """Whether the projected form is also the cheaper one: the factored products need 2*tokens*k*(in_f + out_f) flops per
+    direction, forming the weight 2*tokens*in_f*out_f (+ its generation)."""
+    return k * (in_f + out_f) < in_f * out_f and linear_projection_supported(tokens, in_f, out_f, k)
+
+
+def linear_project(x: torch.Tensor, k: int, out_f: int, seed: int, coef: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Projection state of ``x`` for a matrix-coef bf16 layer: an opaque byte tensor ``(tokens, bytes per token)`` holding ``z = x @ Noise.T`` (tokens, k)
+    in the element orders the consumers' matrix instructions read (all that the forward product and the coef gradient need
+    of ``x``) and, when ``coef`` (out_f, k) is given in bf16, the transposed coefficients for the input gradient."""
+    _need_gpu("linear_project", x, coef)
     x = _act(x)
     if x.dtype != torch.bfloat16:
         raise ValueError("linear_project computes in bf16")
     d = _proj_desc(x.shape[0], x.shape[1], out_f, k, seed)
-    z = torch.empty((x.shape[0], k), dtype=torch.bfloat16, device=x.device)
+    L = _lib.load()
+    nbytes = L.rdb_linear_projection_bytes(ctypes.byref(d))
+    if nbytes <= 0:
+        _lib.check(L.rdb_linear_project(None, None, x.stride(0), None, ctypes.byref(d), None), "rdb_linear_project")
+    # 2-D so that the token count travels with the tensor: (tokens, bytes per token rounded up)
+    state = torch.empty((x.shape[0], -(-nbytes // x.shape[0])), dtype=torch.uint8, device=x.device)
+    c = None
+    if coef is not None and coef.dtype == torch.bfloat16:
+        c = coef.contiguous()
+        if tuple(c.shape) != (out_f, k):
+            raise ValueError(f"coef must be ({out_f}, {k}), got {tuple(c.shape)}")
     with torch.cuda.device(x.device):
-        rc = _lib.load().rdb_linear_project(_p(z), _p(x), x.stride(0), ctypes.byref(d), _stream(x.device))
+        rc = L.rdb_linear_project(_p(state), _p(x), x.stride(0), _p(c), ctypes.byref(d), _stream(x.device))
     _lib.check(rc, "rdb_linear_project")
-    return z
+    return state
 
 
-def linear_fwd_projected(z: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``y = z @ coef.T (+ bias)`` for matrix-coef ``coef`` (out_f, k) in bf16."""
-    _need_gpu("linear_fwd_projected", z, coef)
+def projection_unpack(state: torch.Tensor, in_f: int, out_f: int, k: int) -> dict:
+    """The pieces of a projection state as ordinary row-major tensors, for tools and tests (a layout decode, no arithmetic):
+    ``z`` (tokens, k) as the forward product reads it, ``z_t`` (k, tokens) as the coef gradient reads it, and ``coef_t``
+    (k, out_f), the transposed coefficients, or ``None`` when the state was written without them."""
+    tokens = state.shape[0]
+    d = _proj_desc(tokens, in_f, out_f, k, 0)
+    _check_state(state, d, "projection_unpack")
+    info = (ctypes.c_int64 * 8)()
+    _lib.check(_lib.load().rdb_linear_projection_layout(ctypes.byref(d), info), "rdb_linear_projection_layout")
+    zf_off, frag_fwd, ztf_off, ctf_off, kpad, tok32, tok64, out64 = (int(v) for v in info)
+    flat = state.reshape(-1)
+    dev = state.device
+
+    def piece(off, nelem):
+        return flat[off:off + 2 * nelem].view(torch.bfloat16)
+
+    def frag_gather(buf, rows, kks, ksteps):
+        r = torch.arange(rows, device=dev).view(-1, 1)
+        c = torch.arange(kks, device=dev).view(1, -1)
+        idx = ((r // 32) * ksteps + c // 16) * 512 + (((c // 8) % 2) * 32 + r % 32) * 8 + c % 8
+        return buf[idx]
+
+    if frag_fwd:
+        z = frag_gather(piece(zf_off, tok32 * kpad), tokens, k, kpad // 16)
+    else:
+        z = piece(zf_off, tokens * k).view(tokens, k).clone()
+    z_t = frag_gather(piece(ztf_off, tok64 * kpad), k, tokens, tok64 // 16)
+    has_c = int(flat[:4].view(torch.int32)[0]) == 1
+    coef_t = frag_gather(piece(ctf_off, out64 * kpad), k, out_f, out64 // 16) if has_c else None
+    return {"z": z, "z_t": z_t, "coef_t": coef_t}
+
+
+def _check_state(state: torch.Tensor, d: LinearDesc, who: str) -> None:
+    need = _lib.load().rdb_linear_projection_bytes(ctypes.byref(d))
+    if state.dtype != torch.uint8 or state.dim() != 2 or not state.is_contiguous() or state.numel() < need or need <= 0:
+        raise ValueError(f"{who}: the projection state must be the byte tensor linear_project returned for this layer and token "
+                         f"count ({need} bytes), got {tuple(state.shape)} {state.dtype}")
+
+
+def linear_fwd_projected(state: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int,
+                         bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``y = z @ coef.T (+ bias)`` for matrix-coef ``coef`` (out_f, k) in bf16; ``state`` from :func:`linear_project`."""
+    _need_gpu("linear_fwd_projected", state, coef)
     c = _native(coef)
-    z = z.contiguous()
     out_f, k = c.shape
-    d = _proj_desc(z.shape[0], in_f, out_f, k, seed, c.dtype)
-    b = None if bias is None else bias.to(z.dtype).contiguous()
-    y = torch.empty((z.shape[0], out_f), dtype=z.dtype, device=z.device)
-    with torch.cuda.device(z.device):
-        rc = _lib.load().rdb_linear_fwd_projected(_p(y), y.stride(0), _p(z), _p(c), _p(b), ctypes.byref(d), _stream(z.device))
+    tokens = state.shape[0]
+    d = _proj_desc(tokens, in_f, out_f, k, seed, c.dtype)
+    _check_state(state, d, "linear_fwd_projected")
+    b = None if bias is None else bias.to(torch.bfloat16).contiguous()
+    y = torch.empty((tokens, out_f), dtype=torch.bfloat16, device=state.device)
+    with torch.cuda.device(state.device):
+        rc = _lib.load().rdb_linear_fwd_projected(_p(y), y.stride(0), _p(state), _p(c), _p(b), ctypes.byref(d), _stream(state.device))
     _lib.check(rc, "rdb_linear_fwd_projected")
     return y
 
 
-def linear_bwd_dcoef_projected(dy: torch.Tensor, z: torch.Tensor, in_f: int, seed: int) -> torch.Tensor:
-    """``dcoef = dy.T @ z`` (out_f, k) in fp32."""
-    _need_gpu("linear_bwd_dcoef_projected", dy, z)
+def linear_bwd_dcoef_projected(dy: torch.Tensor, state: torch.Tensor, k: int, in_f: int, seed: int) -> torch.Tensor:
+    """``dcoef = dy.T @ z`` (out_f, k) in fp32; ``state`` from :func:`linear_project`."""
+    _need_gpu("linear_bwd_dcoef_projected", dy, state)
     dy = _act(dy)
-    z = z.contiguous()
-    out_f, k = dy.shape[1], z.shape[1]
+    out_f = dy.shape[1]
     d = _proj_desc(dy.shape[0], in_f, out_f, k, seed)
+    _check_state(state, d, "linear_bwd_dcoef_projected")
     dcoef = torch.empty((out_f, k), dtype=torch.float32, device=dy.device)
     with torch.cuda.device(dy.device):
-        rc = _lib.load().rdb_linear_bwd_dcoef_projected(_p(dcoef), _p(dy), dy.stride(0), _p(z), ctypes.byref(d), _stream(dy.device))
+        rc = _lib.load().rdb_linear_bwd_dcoef_projected(_p(dcoef), _p(dy), dy.stride(0), _p(state), ctypes.byref(d), _stream(dy.device))
     _lib.check(rc, "rdb_linear_bwd_dcoef_projected")
     return dcoef
 
 
-def linear_bwd_projected(dy: torch.Tensor, z: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int, ordered_sums: bool = True):
-    """Whole backward pass of a matrix-coef bf16 layer from the saved projection: ``(dx, dcoef)`` with ``dx = dy @ W`` in
+def linear_bwd_projected(dy: torch.Tensor, state: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int, ordered_sums: bool = True):
+    """Whole backward pass of a matrix-coef bf16 layer from the projection state: ``(dx, dcoef)`` with ``dx = dy @ W`` in
     bf16 and ``dcoef = dy.T @ z`` in fp32, in two kernel launches.  ``ordered_sums`` gives the library room for the partial
     sums of ``dcoef`` (added in a fixed order: bit-reproducible); without it they are combined with fp32 atomics."""
-    _need_gpu("linear_bwd_projected", dy, z, coef)
+    _need_gpu("linear_bwd_projected", dy, state, coef)
     dy = _act(dy)
-    z = z.contiguous()
     c = _native(coef)
     out_f, k = c.shape
     d = _proj_desc(dy.shape[0], in_f, out_f, k, seed, c.dtype)
+    _check_state(state, d, "linear_bwd_projected")
+    z = state
     dx = torch.empty((dy.shape[0], in_f), dtype=dy.dtype, device=dy.device)
     dcoef = torch.empty((out_f, k), dtype=torch.float32, device=dy.device)
     L = _lib.load()

@@ -201,74 +201,78 @@ linear_fwd.register_autograd(_lin_backward, setup_context=_lin_setup_context)
 
 # ------------------------------------------------------------------------------------------------ projected form
 @custom_op("rten::linear_project", mutates_args=())
-def linear_project(x: Tensor, dcoefs_size: int, out_features: int, seed: int) -> Tensor:
-    """``z = x @ Noise.T`` (tokens, k): what the forward product and the coef gradient of a matrix-coef layer need of x."""
-    return hip.linear_project(x, dcoefs_size, out_features, seed)
+def linear_project(x: Tensor, dcoefs_size: int, out_features: int, seed: int, coefs: Optional[Tensor]) -> Tensor:
+    """Projection state of ``x`` (a byte tensor): ``z = x @ Noise.T`` (tokens, k), what the forward product and the coef
+    gradient of a matrix-coef layer need of x, plus, when ``coefs`` is given, the transposed coefficients for the input
+    gradient."""
+    return hip.linear_project(x, dcoefs_size, out_features, seed, coefs)
 
 
 @linear_project.register_fake
-def _(x, dcoefs_size, out_features, seed):
-    return x.new_empty([x.shape[0], dcoefs_size])
+def _(x, dcoefs_size, out_features, seed, coefs):
+    # the size is the library's business; a fake tensor only needs some 1-D byte shape
+    nbytes = hip.linear_projection_bytes(x.shape[0], x.shape[1], out_features, dcoefs_size)
+    return x.new_empty([x.shape[0], -(-nbytes // x.shape[0])], dtype=torch.uint8)
 
 
 @custom_op("rten::linear_fwd_projected", mutates_args=())
-def linear_fwd_projected(z: Tensor, coefs: Tensor, in_features: int, seed: int, bias: Optional[Tensor]) -> Tensor:
-    return hip.linear_fwd_projected(z, coefs, in_features, seed, bias)
+def linear_fwd_projected(state: Tensor, coefs: Tensor, in_features: int, seed: int, bias: Optional[Tensor]) -> Tensor:
+    return hip.linear_fwd_projected(state, coefs, in_features, seed, bias)
 
 
 @linear_fwd_projected.register_fake
-def _(z, coefs, in_features, seed, bias):
-    return z.new_empty([z.shape[0], coefs.shape[0]])
+def _(state, coefs, in_features, seed, bias):
+    return coefs.new_empty([state.shape[0], coefs.shape[0]], dtype=torch.bfloat16)
 
 
 @custom_op("rten::linear_bwd_dcoef_projected", mutates_args=())
-def linear_bwd_dcoef_projected(dy: Tensor, z: Tensor, in_features: int, seed: int) -> Tensor:
-    return hip.linear_bwd_dcoef_projected(dy, z, in_features, seed)
+def linear_bwd_dcoef_projected(dy: Tensor, state: Tensor, dcoefs_size: int, in_features: int, seed: int) -> Tensor:
+    return hip.linear_bwd_dcoef_projected(dy, state, dcoefs_size, in_features, seed)
 
 
 @linear_bwd_dcoef_projected.register_fake
-def _(dy, z, in_features, seed):
-    return dy.new_empty([dy.shape[1], z.shape[1]], dtype=torch.float32)
+def _(dy, state, dcoefs_size, in_features, seed):
+    return dy.new_empty([dy.shape[1], dcoefs_size], dtype=torch.float32)
 
 
 @custom_op("rten::linear_bwd_projected", mutates_args=())
-def linear_bwd_projected(dy: Tensor, z: Tensor, coefs: Tensor, in_features: int, seed: int) -> List[Tensor]:
-    """``[dx, dcoef]`` of a matrix-coef bf16 layer from the saved projection, in one call."""
-    dx, dcoef = hip.linear_bwd_projected(dy, z, coefs, in_features, seed)
+def linear_bwd_projected(dy: Tensor, state: Tensor, coefs: Tensor, in_features: int, seed: int) -> List[Tensor]:
+    """``[dx, dcoef]`` of a matrix-coef bf16 layer from the projection state, in one call."""
+    dx, dcoef = hip.linear_bwd_projected(dy, state, coefs, in_features, seed)
     return [dx, dcoef]
 
 
 @linear_bwd_projected.register_fake
-def _(dy, z, coefs, in_features, seed):
+def _(dy, state, coefs, in_features, seed):
     return [dy.new_empty([dy.shape[0], in_features]), dy.new_empty([coefs.shape[0], coefs.shape[1]], dtype=torch.float32)]
 
 
 class _ProjectedLinear(torch.autograd.Function):
-    """``y = x @ W.T (+ bias)`` for a matrix-coef weight in bf16.  The forward pass computes ``z = x @ Noise.T`` once and
-    saves it for the backward pass in place of ``x`` (``k / in_features`` of its size); the reference's autograd saves
-    ``x`` and materialises ``W`` again (RandumbTensor.py:942-946, 979-990)."""
+    """``y = x @ W.T (+ bias)`` for a matrix-coef weight in bf16.  The forward pass computes the projection state
+    (``z = x @ Noise.T`` and the transposed coefficients) once and saves it for the backward pass in place of ``x``; the
+    reference's autograd saves ``x`` and materialises ``W`` again (RandumbTensor.py:942-946, 979-990)."""
 
     @staticmethod
     def forward(ctx, x, coefs, in_features, out_features, seed, bias):
-        z = linear_project(x, coefs.shape[1], out_features, seed)
-        ctx.save_for_backward(z, coefs)
+        state = linear_project(x, coefs.shape[1], out_features, seed, coefs)
+        ctx.save_for_backward(state, coefs)
         ctx.meta = (in_features, out_features, seed)
         ctx.bias_dtype = None if bias is None else bias.dtype
-        return linear_fwd_projected(z, coefs, in_features, seed, bias)
+        return linear_fwd_projected(state, coefs, in_features, seed, bias)
 
     @staticmethod
     def backward(ctx, dy):
-        z, coefs = ctx.saved_tensors
+        state, coefs = ctx.saved_tensors
         in_f, out_f, seed = ctx.meta
         dy = dy.contiguous()
         dx = dcoefs = dbias = None
         if ctx.needs_input_grad[0] and ctx.needs_input_grad[1]:
-            dx, dc = linear_bwd_projected(dy, z, coefs, in_f, seed)
+            dx, dc = linear_bwd_projected(dy, state, coefs, in_f, seed)
             dcoefs = dc.to(coefs.dtype)
         elif ctx.needs_input_grad[0]:
             dx = linear_bwd_dx(dy, coefs, in_f, out_f, in_f, 1, seed, None)
         elif ctx.needs_input_grad[1]:
-            dcoefs = linear_bwd_dcoef_projected(dy, z, in_f, seed).to(coefs.dtype)
+            dcoefs = linear_bwd_dcoef_projected(dy, state, coefs.shape[1], in_f, seed).to(coefs.dtype)
         if ctx.bias_dtype is not None and ctx.needs_input_grad[5]:
             dbias = dy.sum(0).to(ctx.bias_dtype)
         return dx, dcoefs, None, None, None, dbias
@@ -281,7 +285,7 @@ def linear(x: Tensor, coefs: Tensor, in_features: int, out_features: int, stride
     if (scale_bias is None and coefs.dim() == 2 and coefs.shape[0] == out_features and stride_o == in_features and stride_i == 1
             and x.is_cuda and x.dim() == 2 and x.dtype == torch.bfloat16 and coefs.dtype == torch.bfloat16
             and (bias is None or bias.dtype == torch.bfloat16)
-            and hip.linear_projection_supported(x.shape[0], in_features, out_features, coefs.shape[1])):
+            and hip.linear_projection_preferred(x.shape[0], in_features, out_features, coefs.shape[1])):
         return _ProjectedLinear.apply(x, coefs, in_features, out_features, seed, bias)
     return linear_fwd(x, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias, bias)
 

@@ -355,15 +355,18 @@ def test_linear_projected_form(hip, oracle, T, in_f, out_f, k, seed):
     xn, dyn, cn = x.float().numpy(), dy.float().numpy(), coef.float().numpy()
     assert hip.linear_projection_supported(T, in_f, out_f, k)
     xg, dyg, cg = x.cuda(), dy.cuda(), coef.cuda()
-    z = hip.linear_project(xg, k, out_f, seed)
+    z = hip.linear_project(xg, k, out_f, seed, coef=cg)
     noise = oracle.noise_2d(in_f, k, seed).astype(np.float64)          # noise[i, m] = noise(PRIME*i + m)
     want_z = xn.astype(np.float64) @ noise
-    assert z.shape == (T, k) and z.dtype == torch.bfloat16 and rel_l2(cpu(z), want_z) < 5e-3  # one bf16 rounding of z
+    pieces = hip.projection_unpack(z, in_f, out_f, k)                  # the state holds z twice and the coefficients once
+    assert pieces["z"].shape == (T, k) and rel_l2(cpu(pieces["z"]), want_z) < 5e-3  # one bf16 rounding of z
+    assert torch.equal(pieces["z_t"], pieces["z"].t()) and torch.equal(pieces["coef_t"], cg.t())
+    assert hip.projection_unpack(hip.linear_project(xg, k, out_f, seed), in_f, out_f, k)["coef_t"] is None
     bias = torch.randn(out_f).bfloat16()
     y = hip.linear_fwd_projected(z, cg, in_f, seed, bias=bias.cuda())
     want_y = oracle.linear_fwd(xn, cn, in_f, out_f, seed, bias=bias.float().numpy())
     assert y.shape == (T, out_f) and rel_l2(cpu(y), want_y) < BF16_TOL
-    dc = hip.linear_bwd_dcoef_projected(dyg, z, in_f, seed)
+    dc = hip.linear_bwd_dcoef_projected(dyg, z, k, in_f, seed)
     _, want_dc, _ = oracle.linear_bwd(xn, dyn, cn, in_f, out_f, seed)
     assert dc.shape == (out_f, k) and rel_l2(cpu(dc), want_dc) < BF16_TOL
     # the one-call entry points do the same arithmetic: equal up to the order of the fp32 atomics
@@ -380,10 +383,13 @@ def test_linear_bwd_projected_one_call(hip, oracle, T, in_f, out_f, k, seed):
     print(f"case bwd projected T={T} in={in_f} out={out_f} k={k}", flush=True)
     x, dy, coef = _inputs(T, in_f, out_f, k, True, torch.bfloat16, seed)
     want_dx, want_dc, _ = oracle.linear_bwd(x.float().numpy(), dy.float().numpy(), coef.float().numpy(), in_f, out_f, seed)
-    z = hip.linear_project(x.cuda(), k, out_f, seed)
     dyc, cc = dy.cuda(), coef.cuda()
+    z_plain = hip.linear_project(x.cuda(), k, out_f, seed)            # without the transposed coefficients: dy.C reads C through LDS
+    z = hip.linear_project(x.cuda(), k, out_f, seed, coef=cc)          # with them: dy.C takes them straight into registers
     dx_sep = hip.linear_bwd_dx(dyc, cc, in_f, out_f, in_f, 1, seed, algo=3)
-    dc_sep = hip.linear_bwd_dcoef_projected(dyc, z, in_f, seed)
+    dc_sep = hip.linear_bwd_dcoef_projected(dyc, z, k, in_f, seed)
+    dx_plain, dc_plain = hip.linear_bwd_projected(dyc, z_plain, cc, in_f, seed)
+    assert torch.equal(dx_plain, dx_sep) and rel_l2(cpu(dc_plain), want_dc) < BF16_TOL
     for ordered in (True, False):   # partial sums added in order (bigger workspace) / combined with atomics
         runs = []
         for _ in range(2):   # the second call finds dcoef's buffer dirty in the allocator: it must be overwritten by the call
@@ -404,7 +410,9 @@ def test_projected_form_rejects_what_it_cannot_do(hip):
     x = torch.randn(64, 100, device="cuda").bfloat16()
     with pytest.raises(RandumbHipError):
         hip.linear_project(x, 16, 32, 0)
-    z = torch.randn(64, 16, device="cuda").bfloat16()
+    with pytest.raises(ValueError):                                    # not a projection state
+        hip.linear_fwd_projected(torch.randn(64, 16, device="cuda").bfloat16(), torch.randn(32, 16, device="cuda").bfloat16(), 96, 0)
+    z = hip.linear_project(torch.randn(64, 96, device="cuda").bfloat16(), 16, 32, 0)
     c32 = torch.randn(32, 16, device="cuda")                          # fp32 coefficients: not in the projected forward
     with pytest.raises(RandumbHipError):
         hip.linear_fwd_projected(z, c32, 96, 0)

@@ -174,7 +174,7 @@ def test_default_layer_with_biases_trains(ra, oracle):
 def test_bf16_layer_matches_oracle(ra, oracle):
     print("case bf16 layer", flush=True)
     g = torch.Generator().manual_seed(3)
-    in_f, out_f, k, seed, T = 768, 384, 256, 0, 512
+    in_f, out_f, k, seed, T = 768, 512, 256, 0, 512   # k*(in+out) < in*out: the factored products are the cheaper form
     l = ra.SillyLinear(in_f, out_f, [k, k], [seed, 1], bias=False, matrix_coef=True)
     with torch.no_grad():
         l.weight_coef.copy_(torch.randn(out_f, k, generator=g) * math.sqrt(3 * 0.02**2 / k))

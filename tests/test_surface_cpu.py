@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_lib.SO_PATH)
     for name in declared:
         assert hasattr(lib, name), name
-    assert _lib.load().rdb_abi_version() == 3
+    assert _lib.load().rdb_abi_version() == 4
     assert ctypes.sizeof(_lib.LinearDesc) == 7 * 8 + 4 * 4
 
 
@@ -62,10 +62,24 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     d = desc(8192, 768, 3072, 256)
     r = ctypes.byref(d)
     zbytes = 8192 * 256 * 2
-    assert L.rdb_linear_projection_bytes(r) == zbytes
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, r) == zbytes
+
+    def state_bytes(tokens, out_f, k):
+        # header + z for the forward product (tokens to 32 when k <= 256) + z transposed (tokens to 64) + C transposed (out to 64)
+        up = lambda n, m: -(-n // m) * m
+        kpad = up(k, 64)
+        zf = up(tokens, 32) * kpad * 2 if k <= 256 else tokens * k * 2
+        return 256 + up(zf, 256) + up(up(tokens, 64) * kpad * 2, 256) + up(up(out_f, 64) * kpad * 2, 256)
+
+    assert state_bytes(8192, 3072, 256) == 256 + 2 * zbytes + 3072 * 256 * 2
+    assert L.rdb_linear_projection_bytes(r) == state_bytes(8192, 3072, 256)
+    info = (ctypes.c_int64 * 8)()
+    assert L.rdb_linear_projection_layout(r, info) == 0
+    assert list(info) == [256, 1, 256 + zbytes, 256 + 2 * zbytes, 256, 8192, 8192, 3072]
+    assert L.rdb_linear_projection_bytes(ctypes.byref(desc(1000, 200, 328, 72))) == state_bytes(1000, 328, 72)
+    assert L.rdb_linear_projection_bytes(ctypes.byref(desc(4096, 4096, 14336, 1024))) == state_bytes(4096, 14336, 1024)
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, r) == state_bytes(8192, 3072, 256)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, r) == zbytes
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DCOEF, r) == zbytes
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DCOEF, r) == state_bytes(8192, 3072, 256)
     # whole backward pass: dy.C plus the partial sums of the coefficient gradient, one [out x k] fp32 matrix per token split
     extra = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_PROJECTED, r) - zbytes
     assert extra > 0 and extra % (3072 * 256 * 4) == 0
@@ -82,21 +96,22 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     assert L.rdb_linear_projection_bytes(None) == 0
     # operands of 2^29 elements or more are outside the engine's 32-bit buffer addressing: no projected form
     assert L.rdb_linear_projection_bytes(ctypes.byref(desc(1 << 21, 768, 3072, 256))) == 0          # tokens*k = 2^29
-    assert L.rdb_linear_projection_bytes(ctypes.byref(desc((1 << 21) - 8, 768, 3072, 256))) == ((1 << 21) - 8) * 256 * 2
+    assert L.rdb_linear_projection_bytes(ctypes.byref(desc((1 << 21) - 8, 768, 3072, 256))) == 0    # tokens rounded up to 64
+    assert L.rdb_linear_projection_bytes(ctypes.byref(desc((1 << 21) - 64, 768, 3072, 256))) == state_bytes((1 << 21) - 64, 3072, 256)
     # fp32, small k: one partial [tokens x k] matrix per 256 values of the longer side
     f32 = desc(16, 4096, 4096, 16, act=_lib.RDB_F32, coef=_lib.RDB_F32)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(f32)) == 16 * 16 * 16 * 4
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(16, 4096, 4096, 128, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 0
 
     bad = ctypes.byref(desc(64, 100, 32, 16))
-    assert L.rdb_linear_project(None, None, 100, bad, None) == -5  # RDB_E_UNSUPPORTED
+    assert L.rdb_linear_project(None, None, 100, None, bad, None) == -5  # RDB_E_UNSUPPORTED
     assert b"projected form" in L.rdb_last_error_string()
-    assert L.rdb_linear_project(None, None, 768, r, None) == -1                                          # NULL pointers
+    assert L.rdb_linear_project(None, None, 768, None, r, None) == -1                                    # NULL pointers
     assert L.rdb_linear_fwd_projected(None, 3072, None, None, None, r, None) == -1
     assert L.rdb_linear_bwd_dcoef_projected(None, None, 3072, None, r, None) == -1
     assert L.rdb_linear_bwd_projected(None, 768, None, None, 3072, None, None, r, None, 0, None) == -1
     assert L.rdb_linear_fwd_projected(ctypes.c_void_p(16), 8, ctypes.c_void_p(16), ctypes.c_void_p(16), None, r, None) == -2  # ldy < out_f
-    assert L.rdb_linear_project(None, None, 768, None, None) == -1
+    assert L.rdb_linear_project(None, None, 768, None, None, None) == -1
 
 
 def test_view_ops_stay_lazy_and_only_change_shape_and_stride():
@@ -215,3 +230,22 @@ def test_materialised_weight_has_the_target_std(oracle):
     c = torch.randn(k, generator=g) * math.sqrt(3 * std**2 / k)
     W1 = oracle.materialize_fwd(c.numpy(), (64, 768), (768, 1), 5)
     assert abs(W1.std() / std - 1) < 0.1
+
+
+def test_projected_form_is_chosen_only_where_it_runs_and_pays():
+    """ops.linear takes the projected form only for layers whose activations fit the kernels' addressing and for which the
+    factored products are cheaper than forming the weight; everything else goes to rten::linear_fwd (whose backward cannot
+    be refused late, in the backward pass)."""
+    from randumb_amd import hip
+
+    assert hip.linear_projection_supported(8192, 768, 3072, 256) and hip.linear_projection_preferred(8192, 768, 3072, 256)
+    # tokens*out_f >= 2^29 (65536 tokens x 14336): the projection exists but dy would not fit the kernels' addressing
+    assert hip.linear_projection_bytes(65536, 4096, 14336, 256) > 0
+    assert not hip.linear_projection_supported(65536, 4096, 14336, 256)
+    assert not hip.linear_projection_preferred(65536, 4096, 14336, 256)
+    # tokens*in_f >= 2^29
+    assert not hip.linear_projection_supported(1 << 17, 4096, 64, 8)
+    # k >= in*out/(in+out): forming the weight is cheaper (768 -> 384 at k = 256 is exactly on the boundary)
+    assert hip.linear_projection_supported(512, 768, 384, 256) and not hip.linear_projection_preferred(512, 768, 384, 256)
+    assert hip.linear_projection_preferred(512, 768, 512, 256)
+    assert not hip.linear_projection_preferred(64, 8, 8, 8)
