@@ -10,6 +10,14 @@ namespace rdb {
 
 constexpr int B_BK = 64;
 
+// unroll and prefetch depth (in stages of 64) of the dy stream in the coefficient gradient's contraction
+#ifndef RDB_DC_TRIP
+#define RDB_DC_TRIP 2
+#define RDB_DC_DSTG 2
+#define RDB_DC_RD 2
+#define RDB_DC_BK 64
+#endif
+
 // ----------------------------------------------------------------------------------------------- dC = dy^T . z
 // tile: 128 output features (engine rows "a") x 128 coefficients (engine rows "b"), contraction over a token range
 constexpr int KD_BO = 128, KD_BM = 128;
@@ -28,11 +36,38 @@ struct DcParams {
 };
 
 // Stores (or adds) a block's 128 x 128 sums: acc[mi][ni][j] is o = o0 + wm*64 + mi*32 + 8*(j/4) + 4*g + j%4,
-// m = m0 + wn*64 + ni*32 + r (32 consecutive m per store: coalesced).
-__device__ __forceinline__ void dc_store(const DcParams &p, const f32x16 (&acc)[KD_BO / 64][KD_BM / 64], int o0, int m0, int split)
+// m = m0 + wn*64 + ni*32 + r.  Partial sums go through LDS (`lds`: 64 x 68 floats per wave, free on entry) so that every
+// lane stores 16 bytes of a row; atomic adds go straight from the registers (32 consecutive m per instruction).
+__device__ __forceinline__ void dc_store(const DcParams &p, const f32x16 (&acc)[KD_BO / 64][KD_BM / 64], bf16_t *lds, int o0, int m0, int split)
 {
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
     float *out = p.partial ? p.partial + (int64_t)split * p.out_f * p.k : p.dcoef;
+#ifdef RDB_DC_NO_STORE
+    if (p.partial) return;
+#endif
+    if (p.partial) {
+        // this wave's 64 (o) x 64 (m) quadrant, one 32-row half at a time: registers -> patch[o][m] (row stride 68 floats: the
+        // column writes of 32 lanes and the row reads of 16 lanes both spread over the banks) -> 16-byte row pieces
+        constexpr int LDP = 68;
+        float *patch = reinterpret_cast<float *>(lds) + wave * 32 * LDP;
+#pragma unroll
+        for (int mi = 0; mi < KD_BO / 64; ++mi) {
+#pragma unroll
+            for (int ni = 0; ni < KD_BM / 64; ++ni)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) patch[(8 * (j / 4) + 4 * g + (j % 4)) * LDP + ni * 32 + r] = acc[mi][ni][j];
+            __builtin_amdgcn_wave_barrier();   // LDS serves a wave's instructions in order: the reads see these writes
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int row = q * 4 + (lane >> 4), col = (lane & 15) * 4;   // 16 lanes cover a row of 64 floats
+                const int o = o0 + wm * 64 + mi * 32 + row, m = m0 + wn * 64 + col;
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(patch + row * LDP + col);
+                if (o < p.out_f && m < p.k) *reinterpret_cast<f32x4 *>(out + (int64_t)o * p.k + m) = v;   // k is a multiple of 8
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+        return;
+    }
 #pragma unroll
     for (int ni = 0; ni < KD_BM / 64; ++ni) {
         const int m = m0 + wn * 64 + ni * 32 + r;
@@ -42,12 +77,7 @@ __device__ __forceinline__ void dc_store(const DcParams &p, const f32x16 (&acc)[
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
                 const int o = o0 + wm * 64 + mi * 32 + 8 * (j / 4) + 4 * g + (j % 4);
-                if (o < p.out_f) {
-                    if (p.partial)
-                        out[(int64_t)o * p.k + m] = acc[mi][ni][j];
-                    else
-                        unsafeAtomicAdd(out + (int64_t)o * p.k + m, acc[mi][ni][j]);
-                }
+                if (o < p.out_f) unsafeAtomicAdd(out + (int64_t)o * p.k + m, acc[mi][ni][j]);
             }
     }
 }
@@ -70,7 +100,7 @@ __device__ __forceinline__ void dc_block(const DcParams &p, bf16_t *lds, int blo
     GlobalOperand<KD_BO, B_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
     GlobalOperand<KD_BM, B_BK, M_CONT> opz = {p.z, (int64_t)p.k, m0, p.k, t_end, (int64_t)p.tokens * p.k};
     gemm_mainloop<KD_BO, KD_BM, B_BK, 1, 1>(acc, lds, opdy, opz, t_begin, (t_end - t_begin + B_BK - 1) / B_BK);
-    dc_store(p, acc, o0, m0, split);
+    dc_store(p, acc, lds, o0, m0, split);
     RDB_STAMP(3);
 }
 
@@ -90,12 +120,13 @@ __device__ __forceinline__ void dc_block_direct(const DcParams &p, bf16_t *lds, 
 #pragma unroll
         for (int ni = 0; ni < KD_BM / 64; ++ni) acc[mi][ni] = zero16();
     // staged "A": dy[tok][o], tile rows = o (contiguous in memory), contraction = tokens
-    GlobalOperand<KD_BO, B_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
+    GlobalOperand<KD_BO, RDB_DC_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
     // direct "B": z^T fragments of this wave's 64 coefficients
     FragSource fz;
     fz.init(p.ztf, (int64_t)p.kpad * p.tsteps * 16, p.tsteps, (m0 + wn * 64) >> 5, lane);
-    direct_mainloop<KD_BO / 64, KD_BM / 64, true, 2, 2>(acc, lds, opdy, fz, t_begin, (t_end - t_begin + B_BK - 1) / B_BK, wm * 64, lane);
-    dc_store(p, acc, o0, m0, split);
+    direct_mainloop<KD_BO / 64, KD_BM / 64, RDB_DC_BK / 16, true, RDB_DC_TRIP, RDB_DC_DSTG, RDB_DC_RD>(acc, lds, opdy, fz, t_begin, (t_end - t_begin + RDB_DC_BK - 1) / RDB_DC_BK,
+                                                                                                     wm * 64, lane);
+    dc_store(p, acc, lds, o0, m0, split);
     RDB_STAMP(3);
 }
 

@@ -80,43 +80,47 @@ struct FragSource {
     }
 };
 
-// One stage (BK = 64: four k-steps) with the staged operand in LDS buffer `cur` and the direct operand's fragments in
-// ring[U * 4 .. U * 4 + 3].  Between the MFMAs: the staged operand's registers (the stage after this one) go to the idle
-// buffer and are refilled with stage next_s; the ring slots just used are refilled with k-steps ring_next .. ring_next + 3.
-template <int SI, int DI, bool STAGED_IS_A, int U, int RING, bool STORE, bool RELOAD, class PS>
+// One stage (KS k-steps of 16) with the staged operand in LDS buffer `cur` and the direct operand's fragments in
+// ring[U * KS .. U * KS + KS - 1].  Between the MFMAs: the staged operand's registers (the stage after this one) go to the idle
+// buffer and are refilled with stage next_s; the ring slots just used are refilled with k-steps ring_next .. ring_next + KS - 1.
+template <int SI, int DI, int KS, bool STAGED_IS_A, int U, int RING, bool STORE, bool RELOAD, class PS>
 __device__ __forceinline__ void direct_stage(f32x16 (&acc)[STAGED_IS_A ? SI : DI][STAGED_IS_A ? DI : SI], const bf16_t *__restrict__ cur,
                                              bf16_t *__restrict__ oth, f32x4 (&rs)[PS::Tile::PER_THREAD], const PS &ps, int next_s,
                                              bf16x8 (&ring)[RING][DI], const FragSource &fd, int ring_next, int srow, int lane)
 {
     typedef typename PS::Tile TS;
-    constexpr int KS = 4;
-    constexpr int FRAG_OPS = SI * (TS::LAYOUT_ID == M_CONT ? 2 : 1);
-    constexpr int COPY_OPS = ((STORE ? 1 : 0) + (RELOAD ? 1 : 0)) * ((TS::PER_THREAD + KS - 1) / KS) + (RELOAD ? DI : 0);
-    constexpr int MEM_PER_MFMA = (FRAG_OPS + COPY_OPS + SI * DI - 1) / (SI * DI);
-    bf16x8 fs[2][SI];
+    constexpr int COPY_OPS = ((STORE ? 1 : 0) + (RELOAD ? 1 : 0)) * ((TS::PER_THREAD + KS - 1) / KS) + (RELOAD ? DI : 0) +
+                             (KS > 4 ? SI * (TS::LAYOUT_ID == M_CONT ? 2 : 1) : 0);
+    constexpr int MEM_PER_MFMA = (COPY_OPS + SI * DI - 1) / (SI * DI);
+    // fragment reads run FA k-steps ahead of the MFMAs that use them (LDS returns them in order, each k-step waits for its own
+    // only): a k-step is 64 to 128 clocks of matrix work, a fragment read takes longer than that to come back
+    constexpr int FA = KS < 4 ? KS : 4;
+    bf16x8 fs[KS][SI];
 #pragma unroll
-    for (int i = 0; i < SI; ++i) fs[0][i] = TS::frag(cur, srow + i * 32, 0, lane);
+    for (int ks = 0; ks < FA; ++ks)
+#pragma unroll
+        for (int i = 0; i < SI; ++i) fs[ks][i] = TS::frag(cur, srow + i * 32, ks, lane);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-        const int c = ks & 1, n = c ^ 1;
+        if (ks + FA < KS) {
+#pragma unroll
+            for (int i = 0; i < SI; ++i) fs[ks + FA][i] = TS::frag(cur, srow + i * 32, ks + FA, lane);
+        }
 #pragma unroll
         for (int p = 0; p < TS::PER_THREAD; ++p)
             if (p % KS == ks) {
                 if (STORE) TS::store_piece(oth, rs[p], p);
                 if (RELOAD) ps.load_piece(rs[p], p, next_s);
             }
-        if (ks + 1 < KS) {
-#pragma unroll
-            for (int i = 0; i < SI; ++i) fs[n][i] = TS::frag(cur, srow + i * 32, ks + 1, lane);
-        }
 #pragma unroll
         for (int i = 0; i < SI; ++i)
 #pragma unroll
             for (int j = 0; j < DI; ++j) {
                 if (STAGED_IS_A)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fs[c][i], ring[U * KS + ks][j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fs[ks][i], ring[U * KS + ks][j], acc[i][j], 0, 0, 0);
                 else
-                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[U * KS + ks][j], fs[c][i], acc[j][i], 0, 0, 0);
+                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ring[U * KS + ks][j], fs[ks][i], acc[j][i], 0, 0, 0);
             }
         if (RELOAD) {
 #pragma unroll
@@ -132,19 +136,21 @@ __device__ __forceinline__ void direct_stage(f32x16 (&acc)[STAGED_IS_A ? SI : DI
     __syncthreads();
 }
 
-// Main loop: D += S . Dm over `nstage` stages of 64 starting at contraction index k_begin (a multiple of 16).
+// Main loop: D += S . Dm over `nstage` stages of BK = 16 KS starting at contraction index k_begin (a multiple of 16).
 // S: staged operand (provider PS, rows split over WS waves, SI = rows / (32 WS) fragments per wave);
 // Dm: direct operand, DI row blocks per wave, fragments of k-step q at fd.load(j, q) (absolute k-step numbers).
-// TRIP (2 or 4): stages per unrolled trip = depth of the ring of direct fragments, in stages; DSTG (1 or 2): how many
-// stages ahead of the LDS copy the staged operand's registers are loaded.  `lds` holds 2 * PS::Tile::LDS_ELEMS elements.
-template <int SI, int DI, bool STAGED_IS_A, int TRIP, int DSTG, class PS>
+// TRIP (2 or 4): stages per unrolled trip; DSTG (1, 2 or 4, dividing TRIP): how many stages ahead of the LDS copy the staged
+// operand's registers are loaded (it comes from HBM: a load takes several stages to return under load); RD (1 or 2, dividing
+// TRIP): depth of the ring of direct fragments, in stages (they come from L2).  `lds` holds 2 * PS::Tile::LDS_ELEMS elements.
+template <int SI, int DI, int KS, bool STAGED_IS_A, int TRIP, int DSTG, int RD, class PS>
 __device__ __forceinline__ void direct_mainloop(f32x16 (&acc)[STAGED_IS_A ? SI : DI][STAGED_IS_A ? DI : SI], bf16_t *__restrict__ lds, PS &ps,
                                                 const FragSource &fd, int k_begin, int nstage, int srow, int lane)
 {
     typedef typename PS::Tile TS;
     static_assert(TRIP == 2 || TRIP == 4, "the LDS double buffer needs an even trip");
-    static_assert(DSTG == 1 || DSTG == 2, "prefetch depth of the staged operand");
-    constexpr int RING = TRIP * 4, STAGE = TS::LDS_ELEMS;
+    static_assert((DSTG == 1 || DSTG == 2 || DSTG == 4) && TRIP % DSTG == 0, "prefetch depth of the staged operand");
+    static_assert((RD == 1 || RD == 2) && TRIP % RD == 0, "depth of the fragment ring");
+    constexpr int RING = RD * KS, STAGE = TS::LDS_ELEMS;
     if (nstage <= 0) return;
     RDB_STAMP(0);
     ps.init(k_begin);
@@ -165,36 +171,40 @@ __device__ __forceinline__ void direct_mainloop(f32x16 (&acc)[STAGED_IS_A ? SI :
     __syncthreads();
     RDB_STAMP(1);
     const int nround = (nstage + TRIP - 1) / TRIP * TRIP;
+    // stage s + u: LDS buffer u % 2; register slot (u + 1) % DSTG holds stage s + u + 1 and is refilled with stage s + u + 1 + DSTG;
+    // ring slots (u % RD) * KS .. hold its k-steps and are refilled with those of stage s + u + RD
+#define RDB_DIRECT_STAGE(U, ST, RL, NEXT_S, NEXT_Q)                                                                                  \
+    direct_stage<SI, DI, KS, STAGED_IS_A, (U) % RD, RING, ST, RL>(acc, lds + ((U) & 1) * STAGE, lds + (((U) & 1) ^ 1) * STAGE, rs[((U) + 1) % DSTG], \
+                                                               ps, NEXT_S, ring, fd, NEXT_Q, srow, lane)
     int s = 0;
     for (; s + TRIP < nround; s += TRIP) {
-#pragma unroll
-        for (int u = 0; u < TRIP; ++u) {
-            bf16_t *cur = lds + (u & 1) * STAGE, *oth = lds + ((u & 1) ^ 1) * STAGE;
-            if (u == 0)
-                direct_stage<SI, DI, STAGED_IS_A, 0, RING, true, true>(acc, cur, oth, rs[1 % DSTG], ps, s + 1 + DSTG, ring, fd, q0 + (s + TRIP) * 4, srow, lane);
-            else if (u == 1)
-                direct_stage<SI, DI, STAGED_IS_A, 1, RING, true, true>(acc, cur, oth, rs[2 % DSTG], ps, s + 2 + DSTG, ring, fd, q0 + (s + 1 + TRIP) * 4, srow, lane);
-            else if (u == 2)
-                direct_stage<SI, DI, STAGED_IS_A, 2 % TRIP, RING, true, true>(acc, cur, oth, rs[3 % DSTG], ps, s + 3 + DSTG, ring, fd, q0 + (s + 2 + TRIP) * 4, srow, lane);
-            else
-                direct_stage<SI, DI, STAGED_IS_A, 3 % TRIP, RING, true, true>(acc, cur, oth, rs[4 % DSTG], ps, s + 4 + DSTG, ring, fd, q0 + (s + 3 + TRIP) * 4, srow, lane);
+        RDB_DIRECT_STAGE(0, true, true, s + 1 + DSTG, q0 + (s + RD) * KS);
+        RDB_DIRECT_STAGE(1, true, true, s + 2 + DSTG, q0 + (s + 1 + RD) * KS);
+        if (TRIP == 4) {
+            RDB_DIRECT_STAGE(2, true, true, s + 3 + DSTG, q0 + (s + 2 + RD) * KS);
+            RDB_DIRECT_STAGE(3, true, true, s + 4 + DSTG, q0 + (s + 3 + RD) * KS);
         }
     }
-    // last trip: nothing it would reload is needed, and its last stage has nothing left to hand to LDS
-#pragma unroll
-    for (int u = 0; u < TRIP; ++u) {
-        bf16_t *cur = lds + (u & 1) * STAGE, *oth = lds + ((u & 1) ^ 1) * STAGE;
-        if (u == 0)
-            direct_stage<SI, DI, STAGED_IS_A, 0, RING, true, false>(acc, cur, oth, rs[1 % DSTG], ps, 0, ring, fd, 0, srow, lane);
-        else if (u == 1 && TRIP == 2)
-            direct_stage<SI, DI, STAGED_IS_A, 1, RING, false, false>(acc, cur, oth, rs[2 % DSTG], ps, 0, ring, fd, 0, srow, lane);
-        else if (u == 1)
-            direct_stage<SI, DI, STAGED_IS_A, 1, RING, true, false>(acc, cur, oth, rs[2 % DSTG], ps, 0, ring, fd, 0, srow, lane);
-        else if (u == 2)
-            direct_stage<SI, DI, STAGED_IS_A, 2 % TRIP, RING, true, false>(acc, cur, oth, rs[3 % DSTG], ps, 0, ring, fd, 0, srow, lane);
-        else
-            direct_stage<SI, DI, STAGED_IS_A, 3 % TRIP, RING, false, false>(acc, cur, oth, rs[4 % DSTG], ps, 0, ring, fd, 0, srow, lane);
+    // last trip: the staged operand has nothing more to load (everything past the end reads as zeros anyway), the ring is
+    // refilled only as far as the trip itself still needs, and the last stage has nothing left to hand to LDS
+    if (TRIP == 2) {
+        if (RD == 2) RDB_DIRECT_STAGE(0, true, false, 0, 0);
+        else RDB_DIRECT_STAGE(0, true, true, nround, q0 + (s + 1) * KS);   // the ring holds one stage: the last one is still to be fetched
+        RDB_DIRECT_STAGE(1, false, false, 0, 0);
+    } else {
+        if (RD == TRIP) {
+            RDB_DIRECT_STAGE(0, true, false, 0, 0);
+            RDB_DIRECT_STAGE(1, true, false, 0, 0);
+        } else {   // the ring holds stages s, s + 1 (RD = 2) or s (RD = 1): stages s + RD .. s + 3 are still to be fetched
+            RDB_DIRECT_STAGE(0, true, true, nround, q0 + (s + RD) * KS);
+            if (RD == 1) RDB_DIRECT_STAGE(1, true, true, nround, q0 + (s + 1 + RD) * KS);
+            else RDB_DIRECT_STAGE(1, true, true, nround, q0 + (s + 1 + RD) * KS);
+        }
+        if (RD == 1) RDB_DIRECT_STAGE(2, true, true, nround, q0 + (s + 2 + RD) * KS);
+        else RDB_DIRECT_STAGE(2, true, false, 0, 0);
+        RDB_DIRECT_STAGE(3, false, false, 0, 0);
     }
+#undef RDB_DIRECT_STAGE
     RDB_STAMP(2);
 }
 

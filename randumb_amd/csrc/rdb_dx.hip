@@ -73,10 +73,14 @@ __device__ __forceinline__ void dyc_block_direct(const DyCParams &p, bf16_t *lds
     f32x16 acc[1][K1_BT / 32];
 #pragma unroll
     for (int ni = 0; ni < K1_BT / 32; ++ni) acc[0][ni] = zero16();
-    GlobalOperand<K1_BT, X_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
+    // stages of 128: half as many barriers (and waits for the first fragments after them) as with 64, for the same LDS
+    constexpr int BKD = 128;
+    GlobalOperand<K1_BT, BKD, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
     FragSource fc;
     fc.init(p.ctf, (int64_t)p.kpad * p.osteps * 16, p.osteps, (m0 >> 5) + wave, lane);
-    direct_mainloop<K1_BT / 32, 1, false, 2, 2>(acc, lds, opdy, fc, 0, (p.out_f + X_BK - 1) / X_BK, 0, lane);
+    // these blocks are the longer ones of the launch they share with the coefficient-gradient blocks: their waves issue first
+    __builtin_amdgcn_s_setprio(2);
+    direct_mainloop<K1_BT / 32, 1, BKD / 16, false, 2, 2, 1>(acc, lds, opdy, fc, 0, (p.out_f + BKD - 1) / BKD, 0, lane);
     if (p.frag_ksteps)
         store_tile_bf16_frag<K1_BC, K1_BT, 4>(acc, lds, p.t, p.frag_ksteps, m0, p.frag_ksteps * 16, tok0, (p.tokens + 31) / 32 * 32,
                                               4.656612873077392578125e-10f);

@@ -44,7 +44,10 @@ template <int ROWS, int BK, int LAYOUT> struct OperandTile {
     //         chunk from each of 16 consecutive rows, which the swizzle spreads over all 16 chunk positions of a row pair.
     // M_CONT: rows (one per k) of ROWS elements plus 64 bytes of padding, so the 4 k-rows one ds_read_b64_tr_b16 phase
     //         touches (64 bytes each) tile the 64 banks exactly.
-    static_assert(LAYOUT == M_CONT || BK == 64, "the swizzled K_CONT layout is laid out for 64-element rows");
+    // K_CONT with BK = 128: rows of 256 bytes, chunk c of row r at position c ^ (r & 15): a read phase (one chunk from each
+    //         of 16 consecutive rows) and a store phase (one whole row) both touch all 16 chunk positions once.
+    static_assert(LAYOUT == M_CONT || BK == 64 || BK == 128, "the swizzled K_CONT layout is laid out for rows of 64 or 128 elements");
+    __device__ static __forceinline__ int swz(int row) { return BK == 64 ? ((row >> 1) & 7) : (row & 15); }
     static constexpr int PAD = (LAYOUT == K_CONT) ? 0 : 32;
     static constexpr int LAYOUT_ID = LAYOUT;
     static constexpr int LD = (LAYOUT == K_CONT) ? (BK + PAD) : (ROWS + PAD);     // LDS row stride, elements
@@ -96,7 +99,7 @@ template <int ROWS, int BK, int LAYOUT> struct OperandTile {
         int off;
         if (LAYOUT == K_CONT) {
             const int row = idx / (BK / 8), c = idx % (BK / 8);
-            off = row * LD + ((c ^ ((row >> 1) & 7)) * 8);
+            off = row * LD + ((c ^ swz(row)) * 8);
         } else {
             off = (idx / (ROWS / 8)) * LD + (idx % (ROWS / 8)) * 8;
         }
@@ -116,7 +119,7 @@ template <int ROWS, int BK, int LAYOUT> struct OperandTile {
         const int r = lane & 31, g = lane >> 5;
         if (LAYOUT == K_CONT) {
             // rb is a multiple of 32, so the swizzle depends on the lane only
-            f.v = *reinterpret_cast<const bf16x8 *>(lds + (rb + r) * LD + (((ks * 2 + g) ^ ((r >> 1) & 7)) * 8));
+            f.v = *reinterpret_cast<const bf16x8 *>(lds + (rb + r) * LD + (((ks * 2 + g) ^ swz(r)) * 8));
         } else {
             // 16-lane group q = (lane / 16) & 1 covers rows rb + 16q .. +15; source lane s of the group addresses
             // k = kb + s / 4, rows 4*(s % 4) .. +3; the result lane c receives rows' column c for k = kb .. kb+3.
