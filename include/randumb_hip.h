@@ -158,6 +158,17 @@ int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, const void 
                    const void *scale_bias, const void *bias, const rdb_linear_desc *desc, void *workspace,
                    int64_t workspace_bytes, void *stream);
 
+/* rdb_linear_fwd for callers that can neither allocate a workspace nor hand one over (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid allocation); it has no counterpart in the reference.  Same arguments and results as
+ * rdb_linear_fwd without the workspace: the scratch its kernels use (the projection of x) lies in a static device array of
+ * the library, rdb_linear_fwd_static_max_bytes() = 16 MiB per device.  A layer whose kernels would use more returns
+ * RDB_E_WORKSPACE and launches nothing (8192 tokens at k = 256, out_f = 3072 use 9.5 MiB).  The call allocates and frees
+ * nothing.  All calls on one device share the array: calls that overlap in time on one device (different streams or
+ * threads) race; on one stream they are ordered.  Nothing in the array has to be cleared between calls. */
+int rdb_linear_fwd_static(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef,
+                          const void *scale_bias, const void *bias, const rdb_linear_desc *desc, void *stream);
+int64_t rdb_linear_fwd_static_max_bytes(void);
+
 /* Replaces autograd's MmBackward on the materialised weight (second materialize() + dense product).
  * dx[t, i] = sum_o dy[t, o] * W[o, i]. */
 int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef,

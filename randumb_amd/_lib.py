@@ -32,6 +32,8 @@ EXPORTS = [
     "rdb_embed_bwd_workspace_bytes",
     "rdb_linear_workspace_bytes",
     "rdb_linear_fwd",
+    "rdb_linear_fwd_static",
+    "rdb_linear_fwd_static_max_bytes",
     "rdb_linear_bwd_dx",
     "rdb_linear_bwd_dcoef",
     "rdb_linear_projection_bytes",
@@ -101,6 +103,10 @@ def load() -> ctypes.CDLL:
     L.rdb_linear_workspace_bytes.argtypes = [ci, dp]
     L.rdb_linear_workspace_bytes.restype = i64
     L.rdb_linear_fwd.argtypes = [vp, i64, vp, i64, vp, vp, vp, dp, vp, i64, vp]
+    L.rdb_linear_fwd_static.argtypes = [vp, i64, vp, i64, vp, vp, vp, dp, vp]
+    L.rdb_linear_fwd_static.restype = ci
+    L.rdb_linear_fwd_static_max_bytes.argtypes = []
+    L.rdb_linear_fwd_static_max_bytes.restype = i64
     L.rdb_linear_bwd_dx.argtypes = [vp, i64, vp, i64, vp, vp, dp, vp, i64, vp]
     L.rdb_linear_bwd_dcoef.argtypes = [vp, vp, vp, i64, vp, i64, dp, vp, i64, vp]
     L.rdb_linear_projection_bytes.argtypes = [dp]

@@ -521,6 +521,49 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
                : launch(linear_dcoef_kernel<float, false>, grid, smem_dcoef<float>(), s, p, "linear_dcoef_kernel<f32,vector>");
 }
 
+// ----------------------------------------------------------------------------------------------- forward without a caller's workspace
+// Scratch of rdb_linear_fwd_static: one copy per device that loads this library, held until the process ends.
+#define RDB_STATIC_SCRATCH_BYTES (16ll << 20)
+static __device__ __align__(256) unsigned char rdb_static_scratch[RDB_STATIC_SCRATCH_BYTES];
+
+// Device address of the scratch array on the current device.  In host code the array's name is only a handle: the address
+// is asked for once per device (with that device current) and kept.
+static int static_scratch_ptr(void **out)
+{
+    static void *ptrs[64] = {nullptr};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return set_error((int)e, "rdb_linear_fwd_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= 64) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd_static: device index %d outside 0..63", dev);
+    void *p = __atomic_load_n(&ptrs[dev], __ATOMIC_ACQUIRE);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(rdb_static_scratch));
+        if (e != hipSuccess || !p) return set_error(e != hipSuccess ? (int)e : RDB_E_UNSUPPORTED, "rdb_linear_fwd_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        __atomic_store_n(&ptrs[dev], p, __ATOMIC_RELEASE);   // every thread that gets here asks for the same address
+    }
+    *out = p;
+    return RDB_OK;
+}
+
+extern "C" int64_t rdb_linear_fwd_static_max_bytes(void) { return RDB_STATIC_SCRATCH_BYTES; }
+
+extern "C" int rdb_linear_fwd_static(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias,
+                                     const void *bias, const rdb_linear_desc *d, void *stream)
+{
+    int rc = check_desc("rdb_linear_fwd_static", d);
+    if (rc) return rc;
+    const int64_t need = rdb_linear_workspace_bytes(RDB_OP_LINEAR_FWD, d);
+    if (need > RDB_STATIC_SCRATCH_BYTES)
+        return set_error(RDB_E_WORKSPACE, "rdb_linear_fwd_static: this layer's kernels use %lld bytes of scratch, the library's static scratch holds "
+                                          "%lld: call rdb_linear_fwd with a workspace of the caller's", (long long)need, (long long)RDB_STATIC_SCRATCH_BYTES);
+    void *scratch = nullptr;
+    if (need > 0) {
+        rc = static_scratch_ptr(&scratch);
+        if (rc) return rc;
+    }
+    return rdb_linear_fwd(y, ldy, x, ldx, coef, scale_bias, bias, d, scratch, need > 0 ? RDB_STATIC_SCRATCH_BYTES : 0, stream);
+}
+
 // ----------------------------------------------------------------------------------------------- projected entry points
 static int check_projected(const char *who, const rdb_linear_desc *d)
 {
