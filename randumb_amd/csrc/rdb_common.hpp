@@ -12,6 +12,7 @@ namespace rdb {
 // ----------------------------------------------------------------------------------------------- errors
 int set_error(int code, const char *fmt, ...);  // records the message for rdb_last_error_string, returns code
 int check_launch(const char *what);             // hipGetLastError -> positive code + message
+int reserve_lds(const void *kernel, size_t smem, const char *name);  // dynamic-LDS limit of a kernel, set once per device
 
 // ----------------------------------------------------------------------------------------------- noise
 // Squirrel5 constants and the row/column mixing prime (reference: src/rten_cpp/RandumbTensor.py:140-145,

@@ -166,9 +166,7 @@ int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, co
     const size_t main_bytes = 2 * (TA::LDS_ELEMS + TB::LDS_ELEMS) * sizeof(bf16_t);
     const size_t epi_bytes = (size_t)(DC_BO + DC_MC) * (DC_BI + 8) * sizeof(bf16_t);
     const size_t smem = main_bytes > epi_bytes ? main_bytes : epi_bytes;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(linear_dcoef_fast_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)smem);
-    if (e != hipSuccess) return set_error((int)e, "linear_dcoef_fast_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+    if (int rl = reserve_lds(reinterpret_cast<const void *>(linear_dcoef_fast_kernel), smem, "linear_dcoef_fast_kernel")) return rl;
     linear_dcoef_fast_kernel<<<xcd_grid_size(ti * to * splits), 256, smem, s>>>(p);
     return check_launch("linear_dcoef_fast_kernel");
 }

@@ -328,8 +328,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
         if (tn_stationary_ok(d, lddx)) a.dyc.frag_ksteps = (int)cdiv(d->k, 64) * 4;   // the t.N kernel below keeps t in registers
         a.dc_blocks = xcd_grid_size(dc_items);
         size_t smem = smem_dc > smem_dyc ? smem_dc : smem_dyc;
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dc_dyc_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return set_error((int)e, "bwd_dc_dyc_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+        if (int rl = reserve_lds(reinterpret_cast<const void *>(bwd_dc_dyc_kernel), smem, "bwd_dc_dyc_kernel")) return rl;
         bwd_dc_dyc_kernel<<<a.dc_blocks + xcd_grid_size(p1.tiles_c * p1.tiles_t), 256, smem, s>>>(a);
         int rc = check_launch("bwd_dc_dyc_kernel");
         if (rc) return rc;
@@ -351,8 +350,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
             const size_t smem_s = stationary_smem(kg);
             const void *fn = kg == 1 ? (const void *)bwd_tns_red_kernel<1> : kg == 2 ? (const void *)bwd_tns_red_kernel<2>
                            : kg == 3 ? (const void *)bwd_tns_red_kernel<3> : (const void *)bwd_tns_red_kernel<4>;
-            e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_s);
-            if (e != hipSuccess) return set_error((int)e, "bwd_tns_red_kernel: cannot reserve %zu bytes of LDS: %s", smem_s, hipGetErrorString(e));
+            if (int rl = reserve_lds(fn, smem_s, "bwd_tns_red_kernel")) return rl;
             const dim3 grid(bs.tn_blocks + rblocks), block(ST_THREADS);
             switch (kg) {
             case 1: bwd_tns_red_kernel<1><<<grid, block, smem_s, s>>>(bs); break;
@@ -370,8 +368,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
         if (red_blocks > num_cus) red_blocks = num_cus;
         if (red_blocks < 1) red_blocks = 1;
         if (direct) red_blocks = 0;
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_tn_red_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_tn);
-        if (e != hipSuccess) return set_error((int)e, "bwd_tn_red_kernel: cannot reserve %zu bytes of LDS: %s", smem_tn, hipGetErrorString(e));
+        if (int rl = reserve_lds(reinterpret_cast<const void *>(bwd_tn_red_kernel), smem_tn, "bwd_tn_red_kernel")) return rl;
         bwd_tn_red_kernel<<<b.tn_blocks + red_blocks, 256, smem_tn, s>>>(b);
         return check_launch("bwd_tn_red_kernel");
     }
@@ -386,8 +383,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
     const int tn_items = make_tn_params(p.tn, dx, lddx, workspace, d);
     p.dc_blocks = xcd_grid_size(dc_items);
     const size_t smem = smem_dc > smem_tn ? smem_dc : smem_tn;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dc_tn_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return set_error((int)e, "bwd_dc_tn_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+    if (int rl = reserve_lds(reinterpret_cast<const void *>(bwd_dc_tn_kernel), smem, "bwd_dc_tn_kernel")) return rl;
     bwd_dc_tn_kernel<<<p.dc_blocks + xcd_grid_size(tn_items), 256, smem, s>>>(p);
     return check_launch("bwd_dc_tn_kernel");
 }

@@ -454,8 +454,7 @@ template <int BM, int BN, int BK, int LA, int LB> inline size_t engine_smem()
 // Launches an engine kernel over `items` work items (one 256-thread block each, XCD-aware numbering).
 template <class K, class P> inline int launch_engine(K kernel, const P &p, int items, size_t smem, hipStream_t s, const char *name)
 {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return set_error((int)e, "%s: cannot reserve %zu bytes of LDS: %s", name, smem, hipGetErrorString(e));
+    if (int rl = reserve_lds(reinterpret_cast<const void *>(kernel), smem, name)) return rl;
     kernel<<<xcd_grid_size(items), 256, smem, s>>>(p);
     return check_launch(name);
 }

@@ -351,8 +351,7 @@ static WeightSpec make_spec(const rdb_linear_desc *d, const void *coef, const vo
 template <typename K> static int launch(K kernel, dim3 grid, size_t smem, hipStream_t s, const LinParams &p, const char *name)
 {
     if (smem > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (e != hipSuccess) return set_error((int)e, "%s: cannot reserve %zu bytes of LDS: %s", name, smem, hipGetErrorString(e));
+        if (int rl = reserve_lds(reinterpret_cast<const void *>(kernel), smem, name)) return rl;
     }
     kernel<<<grid, TILE_THREADS, smem, s>>>(p);
     return check_launch(name);

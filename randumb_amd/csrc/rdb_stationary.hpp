@@ -312,8 +312,7 @@ inline int make_stationary_grid(StParams &q, int64_t tokens, int64_t out_f, int 
 
 template <class K> inline int launch_stationary(K kernel, const StParams &q, int items, size_t smem, hipStream_t s, const char *name)
 {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return set_error((int)e, "%s: cannot reserve %zu bytes of LDS: %s", name, smem, hipGetErrorString(e));
+    if (int rl = reserve_lds(reinterpret_cast<const void *>(kernel), smem, name)) return rl;
     kernel<<<xcd_grid_size(items), ST_THREADS, smem, s>>>(q);
     return check_launch(name);
 }

@@ -301,8 +301,7 @@ template <int BO, int CMODE> static int launch_strip_mode(const StripParams &p, 
 {
     const size_t smem = (size_t)BO * p.in_pad * sizeof(bf16_t);
     auto kern = linear_fwd_strip_kernel<BO, 4, CMODE>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return set_error((int)e, "linear_fwd_strip_kernel: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+    if (int rl = reserve_lds(reinterpret_cast<const void *>(kern), smem, "linear_fwd_strip_kernel")) return rl;
     kern<<<strips * p.splits, 256, smem, s>>>(p);
     return check_launch("linear_fwd_strip_kernel");
 }
