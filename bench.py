@@ -483,8 +483,23 @@ def main():
             return {"fwd_strip": t["fwd"], "dx_noise_strip": t["dx"], "dcoef_dw_tile": t["dcoef"],
                     "step": round(t["fwd"] + t["dx"] + t["dcoef"], 4), "dx_tile": onecall_ms(_lib.RDB_ALGO_TILE)["dx"]}
 
+        def scale_bias_ms():
+            # the reference's default layer: W = C.N + s.noise1d (zero coefficients and a fused random bias at initialisation).
+            # forward: the strip kernel; dx: factored share + hashed random-bias share; dcoef and ds: dW tiles
+            sb = torch.tensor([0.02], device=dev).bfloat16()
+            ds = torch.empty(1, dtype=torch.float32, device=dev)
+            psb, pds, r = ctypes.c_void_p(sb.data_ptr()), ctypes.c_void_p(ds.data_ptr()), main_set.dref
+            fwd = lambda: _lib.check(L.rdb_linear_fwd(p["y"], OUT_F, p["x"], IN_F, p["C"], psb, None, r, p["ws"], ws_bytes, stream), "rdb_linear_fwd")
+            dxf = lambda: _lib.check(L.rdb_linear_bwd_dx(p["dx"], IN_F, p["dy"], OUT_F, p["C"], psb, r, p["ws"], ws_bytes, stream), "rdb_linear_bwd_dx")
+            dcf = lambda: _lib.check(L.rdb_linear_bwd_dcoef(p["dC"], pds, p["dy"], OUT_F, p["x"], IN_F, r, p["ws"], ws_bytes, stream),
+                                     "rdb_linear_bwd_dcoef")
+            t = {"fwd": round(event_ms(fwd, 20), 4), "dx": round(event_ms(dxf, 20), 4), "dcoef_and_dscale": round(event_ms(dcf, 20), 4)}
+            t["step"] = round(sum(t.values()), 4)
+            return t
+
         compare = {
             "one_call_entry_points_ms": onecall_ms(_lib.RDB_ALGO_AUTO),
+            "layer_with_fused_random_bias_ms": scale_bias_ms(),
             "w_tiles_formed_on_chip_ms": strip_ms(),
             "vendor_gemm_on_the_factored_shapes_ms": vendor_skinny(),
             "materialize_then_gemm_ms": round(event_ms(mat_gemm_step, 10), 4),

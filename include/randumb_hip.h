@@ -142,7 +142,10 @@ enum {
     RDB_ALGO_FACTORED = 3 /* matrix-coef only: use W = C.N associatively so that no weight tile is formed at all:
                              y = (x.N^T).C^T, dx = (dy.C).N, dcoef = dy^T.(x.N^T); the [tokens x k] intermediate lives
                              in the caller's workspace.  bf16 activations and coef: matrix-core kernels; fp32 with
-                             k <= 64 and tokens <= 4096 (the GEMV-like regime): vector-ALU kernels, bit-reproducible. */
+                             k <= 64 and tokens <= 4096 (the GEMV-like regime): vector-ALU kernels, bit-reproducible.
+                             With scale_bias (W = C.N + s.R, R the fused random bias, full rank) the input gradient adds
+                             s * dy.R on top with R hashed into the matrix pipeline; forward and dcoef then need the
+                             kernels that form W (RDB_ALGO_AUTO picks them). */
 };
 
 enum { RDB_OP_LINEAR_FWD = 0, RDB_OP_LINEAR_BWD_DX = 1, RDB_OP_LINEAR_BWD_DCOEF = 2, RDB_OP_LINEAR_BWD_PROJECTED = 3 };

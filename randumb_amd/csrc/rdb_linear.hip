@@ -313,6 +313,9 @@ int64_t linear_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus);
 int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias,
                        const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
 
+// rdb_rbias.hip
+int linear_dx_rbias_add(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *scale_bias, const rdb_linear_desc *d, hipStream_t s);
+
 // rdb_dcoef.hip
 int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d,
                       int num_cus, hipStream_t s);
@@ -431,12 +434,21 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
     if (!dx || (!dy && d->out_f > 0) || (!coef && d->k > 0)) return set_error(RDB_E_NULL, "rdb_linear_bwd_dx: dx, dy or coef is NULL");
     if (lddx < d->in_f || lddy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dx: leading dimension smaller than the row");
     if (d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) {
+        if (scale_bias && d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16 && d->tokens * lddx < (1ll << 29)) {
+            // W = C.N + s.R: the low-rank share through the factored kernels, then the random-bias share added on top
+            rc = linear_dx_factored(dx, lddx, dy, lddy, coef, nullptr, d, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
+            if (rc == RDB_OK) {
+                rc = linear_dx_rbias_add(dx, lddx, dy, lddy, scale_bias, d, (hipStream_t)stream);
+                if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dx: internal: the random-bias share refused a request the factored share took");
+            }
+            if (rc != RDB_E_UNSUPPORTED) return rc;
+        }
         rc = linear_dx_factored(dx, lddx, dy, lddy, coef, scale_bias, d, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
         if (rc != RDB_E_UNSUPPORTED) return rc;
         rc = linear_dx_smallk(dx, lddx, dy, lddy, coef, scale_bias, d, workspace, workspace_bytes, (hipStream_t)stream);
         if (rc != RDB_E_UNSUPPORTED) return rc;
         if (d->algo == RDB_ALGO_FACTORED)
-            return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dx: the factored algorithm needs matrix-coef, no scale_bias, a workspace of "
+            return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dx: the factored algorithm needs matrix-coef, a workspace of "
                                                 "rdb_linear_workspace_bytes() bytes and either bf16 (activations and coef; sizes that are "
                                                 "multiples of 8; aligned rows) or fp32 with k <= 64 and tokens <= 4096");
     }

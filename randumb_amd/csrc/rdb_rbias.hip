@@ -1,0 +1,135 @@
+// The fused random bias in the fast input-gradient path.
+//
+// With scale_bias the weight is W = C . N + s . R,  R[o, i] = noise1d(o*in_f + i)  (src/rten_cpp/RandumbTensor.py:286-289;
+// it is what the reference's default initialisation starts from: zero coefficients, random bias,
+// src/rten_cpp/SillyLayers.py:122-133, 218-221).  R is a full-rank pseudorandom matrix, so its share of a product is a
+// dense contraction whatever is done about C . N; the low-rank share keeps its factored kernels and this file adds
+//     dx[t, i] += s * sum_o dy[t, o] * R[o, i]
+// on the tile engine with R as a hashed operand: a tile of 64 input features x 256 tokens, R hashed once per block and
+// stage straight into the pipeline's registers (as 2^31 * noise in bf16, the scale folded into the epilogue), two blocks
+// per compute unit so that one block's hashing runs under the other's matrix work.  R never exists in memory.
+#include "rdb_gemm.hpp"
+#include "rdb_tile.hpp"
+
+namespace rdb {
+
+constexpr int RB_BI = 64, RB_BT = 256, RB_BK = 64;
+
+// Hashed operand: element (row, k) = 2^31 * noise1d((row0 + row) * sR + k * sK) as bf16.
+template <int ROWS, int BK> struct Noise1DOperand {
+    typedef OperandTile<ROWS, BK, K_CONT> Tile;
+    int row0;
+    uint32_t sR, sK, seed;
+    int k_begin;
+    __device__ __forceinline__ void init(int kb) { k_begin = kb; }
+    __device__ __forceinline__ void load_piece(f32x4 &reg, int p, int stage) const
+    {
+        const int idx = p * 256 + threadIdx.x, k0 = k_begin + stage * BK;
+        const uint32_t row = (uint32_t)(row0 + idx / (BK / 8)), k = (uint32_t)(k0 + (idx % (BK / 8)) * 8);
+        const uint32_t step = sK * SQ5_N1, first = (row * sR + k * sK) * SQ5_N1 + seed;
+        uint32_t b[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) b[e] = sq5_tail(first + (uint32_t)e * step);
+        Frag8 f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) f.u[e] = f32x2_to_bf16x2((float)(int32_t)b[2 * e], (float)(int32_t)b[2 * e + 1]);
+        reg = f.f4;
+    }
+    __device__ __forceinline__ void load(f32x4 (&regs)[Tile::PER_THREAD], int stage) const
+    {
+#pragma unroll
+        for (int p = 0; p < Tile::PER_THREAD; ++p) load_piece(regs[p], p, stage);
+    }
+};
+
+struct RBiasDxParams {
+    const bf16_t *dy;
+    const bf16_t *scale_bias;   // one bf16 value
+    bf16_t *dx;
+    int64_t lddy, lddx;
+    int tokens, in_f, out_f;
+    int tiles_i, tiles_t;
+    uint32_t seed;
+};
+
+__global__ __launch_bounds__(256, 2) void rbias_dx_add_kernel(RBiasDxParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
+    // work item = (token tile, feature tile), feature tile fastest: neighbours share the dy tile
+    const int w = xcd_work_item(blockIdx.x, p.tiles_i * p.tiles_t);
+    if (w >= p.tiles_i * p.tiles_t) return;
+    const int i0 = (w % p.tiles_i) * RB_BI, tok0 = (w / p.tiles_i) * RB_BT;
+    constexpr int MI = RB_BI / 32, NI = RB_BT / 128;
+    f32x16 acc[MI][NI];
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = zero16();
+    // "A": 2^31 * R[o, i], rows = i, contraction = o: the noise index o*in_f + i moves by 1 per row and by in_f per k
+    Noise1DOperand<RB_BI, RB_BK> opr = {i0, 1u, (uint32_t)p.in_f, p.seed};
+    // "B": dy[tok][o]; output rows past out_f read as zeros, whatever the hash says there
+    GlobalOperand<RB_BT, RB_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
+    gemm_mainloop<RB_BI, RB_BT, RB_BK, 1, 2, 1>(acc, lds, opr, opdy, 0, (p.out_f + RB_BK - 1) / RB_BK);
+    // dx += s * 2^-31 * acc, through LDS as fp32 so that every lane updates 8 consecutive features of a token's row
+    const float scale = bf16_to_f32(*p.scale_bias) * 4.656612873077392578125e-10f;
+    constexpr int LDF = RB_BI + 4;   // floats per token row of the staging tile
+    float *stage = reinterpret_cast<float *>(smem_raw);
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int jq = 0; jq < 4; ++jq) {
+                const int b = wave * NI * 32 + ni * 32 + r, a = mi * 32 + 8 * jq + 4 * g;
+                const f32x4 v = {acc[mi][ni][jq * 4] * scale, acc[mi][ni][jq * 4 + 1] * scale, acc[mi][ni][jq * 4 + 2] * scale,
+                                 acc[mi][ni][jq * 4 + 3] * scale};
+                *reinterpret_cast<f32x4 *>(stage + b * LDF + a) = v;
+            }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < RB_BI * RB_BT / 8 / 256; ++q) {
+        const int idx = q * 256 + t, b = idx / (RB_BI / 8), a = (idx % (RB_BI / 8)) * 8;
+        if (tok0 + b < p.tokens && i0 + a < p.in_f) {   // in_f is a multiple of 8: a piece lies inside or outside
+            bf16_t *dst = p.dx + (int64_t)(tok0 + b) * p.lddx + i0 + a;
+            Frag8 old;
+            old.f4 = *reinterpret_cast<const f32x4 *>(dst);
+            const f32x4 lo = *reinterpret_cast<const f32x4 *>(stage + b * LDF + a), hi = *reinterpret_cast<const f32x4 *>(stage + b * LDF + a + 4);
+            Frag8 nw;
+            nw.u[0] = f32x2_to_bf16x2(__uint_as_float(old.u[0] << 16) + lo[0], __uint_as_float(old.u[0] & 0xffff0000u) + lo[1]);
+            nw.u[1] = f32x2_to_bf16x2(__uint_as_float(old.u[1] << 16) + lo[2], __uint_as_float(old.u[1] & 0xffff0000u) + lo[3]);
+            nw.u[2] = f32x2_to_bf16x2(__uint_as_float(old.u[2] << 16) + hi[0], __uint_as_float(old.u[2] & 0xffff0000u) + hi[1]);
+            nw.u[3] = f32x2_to_bf16x2(__uint_as_float(old.u[3] << 16) + hi[2], __uint_as_float(old.u[3] & 0xffff0000u) + hi[3]);
+            *reinterpret_cast<f32x4 *>(dst) = nw.f4;
+        }
+    }
+}
+
+// dx += s * dy . R on the launch stream, after the kernels that wrote dx.  Returns RDB_E_UNSUPPORTED (without setting an
+// error) when the request does not fit.
+int linear_dx_rbias_add(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *scale_bias, const rdb_linear_desc *d, hipStream_t s)
+{
+    if (d->act_dtype != RDB_BF16 || d->coef_dtype != RDB_BF16 || d->coef_rows == 0 || !scale_bias) return RDB_E_UNSUPPORTED;
+    if (d->in_f % 8 || d->out_f % 8 || d->tokens < 1 || d->in_f < 1 || d->out_f < 1) return RDB_E_UNSUPPORTED;
+    if (lddy % 8 || lddx % 8 || ((uintptr_t)dy & 15) || ((uintptr_t)dx & 15)) return RDB_E_UNSUPPORTED;
+    if (d->tokens * lddy >= (1ll << 29) || d->tokens * lddx >= (1ll << 29)) return RDB_E_UNSUPPORTED;
+    RBiasDxParams p;
+    p.dy = (const bf16_t *)dy;
+    p.scale_bias = (const bf16_t *)scale_bias;
+    p.dx = (bf16_t *)dx;
+    p.lddy = lddy;
+    p.lddx = lddx;
+    p.tokens = (int)d->tokens;
+    p.in_f = (int)d->in_f;
+    p.out_f = (int)d->out_f;
+    p.tiles_i = (int)cdiv(d->in_f, RB_BI);
+    p.tiles_t = (int)cdiv(d->tokens, RB_BT);
+    p.seed = d->seed;
+    size_t smem = engine_smem<RB_BI, RB_BT, RB_BK, K_CONT, K_CONT>();
+    const size_t stage = (size_t)RB_BT * (RB_BI + 4) * sizeof(float);
+    if (smem < stage) smem = stage;
+    return launch_engine(rbias_dx_add_kernel, p, p.tiles_i * p.tiles_t, smem, s, "rbias_dx_add_kernel");
+}
+
+}  // namespace rdb

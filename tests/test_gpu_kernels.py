@@ -426,9 +426,8 @@ def test_factored_dx_needs_what_it_says(hip):
     with pytest.raises(RandumbHipError):
         hip.linear_bwd_dx(dy, c, 40, 48, 40, 1, 0, algo=RDB_ALGO_FACTORED)
     C = torch.randn(48, 16, device="cuda").bfloat16()
-    sb = torch.tensor([0.1], device="cuda").bfloat16()      # neither has the random-bias term
-    with pytest.raises(RandumbHipError):
-        hip.linear_bwd_dx(dy, C, 40, 48, 40, 1, 0, scale_bias=sb, algo=RDB_ALGO_FACTORED)
+    sb = torch.tensor([0.1], device="cuda").bfloat16()      # the random-bias term rides on top of the factored input gradient
+    assert hip.linear_bwd_dx(dy, C, 40, 48, 40, 1, 0, scale_bias=sb, algo=RDB_ALGO_FACTORED).shape == (64, 40)
     assert hip.linear_bwd_dx(dy, C, 40, 48, 40, 1, 0, scale_bias=sb).shape == (64, 40)
     x = torch.randn(64, 40, device="cuda").bfloat16()
     with pytest.raises(RandumbHipError):
@@ -439,6 +438,35 @@ def test_factored_dx_needs_what_it_says(hip):
         hip.linear_bwd_dcoef(dy, x, 16, 0, 40, 48, 40, 1, 0, algo=RDB_ALGO_FACTORED)
     with pytest.raises(RandumbHipError):
         hip.linear_bwd_dcoef(dy, x, 16, 48, 40, 48, 40, 1, 0, want_scale_bias_grad=True, algo=RDB_ALGO_FACTORED)
+
+
+@pytest.mark.parametrize("T,in_f,out_f,k", [(2048, 768, 3072, 256), (200, 72, 136, 40)])
+def test_default_layer_fast_path_with_scale_bias(hip, oracle, T, in_f, out_f, k):
+    """The reference's default layer starts from zero coefficients and a fused random bias (SillyLayers.py:122-133, 218-221):
+    W = C.N + s.noise1d.  Forward, input gradient (factored share + hashed random-bias share), coefficient gradient and the
+    gradient of s through the entry points AUTO picks, against the oracle, with s != 0 and C != 0 and with C = 0."""
+    print(f"case scale_bias fast path T={T} in={in_f} out={out_f} k={k}", flush=True)
+    x, dy, coef = _inputs(T, in_f, out_f, k, True, torch.bfloat16, 21)
+    sbv = 0.0625     # exact in bf16; the weight's random share then has the size of the low-rank share
+    sb = torch.tensor([sbv]).bfloat16()
+    for c in (coef, torch.zeros_like(coef)):
+        xn, dyn, cn = x.float().numpy(), dy.float().numpy(), c.float().numpy()
+        want_y = oracle.linear_fwd(xn, cn, in_f, out_f, 9, scale_bias=sbv)
+        want_dx, want_dc, dW = oracle.linear_bwd(xn, dyn, cn, in_f, out_f, 9, scale_bias=sbv)
+        want_ds = float(oracle.scale_bias_bwd(dW.astype(np.float32), 9)[0])
+        xg, dyg, cg, sg = x.cuda(), dy.cuda(), c.cuda(), sb.cuda()
+        y = hip.linear_fwd(xg, cg, in_f, out_f, in_f, 1, 9, scale_bias=sg)
+        dx = hip.linear_bwd_dx(dyg, cg, in_f, out_f, in_f, 1, 9, scale_bias=sg)
+        dc, ds = hip.linear_bwd_dcoef(dyg, xg, k, out_f, in_f, out_f, in_f, 1, 9, want_scale_bias_grad=True)
+        assert rel_l2(cpu(y), want_y) < BF16_TOL
+        assert rel_l2(cpu(dx), want_dx) < BF16_TOL
+        assert rel_l2(cpu(dc), want_dc) < BF16_TOL
+        assert abs(float(ds) - want_ds) < BF16_TOL * max(abs(want_ds), float(np.linalg.norm(dW)))
+        # the same input gradient from the general kernel that forms the weight block by block
+        from randumb_amd._lib import RDB_ALGO_TILE
+        if T <= 256:
+            dx_t = hip.linear_bwd_dx(dyg, cg, in_f, out_f, in_f, 1, 9, scale_bias=sg, algo=RDB_ALGO_TILE)
+            assert rel_l2(cpu(dx), cpu(dx_t)) < 1e-2
 
 
 def test_projected_path_random_shapes(hip, oracle):
