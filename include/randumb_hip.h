@@ -204,11 +204,20 @@ int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const void *dy, int6
  * 2 * tokens * k * 2 bytes with k rounded up to 64) and, if rdb_linear_project was given the coefficients, C transposed for
  * the input gradient (out_f * k * 2 bytes): the kernels then fetch these small operands straight into registers and only
  * the large operand (dy) is staged through on-chip memory.  Needs: coef_rows == out_f, act_dtype RDB_BF16,
- * tokens/in_f/out_f/k > 0, in_f, out_f, k multiples of 8, tokens*k and out_f*k (k rounded up to 64, tokens and out_f to
- * 64) below 2^29, 16-byte aligned pointers, leading dimensions multiples of 8; otherwise RDB_E_UNSUPPORTED. */
+ * tokens/in_f/out_f/k > 0, in_f, out_f, k multiples of 8, out_f*k (k and out_f rounded up to 64) below 2^29, 16-byte
+ * aligned pointers, leading dimensions multiples of 8; otherwise RDB_E_UNSUPPORTED. */
 
 /* Bytes of the projection state for `desc`, or 0 when the projected form does not apply to it. */
 int64_t rdb_linear_projection_bytes(const rdb_linear_desc *desc);
+
+/* One launch addresses at most 2^29 elements of x, y, dy or dx.  The projected entry points take any number of tokens all
+ * the same: tokens are independent in y and dx and additive in dcoef, so a layer with more is run in chunks of tokens (a
+ * multiple of 256 each), every chunk with a projection state of its own, one after the other in the state buffer; dcoef is
+ * added up in chunk order (the same bits from run to run) and one workspace serves the chunks in turn.  The reference has
+ * no such limit and no counterpart of this (R.py:942-946 is one dense product).  Returns the number of chunks (1 for every
+ * layer whose activations fit one launch, 0 when the projected form does not apply) and, if chunk_tokens != NULL, the tokens
+ * per chunk (the last chunk may hold fewer).  Leading dimensions may exceed the row length by up to a factor of two. */
+int rdb_linear_projection_chunks(const rdb_linear_desc *desc, int64_t *chunk_tokens);
 
 /* Where the pieces lie inside the state, for tools and tests that want to look at z (no reference counterpart: the
  * reference keeps x).  Returns 0 and fills info[0..7], or RDB_E_UNSUPPORTED:

@@ -37,6 +37,7 @@ EXPORTS = [
     "rdb_linear_bwd_dx",
     "rdb_linear_bwd_dcoef",
     "rdb_linear_projection_bytes",
+    "rdb_linear_projection_chunks",
     "rdb_linear_projection_layout",
     "rdb_linear_project",
     "rdb_linear_fwd_projected",
@@ -111,6 +112,8 @@ def load() -> ctypes.CDLL:
     L.rdb_linear_bwd_dcoef.argtypes = [vp, vp, vp, i64, vp, i64, dp, vp, i64, vp]
     L.rdb_linear_projection_bytes.argtypes = [dp]
     L.rdb_linear_projection_bytes.restype = i64
+    L.rdb_linear_projection_chunks.argtypes = [dp, ctypes.POINTER(i64)]
+    L.rdb_linear_projection_chunks.restype = ci
     L.rdb_linear_projection_layout.argtypes = [dp, ctypes.POINTER(i64)]
     L.rdb_linear_projection_layout.restype = ci
     L.rdb_linear_project.argtypes = [vp, vp, i64, vp, dp, vp]

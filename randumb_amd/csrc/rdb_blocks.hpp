@@ -137,6 +137,7 @@ struct RedParams {
     float *out;            // [n]
     int64_t n;             // multiple of 4
     int splits;
+    int accumulate;        // 0: out = sum of the splits; 1: out += that sum (a later chunk of tokens of the same layer)
 };
 
 __device__ __forceinline__ void red_block(const RedParams &p, int block, int nblocks)
@@ -146,6 +147,7 @@ __device__ __forceinline__ void red_block(const RedParams &p, int block, int nbl
     for (int64_t e = (int64_t)block * blockDim.x + threadIdx.x; e < n4; e += (int64_t)nblocks * blockDim.x) {
         const f32x4 *src = reinterpret_cast<const f32x4 *>(p.partial) + e;
         f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (p.accumulate) v = reinterpret_cast<const f32x4 *>(p.out)[e];
         // eight loads in flight at a time (a loop of single loads would wait out the memory latency once per split);
         // the additions stay in split order
         for (int s0 = 0; s0 < p.splits; s0 += 8) {

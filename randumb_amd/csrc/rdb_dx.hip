@@ -215,12 +215,13 @@ int64_t linear_dx_factored_workspace(const rdb_linear_desc *d)
 static int64_t align256(int64_t n) { return (n + 255) / 256 * 256; }
 
 // Workspace of the regrouped backward pass: t, then the partial sums of the coefficient gradient.
-int64_t linear_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus)
+// force_partial: also with a single token range (the call adds to dcoef instead of overwriting it).
+int64_t linear_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus, bool force_partial)
 {
     if (!dx_factored_ok(d)) return 0;
     DcParams dc;
     make_dc_params(dc, nullptr, nullptr, d->out_f, nullptr, d, num_cus);
-    if (dc.splits == 1) return linear_dx_factored_workspace(d);   // a single token range is stored straight into dcoef
+    if (dc.splits == 1 && !force_partial) return linear_dx_factored_workspace(d);   // a single token range is stored straight into dcoef
     return align256(linear_dx_factored_workspace(d)) + (int64_t)dc.splits * d->out_f * d->k * (int64_t)sizeof(float);
 }
 
@@ -298,8 +299,9 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
 
 // Whole backward pass of the layer from the saved projection z: dx = (dy.C).N and dcoef = dy^T.z in two launches.
 // Returns RDB_E_UNSUPPORTED (without setting an error) when the request does not fit.
+// accumulate: dcoef += instead of dcoef = (a later chunk of tokens of a layer whose activations are passed in chunks).
 int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z, const void *coef,
-                         const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s)
+                         const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, bool accumulate, hipStream_t s)
 {
     if (!dx_factored_ok(d)) return RDB_E_UNSUPPORTED;
     if (!workspace || workspace_bytes < linear_dx_factored_workspace(d) || ((uintptr_t)workspace & 15)) return RDB_E_UNSUPPORTED;
@@ -310,12 +312,12 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
     make_dyc_params(p1, dy, lddy, coef, workspace, d);
     const size_t smem_dc = engine_smem<KD_BO, KD_BM, X_BK, M_CONT, M_CONT>(), smem_tn = engine_smem<K2_BI, K2_BT, X_BK, K_CONT, K_CONT>();
     const size_t smem_dyc = engine_smem<K1_BC, K1_BT, X_BK, M_CONT, K_CONT>();
-    if (workspace_bytes >= linear_bwd_projected_workspace(d, num_cus)) {
+    if (workspace_bytes >= linear_bwd_projected_workspace(d, num_cus, accumulate)) {
         BwdAParams a;
         const int dc_items = make_dc_params(a.dc, dcoef, dy, lddy, nullptr, d, num_cus);
         dc_params_from_state(a.dc, z, d);
         // one token range only: its sums are the result, stored straight into dcoef, and nothing is left to add up
-        const bool direct = a.dc.splits == 1;
+        const bool direct = a.dc.splits == 1 && !accumulate;
         a.dc.partial = direct ? dcoef : reinterpret_cast<float *>(static_cast<char *>(workspace) + align256(linear_dx_factored_workspace(d)));
         a.dyc = p1;
         {   // the transposed coefficients, if the forward pass left them in the state (its header says so)
@@ -337,6 +339,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
         red.out = dcoef;
         red.n = d->out_f * d->k;
         red.splits = a.dc.splits;
+        red.accumulate = accumulate ? 1 : 0;
         if (tn_stationary_ok(d, lddx)) {
             BwdBsParams bs;
             const int items = make_tns_params(bs.tn, dx, lddx, workspace, d, num_cus);
@@ -373,7 +376,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
         return check_launch("bwd_tn_red_kernel");
     }
     // workspace for t only: dy.C first (clearing dcoef on the side), then the coefficient gradient with atomics beside t.N
-    p1.zero = dcoef;
+    p1.zero = accumulate ? nullptr : dcoef;
     p1.zero_n = d->out_f * d->k;
     int rc = launch_engine(dx_dyc_kernel, p1, p1.tiles_c * p1.tiles_t, smem_dyc, s, "dx_dyc_kernel");
     if (rc) return rc;

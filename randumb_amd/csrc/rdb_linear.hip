@@ -9,6 +9,8 @@
 // contraction in steps of 32.  Reference behaviour replaced: materialize() + dense product per aten.mm
 // (src/rten_cpp/RandumbTensor.py:942-952, 771-791), autograd's MmBackward on the dense weight, and
 // RandumbTensorConstructor.backward -> materialize_bwd / scale_bias_bwd (RandumbTensor.py:979-990).
+#include <algorithm>
+
 #include "rdb_direct.hpp"
 #include "rdb_tile.hpp"
 
@@ -307,9 +309,9 @@ int linear_dcoef_smallk(float *dcoef, const void *dy, int64_t lddy, const void *
 
 // rdb_dx.hip
 int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z, const void *coef,
-                         const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
+                         const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, bool accumulate, hipStream_t s);
 int64_t linear_dx_factored_workspace(const rdb_linear_desc *d);
-int64_t linear_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus);
+int64_t linear_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus, bool force_partial);
 int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias,
                        const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
 
@@ -364,6 +366,8 @@ template <typename K> static int launch(K kernel, dim3 grid, size_t smem, hipStr
 
 using namespace rdb;
 
+static int64_t bwd_projected_workspace(const rdb_linear_desc *d);
+
 extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
 {
     if (!d) return 0;
@@ -374,7 +378,7 @@ extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
         return (op == RDB_OP_LINEAR_FWD || op == RDB_OP_LINEAR_BWD_DX || op == RDB_OP_LINEAR_BWD_DCOEF) ? linear_smallk_workspace(&dd) : 0;
     }
     if (op == RDB_OP_LINEAR_BWD_DX) return linear_dx_factored_workspace(d);
-    if (op == RDB_OP_LINEAR_BWD_PROJECTED) return linear_bwd_projected_workspace(d, num_compute_units());
+    if (op == RDB_OP_LINEAR_BWD_PROJECTED) return bwd_projected_workspace(d);
     if (op == RDB_OP_LINEAR_FWD) return d->coef_dtype == RDB_BF16 ? linear_projection_bytes(d) : 0;
     if (op == RDB_OP_LINEAR_BWD_DCOEF) return linear_projection_bytes(d);  // reads no coefficients: their dtype does not matter
     return 0;
@@ -576,23 +580,70 @@ extern "C" int rdb_linear_fwd_static(void *y, int64_t ldy, const void *x, int64_
 }
 
 // ----------------------------------------------------------------------------------------------- projected entry points
-static int check_projected(const char *who, const rdb_linear_desc *d)
+// The kernels address activations with 32-bit byte offsets: one launch takes at most 2^29 elements of x, y, dy or dx.  Tokens
+// are independent in y and dx and additive in dcoef, so a layer with more than that is run in chunks of tokens: every chunk
+// is a layer of its own with its own projection state (the states lie one after the other in the caller's buffer), the
+// chunks' dcoef are added up in chunk order (still the same bits from run to run), and one workspace serves them in turn.
+struct ChunkPlan {
+    int64_t chunk_tokens;  // tokens of every chunk but the last (a multiple of 256)
+    int nchunks;           // 0: the projected form does not apply
+    int64_t state_stride;  // bytes from one chunk's projection state to the next
+};
+
+static rdb_linear_desc chunk_desc(const rdb_linear_desc *d, const ChunkPlan &pl, int c)
+{
+    rdb_linear_desc dd = *d;
+    const int64_t left = d->tokens - (int64_t)c * pl.chunk_tokens;
+    dd.tokens = left < pl.chunk_tokens ? left : pl.chunk_tokens;
+    return dd;
+}
+
+static ChunkPlan chunk_plan(const rdb_linear_desc *d)
+{
+    ChunkPlan pl = {0, 0, 0};
+    if (!d || d->tokens <= 0 || d->in_f <= 0 || d->out_f <= 0 || d->k <= 0) return pl;
+    const int64_t widest = std::max(std::max(d->in_f, d->out_f), cdiv(d->k, 64) * 64);
+    // half the addressing limit, so that leading dimensions may exceed the row length by up to a factor of two
+    int64_t per_chunk = ((1ll << 28) / widest) / 256 * 256;
+    if (per_chunk < 256) return pl;
+    int nchunks = (int)cdiv(d->tokens, per_chunk);
+    if (nchunks > 1) per_chunk = cdiv(cdiv(d->tokens, nchunks), 256) * 256;   // chunks of about equal size
+    else per_chunk = d->tokens;
+    pl.chunk_tokens = per_chunk;
+    pl.nchunks = (int)cdiv(d->tokens, per_chunk);
+    const rdb_linear_desc first = chunk_desc(d, pl, 0);
+    pl.state_stride = linear_projection_bytes(&first);
+    if (pl.state_stride <= 0) pl.nchunks = 0;
+    return pl;
+}
+
+static int check_projected(const char *who, const rdb_linear_desc *d, ChunkPlan *plan)
 {
     int rc = check_desc(who, d);
     if (rc) return rc;
-    if (linear_projection_bytes(d) == 0)
+    const ChunkPlan pl = chunk_plan(d);
+    if (pl.nchunks == 0)
         return set_error(RDB_E_UNSUPPORTED, "%s: the projected form needs matrix-coef, bf16 activations, non-empty sizes that are "
-                                            "multiples of 8, and tokens*k and out_f*k (k rounded up to 64) below 2^29", who);
+                                            "multiples of 8, and out_f*k (k rounded up to 64) below 2^29", who);
+    if (plan) *plan = pl;
     return RDB_OK;
 }
 
-extern "C" int64_t rdb_linear_projection_bytes(const rdb_linear_desc *d) { return d ? linear_projection_bytes(d) : 0; }
+extern "C" int64_t rdb_linear_projection_bytes(const rdb_linear_desc *d)
+{
+    const ChunkPlan pl = chunk_plan(d);
+    return pl.nchunks * pl.state_stride;
+}
 
 extern "C" int rdb_linear_projection_layout(const rdb_linear_desc *d, int64_t *info)
 {
-    int rc = check_projected("rdb_linear_projection_layout", d);
+    ChunkPlan pl;
+    int rc = check_projected("rdb_linear_projection_layout", d, &pl);
     if (rc) return rc;
     if (!info) return set_error(RDB_E_NULL, "rdb_linear_projection_layout: info is NULL");
+    if (pl.nchunks != 1) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_projection_layout: this layer's state is %d states of %lld tokens, one "
+                                                            "after the other, %lld bytes apart: ask for the layout of one of them",
+                                          pl.nchunks, (long long)pl.chunk_tokens, (long long)pl.state_stride);
     const ProjLayout L = proj_layout(d);
     info[0] = L.zf_off;
     info[1] = L.frag_fwd ? 1 : 0;
@@ -605,59 +656,111 @@ extern "C" int rdb_linear_projection_layout(const rdb_linear_desc *d, int64_t *i
     return RDB_OK;
 }
 
+// number of token chunks the projected entry points run `desc` in (1 for every layer whose activations fit one launch)
+extern "C" int rdb_linear_projection_chunks(const rdb_linear_desc *d, int64_t *chunk_tokens)
+{
+    const ChunkPlan pl = chunk_plan(d);
+    if (chunk_tokens) *chunk_tokens = pl.chunk_tokens;
+    return pl.nchunks;
+}
+
+static char *at_bytes(const void *p, int64_t bytes) { return static_cast<char *>(const_cast<void *>(p)) + bytes; }
+
 extern "C" int rdb_linear_project(void *state, const void *x, int64_t ldx, const void *coef, const rdb_linear_desc *d, void *stream)
 {
-    int rc = check_projected("rdb_linear_project", d);
+    ChunkPlan pl;
+    int rc = check_projected("rdb_linear_project", d, &pl);
     if (rc) return rc;
     if (!state || !x) return set_error(RDB_E_NULL, "rdb_linear_project: state or x is NULL");
     if (ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_project: leading dimension smaller than the row");
     if (coef && !aligned16(coef)) return set_error(RDB_E_ALIGN, "rdb_linear_project: coef must be 16-byte aligned");
-    rc = linear_project(state, x, ldx, coef, d, (hipStream_t)stream);
-    if (rc == RDB_E_UNSUPPORTED)
-        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_project: x and state must be 16-byte aligned, ldx a multiple of 8, tokens*ldx < 2^29");
-    return rc;
+    if (pl.chunk_tokens * ldx >= (1ll << 29) || ldx % 8 || !aligned16(x) || !aligned16(state))
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_project: x and state must be 16-byte aligned, ldx a multiple of 8 and below twice in_f");
+    for (int c = 0; c < pl.nchunks; ++c) {
+        const rdb_linear_desc dd = chunk_desc(d, pl, c);
+        rc = linear_project(at_bytes(state, c * pl.state_stride), at_bytes(x, c * pl.chunk_tokens * ldx * 2), ldx, coef, &dd, (hipStream_t)stream);
+        if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_project: internal: chunk %d of %d refused", c, pl.nchunks);
+        if (rc) return rc;
+    }
+    return RDB_OK;
 }
 
 extern "C" int rdb_linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, const void *bias, const rdb_linear_desc *d,
                                         void *stream)
 {
-    int rc = check_projected("rdb_linear_fwd_projected", d);
+    ChunkPlan pl;
+    int rc = check_projected("rdb_linear_fwd_projected", d, &pl);
     if (rc) return rc;
     if (!y || !z || !coef) return set_error(RDB_E_NULL, "rdb_linear_fwd_projected: y, z or coef is NULL");
     if (ldy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_fwd_projected: leading dimension smaller than the row");
-    rc = linear_fwd_projected(y, ldy, z, coef, bias, d, num_compute_units(), (hipStream_t)stream);
-    if (rc == RDB_E_UNSUPPORTED)
-        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd_projected: coefficients must be bf16; y, state and coef 16-byte aligned; ldy "
-                                            "a multiple of 8; with k <= 256 also bias 8-byte aligned and tokens*ldy < 2^29");
-    return rc;
+    if (d->coef_dtype != RDB_BF16 || ldy % 8 || !aligned16(y) || !aligned16(z) || !aligned16(coef) || ((uintptr_t)bias & 7) ||
+        pl.chunk_tokens * ldy >= (1ll << 29))
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd_projected: coefficients must be bf16; y, state and coef 16-byte aligned, bias 8-byte; "
+                                            "ldy a multiple of 8 and below twice out_f");
+    for (int c = 0; c < pl.nchunks; ++c) {
+        const rdb_linear_desc dd = chunk_desc(d, pl, c);
+        rc = linear_fwd_projected(at_bytes(y, c * pl.chunk_tokens * ldy * 2), ldy, at_bytes(z, c * pl.state_stride), coef, bias, &dd,
+                                  num_compute_units(), (hipStream_t)stream);
+        if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd_projected: internal: chunk %d of %d refused", c, pl.nchunks);
+        if (rc) return rc;
+    }
+    return RDB_OK;
 }
 
 extern "C" int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *z, const rdb_linear_desc *d, void *stream)
 {
-    int rc = check_projected("rdb_linear_bwd_dcoef_projected", d);
+    ChunkPlan pl;
+    int rc = check_projected("rdb_linear_bwd_dcoef_projected", d, &pl);
     if (rc) return rc;
     if (!dcoef || !dy || !z) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef_projected: dcoef, dy or z is NULL");
     if (lddy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dcoef_projected: leading dimension smaller than the row");
-    if (lddy % 8 || !aligned16(dy) || !aligned16(z) || d->tokens * lddy >= (1ll << 29))
-        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dcoef_projected: dy and z must be 16-byte aligned, lddy a multiple of 8, "
-                                            "tokens*lddy < 2^29");
+    if (lddy % 8 || !aligned16(dy) || !aligned16(z) || pl.chunk_tokens * lddy >= (1ll << 29))
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dcoef_projected: dy and z must be 16-byte aligned, lddy a multiple of 8 and below "
+                                            "twice out_f");
     hipStream_t s = (hipStream_t)stream;
     rc = fill_zero(dcoef, d->coef_rows * d->k, s);
     if (rc) return rc;
-    return linear_dcoef_projected(dcoef, dy, lddy, z, d, num_compute_units(), s);
+    for (int c = 0; c < pl.nchunks; ++c) {   // every chunk adds its share with atomics
+        const rdb_linear_desc dd = chunk_desc(d, pl, c);
+        rc = linear_dcoef_projected(dcoef, at_bytes(dy, c * pl.chunk_tokens * lddy * 2), lddy, at_bytes(z, c * pl.state_stride), &dd, num_compute_units(), s);
+        if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dcoef_projected: internal: chunk %d of %d refused", c, pl.nchunks);
+        if (rc) return rc;
+    }
+    return RDB_OK;
+}
+
+// workspace of rdb_linear_bwd_projected: that of the largest chunk; chunks after the first add to dcoef and so always keep
+// their sums in the workspace first
+static int64_t bwd_projected_workspace(const rdb_linear_desc *d)
+{
+    const ChunkPlan pl = chunk_plan(d);
+    if (pl.nchunks == 0) return 0;
+    const rdb_linear_desc first = chunk_desc(d, pl, 0);
+    return linear_bwd_projected_workspace(&first, num_compute_units(), pl.nchunks > 1);
 }
 
 extern "C" int rdb_linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z, const void *coef,
                                         const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
 {
-    int rc = check_projected("rdb_linear_bwd_projected", d);
+    ChunkPlan pl;
+    int rc = check_projected("rdb_linear_bwd_projected", d, &pl);
     if (rc) return rc;
     if (!dx || !dcoef || !dy || !z || !coef) return set_error(RDB_E_NULL, "rdb_linear_bwd_projected: dx, dcoef, dy, z or coef is NULL");
     if (lddy < d->out_f || lddx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_projected: leading dimension smaller than the row");
-    rc = linear_bwd_projected(dx, lddx, dcoef, dy, lddy, z, coef, d, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
-    if (rc == RDB_E_UNSUPPORTED)
+    const rdb_linear_desc first = chunk_desc(d, pl, 0);
+    if (d->coef_dtype != RDB_BF16 || lddy % 8 || lddx % 8 || !aligned16(dy) || !aligned16(dx) || !aligned16(z) || !aligned16(coef) ||
+        !aligned16(dcoef) || !aligned16(workspace) || pl.chunk_tokens * lddy >= (1ll << 29) || pl.chunk_tokens * lddx >= (1ll << 29) || !workspace ||
+        workspace_bytes < linear_dx_factored_workspace(&first))
         return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_projected: coefficients must be bf16; all pointers 16-byte aligned; lddy, lddx "
-                                            "multiples of 8; tokens*lddy < 2^29; workspace of rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX) "
-                                            "bytes");
-    return rc;
+                                            "multiples of 8 and below twice the row; workspace of rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX) "
+                                            "bytes at least");
+    for (int c = 0; c < pl.nchunks; ++c) {
+        const rdb_linear_desc dd = chunk_desc(d, pl, c);
+        rc = linear_bwd_projected(at_bytes(dx, c * pl.chunk_tokens * lddx * 2), lddx, dcoef, at_bytes(dy, c * pl.chunk_tokens * lddy * 2), lddy,
+                                  at_bytes(z, c * pl.state_stride), coef, &dd, num_compute_units(), workspace, workspace_bytes, c > 0,
+                                  (hipStream_t)stream);
+        if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_projected: internal: chunk %d of %d refused", c, pl.nchunks);
+        if (rc) return rc;
+    }
+    return RDB_OK;
 }

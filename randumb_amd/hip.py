@@ -271,10 +271,8 @@ def linear_projection_bytes(tokens: int, in_f: int, out_f: int, k: int) -> int:
 
 
 def linear_projection_supported(tokens: int, in_f: int, out_f: int, k: int) -> bool:
-    """Whether the projected entry points run a layer of these sizes: matrix-coef bf16, sizes in multiples of 8, and
-    activations and gradients inside the kernels' 32-bit addressing (tokens*in_f, tokens*out_f < 2^29)."""
-    if tokens * in_f >= 2**29 or tokens * out_f >= 2**29:
-        return False
+    """Whether the projected entry points run a layer of these sizes: matrix-coef bf16, sizes in multiples of 8 (any number
+    of tokens: activations beyond one launch's 2^29 elements are run in chunks of tokens by the library)."""
     return linear_projection_bytes(tokens, in_f, out_f, k) > 0
 
 

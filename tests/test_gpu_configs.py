@@ -132,6 +132,40 @@ def test_projected_form_against_the_kernels_that_form_the_weight(hip, T, in_f, o
     assert rel_l2(cpu(dC), cpu(dC_w)) < 1e-2
 
 
+def test_more_tokens_than_one_launch_addresses(hip, oracle):
+    """65536 tokens through 4096 -> 14336 (k = 256): dy and y hold 2^29.8 elements, more than one launch addresses, so the
+    projected entry points run the layer in 4 chunks of 16384 tokens.  y and dx on tokens from every chunk (and both sides of
+    every chunk boundary) against the oracle; dC rows against dy^T.(x.N^T) over ALL tokens in fp64 with the oracle's noise;
+    dC the same bits on a second run (the chunks' sums are added in chunk order)."""
+    print("case config: 65536 tokens x 4096->14336 k=256, chunked", flush=True)
+    T, in_f, out_f, k, seed = 65536, 4096, 14336, 256, 5
+    assert hip.linear_projection_supported(T, in_f, out_f, k)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn(T, in_f, generator=g, device="cuda", dtype=torch.float32).bfloat16()
+    C = (torch.randn(out_f, k, generator=g, device="cuda") * (3.0 / k) ** 0.5 / 64.0).bfloat16()
+    osel = np.sort(np.random.default_rng(0).choice(out_f, size=96, replace=False))
+    tok = np.array([0, 1, 16383, 16384, 16385, 32767, 32768, 40000, 49151, 49152, 65534, 65535])
+    # dy non-zero on the chosen output rows only (dx then needs only those rows of W), but on every token
+    dy = torch.zeros(T, out_f, device="cuda", dtype=torch.bfloat16)
+    dy[:, torch.from_numpy(osel).cuda()] = torch.randn(T, len(osel), generator=g, device="cuda").bfloat16()
+    state = hip.linear_project(x, k, out_f, seed, coef=C)
+    y = hip.linear_fwd_projected(state, C, in_f, seed)
+    dx, dC = hip.linear_bwd_projected(dy, state, C, in_f, seed)
+    dx2, dC2 = hip.linear_bwd_projected(dy, state, C, in_f, seed)
+    torch.cuda.synchronize()
+    assert y.shape == (T, out_f) and dx.shape == (T, in_f) and dC.shape == (out_f, k)
+    assert torch.equal(dC, dC2) and torch.equal(dx, dx2)
+    xs, Cs = cpu(x[tok]), cpu(C)[osel]
+    assert rel_l2(cpu(y[tok])[:, osel], oracle.linear_fwd(xs, Cs, in_f, len(osel), seed)) < BF16_TOL
+    want_dx, _, _ = oracle.linear_bwd(xs, cpu(dy[tok])[:, osel], Cs, in_f, len(osel), seed)
+    assert rel_l2(cpu(dx[tok]), want_dx) < BF16_TOL
+    noise = torch.from_numpy(oracle.noise_2d(in_f, k, seed)).cuda().double()
+    want_dC = dy[:, torch.from_numpy(osel).cuda()].double().t() @ (x.double() @ noise)
+    assert rel_l2(cpu(dC)[osel], want_dC.cpu().numpy()) < BF16_TOL
+    rest = np.setdiff1d(np.arange(out_f), osel)[:64]
+    assert float(dC[torch.from_numpy(rest).cuda()].abs().max()) == 0.0   # rows whose dy is zero
+
+
 @pytest.mark.parametrize("batch", [1, 16, 256])
 @pytest.mark.parametrize("matrix", [True, False])
 def test_small_k_fp32_regime(hip, oracle, batch, matrix):

@@ -94,10 +94,23 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     assert L.rdb_linear_projection_bytes(ctypes.byref(desc(64, 96, 32, 16, rows=0))) == 0              # vector-coef
     assert L.rdb_linear_projection_bytes(ctypes.byref(desc(64, 96, 32, 16, act=_lib.RDB_F32))) == 0    # fp32 activations
     assert L.rdb_linear_projection_bytes(None) == 0
-    # operands of 2^29 elements or more are outside the engine's 32-bit buffer addressing: no projected form
-    assert L.rdb_linear_projection_bytes(ctypes.byref(desc(1 << 21, 768, 3072, 256))) == 0          # tokens*k = 2^29
-    assert L.rdb_linear_projection_bytes(ctypes.byref(desc((1 << 21) - 8, 768, 3072, 256))) == 0    # tokens rounded up to 64
-    assert L.rdb_linear_projection_bytes(ctypes.byref(desc((1 << 21) - 64, 768, 3072, 256))) == state_bytes((1 << 21) - 64, 3072, 256)
+    # activations of 2^29 elements or more are outside one launch's 32-bit addressing: the layer is run in chunks of tokens,
+    # each with a state of its own (chunks of at most 2^28 / widest row tokens, a multiple of 256, about equal)
+    ct = ctypes.c_int64()
+    assert L.rdb_linear_projection_chunks(r, ctypes.byref(ct)) == 1 and ct.value == 8192
+    big = desc(65536, 4096, 14336, 256)
+    assert L.rdb_linear_projection_chunks(ctypes.byref(big), ctypes.byref(ct)) == 4 and ct.value == 16384   # 2^28 / 14336 = 18724 -> 18688
+    assert L.rdb_linear_projection_bytes(ctypes.byref(big)) == 4 * state_bytes(16384, 14336, 256)
+    odd = desc(40000, 4096, 14336, 256)                                                   # 3 chunks of 13568, 13568, 12864
+    assert L.rdb_linear_projection_chunks(ctypes.byref(odd), ctypes.byref(ct)) == 3 and ct.value == 13568
+    assert L.rdb_linear_projection_bytes(ctypes.byref(odd)) == 3 * state_bytes(13568, 14336, 256)
+    assert L.rdb_linear_projection_chunks(ctypes.byref(desc(1 << 21, 768, 3072, 256)), ctypes.byref(ct)) == 25 and ct.value % 256 == 0
+    assert ct.value * 3072 < (1 << 28) + 256 * 3072
+    # chunks after the first add to dcoef: their sums pass through the workspace even when a chunk is a single token range
+    w_big = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_PROJECTED, ctypes.byref(big))
+    w_one = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_PROJECTED, ctypes.byref(desc(16384, 4096, 14336, 256)))
+    assert w_big >= w_one >= 16384 * 256 * 2 and (w_big - 16384 * 256 * 2) % (14336 * 256 * 4) == 0
+    assert L.rdb_linear_projection_layout(ctypes.byref(big), info) == -5 and b"4 states" in L.rdb_last_error_string()
     # fp32, small k: one partial [tokens x k] matrix per 256 values of the longer side
     f32 = desc(16, 4096, 4096, 16, act=_lib.RDB_F32, coef=_lib.RDB_F32)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(f32)) == 16 * 16 * 16 * 4
@@ -239,12 +252,10 @@ def test_projected_form_is_chosen_only_where_it_runs_and_pays():
     from randumb_amd import hip
 
     assert hip.linear_projection_supported(8192, 768, 3072, 256) and hip.linear_projection_preferred(8192, 768, 3072, 256)
-    # tokens*out_f >= 2^29 (65536 tokens x 14336): the projection exists but dy would not fit the kernels' addressing
+    # tokens*out_f >= 2^29 (65536 tokens x 14336): run in chunks of tokens by the library, so still the projected form
     assert hip.linear_projection_bytes(65536, 4096, 14336, 256) > 0
-    assert not hip.linear_projection_supported(65536, 4096, 14336, 256)
-    assert not hip.linear_projection_preferred(65536, 4096, 14336, 256)
-    # tokens*in_f >= 2^29
-    assert not hip.linear_projection_supported(1 << 17, 4096, 64, 8)
+    assert hip.linear_projection_supported(65536, 4096, 14336, 256) and hip.linear_projection_preferred(65536, 4096, 14336, 256)
+    assert hip.linear_projection_supported(1 << 17, 4096, 64, 8)
     # k >= in*out/(in+out): forming the weight is cheaper (768 -> 384 at k = 256 is exactly on the boundary)
     assert hip.linear_projection_supported(512, 768, 384, 256) and not hip.linear_projection_preferred(512, 768, 384, 256)
     assert hip.linear_projection_preferred(512, 768, 512, 256)
