@@ -293,6 +293,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
     ap.add_argument("--no-compare", action="store_true", help="skip the comparison legs and the other configurations")
     ap.add_argument("--no-graph", action="store_true", help="time eager calls only (profiling runs: one kernel record per launch)")
+    ap.add_argument("--vector-coef-only", action="store_true",
+                    help="run only the vector-coef (reference form) materialise kernels a few times and exit (counter runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch plain device copies of 256 MiB (a known 256 MiB read + 256 MiB written per launch) so that "
                          "hardware byte counters collected over this run can be scaled")
@@ -311,6 +313,15 @@ def main():
     L = _lib.load()
 
     g = torch.Generator().manual_seed(0)
+    if args.vector_coef_only:
+        c1 = (torch.randn(K, generator=g) * (3 * 0.02**2 / K) ** 0.5).to(dev)
+        dW = torch.randn(OUT_F, IN_F, generator=g).to(dev)
+        for _ in range(5):
+            hip.materialize_fwd(c1, (OUT_F, IN_F), (IN_F, 1), SEED, None, False)
+            hip.materialize_bwd(dW, K, SEED)
+        torch.cuda.synchronize()
+        print(json.dumps({"ran": "vector-coef materialize_fwd / materialize_bwd, 768x3072, k=256, 5 times each"}))
+        return
     main_set = LayerBuffers(L, _lib, torch, dev, g)
     sets = [main_set] + [LayerBuffers(L, _lib, torch, dev, g, share_inputs_of=main_set) for _ in range(2)]
     set_mb = sum(t.numel() * t.element_size() for t in (main_set.x, main_set.dy, main_set.y, main_set.dx, main_set.dC, main_set.ws,

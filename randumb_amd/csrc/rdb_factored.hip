@@ -19,10 +19,9 @@ constexpr float INV_2_31 = 4.656612873077392578125e-10f;
 constexpr int F_BK = 64;
 
 // ----------------------------------------------------------------------------------------------- z = x . N^T
-// tile: 32 coefficients (engine rows "a", hashed) x 256 tokens (engine rows "b"), 4 waves side by side along the tokens,
-// contraction over in_f; two blocks per CU.  The noise tile is hashed once per block, so the hash work of the kernel is
-// (tokens / 256) * in_f * k: the token tile is as long as the accumulators allow and the coefficient tile as short.
-constexpr int KZ_BM = 32, KZ_BT = 256, KZ_WM = 1;
+// tile: 32 coefficients (hashed) x 256 tokens, contraction over in_f.  The noise tile is hashed once per block, so the hash
+// work of the kernel is (tokens / 256) * in_f * k: the token tile is long and the coefficient tile short.
+constexpr int KZ_BM = 32, KZ_BT = 256;
 
 struct ZParams {
     const bf16_t *x;
@@ -38,59 +37,138 @@ struct ZParams {
     uint32_t seed;
 };
 
-__global__ __launch_bounds__(256, 2) void factored_z_kernel(ZParams p)
+// Eight waves, two to a SIMD: the tile's noise is hashed once per stage by all 512 threads (4 values each) on the vector ALU,
+// and while one wave of a SIMD hashes or waits for its x pieces the other one's MFMAs run.  Per stage of 64 input features:
+// x pieces (loaded two stages ahead) and the next stage's noise go registers -> LDS, 4 MFMAs per wave (its 32 tokens), one
+// barrier.  Written without the 256-thread tile engine; the LDS layouts and fragment reads are the engine's (OperandTile).
+constexpr int KZ_THREADS = 512;
+
+__global__ __launch_bounds__(KZ_THREADS, 1) void factored_z_kernel(ZParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
     if (blockIdx.x == 0 && t == 0) *p.flag = p.coef ? 1u : 0u;
-    if (p.coef) {
-        // C transposed into fragment order, a 1 KB unit (32 coefficients x 16 output features) per wave and turn: lane (r, g)
-        // gathers C[o0 + 8 g + j][m0 + r], j = 0..7 (32 lanes read 64 consecutive bytes of a row) and stores its 16 bytes
-        const int osteps = p.out64 >> 4, units = (p.kpad >> 5) * osteps, r = lane & 31, g = lane >> 5;
-        for (int u = blockIdx.x * 4 + wave; u < units; u += gridDim.x * 4) {
-            const int mb = u / osteps, os = u % osteps, m = mb * 32 + r;
-            uint32_t w[4];
+    // C transposed into fragment order, a 1 KB unit (32 coefficients x 16 output features) per wave and turn: lane (r, g)
+    // gathers C[o0 + 8 g + j][m0 + r], j = 0..7 (32 lanes read 64 consecutive bytes of a row) and stores its 16 bytes.
+    // The first turn's loads are issued here and stored after the tile's main loop, which hides their latency.
+    const int osteps = p.out64 >> 4, units = p.coef ? (p.kpad >> 5) * osteps : 0;
+    auto gather_unit = [&](int u, uint32_t (&w)[8]) {   // the raw values: combining them would wait for the loads
+        const int mb = u / osteps, os = u % osteps, m = mb * 32 + (lane & 31);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int o = os * 16 + g * 8 + 2 * j;   // out_f is even: o and o + 1 exist together
-                const bool in = m < p.k && o < p.out_f;
-                const uint32_t lo = in ? p.coef[(int64_t)o * p.k + m] : 0u, hi = in ? p.coef[(int64_t)(o + 1) * p.k + m] : 0u;
-                w[j] = lo | (hi << 16);
-            }
-            const i32x4 v = {(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
-            *reinterpret_cast<i32x4 *>(p.ctf + (int64_t)u * 512 + lane * 8) = v;
+        for (int j = 0; j < 8; ++j) {
+            const int o = os * 16 + (lane >> 5) * 8 + j;
+            w[j] = (m < p.k && o < p.out_f) ? p.coef[(int64_t)o * p.k + m] : 0u;
         }
-    }
+    };
+    auto store_unit = [&](int u, const uint32_t (&w)[8]) {
+        const i32x4 v = {(int)(w[0] | (w[1] << 16)), (int)(w[2] | (w[3] << 16)), (int)(w[4] | (w[5] << 16)), (int)(w[6] | (w[7] << 16))};
+        *reinterpret_cast<i32x4 *>(p.ctf + (int64_t)u * 512 + lane * 8) = v;
+    };
+    const int unit0 = blockIdx.x * (KZ_THREADS / 64) + wave, unit_step = gridDim.x * (KZ_THREADS / 64);
+    uint32_t cw0[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+    if (unit0 < units) gather_unit(unit0, cw0);
+    auto finish_units = [&]() {
+        if (unit0 < units) store_unit(unit0, cw0);
+        for (int u = unit0 + unit_step; u < units; u += unit_step) {
+            uint32_t w[8];
+            gather_unit(u, w);
+            store_unit(u, w);
+        }
+    };
     // work item = (token tile, coefficient tile), coefficient tile fastest: neighbours share the x tile
     const int w = xcd_work_item(blockIdx.x, p.tiles_m * p.tiles_t);
-    if (w >= p.tiles_m * p.tiles_t) return;
+    if (w >= p.tiles_m * p.tiles_t) {
+        finish_units();
+        return;
+    }
     const int m0 = (w % p.tiles_m) * KZ_BM, tok0 = (w / p.tiles_m) * KZ_BT;
-    constexpr int MI = KZ_BM / (32 * KZ_WM), NI = KZ_BT / (128 / KZ_WM);
-    f32x16 acc[MI][NI];
+    RDB_STAMP(0);
+    typedef OperandTile<KZ_BM, F_BK, K_CONT> TN;   // noise tile: rows = coefficients, contraction = input features
+    typedef OperandTile<KZ_BT, F_BK, K_CONT> TX;   // x tile: rows = tokens
+    constexpr int STAGE = TN::LDS_ELEMS + TX::LDS_ELEMS, XP = KZ_BT * F_BK / 8 / KZ_THREADS;   // x pieces per thread and stage: 4
+    const int nstage = (p.in_f + F_BK - 1) / F_BK;
+    const __amdgpu_buffer_rsrc_t rs_x =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.x), 0, (int)(((int64_t)(p.tokens - 1) * p.ldx + p.in_f) * 2), 0x00020000);
+    // this thread's x pieces: rows idx / 8, 16-byte chunk idx % 8 of the stage's 64 features
+    uint32_t xoff[XP];
+    int xlds[XP];
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
+    for (int q = 0; q < XP; ++q) {
+        const int idx = q * KZ_THREADS + t, row = idx >> 3, c = idx & 7;
+        xoff[q] = (tok0 + row < p.tokens) ? (uint32_t)(((int64_t)(tok0 + row) * p.ldx + c * 8) * 2) : BUFFER_OOB;
+        xlds[q] = row * TX::LD + ((c ^ TX::swz(row)) * 8);
+    }
+    const int xc8 = (t & 7) * 8;   // the same for all of a thread's pieces (512 % 8 == 0)
+    auto load_x = [&](f32x4 (&r)[XP], int stage) {
+        const uint32_t adv = (stage * F_BK + xc8 < p.in_f) ? (uint32_t)(stage * F_BK * 2) : BUFFER_OOB;   // in_f % 8 == 0
 #pragma unroll
-        for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = zero16();
-    // "A": 2^31 * noise(i, m), rows = m, contraction = i; values for i >= in_f meet zero columns of x
-    NoiseOperandRowsAreCoefs<KZ_BM, F_BK> opn = {m0, p.seed};
-    GlobalOperand<KZ_BT, F_BK, K_CONT> opx = {p.x, p.ldx, tok0, p.tokens, p.in_f, (int64_t)(p.tokens - 1) * p.ldx + p.in_f};
-    gemm_mainloop<KZ_BM, KZ_BT, F_BK, 1, 1, KZ_WM>(acc, lds, opn, opx, 0, (p.in_f + F_BK - 1) / F_BK);
+        for (int q = 0; q < XP; ++q) r[q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs_x, (int)(xoff[q] + adv), 0, 0));
+    };
+    auto store_x = [&](bf16_t *buf, const f32x4 (&r)[XP]) {
+#pragma unroll
+        for (int q = 0; q < XP; ++q) *reinterpret_cast<f32x4 *>(buf + TN::LDS_ELEMS + xlds[q]) = r[q];
+    };
+    // this thread's share of the noise tile: coefficient row t / 16, features (t % 16) * 4 .. + 3 of the stage (8 bytes);
+    // values for features past in_f meet zero columns of x
+    const int nrow = t >> 4, nk = (t & 15) * 4;
+    const int nlds = nrow * TN::LD + (((nk >> 3) ^ TN::swz(nrow)) * 8) + (nk & 7);
+    const uint32_t nfirst = sq5_first((uint32_t)nk, (uint32_t)(m0 + nrow), p.seed);   // noise(i, m): first(i, m), + PN1 per feature
+    auto hash_noise = [&](bf16_t *buf, int stage) {
+        const uint32_t f0 = nfirst + (uint32_t)(stage * F_BK) * PN1;
+        uint2 v;
+        v.x = f32x2_to_bf16x2((float)(int32_t)sq5_tail(f0), (float)(int32_t)sq5_tail(f0 + PN1));
+        v.y = f32x2_to_bf16x2((float)(int32_t)sq5_tail(f0 + 2u * PN1), (float)(int32_t)sq5_tail(f0 + 3u * PN1));
+        *reinterpret_cast<uint2 *>(buf + nlds) = v;
+    };
+    f32x16 acc = zero16();
+    f32x4 rx[2][XP];
+    {
+        f32x4 rx0[XP];
+        load_x(rx0, 0);
+        load_x(rx[1], 1);
+        load_x(rx[0], 2);
+        hash_noise(lds, 0);
+        store_x(lds, rx0);
+    }
+    RDB_STAMP(1);
+    auto stage_body = [&](int s, int u, bool more) {   // stage s in LDS buffer u (= s % 2); slot (u ^ 1) of rx holds stage s + 1
+        bf16_t *cur = lds + u * STAGE, *oth = lds + (u ^ 1) * STAGE;
+        __syncthreads();   // stage s is complete in `cur`; everybody has finished reading `oth` (stage s - 1)
+        bf16x8 fa[4], fb[4];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            fa[ks] = TN::frag(cur, 0, ks, lane);
+            fb[ks] = TX::frag(cur + TN::LDS_ELEMS, wave * 32, ks, lane);
+        }
+        if (more) {
+            store_x(oth, rx[u ^ 1]);
+            load_x(rx[u ^ 1], s + 3);
+            hash_noise(oth, s + 1);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks], fb[ks], acc, 0, 0, 0);
+    };
+    int s = 0;
+    for (; s + 2 < nstage; s += 2) {
+        stage_body(s, 0, true);
+        stage_body(s + 1, 1, true);
+    }
+    stage_body(s, 0, s + 1 < nstage);
+    if (s + 1 < nstage) stage_body(s + 1, 1, false);
+    finish_units();
+    __syncthreads();   // the last stage's fragment reads are done: the tile buffers may be reused
+    RDB_STAMP(2);
     // The tile D[a = coefficient][b = token] goes to LDS once, as bf16 rows of tokens (LD elements apart), and leaves in
     // up to two orders.  Rows of tokens past the end and coefficients past k hold zeros or finite values: every byte of the
     // state's z pieces is written, so that their consumers may multiply padding with zeros.
-    static_assert(MI == 1 && KZ_WM == 1, "the epilogue below is written for one 32-coefficient row block per wave");
     constexpr int LD = KZ_BM + 8;
     {
-        const int r = lane & 31, g = lane >> 5;
+        const int r = lane & 31, g = lane >> 5, b = wave * 32 + r;
 #pragma unroll
         for (int jq = 0; jq < 4; ++jq)
-#pragma unroll
-            for (int ni = 0; ni < NI; ++ni) {
-                const int b = wave * NI * 32 + ni * 32 + r;
-                store4<bf16_t>(lds + b * LD + 8 * jq + 4 * g, acc[0][ni][jq * 4 + 0] * INV_2_31, acc[0][ni][jq * 4 + 1] * INV_2_31,
-                               acc[0][ni][jq * 4 + 2] * INV_2_31, acc[0][ni][jq * 4 + 3] * INV_2_31);
-            }
+            store4<bf16_t>(lds + b * LD + 8 * jq + 4 * g, acc[jq * 4 + 0] * INV_2_31, acc[jq * 4 + 1] * INV_2_31, acc[jq * 4 + 2] * INV_2_31,
+                           acc[jq * 4 + 3] * INV_2_31);
     }
     __syncthreads();
     constexpr int PIECES = KZ_BM * KZ_BT / 8;
@@ -98,8 +176,8 @@ __global__ __launch_bounds__(256, 2) void factored_z_kernel(ZParams p)
         // rows = tokens, k = coefficients: a piece is 8 coefficients of one token, neighbouring lanes take neighbouring tokens
         const int ksteps = p.kpad >> 4;
 #pragma unroll
-        for (int q = 0; q < PIECES / 256; ++q) {
-            const int idx = q * 256 + t, b = idx % KZ_BT, a = (idx / KZ_BT) * 8;
+        for (int q = 0; q < PIECES / KZ_THREADS; ++q) {
+            const int idx = q * KZ_THREADS + t, b = idx % KZ_BT, a = (idx / KZ_BT) * 8;
             const int gb = tok0 + b, ga = m0 + a;
             if (gb < p.tok32)
                 *reinterpret_cast<f32x4 *>(p.zf + ((int64_t)(gb >> 5) * ksteps + (ga >> 4)) * 512 + (((ga >> 3) & 1) * 32 + (gb & 31)) * 8) =
@@ -107,20 +185,20 @@ __global__ __launch_bounds__(256, 2) void factored_z_kernel(ZParams p)
         }
     } else {
 #pragma unroll
-        for (int q = 0; q < PIECES / 256; ++q) {
-            const int idx = q * 256 + t, b = idx / (KZ_BM / 8), a = (idx % (KZ_BM / 8)) * 8;
+        for (int q = 0; q < PIECES / KZ_THREADS; ++q) {
+            const int idx = q * KZ_THREADS + t, b = idx / (KZ_BM / 8), a = (idx % (KZ_BM / 8)) * 8;
             if (tok0 + b < p.tokens && m0 + a < p.k)
                 *reinterpret_cast<f32x4 *>(p.zf + (int64_t)(tok0 + b) * p.k + m0 + a) = *reinterpret_cast<const f32x4 *>(lds + b * LD + a);
         }
     }
     {
         // rows = coefficients, k = tokens: the LDS transpose read turns 16 token rows x 32 coefficients into the fragment
-        const int tsteps = p.tok64 >> 4, s = lane & 15, qq = (lane >> 4) & 1, g = lane >> 5;
+        const int tsteps = p.tok64 >> 4, sl = lane & 15, qq = (lane >> 4) & 1, g = lane >> 5;
 #pragma unroll
-        for (int q = 0; q < KZ_BT / 16 / 4; ++q) {
-            const int ks = wave * (KZ_BT / 16 / 4) + q;   // token k-step inside the tile
+        for (int q = 0; q < KZ_BT / 16 / (KZ_THREADS / 64); ++q) {
+            const int ks = wave * (KZ_BT / 16 / (KZ_THREADS / 64)) + q;   // token k-step inside the tile
             if (tok0 + ks * 16 >= p.tok64) continue;
-            const bf16_t *src = lds + (ks * 16 + g * 8 + (s >> 2)) * LD + qq * 16 + (s & 3) * 4;
+            const bf16_t *src = lds + (ks * 16 + g * 8 + (sl >> 2)) * LD + qq * 16 + (sl & 3) * 4;
             Frag8 f;
             f.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(src));
             f.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(src + 4 * LD));
@@ -232,7 +310,10 @@ int linear_project(void *state, const void *x, int64_t ldx, const void *coef, co
     p.seed = d->seed;
     p.tiles_m = L.kpad / KZ_BM;   // every coefficient row block of the padded pieces is written
     p.tiles_t = (int)cdiv(d->tokens, KZ_BT);
-    return launch_engine(factored_z_kernel, p, p.tiles_m * p.tiles_t, engine_smem<KZ_BM, KZ_BT, F_BK, K_CONT, K_CONT>(), s, "factored_z_kernel");
+    const size_t smem = engine_smem<KZ_BM, KZ_BT, F_BK, K_CONT, K_CONT>();
+    if (int rl = reserve_lds(reinterpret_cast<const void *>(factored_z_kernel), smem, "factored_z_kernel")) return rl;
+    factored_z_kernel<<<xcd_grid_size(p.tiles_m * p.tiles_t), KZ_THREADS, smem, s>>>(p);
+    return check_launch("factored_z_kernel");
 }
 
 int linear_fwd_projected(void *y, int64_t ldy, const void *state, const void *coef, const void *bias, const rdb_linear_desc *d, int num_cus,
