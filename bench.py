@@ -432,10 +432,15 @@ def main():
     traffic = profiled_traffic(dom_kernels)
     executed_frac = dom_exec / (dom_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS
     hbm_frac = None if traffic is None else traffic / (dom_ms * 1e-3) / 1e12 / HBM_PEAK_TBPS
+    # bytes the call has to move whatever the algorithm: its inputs once, its outputs once
+    min_bytes = 2.0 * (T * OUT_F + OUT_F * K + T * IN_F) + 4.0 * OUT_F * K if dom == "backward" else 2.0 * (T * IN_F + OUT_F * K + T * OUT_F)
+    hbm_min_frac = min_bytes / (dom_ms * 1e-3) / 1e12 / HBM_PEAK_TBPS
     roofline = {
-        # the nearer of the two rooflines; neither pipe is saturated: the kernels are bound by LDS / vector-memory issue and
-        # memory latency, see the SQ counters under profiles/
-        "bound": "mfma" if hbm_frac is None or executed_frac >= hbm_frac else "hbm",
+        # the roofline of the metric (share of the MFMA peak).  On the flops the factored algorithm executes the call is at
+        # `executed_frac` of that peak and, on the bytes it has to move, at `hbm_min_frac` of the HBM peak (`hbm_frac`: on the bytes
+        # the counters saw): the matrix cores are the nearer wall, neither is reached; the kernels are held by LDS /
+        # vector-memory issue and memory latency, see the SQ counters under profiles/
+        "bound": "mfma",
         "kernel": f"{dom} call ({' + '.join(dom_kernels)})",
         "achieved": round(achieved, 3), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 5),
         "traffic": traffic, "traffic_source": "profiles/bench_c2_hbm_traffic.md" if traffic is not None else None,
@@ -444,6 +449,7 @@ def main():
         "executed_gflop_per_launch": round(dom_exec / 1e9, 3),
         "executed_achieved": round(dom_exec / (dom_ms * 1e-3) / 1e12, 3), "executed_frac": round(executed_frac, 5),
         "hbm_frac": None if hbm_frac is None else round(hbm_frac, 5),
+        "hbm_min_bytes_per_launch": min_bytes, "hbm_min_frac": round(hbm_min_frac, 5),
         "calls_ms": {n: round(v, 5) for n, v in calls.items()},
     }
 
