@@ -441,6 +441,7 @@ def main():
         # the counters saw): the matrix cores are the nearer wall, neither is reached; the kernels are held by LDS /
         # vector-memory issue and memory latency, see the SQ counters under profiles/
         "bound": "mfma",
+        "bound_observed": "neither pipe: waits on vector memory and LDS issue (profiles/bench_c2_sq_counters.md)",
         "kernel": f"{dom} call ({' + '.join(dom_kernels)})",
         "achieved": round(achieved, 3), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 5),
         "traffic": traffic, "traffic_source": "profiles/bench_c2_hbm_traffic.md" if traffic is not None else None,

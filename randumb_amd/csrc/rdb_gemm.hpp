@@ -176,8 +176,9 @@ template <int ROWS, int BK, int LAYOUT> struct GlobalOperand {
         uint32_t adv;
         if (LAYOUT == K_CONT)
             adv = (k_begin + stage * BK + kk < klim) ? (uint32_t)(stage * BK * 2) : BUFFER_OOB;
-        else
-            adv = (uint32_t)stage * (uint32_t)(BK * 2) * (uint32_t)ld;
+        else   // stages that begin at or past klim (round-up of the trip count, prefetch past the end) must not depend on the
+               // 32-bit product below staying out of bounds: with a huge leading dimension it could wrap back into the buffer
+            adv = (k_begin + stage * BK < klim) ? (uint32_t)stage * (uint32_t)(BK * 2) * (uint32_t)ld : BUFFER_OOB;
         Tile::load_piece(reg, rsrc, q, p, adv);
     }
     __device__ __forceinline__ void load(f32x4 (&regs)[Tile::PER_THREAD], int stage) const

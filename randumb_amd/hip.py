@@ -40,6 +40,8 @@ def _stream(device) -> ctypes.c_void_p:
 
 
 def _workspace(nbytes: int, device) -> Optional[torch.Tensor]:
+    # torch's caching allocator is the reusable pool: a block freed by the previous call on this stream comes back without
+    # a device allocation, and blocks are never handed to another stream while work on them is pending
     return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes > 0 else None
 
 
@@ -114,9 +116,9 @@ def materialize_bwd(dout: torch.Tensor, dcoefs_size: int, seed: int, coef_rows: 
     row_len = 0 if coef_rows == 0 else Nw // max(coef_rows, 1)
     dcoefs = torch.empty(shape, dtype=torch.float32, device=d.device)
     L = _lib.load()
-    ws_bytes = L.rdb_materialize_bwd_workspace_bytes(coef_rows, k, row_len, Nw)
-    ws = _workspace(ws_bytes, d.device)
     with torch.cuda.device(d.device):
+        ws_bytes = L.rdb_materialize_bwd_workspace_bytes(coef_rows, k, row_len, Nw)
+        ws = _workspace(ws_bytes, d.device)
         rc = L.rdb_materialize_bwd(_p(dcoefs), _p(d), _DT[d.dtype], coef_rows, k, row_len, Nw, _seed(seed), _p(ws), ws_bytes,
                                    _stream(d.device))
     _lib.check(rc, "rdb_materialize_bwd")
@@ -130,9 +132,9 @@ def scale_bias_bwd(dout: torch.Tensor, seed: int) -> torch.Tensor:
     d = _native(dout)
     ds = torch.empty((1,), dtype=torch.float32, device=d.device)
     L = _lib.load()
-    ws_bytes = L.rdb_scale_bias_bwd_workspace_bytes(d.numel())
-    ws = _workspace(ws_bytes, d.device)
     with torch.cuda.device(d.device):
+        ws_bytes = L.rdb_scale_bias_bwd_workspace_bytes(d.numel())
+        ws = _workspace(ws_bytes, d.device)
         rc = L.rdb_scale_bias_bwd(_p(ds), _p(d), _DT[d.dtype], d.numel(), _seed(seed), _p(ws), ws_bytes, _stream(d.device))
     _lib.check(rc, "rdb_scale_bias_bwd")
     return ds
@@ -160,9 +162,9 @@ def embed_bwd(idx: torch.Tensor, dout: torch.Tensor, dcoefs_size: int, rowsize: 
     k = int(dcoefs_size)
     dcoefs = torch.empty((k,), dtype=torch.float32, device=d.device)
     L = _lib.load()
-    ws_bytes = L.rdb_embed_bwd_workspace_bytes(ix.numel(), int(rowsize), k)
-    ws = _workspace(ws_bytes, d.device)
     with torch.cuda.device(d.device):
+        ws_bytes = L.rdb_embed_bwd_workspace_bytes(ix.numel(), int(rowsize), k)
+        ws = _workspace(ws_bytes, d.device)
         rc = L.rdb_embed_bwd(_p(dcoefs), _p(ix), ix.numel(), _p(d), _DT[d.dtype], k, int(rowsize), _seed(seed), _p(ws), ws_bytes,
                              _stream(d.device))
     _lib.check(rc, "rdb_embed_bwd")
@@ -204,9 +206,9 @@ def linear_fwd(x: torch.Tensor, coef: torch.Tensor, in_f: int, out_f: int, sO: i
     y = torch.empty((x.shape[0], out_f), dtype=x.dtype, device=x.device)
     d = _desc(x.shape[0], in_f, out_f, c, sO, sI, seed, x.dtype, algo)
     L = _lib.load()
-    ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_FWD, ctypes.byref(d))
-    ws = _workspace(ws_bytes, x.device)
     with torch.cuda.device(x.device):
+        ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_FWD, ctypes.byref(d))
+        ws = _workspace(ws_bytes, x.device)
         rc = L.rdb_linear_fwd(_p(y), y.stride(0), _p(x), x.stride(0), _p(c), _p(sb), _p(b), ctypes.byref(d), _p(ws), ws_bytes,
                               _stream(x.device))
     _lib.check(rc, "rdb_linear_fwd")
@@ -223,9 +225,9 @@ def linear_bwd_dx(dy: torch.Tensor, coef: torch.Tensor, in_f: int, out_f: int, s
     dx = torch.empty((dy.shape[0], in_f), dtype=dy.dtype, device=dy.device)
     d = _desc(dy.shape[0], in_f, out_f, c, sO, sI, seed, dy.dtype, algo)
     L = _lib.load()
-    ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX, ctypes.byref(d))
-    ws = _workspace(ws_bytes, dy.device)
     with torch.cuda.device(dy.device):
+        ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX, ctypes.byref(d))
+        ws = _workspace(ws_bytes, dy.device)
         rc = L.rdb_linear_bwd_dx(_p(dx), dx.stride(0), _p(dy), dy.stride(0), _p(c), _p(sb), ctypes.byref(d), _p(ws), ws_bytes,
                                  _stream(dy.device))
     _lib.check(rc, "rdb_linear_bwd_dx")
@@ -247,9 +249,9 @@ def linear_bwd_dcoef(dy: torch.Tensor, x: torch.Tensor, k: int, coef_rows: int, 
     d.sO, d.sI, d.seed = int(sO), int(sI), _seed(seed)
     d.act_dtype, d.coef_dtype, d.algo = _DT[dy.dtype], RDB_F32, int(algo)
     L = _lib.load()
-    ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DCOEF, ctypes.byref(d))
-    ws = _workspace(ws_bytes, dy.device)
     with torch.cuda.device(dy.device):
+        ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DCOEF, ctypes.byref(d))
+        ws = _workspace(ws_bytes, dy.device)
         rc = L.rdb_linear_bwd_dcoef(_p(dcoef), _p(dsb), _p(dy), dy.stride(0), _p(x), x.stride(0), ctypes.byref(d), _p(ws), ws_bytes,
                                     _stream(dy.device))
     _lib.check(rc, "rdb_linear_bwd_dcoef")
@@ -392,9 +394,9 @@ def linear_bwd_projected(dy: torch.Tensor, state: torch.Tensor, coef: torch.Tens
     dx = torch.empty((dy.shape[0], in_f), dtype=dy.dtype, device=dy.device)
     dcoef = torch.empty((out_f, k), dtype=torch.float32, device=dy.device)
     L = _lib.load()
-    ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_PROJECTED if ordered_sums else RDB_OP_LINEAR_BWD_DX, ctypes.byref(d))
-    ws = _workspace(ws_bytes, dy.device)
     with torch.cuda.device(dy.device):
+        ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_PROJECTED if ordered_sums else RDB_OP_LINEAR_BWD_DX, ctypes.byref(d))
+        ws = _workspace(ws_bytes, dy.device)
         rc = L.rdb_linear_bwd_projected(_p(dx), dx.stride(0), _p(dcoef), _p(dy), dy.stride(0), _p(z), _p(c), ctypes.byref(d), _p(ws),
                                         ws_bytes, _stream(dy.device))
     _lib.check(rc, "rdb_linear_bwd_projected")
