@@ -7,17 +7,17 @@ activations with fp32 accumulation, x ~ N(0,1), dy ~ N(0,1), C ~ N(0, 3*0.02^2/k
 
 A "step" is one pass of the hot path, y = x W^T, dx = dy W, dC = (dy^T x) N^T with W = C N never stored, through
 the C ABI of librandumb_hip.so with inputs already resident in HBM, the way a training step calls it:
-  forward   rdb_linear_project (z = x N^T and the transposed coefficients, kept for the backward pass in place of x)
-            + rdb_linear_fwd_projected
+  forward   rdb_linear_project_fwd (z = x N^T and the transposed coefficients, kept for the backward pass in place of x,
+            and y = z C^T, in one launch)
   backward  rdb_linear_bwd_projected (dx and dC from dy, the projection state and C, in two launches)
 Every buffer (inputs, outputs, projection state, workspace) is allocated before the timed region.
 
 What the printed JSON line says, and with which clock:
   ms_per_step            host clock (time.perf_counter) around exactly --steps steps, a device synchronisation on both sides,
                          every step on the SAME buffers: about 150 MB per step, which the 256 MB last-level cache holds from
-                         one step to the next.  A step is five launches of 10 to 40 us; Python issues them more slowly than
+                         one step to the next.  A step is three launches of 10 to 40 us; Python may issue them more slowly than
                          the GPU runs them, so the step is recorded into a HIP graph once and a timed step is one replay
-                         (ms_per_step_graph); ms_per_step_eager is the same loop with the three C-ABI calls issued one by one.
+                         (ms_per_step_graph); ms_per_step_eager is the same loop with the two C-ABI calls issued one by one.
                          ms_per_step is the smaller of the two and `launch` says which
   ms_per_step_rotating   the same loop over 3 buffer sets in turn (480 MB: nothing a step reads is left in a cache by the
                          step before): the number to expect inside a real training step
@@ -59,7 +59,7 @@ F_STEP = 3.0 * F_PER_PRODUCT
 EXEC_FWD = 2.0 * T * K * (IN_F + OUT_F)
 EXEC_BWD = 2.0 * T * K * (OUT_F + IN_F) + 2.0 * T * K * OUT_F
 EXEC_STEP = EXEC_FWD + EXEC_BWD
-FWD_KERNELS = ("factored_z_kernel", "factored_ys_kernel")
+FWD_KERNELS = ("factored_zy_kernel",)
 BWD_KERNELS = ("bwd_dc_dyc_kernel", "bwd_tns_red_kernel")
 SETTLE_STEPS = 400   # untimed, before the warm-up steps: about 30 ms of continuous work
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_c2_hbm_traffic.md")
@@ -111,16 +111,20 @@ class LayerBuffers:
         self.state = torch.empty(self.state_bytes, dtype=torch.uint8, device=dev)
         self.stream = vp(torch.cuda.current_stream().cuda_stream)
         self.p = p = {n: vp(getattr(self, n).data_ptr()) for n in ("x", "dy", "C", "y", "dx", "dC", "ws", "state")}
-        # the three calls of a step with their arguments marshalled once: the timed loop is the calls and nothing else
+        # the two calls of a step with their arguments marshalled once: the timed loop is the calls and nothing else
         self._step_calls = (
-            (L.rdb_linear_project, (p["state"], p["x"], IN_F, p["C"], self.dref, self.stream)),
-            (L.rdb_linear_fwd_projected, (p["y"], OUT_F, p["state"], p["C"], None, self.dref, self.stream)),
+            (L.rdb_linear_project_fwd, (p["y"], OUT_F, p["state"], p["x"], IN_F, p["C"], None, self.dref, self.stream)),
             (L.rdb_linear_bwd_projected, (p["dx"], IN_F, p["dC"], p["dy"], OUT_F, p["state"], p["C"], self.dref, p["ws"], self.ws_bytes, self.stream)),
         )
 
     def project(self):
         p = self.p
         self._lib.check(self.L.rdb_linear_project(p["state"], p["x"], IN_F, p["C"], self.dref, self.stream), "rdb_linear_project")
+
+    def project_fwd(self):
+        p = self.p
+        self._lib.check(self.L.rdb_linear_project_fwd(p["y"], OUT_F, p["state"], p["x"], IN_F, p["C"], None, self.dref, self.stream),
+                        "rdb_linear_project_fwd")
 
     def fwd_projected(self):
         p = self.p
@@ -142,7 +146,7 @@ class LayerBuffers:
                         "rdb_linear_bwd_dcoef_projected")
 
     def step(self, stream=None):
-        """the three calls; `stream` (a ctypes pointer) replaces the stream they were marshalled for (graph capture)"""
+        """the two calls; `stream` (a ctypes pointer) replaces the stream they were marshalled for (graph capture)"""
         rc = 0
         for fn, a in self._step_calls:
             rc |= fn(*a) if stream is None else fn(*a[:-1], stream)
@@ -373,7 +377,7 @@ def main():
         except Exception as e:   # capture not available: the eager loop is the measurement
             print(f"bench.py: HIP graph capture of the step failed ({e}); timing eager calls", file=sys.stderr)
     if ms_graph is not None and ms_graph < ms_eager:
-        ms_per_step, launch = ms_graph, "one HIP graph replay per step (the step's five launches captured once)"
+        ms_per_step, launch = ms_graph, "one HIP graph replay per step (the step's three launches captured once)"
     else:
         ms_per_step = ms_eager
     value = F_STEP / (ms_per_step * 1e-3) / 1e12
@@ -416,13 +420,14 @@ def main():
 
     iters = max(10, min(args.steps, 50))
     calls = {
-        "rdb_linear_project": event_ms(main_set.project, iters),
-        "rdb_linear_fwd_projected": event_ms(main_set.fwd_projected, iters),
+        "rdb_linear_project_fwd": event_ms(main_set.project_fwd, iters),
+        "rdb_linear_project (separate call)": event_ms(main_set.project, iters),
+        "rdb_linear_fwd_projected (separate call)": event_ms(main_set.fwd_projected, iters),
         "rdb_linear_bwd_projected": event_ms(main_set.bwd, iters),
         "rdb_linear_bwd_dx (separate call)": event_ms(main_set.dx_separate, iters),
         "rdb_linear_bwd_dcoef_projected (separate call)": event_ms(main_set.dcoef_separate, iters),
     }
-    fwd_ms = calls["rdb_linear_project"] + calls["rdb_linear_fwd_projected"]
+    fwd_ms = calls["rdb_linear_project_fwd"]
     bwd_ms = calls["rdb_linear_bwd_projected"]
     if bwd_ms >= fwd_ms:
         dom, dom_ms, dom_flops, dom_exec, dom_kernels = "backward", bwd_ms, 2 * F_PER_PRODUCT, EXEC_BWD, BWD_KERNELS

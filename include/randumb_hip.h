@@ -237,6 +237,16 @@ int rdb_linear_projection_layout(const rdb_linear_desc *desc, int64_t *info);
 int rdb_linear_project(void *state, const void *x, int64_t ldx, const void *coef, const rdb_linear_desc *desc,
                        void *stream);
 
+/* rdb_linear_project (with coef) and rdb_linear_fwd_projected in one call: state <- projection of x and transposed coef,
+ * y[t, o] = sum_m z[t, m] * coef[o, m] (+ bias[o]); coef must be bf16.  The forward pass of a training step (R.py:942-946
+ * with what autograd saves replaced by the state).  With k <= 256 it is a single kernel launch: the blocks that multiply
+ * start as the blocks that project leave the compute units, each waiting only for the 256 tokens it reads (per-tile tags
+ * inside the state, unique to the launch; the hardware hands out a launch's blocks in index order, so the waiting blocks
+ * cannot starve the ones they wait for; the wait is bounded and a block that gives up sets the state's second 32-bit word,
+ * which no run has shown).  Results are bit for bit those of the two separate calls. */
+int rdb_linear_project_fwd(void *y, int64_t ldy, void *state, const void *x, int64_t ldx, const void *coef,
+                           const void *bias, const rdb_linear_desc *desc, void *stream);
+
 /* y[t, o] = sum_m z[t, m] * coef[o, m] (+ bias[o]); coef must be bf16. */
 int rdb_linear_fwd_projected(void *y, int64_t ldy, const void *state, const void *coef, const void *bias,
                              const rdb_linear_desc *desc, void *stream);

@@ -40,6 +40,7 @@ EXPORTS = [
     "rdb_linear_projection_chunks",
     "rdb_linear_projection_layout",
     "rdb_linear_project",
+    "rdb_linear_project_fwd",
     "rdb_linear_fwd_projected",
     "rdb_linear_bwd_dcoef_projected",
     "rdb_linear_bwd_projected",
@@ -117,12 +118,14 @@ def load() -> ctypes.CDLL:
     L.rdb_linear_projection_layout.argtypes = [dp, ctypes.POINTER(i64)]
     L.rdb_linear_projection_layout.restype = ci
     L.rdb_linear_project.argtypes = [vp, vp, i64, vp, dp, vp]
+    L.rdb_linear_project_fwd.argtypes = [vp, i64, vp, vp, i64, vp, vp, dp, vp]
     L.rdb_linear_fwd_projected.argtypes = [vp, i64, vp, vp, vp, dp, vp]
     L.rdb_linear_bwd_dcoef_projected.argtypes = [vp, vp, i64, vp, dp, vp]
     L.rdb_linear_bwd_projected.argtypes = [vp, i64, vp, vp, i64, vp, vp, dp, vp, i64, vp]
     for name in ("rdb_sq5_fill_2d", "rdb_sq5_fill_1d", "rdb_materialize_fwd", "rdb_materialize_bwd", "rdb_scale_bias_bwd",
                  "rdb_embed_fwd", "rdb_embed_bwd", "rdb_linear_fwd", "rdb_linear_bwd_dx", "rdb_linear_bwd_dcoef",
-                 "rdb_linear_project", "rdb_linear_fwd_projected", "rdb_linear_bwd_dcoef_projected", "rdb_linear_bwd_projected"):
+                 "rdb_linear_project", "rdb_linear_project_fwd", "rdb_linear_fwd_projected", "rdb_linear_bwd_dcoef_projected",
+                 "rdb_linear_bwd_projected"):
         getattr(L, name).restype = ci
     _lib = L
     return L

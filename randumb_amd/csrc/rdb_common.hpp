@@ -101,6 +101,53 @@ inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // finds, per block, 4 kernels x 4 slots of two counters: the constant-rate wall clock (comparable across compute units) and
 // the shader clock.  Which of the 4 kernels a launch is, the harness says with an expression RDB_STAMP_KERNEL_ID over the
 // launch geometry (no extra registers or LDS in the kernels, so their occupancy is that of the library's build).
+// 16-byte store of data that the kernel which writes it does not read again (it is for the next launch, on other dies):
+// non-temporal, so the line does not wait dirty in this die's L2 for the write-back at the end of the kernel.
+template <class V> __device__ __forceinline__ void store_stream(V *dst, const V &v)
+{
+#ifdef RDB_NO_STREAM_STORES
+    *dst = v;
+#else
+    __builtin_nontemporal_store(v, dst);
+#endif
+}
+
+// ----------------------------------------------------------------------------------------------- producer -> consumer blocks of one launch
+// Blocks of one launch that consume what earlier blocks of the same launch produce: a producer publishes a 64-bit tag, unique
+// to the launch, in a slot of its own when its output is in memory; a consumer polls the slots it depends on.  Hardware
+// queues hand out the blocks of a launch in index order (per die), so a consumer that only waits for blocks with lower
+// indices cannot starve them.  The wait is bounded all the same: after SYNC_SPIN_LIMIT polls (a fraction of a second) the
+// consumer gives up, records it in *err and goes on with whatever is there.
+//
+// The dies' L2 caches are not coherent with each other, and the fences that make them so (write back / invalidate a whole
+// L2) cost microseconds per block.  So the data that passes from producer to consumer goes around them instead: stored and
+// loaded with device scope (SCOPE_DEVICE below: write-through, and read from memory), as the tags are.
+constexpr int SYNC_SPIN_LIMIT = 1 << 17;
+constexpr int SCOPE_DEVICE = 16;   // cache-policy argument of the raw buffer loads and stores: sc1
+
+// All threads of the block call this after their last store (with SCOPE_DEVICE) of the block's output.
+__device__ __forceinline__ void publish_tag(unsigned long long *slot, unsigned long long tag)
+{
+    __builtin_amdgcn_s_waitcnt(0);   // this wave's stores have been acknowledged at their scope
+    __syncthreads();                 // ... and every other wave's
+    if (threadIdx.x == 0) __hip_atomic_store(slot, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// One wave calls this: lanes 0 .. n - 1 (n <= 64) poll slots[0 .. n - 1].  Returns false after the spin limit.  Loads of the
+// producers' data that follow must use SCOPE_DEVICE.
+__device__ __forceinline__ bool await_tags(const unsigned long long *slots, int n, unsigned long long tag, unsigned int *err)
+{
+    const int lane = threadIdx.x & 63;
+    const unsigned long long *mine = slots + (lane < n ? lane : 0);
+    for (int it = 0; it < SYNC_SPIN_LIMIT; ++it) {
+        const unsigned long long v = __hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (__all(v == tag)) return true;
+        __builtin_amdgcn_s_sleep(20);
+    }
+    if (lane == 0) atomicOr(err, 2u);
+    return false;
+}
+
 #ifdef RDB_STAMPS
 #ifndef RDB_STAMP_KERNEL_ID
 #define RDB_STAMP_KERNEL_ID 0

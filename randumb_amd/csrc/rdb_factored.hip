@@ -12,6 +12,10 @@
 // (src/rten_cpp/RandumbTensor.py:942-946) and MmBackward's dW followed by materialize_bwd (RandumbTensor.py:979-990, 304-359).
 #include "rdb_blocks.hpp"
 #include "rdb_stationary.hpp"
+#include <algorithm>
+#include <atomic>
+#include <random>
+#include <unistd.h>
 
 namespace rdb {
 
@@ -35,6 +39,8 @@ struct ZParams {
     int kpad, tok32, tok64, out64, frag_fwd;
     int tiles_m, tiles_t;
     uint32_t seed;
+    unsigned long long *sync;   // NULL, or slots [tiles_t][tiles_m]: a block sets its slot to sync_tag when its tile is in memory
+    unsigned long long sync_tag;
 };
 
 // Eight waves, two to a SIMD: the tile's noise is hashed once per stage by all 512 threads (4 values each) on the vector ALU,
@@ -43,12 +49,15 @@ struct ZParams {
 // barrier.  Written without the 256-thread tile engine; the LDS layouts and fragment reads are the engine's (OperandTile).
 constexpr int KZ_THREADS = 512;
 
-__global__ __launch_bounds__(KZ_THREADS, 1) void factored_z_kernel(ZParams p)
+// `block` of `nblocks`: index of this block among the blocks that run this body; all KZ_THREADS threads must call.
+__device__ __forceinline__ void z_block(const ZParams &p, unsigned char *smem_raw, int block, int nblocks)
 {
-    extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
-    if (blockIdx.x == 0 && t == 0) *p.flag = p.coef ? 1u : 0u;
+    if (block == 0 && t == 0) {
+        p.flag[0] = p.coef ? 1u : 0u;
+        p.flag[1] = 0u;   // nobody has given up waiting on this state
+    }
     // C transposed into fragment order, a 1 KB unit (32 coefficients x 16 output features) per wave and turn: lane (r, g)
     // gathers C[o0 + 8 g + j][m0 + r], j = 0..7 (32 lanes read 64 consecutive bytes of a row) and stores its 16 bytes.
     // The first turn's loads are issued here and stored after the tile's main loop, which hides their latency.
@@ -63,9 +72,9 @@ __global__ __launch_bounds__(KZ_THREADS, 1) void factored_z_kernel(ZParams p)
     };
     auto store_unit = [&](int u, const uint32_t (&w)[8]) {
         const i32x4 v = {(int)(w[0] | (w[1] << 16)), (int)(w[2] | (w[3] << 16)), (int)(w[4] | (w[5] << 16)), (int)(w[6] | (w[7] << 16))};
-        *reinterpret_cast<i32x4 *>(p.ctf + (int64_t)u * 512 + lane * 8) = v;
+        store_stream(reinterpret_cast<i32x4 *>(p.ctf + (int64_t)u * 512 + lane * 8), v);
     };
-    const int unit0 = blockIdx.x * (KZ_THREADS / 64) + wave, unit_step = gridDim.x * (KZ_THREADS / 64);
+    const int unit0 = block * (KZ_THREADS / 64) + wave, unit_step = nblocks * (KZ_THREADS / 64);
     uint32_t cw0[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
     if (unit0 < units) gather_unit(unit0, cw0);
     auto finish_units = [&]() {
@@ -77,7 +86,7 @@ __global__ __launch_bounds__(KZ_THREADS, 1) void factored_z_kernel(ZParams p)
         }
     };
     // work item = (token tile, coefficient tile), coefficient tile fastest: neighbours share the x tile
-    const int w = xcd_work_item(blockIdx.x, p.tiles_m * p.tiles_t);
+    const int w = xcd_work_item(block, p.tiles_m * p.tiles_t);
     if (w >= p.tiles_m * p.tiles_t) {
         finish_units();
         return;
@@ -174,21 +183,24 @@ __global__ __launch_bounds__(KZ_THREADS, 1) void factored_z_kernel(ZParams p)
     constexpr int PIECES = KZ_BM * KZ_BT / 8;
     if (p.frag_fwd) {
         // rows = tokens, k = coefficients: a piece is 8 coefficients of one token, neighbouring lanes take neighbouring tokens
+        // device scope (written through): blocks of this very launch on other dies may be waiting for the tile
         const int ksteps = p.kpad >> 4;
+        const __amdgpu_buffer_rsrc_t rs_zf = __builtin_amdgcn_make_buffer_rsrc(p.zf, 0, (int)((int64_t)p.tok32 * p.kpad * 2), 0x00020000);
 #pragma unroll
         for (int q = 0; q < PIECES / KZ_THREADS; ++q) {
             const int idx = q * KZ_THREADS + t, b = idx % KZ_BT, a = (idx / KZ_BT) * 8;
             const int gb = tok0 + b, ga = m0 + a;
             if (gb < p.tok32)
-                *reinterpret_cast<f32x4 *>(p.zf + ((int64_t)(gb >> 5) * ksteps + (ga >> 4)) * 512 + (((ga >> 3) & 1) * 32 + (gb & 31)) * 8) =
-                    *reinterpret_cast<const f32x4 *>(lds + b * LD + a);
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, *reinterpret_cast<const f32x4 *>(lds + b * LD + a)), rs_zf,
+                                                       (int)((((gb >> 5) * ksteps + (ga >> 4)) * 512 + (((ga >> 3) & 1) * 32 + (gb & 31)) * 8) * 2), 0,
+                                                       SCOPE_DEVICE);
         }
     } else {
 #pragma unroll
         for (int q = 0; q < PIECES / KZ_THREADS; ++q) {
             const int idx = q * KZ_THREADS + t, b = idx / (KZ_BM / 8), a = (idx % (KZ_BM / 8)) * 8;
             if (tok0 + b < p.tokens && m0 + a < p.k)
-                *reinterpret_cast<f32x4 *>(p.zf + (int64_t)(tok0 + b) * p.k + m0 + a) = *reinterpret_cast<const f32x4 *>(lds + b * LD + a);
+                store_stream(reinterpret_cast<f32x4 *>(p.zf + (int64_t)(tok0 + b) * p.k + m0 + a), *reinterpret_cast<const f32x4 *>(lds + b * LD + a));
         }
     }
     {
@@ -202,10 +214,17 @@ __global__ __launch_bounds__(KZ_THREADS, 1) void factored_z_kernel(ZParams p)
             Frag8 f;
             f.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(src));
             f.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(src + 4 * LD));
-            *reinterpret_cast<f32x4 *>(p.ztf + ((int64_t)(m0 >> 5) * tsteps + (tok0 >> 4) + ks) * 512 + lane * 8) = f.f4;
+            store_stream(reinterpret_cast<f32x4 *>(p.ztf + ((int64_t)(m0 >> 5) * tsteps + (tok0 >> 4) + ks) * 512 + lane * 8), f.f4);
         }
     }
+    if (p.sync) publish_tag(p.sync + (int64_t)(w / p.tiles_m) * p.tiles_m + (w % p.tiles_m), p.sync_tag);
     RDB_STAMP(3);
+}
+
+__global__ __launch_bounds__(KZ_THREADS, 1) void factored_z_kernel(ZParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    z_block(p, smem_raw, blockIdx.x, gridDim.x);
 }
 
 // ----------------------------------------------------------------------------------------------- y = z . C^T
@@ -251,6 +270,25 @@ template <int KG, bool BIAS> __global__ __launch_bounds__(ST_THREADS, 1) void fa
     stationary_block<KG, BIAS, false, true>(p, smem_raw, blockIdx.x);
 }
 
+// Projection and forward product in one launch: blocks 0 .. z_blocks - 1 project (z_block), the others multiply
+// (stationary_block) and wait, tile by tile, for the tags of the projection blocks that feed them.  A multiplying block
+// starts on a compute unit the moment a projecting block leaves it: no drain of the whole chip, no second launch in between.
+struct ZYParams {
+    ZParams z;
+    StParams y;
+    int z_blocks;   // a multiple of 8, so that both kinds keep their numbering over the dies
+};
+
+template <int KG, bool BIAS> __global__ __launch_bounds__(ST_THREADS, 1) void factored_zy_kernel(ZYParams p)
+{
+    static_assert(KZ_THREADS == ST_THREADS && KZ_BT == ST_BT, "one block size and one token tile for both kinds of block");
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    if ((int)blockIdx.x < p.z_blocks)
+        z_block(p.z, smem_raw, blockIdx.x, p.z_blocks);
+    else
+        stationary_block<KG, BIAS, false, true>(p.y, smem_raw, blockIdx.x - p.z_blocks);
+}
+
 // ----------------------------------------------------------------------------------------------- dC = dy^T . z
 // body in rdb_blocks.hpp (dc_block)
 __global__ __launch_bounds__(256, 1) void factored_dc_kernel(DcParams p)
@@ -285,12 +323,14 @@ void dc_params_from_state(DcParams &p, const void *state, const rdb_linear_desc 
 // The entry points below return RDB_E_UNSUPPORTED, without setting an error, when the request does not fit.
 // state <- projection of x (z for the forward product, z transposed for the coefficient gradient) and, when coef is given,
 // the transposed coefficients for the input gradient.
-int linear_project(void *state, const void *x, int64_t ldx, const void *coef, const rdb_linear_desc *d, hipStream_t s)
+int linear_fwd_projected(void *y, int64_t ldy, const void *state, const void *coef, const void *bias, const rdb_linear_desc *d, int num_cus,
+                         hipStream_t s);
+
+static bool fill_z_params(ZParams &p, void *state, const void *x, int64_t ldx, const void *coef, const rdb_linear_desc *d)
 {
     const ProjLayout L = proj_layout(d);
-    if (!L.ok || d->tokens * ldx >= (1ll << 29) || ldx % 8 || !aligned16(x) || !aligned16(state)) return RDB_E_UNSUPPORTED;
+    if (!L.ok || d->tokens * ldx >= (1ll << 29) || ldx % 8 || !aligned16(x) || !aligned16(state)) return false;
     if (coef && d->coef_dtype != RDB_BF16) coef = nullptr;   // the transposed copy is an operand of the bf16 kernels only
-    ZParams p;
     p.x = (const bf16_t *)x;
     p.coef = (const bf16_t *)coef;
     p.zf = state_piece(state, L.zf_off);
@@ -310,10 +350,100 @@ int linear_project(void *state, const void *x, int64_t ldx, const void *coef, co
     p.seed = d->seed;
     p.tiles_m = L.kpad / KZ_BM;   // every coefficient row block of the padded pieces is written
     p.tiles_t = (int)cdiv(d->tokens, KZ_BT);
-    const size_t smem = engine_smem<KZ_BM, KZ_BT, F_BK, K_CONT, K_CONT>();
+    p.sync = nullptr;
+    p.sync_tag = 0;
+    return true;
+}
+
+static size_t z_smem() { return engine_smem<KZ_BM, KZ_BT, F_BK, K_CONT, K_CONT>(); }
+
+int linear_project(void *state, const void *x, int64_t ldx, const void *coef, const rdb_linear_desc *d, hipStream_t s)
+{
+    ZParams p;
+    if (!fill_z_params(p, state, x, ldx, coef, d)) return RDB_E_UNSUPPORTED;
+    const size_t smem = z_smem();
     if (int rl = reserve_lds(reinterpret_cast<const void *>(factored_z_kernel), smem, "factored_z_kernel")) return rl;
     factored_z_kernel<<<xcd_grid_size(p.tiles_m * p.tiles_t), KZ_THREADS, smem, s>>>(p);
     return check_launch("factored_z_kernel");
+}
+
+// The forward product's parameters when the contraction of a token fits in registers (z in fragment order); returns the
+// number of work items, 0 when the request does not fit.
+static int fill_ys_params(StParams &q, void *y, int64_t ldy, const void *state, const void *coef, const void *bias, const rdb_linear_desc *d,
+                          int num_cus)
+{
+    const ProjLayout L = proj_layout(d);
+    if (!L.ok || !L.frag_fwd || d->coef_dtype != RDB_BF16 || ldy % 8 || !aligned16(y) || !aligned16(state) || !aligned16(coef)) return 0;
+    if (((uintptr_t)bias & 7) || d->tokens * ldy >= (1ll << 29)) return 0;
+    q.z = state_piece(state, L.zf_off);
+    q.coef = (const bf16_t *)coef;
+    q.bias = (const bf16_t *)bias;
+    q.y = (bf16_t *)y;
+    q.ldy = ldy;
+    q.k = (int)d->k;
+    q.seed = 0;
+    return make_stationary_grid(q, d->tokens, d->out_f, num_cus);
+}
+
+// A tag no other launch of any process is likely ever to have written where this launch's slots lie: a counter that starts
+// at a random 64-bit value.
+static unsigned long long next_sync_tag()
+{
+    static std::atomic<unsigned long long> counter{[] {
+        std::random_device rd;
+        return ((unsigned long long)rd() << 32) ^ (unsigned long long)rd() ^ ((unsigned long long)getpid() << 17);
+    }()};
+    unsigned long long v = counter.fetch_add(1) + 1;
+    return v ? v : counter.fetch_add(1) + 1;
+}
+
+template <int KG, bool BIAS> static int launch_zy(const ZYParams &p, int y_items, hipStream_t s)
+{
+    const size_t smem = std::max(z_smem(), stationary_smem(KG));
+    if (int rl = reserve_lds(reinterpret_cast<const void *>(factored_zy_kernel<KG, BIAS>), smem, "factored_zy_kernel")) return rl;
+    factored_zy_kernel<KG, BIAS><<<p.z_blocks + xcd_grid_size(y_items), ST_THREADS, smem, s>>>(p);
+    return check_launch("factored_zy_kernel");
+}
+
+// state <- projection of x (with the transposed coefficients if with_ct), y <- forward product, in one launch when the
+// contraction of a token fits in registers (k <= 256), otherwise in two.
+int linear_project_fwd(void *y, int64_t ldy, void *state, const void *x, int64_t ldx, const void *coef, bool with_ct, const void *bias,
+                       const rdb_linear_desc *d, int num_cus, hipStream_t s)
+{
+    ZYParams p;
+    if (!fill_z_params(p.z, state, x, ldx, with_ct ? coef : nullptr, d)) return RDB_E_UNSUPPORTED;
+    const int y_items = fill_ys_params(p.y, y, ldy, state, coef, bias, d, num_cus);
+    if (!y_items || p.z.tiles_m > 64) {
+        // check the second call's conditions before the first launch, so that a refusal leaves nothing half done
+        const ProjLayout L = proj_layout(d);
+        if (d->coef_dtype != RDB_BF16 || ldy % 8 || !aligned16(y) || !aligned16(coef)) return RDB_E_UNSUPPORTED;
+        if (L.frag_fwd && (((uintptr_t)bias & 7) || d->tokens * ldy >= (1ll << 29))) return RDB_E_UNSUPPORTED;
+        if (int rc = linear_project(state, x, ldx, with_ct ? coef : nullptr, d, s)) return rc;
+        return linear_fwd_projected(y, ldy, state, coef, bias, d, num_cus, s);
+    }
+    const ProjLayout L = proj_layout(d);
+    p.z.sync = reinterpret_cast<unsigned long long *>(static_cast<char *>(state) + L.sync_off);
+    p.z.sync_tag = next_sync_tag();
+    p.y.sync = p.z.sync;
+    p.y.sync_tag = p.z.sync_tag;
+    p.y.sync_n = p.z.tiles_m;
+    p.y.sync_err = reinterpret_cast<unsigned int *>(state) + 1;
+    p.z_blocks = xcd_grid_size(p.z.tiles_m * p.z.tiles_t);
+    const int kg = (int)cdiv(d->k, 64);
+    if (bias) {
+        switch (kg) {
+        case 1: return launch_zy<1, true>(p, y_items, s);
+        case 2: return launch_zy<2, true>(p, y_items, s);
+        case 3: return launch_zy<3, true>(p, y_items, s);
+        default: return launch_zy<4, true>(p, y_items, s);
+        }
+    }
+    switch (kg) {
+    case 1: return launch_zy<1, false>(p, y_items, s);
+    case 2: return launch_zy<2, false>(p, y_items, s);
+    case 3: return launch_zy<3, false>(p, y_items, s);
+    default: return launch_zy<4, false>(p, y_items, s);
+    }
 }
 
 int linear_fwd_projected(void *y, int64_t ldy, const void *state, const void *coef, const void *bias, const rdb_linear_desc *d, int num_cus,
@@ -323,16 +453,9 @@ int linear_fwd_projected(void *y, int64_t ldy, const void *state, const void *co
     if (!L.ok || d->coef_dtype != RDB_BF16 || ldy % 8 || !aligned16(y) || !aligned16(state) || !aligned16(coef)) return RDB_E_UNSUPPORTED;
     const bf16_t *zf = state_piece(state, L.zf_off);
     if (L.frag_fwd) {   // the contraction of a token fits in registers; z lies in fragment order
-        if (((uintptr_t)bias & 7) || d->tokens * ldy >= (1ll << 29)) return RDB_E_UNSUPPORTED;
         StParams q;
-        q.z = zf;
-        q.coef = (const bf16_t *)coef;
-        q.bias = (const bf16_t *)bias;
-        q.y = (bf16_t *)y;
-        q.ldy = ldy;
-        q.k = (int)d->k;
-        q.seed = 0;
-        const int items = make_stationary_grid(q, d->tokens, d->out_f, num_cus);
+        const int items = fill_ys_params(q, y, ldy, state, coef, bias, d, num_cus);
+        if (!items) return RDB_E_UNSUPPORTED;
         const int kg = (int)cdiv(d->k, 64);
         const size_t smem = stationary_smem(kg);
         if (bias) {
@@ -386,9 +509,7 @@ int linear_fwd_factored(void *y, int64_t ldy, const void *x, int64_t ldx, const 
     if (d->tokens * ldx >= (1ll << 29) || ldx % 8 || ldy % 8 || !aligned16(x) || !aligned16(coef) || !aligned16(y) || !aligned16(workspace))
         return RDB_E_UNSUPPORTED;
     if (proj_layout(d).frag_fwd && (((uintptr_t)bias & 7) || d->tokens * ldy >= (1ll << 29))) return RDB_E_UNSUPPORTED;
-    int rc = linear_project(workspace, x, ldx, nullptr, d, s);
-    if (rc) return rc;
-    return linear_fwd_projected(y, ldy, workspace, coef, bias, d, num_cus, s);
+    return linear_project_fwd(y, ldy, workspace, x, ldx, coef, false, bias, d, num_cus, s);
 }
 
 // dC = dy^T . (x . N^T) with the projection state in the workspace; dcoef must have been zeroed on the same stream.

@@ -286,6 +286,8 @@ int linear_fwd_strip(void *y, int64_t ldy, const void *x, int64_t ldx, const voi
 // rdb_factored.hip
 int64_t linear_projection_bytes(const rdb_linear_desc *d);
 int linear_project(void *state, const void *x, int64_t ldx, const void *coef, const rdb_linear_desc *d, hipStream_t s);
+int linear_project_fwd(void *y, int64_t ldy, void *state, const void *x, int64_t ldx, const void *coef, bool with_ct, const void *bias,
+                       const rdb_linear_desc *d, int num_cus, hipStream_t s);
 int linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, const void *bias, const rdb_linear_desc *d, int num_cus,
                          hipStream_t s);
 int linear_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *z, const rdb_linear_desc *d, int num_cus, hipStream_t s);
@@ -702,6 +704,28 @@ extern "C" int rdb_linear_fwd_projected(void *y, int64_t ldy, const void *z, con
         rc = linear_fwd_projected(at_bytes(y, c * pl.chunk_tokens * ldy * 2), ldy, at_bytes(z, c * pl.state_stride), coef, bias, &dd,
                                   num_compute_units(), (hipStream_t)stream);
         if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd_projected: internal: chunk %d of %d refused", c, pl.nchunks);
+        if (rc) return rc;
+    }
+    return RDB_OK;
+}
+
+extern "C" int rdb_linear_project_fwd(void *y, int64_t ldy, void *state, const void *x, int64_t ldx, const void *coef, const void *bias,
+                                      const rdb_linear_desc *d, void *stream)
+{
+    ChunkPlan pl;
+    int rc = check_projected("rdb_linear_project_fwd", d, &pl);
+    if (rc) return rc;
+    if (!y || !state || !x || !coef) return set_error(RDB_E_NULL, "rdb_linear_project_fwd: y, state, x or coef is NULL");
+    if (ldx < d->in_f || ldy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_project_fwd: leading dimension smaller than the row");
+    if (d->coef_dtype != RDB_BF16 || ldx % 8 || ldy % 8 || !aligned16(x) || !aligned16(state) || !aligned16(y) || !aligned16(coef) ||
+        ((uintptr_t)bias & 7) || pl.chunk_tokens * ldx >= (1ll << 29) || pl.chunk_tokens * ldy >= (1ll << 29))
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_project_fwd: coefficients must be bf16; x, y, state and coef 16-byte aligned, bias 8-byte; "
+                                            "leading dimensions multiples of 8 and below twice the row");
+    for (int c = 0; c < pl.nchunks; ++c) {
+        const rdb_linear_desc dd = chunk_desc(d, pl, c);
+        rc = linear_project_fwd(at_bytes(y, c * pl.chunk_tokens * ldy * 2), ldy, at_bytes(state, c * pl.state_stride),
+                                at_bytes(x, c * pl.chunk_tokens * ldx * 2), ldx, coef, true, bias, &dd, num_compute_units(), (hipStream_t)stream);
+        if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_project_fwd: internal: chunk %d of %d refused", c, pl.nchunks);
         if (rc) return rc;
     }
     return RDB_OK;

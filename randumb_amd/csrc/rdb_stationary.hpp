@@ -33,6 +33,12 @@ struct StParams {
     int tokens, out_f, k;
     int tiles_t, splits, units_per_split;
     uint32_t seed;       // noise flavour
+    // ZFRAG only: NULL, or slots [token tile of 256][sync_n] that earlier blocks of the same launch set to sync_tag when the tile's
+    // share of z is in memory
+    const unsigned long long *sync;
+    unsigned long long sync_tag;
+    int sync_n;
+    unsigned int *sync_err;
 };
 
 // KG: k rounded up to groups of 64 (compile time: the k loop is one straight line of code).  NOISE: the right operand's
@@ -219,11 +225,23 @@ __device__ __forceinline__ void stationary_block(const StParams &p, unsigned cha
         const int64_t padded = (int64_t)((p.tokens + 31) / 32) * 32 * B::kpad;
         const __amdgpu_buffer_rsrc_t rs_z = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.z), 0, (int)(padded * 2), 0x00020000);
         if (!NOISE) b.issue(b.unit0);
+        if (p.sync) {   // z comes from earlier blocks of this launch
+            if (wave == 0) await_tags(p.sync + (int64_t)(w / p.splits) * p.sync_n, p.sync_n, p.sync_tag, p.sync_err);
+            __syncthreads();
+        }
         const int tile = tok0 >> 5;
+        if (p.sync) {   // written by other dies during this launch: read around this die's L2
 #pragma unroll
-        for (int ks = 0; ks < KG * 4; ++ks) {
-            const uint32_t a = tok0 < p.tokens ? (uint32_t)(((tile * (KG * 4) + ks) * 512 + b.lane * 8) * 2) : BUFFER_OOB;
-            b.zf[ks] = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)a, 0, 0));
+            for (int ks = 0; ks < KG * 4; ++ks) {
+                const uint32_t a = tok0 < p.tokens ? (uint32_t)(((tile * (KG * 4) + ks) * 512 + b.lane * 8) * 2) : BUFFER_OOB;
+                b.zf[ks] = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)a, 0, SCOPE_DEVICE));
+            }
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < KG * 4; ++ks) {
+                const uint32_t a = tok0 < p.tokens ? (uint32_t)(((tile * (KG * 4) + ks) * 512 + b.lane * 8) * 2) : BUFFER_OOB;
+                b.zf[ks] = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(rs_z, (int)a, 0, 0));
+            }
         }
         if (NOISE) b.hash_piece_all(b.unit0);   // the first noise tile is hashed while the loads are in flight
         b.commit(b.Cs);                          // first tile of the right operand; the barrier at the top of step 0 publishes it
@@ -301,6 +319,10 @@ inline int make_stationary_grid(StParams &q, int64_t tokens, int64_t out_f, int 
 {
     q.tokens = (int)tokens;
     q.out_f = (int)out_f;
+    q.sync = nullptr;   // the left operand comes from an earlier launch unless the caller says otherwise afterwards
+    q.sync_tag = 0;
+    q.sync_n = 0;
+    q.sync_err = nullptr;
     q.tiles_t = (int)cdiv(tokens, ST_BT);
     const int units = (int)cdiv(out_f, ST_BO);
     int splits = (int)cdiv(num_cus, q.tiles_t);

@@ -310,6 +310,29 @@ def linear_project(x: torch.Tensor, k: int, out_f: int, seed: int, coef: Optiona
     return state
 
 
+def linear_project_fwd(x: torch.Tensor, coef: torch.Tensor, seed: int, bias: Optional[torch.Tensor] = None):
+    """``(y, state)``: :func:`linear_project` (with ``coef``) and :func:`linear_fwd_projected` in one call, for k <= 256 in a
+    single kernel launch; the forward pass of a training step, ``state`` being what it saves for backward."""
+    _need_gpu("linear_project_fwd", x, coef)
+    x = _act(x)
+    c = _native(coef)
+    if x.dtype != torch.bfloat16 or c.dtype != torch.bfloat16:
+        raise ValueError("linear_project_fwd computes in bf16")
+    out_f, k = c.shape
+    d = _proj_desc(x.shape[0], x.shape[1], out_f, k, seed)
+    L = _lib.load()
+    nbytes = L.rdb_linear_projection_bytes(ctypes.byref(d))
+    if nbytes <= 0:
+        _lib.check(L.rdb_linear_project(None, None, x.stride(0), None, ctypes.byref(d), None), "rdb_linear_project")
+    state = torch.empty((x.shape[0], -(-nbytes // x.shape[0])), dtype=torch.uint8, device=x.device)
+    b = None if bias is None else bias.to(torch.bfloat16).contiguous()
+    y = torch.empty((x.shape[0], out_f), dtype=torch.bfloat16, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = L.rdb_linear_project_fwd(_p(y), y.stride(0), _p(state), _p(x), x.stride(0), _p(c), _p(b), ctypes.byref(d), _stream(x.device))
+    _lib.check(rc, "rdb_linear_project_fwd")
+    return y, state
+
+
 def projection_unpack(state: torch.Tensor, in_f: int, out_f: int, k: int) -> dict:
     """The pieces of a projection state as ordinary row-major tensors, for tools and tests (a layout decode, no arithmetic):
     ``z`` (tokens, k) as the forward product reads it, ``z_t`` (k, tokens) as the coef gradient reads it, and ``coef_t``

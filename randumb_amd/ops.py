@@ -22,7 +22,7 @@ from . import hip
 
 __all__ = [
     "materialize_fwd", "materialize_bwd", "scale_bias_bwd", "embed_fwd", "embed_bwd",
-    "linear_fwd", "linear_bwd_dx", "linear_bwd_dcoef", "linear", "linear_project", "linear_fwd_projected",
+    "linear_fwd", "linear_bwd_dx", "linear_bwd_dcoef", "linear", "linear_project", "linear_project_fwd", "linear_fwd_projected",
     "linear_bwd_dcoef_projected", "linear_bwd_projected", "sq5_gen_2d", "sq5_gen_1d",
 ]
 
@@ -225,6 +225,21 @@ def _(state, coefs, in_features, seed, bias):
     return coefs.new_empty([state.shape[0], coefs.shape[0]], dtype=torch.bfloat16)
 
 
+@custom_op("rten::linear_project_fwd", mutates_args=())
+def linear_project_fwd(x: Tensor, coefs: Tensor, seed: int, bias: Optional[Tensor]) -> List[Tensor]:
+    """``[y, state]``: ``linear_project`` with the coefficients and ``linear_fwd_projected`` in one call (one kernel launch
+    for k <= 256)."""
+    y, state = hip.linear_project_fwd(x, coefs, seed, bias)
+    return [y, state]
+
+
+@linear_project_fwd.register_fake
+def _(x, coefs, seed, bias):
+    nbytes = hip.linear_projection_bytes(x.shape[0], x.shape[1], coefs.shape[0], coefs.shape[1])
+    return [x.new_empty([x.shape[0], coefs.shape[0]], dtype=torch.bfloat16),
+            x.new_empty([x.shape[0], -(-nbytes // x.shape[0])], dtype=torch.uint8)]
+
+
 @custom_op("rten::linear_bwd_dcoef_projected", mutates_args=())
 def linear_bwd_dcoef_projected(dy: Tensor, state: Tensor, dcoefs_size: int, in_features: int, seed: int) -> Tensor:
     return hip.linear_bwd_dcoef_projected(dy, state, dcoefs_size, in_features, seed)
@@ -254,11 +269,11 @@ class _ProjectedLinear(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, coefs, in_features, out_features, seed, bias):
-        state = linear_project(x, coefs.shape[1], out_features, seed, coefs)
+        y, state = linear_project_fwd(x, coefs, seed, bias)
         ctx.save_for_backward(state, coefs)
         ctx.meta = (in_features, out_features, seed)
         ctx.bias_dtype = None if bias is None else bias.dtype
-        return linear_fwd_projected(state, coefs, in_features, seed, bias)
+        return y
 
     @staticmethod
     def backward(ctx, dy):

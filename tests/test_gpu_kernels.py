@@ -376,6 +376,29 @@ def test_linear_projected_form(hip, oracle, T, in_f, out_f, k, seed):
     assert rel_l2(cpu(dc1), cpu(dc)) < 1e-5
 
 
+@pytest.mark.parametrize("T,in_f,out_f,k,seed", BWD_SHAPES + [(8192, 768, 3072, 256, 0), (1000, 200, 328, 72, 5), (300, 128, 256, 512, 2)])
+def test_project_fwd_in_one_call(hip, T, in_f, out_f, k, seed):
+    """Projection and forward product in one call (one launch for k <= 256: the multiplying blocks wait for the tags of the
+    projecting blocks) against the two separate calls: same bits in y and in every piece of the state, on a state buffer
+    that held other bytes before and again on the buffer the first call wrote."""
+    print(f"case project+fwd T={T} in={in_f} out={out_f} k={k}", flush=True)
+    x, _, coef = _inputs(T, in_f, out_f, k, True, torch.bfloat16, seed)
+    xg, cg = x.cuda(), coef.cuda()
+    bias = torch.randn(out_f).bfloat16().cuda()
+    want_state = hip.linear_project(xg, k, out_f, seed, coef=cg)
+    want_y = hip.linear_fwd_projected(want_state, cg, in_f, seed, bias=bias)
+    want = hip.projection_unpack(want_state, in_f, out_f, k)
+    for round_ in range(3):
+        y, state = hip.linear_project_fwd(xg, cg, seed, bias=bias)
+        got = hip.projection_unpack(state, in_f, out_f, k)
+        assert torch.equal(y, want_y), f"y differs in round {round_}"
+        for name in ("z", "z_t", "coef_t"):
+            assert torch.equal(got[name], want[name]), f"{name} differs in round {round_}"
+        assert int(state.view(-1)[:8].view(torch.int32)[1]) == 0, "a block gave up waiting for the projection"
+    y_nb, _ = hip.linear_project_fwd(xg, cg, seed)
+    assert torch.equal(y_nb, hip.linear_fwd_projected(want_state, cg, in_f, seed))
+
+
 @pytest.mark.parametrize("T,in_f,out_f,k,seed", BWD_SHAPES)
 def test_linear_bwd_projected_one_call(hip, oracle, T, in_f, out_f, k, seed):
     """dx and dcoef from one call (two launches, dcoef blocks and dx blocks side by side) against the oracle and against

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_lib.SO_PATH)
     for name in declared:
         assert hasattr(lib, name), name
-    assert _lib.load().rdb_abi_version() == 4
+    assert _lib.load().rdb_abi_version() == 5
     assert ctypes.sizeof(_lib.LinearDesc) == 7 * 8 + 4 * 4
 
 
@@ -65,12 +65,14 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
 
     def state_bytes(tokens, out_f, k):
         # header + z for the forward product (tokens to 32 when k <= 256) + z transposed (tokens to 64) + C transposed (out to 64)
+        # + a 64-bit slot per projection tile (256 tokens x 32 coefficients)
         up = lambda n, m: -(-n // m) * m
         kpad = up(k, 64)
         zf = up(tokens, 32) * kpad * 2 if k <= 256 else tokens * k * 2
-        return 256 + up(zf, 256) + up(up(tokens, 64) * kpad * 2, 256) + up(up(out_f, 64) * kpad * 2, 256)
+        return (256 + up(zf, 256) + up(up(tokens, 64) * kpad * 2, 256) + up(up(out_f, 64) * kpad * 2, 256)
+                + up(-(-tokens // 256) * (kpad // 32) * 8, 256))
 
-    assert state_bytes(8192, 3072, 256) == 256 + 2 * zbytes + 3072 * 256 * 2
+    assert state_bytes(8192, 3072, 256) == 256 + 2 * zbytes + 3072 * 256 * 2 + 32 * 8 * 8
     assert L.rdb_linear_projection_bytes(r) == state_bytes(8192, 3072, 256)
     info = (ctypes.c_int64 * 8)()
     assert L.rdb_linear_projection_layout(r, info) == 0
