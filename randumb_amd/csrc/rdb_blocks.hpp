@@ -13,8 +13,14 @@ constexpr int B_BK = 64;
 // unroll and prefetch depth (in stages of 64) of the dy stream in the coefficient gradient's contraction
 #ifndef RDB_DC_TRIP
 #define RDB_DC_TRIP 2
+#endif
+#ifndef RDB_DC_DSTG
 #define RDB_DC_DSTG 2
+#endif
+#ifndef RDB_DC_RD
 #define RDB_DC_RD 2
+#endif
+#ifndef RDB_DC_BK
 #define RDB_DC_BK 64
 #endif
 

@@ -20,6 +20,23 @@ constexpr int X_BK = 64;
 // tile: 128 coefficient columns (engine rows "a") x 64 tokens (engine rows "b"), contraction over out_f.  The output is
 // small (tokens x k), so the token tile is kept short to have a block for every compute unit; loads run two stages ahead.
 constexpr int K1_BC = 128, K1_BT = 64;
+// pipeline shape of the dy.C blocks that take C^T straight into registers: contraction per stage, stages per unrolled trip,
+// how many stages ahead dy is loaded, depth of the fragment ring in stages, wave priority
+#ifndef RDB_DYC_BKD
+#define RDB_DYC_BKD 128
+#endif
+#ifndef RDB_DYC_TRIP
+#define RDB_DYC_TRIP 2
+#endif
+#ifndef RDB_DYC_DSTG
+#define RDB_DYC_DSTG 2
+#endif
+#ifndef RDB_DYC_RD
+#define RDB_DYC_RD 1
+#endif
+#ifndef RDB_DYC_PRIO
+#define RDB_DYC_PRIO 2
+#endif
 
 struct DyCParams {
     const bf16_t *dy;
@@ -74,13 +91,13 @@ __device__ __forceinline__ void dyc_block_direct(const DyCParams &p, bf16_t *lds
 #pragma unroll
     for (int ni = 0; ni < K1_BT / 32; ++ni) acc[0][ni] = zero16();
     // stages of 128: half as many barriers (and waits for the first fragments after them) as with 64, for the same LDS
-    constexpr int BKD = 128;
+    constexpr int BKD = RDB_DYC_BKD;
     GlobalOperand<K1_BT, BKD, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
     FragSource fc;
     fc.init(p.ctf, (int64_t)p.kpad * p.osteps * 16, p.osteps, (m0 >> 5) + wave, lane);
     // these blocks are the longer ones of the launch they share with the coefficient-gradient blocks: their waves issue first
-    __builtin_amdgcn_s_setprio(2);
-    direct_mainloop<K1_BT / 32, 1, BKD / 16, false, 2, 2, 1>(acc, lds, opdy, fc, 0, (p.out_f + BKD - 1) / BKD, 0, lane);
+    __builtin_amdgcn_s_setprio(RDB_DYC_PRIO);
+    direct_mainloop<K1_BT / 32, 1, BKD / 16, false, RDB_DYC_TRIP, RDB_DYC_DSTG, RDB_DYC_RD>(acc, lds, opdy, fc, 0, (p.out_f + BKD - 1) / BKD, 0, lane);
     if (p.frag_ksteps)
         store_tile_bf16_frag<K1_BC, K1_BT, 4>(acc, lds, p.t, p.frag_ksteps, m0, p.frag_ksteps * 16, tok0, (p.tokens + 31) / 32 * 32,
                                               4.656612873077392578125e-10f);

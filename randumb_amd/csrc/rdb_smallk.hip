@@ -10,6 +10,9 @@
 // Replaces materialize() + dense product (src/rten_cpp/RandumbTensor.py:942-946) and MmBackward's dW followed by
 // materialize_bwd (RandumbTensor.py:979-990, 304-359) in the regime where a stored-W product would be bound by reading W.
 #include "rdb_common.hpp"
+#include <atomic>
+#include <random>
+#include <unistd.h>
 
 namespace rdb {
 
@@ -36,22 +39,37 @@ __device__ __forceinline__ float sum_partials(const float *__restrict__ p, int64
 // compute units; thread = (m % 16, one of 16 interleaved slices of the chunk); the source rows go through LDS (coalesced
 // loads, broadcast reads); slices meet in LDS in slice order.  The block writes a partial result, out[chunk][t][m]; the
 // expanding kernel adds the chunks up in chunk order while it loads them.
-template <bool HASH>
-__global__ __launch_bounds__(256) void smallk_contract_kernel(float *__restrict__ out, const float *__restrict__ src, int64_t lds_src,
-                                                              const float *__restrict__ coef, int T, int J, int k, uint32_t seed)
+struct SkContract {
+    float *out;          // [chunks][T][k] partial sums
+    const float *src;    // [T x J], leading dimension ld_src
+    int64_t ld_src;
+    const float *coef;   // [J x k] (not HASH)
+    int T, J, k;
+    uint32_t seed;
+};
+
+// bx: token tile, by: chunk of 256 values of j.  The partial sums are stored at device scope: blocks of the same launch on
+// another die may be the ones that read them (smallk_fused_kernel).
+template <bool HASH> __device__ __forceinline__ void smallk_contract_block(const SkContract &p, int bx, int by)
 {
     constexpr int JC = 256, MC = SK_MAX_K / 16;
     __shared__ float xs[SK_TT][JC];
     __shared__ float red[16][SK_TT][16];
+    float *__restrict__ out = p.out;
+    const float *__restrict__ src = p.src;
+    const float *__restrict__ coef = p.coef;
+    const int64_t lds_src = p.ld_src;
+    const int T = p.T, J = p.J, k = p.k;
+    const uint32_t seed = p.seed;
     const int tid = threadIdx.x, m16 = tid & 15, slice = tid >> 4;
-    const int t0 = blockIdx.x * SK_TT;
+    const int t0 = bx * SK_TT;
     float acc[MC][SK_TT];
 #pragma unroll
     for (int c = 0; c < MC; ++c)
 #pragma unroll
         for (int tt = 0; tt < SK_TT; ++tt) acc[c][tt] = 0.0f;
     {
-        const int jc = blockIdx.y * JC;
+        const int jc = by * JC;
 #pragma unroll
         for (int tt = 0; tt < SK_TT; ++tt) xs[tt][tid] = (t0 + tt < T && jc + tid < J) ? src[(int64_t)(t0 + tt) * lds_src + jc + tid] : 0.0f;
         __syncthreads();
@@ -83,23 +101,63 @@ __global__ __launch_bounds__(256) void smallk_contract_kernel(float *__restrict_
             float s = 0.0f;
 #pragma unroll
             for (int sl = 0; sl < 16; ++sl) s += red[sl][tt][m16];
-            if (t0 + tt < T && m < k) out[((int64_t)blockIdx.y * T + t0 + tt) * k + m] = s;
+            if (t0 + tt < T && m < k) __hip_atomic_store(out + ((int64_t)by * T + t0 + tt) * k + m, s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         __syncthreads();
     }
 }
 
+template <bool HASH> __global__ __launch_bounds__(256) void smallk_contract_kernel(SkContract p) { smallk_contract_block<HASH>(p, blockIdx.x, blockIdx.y); }
+
 // out[t, c] = sum_m src[t, m] * B(c, m) (+ bias[c]),  B(c, m) = noise(PRIME*c + m) (HASH) or coef[c, m]; c runs over the
 // cols = in_f or out_f.  Block = 256 columns x 16 tokens; a thread owns one column and keeps its 16 B values in registers.
 // src holds `nchunk` partial matrices [T x k] (from the contracting kernel), added up here in chunk order.
-template <bool HASH>
-__global__ __launch_bounds__(256) void smallk_expand_kernel(float *__restrict__ out, int64_t ld_out, const float *__restrict__ src, int nchunk,
-                                                            const float *__restrict__ coef, const float *__restrict__ bias, int T, int cols,
-                                                            int k, uint32_t seed)
+struct SkExpand {
+    float *out;          // [T x cols], leading dimension ld_out
+    int64_t ld_out;
+    const float *src;    // [nchunk][T][k] partial sums
+    int nchunk;
+    const float *coef;   // [cols x k] (not HASH)
+    const float *bias;   // [cols] or NULL
+    int T, cols, k;
+    uint32_t seed;
+    // NULL, or slots [token tiles of SK_TT][nchunk] that contracting blocks of the same launch set to sync_tag
+    const unsigned long long *sync;
+    unsigned long long sync_tag;
+    unsigned int *sync_err;
+};
+
+// bx: block of 256 columns, by: block of SK_ET tokens.
+template <bool HASH> __device__ __forceinline__ void smallk_expand_block(const SkExpand &p, int bx, int by)
 {
     __shared__ __align__(16) float s[SK_ET][SK_MAX_K];
+    float *__restrict__ out = p.out;
+    const float *__restrict__ src = p.src;
+    const float *__restrict__ coef = p.coef;
+    const float *__restrict__ bias = p.bias;
+    const int64_t ld_out = p.ld_out;
+    const int nchunk = p.nchunk, T = p.T, cols = p.cols, k = p.k;
+    const uint32_t seed = p.seed;
     const int tid = threadIdx.x;
-    const int c = blockIdx.x * 256 + tid, t0 = blockIdx.y * SK_ET;
+    const int c = bx * 256 + tid, t0 = by * SK_ET;
+    // this thread's first 16 values of B: fetched (or hashed) before anything is waited for
+    float b0[16];
+    {
+        const int cc = c < cols ? c : cols - 1;
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {  // branch-free: a column from k on reads a valid address and becomes 0
+            const float v = HASH ? sq5_unit(sq5_tail(sq5_first((uint32_t)cc, (uint32_t)m, seed))) : coef[(int64_t)cc * k + ((m < k) ? m : k - 1)];
+            b0[m] = (m < k) ? v : 0.0f;
+        }
+    }
+    if (p.sync) {   // the partial sums of these tokens come from earlier blocks of this launch
+        if (tid < 64) {
+            const int tile0 = t0 / SK_TT, tiles = (T + SK_TT - 1) / SK_TT;
+            const int ntile = (tile0 + SK_ET / SK_TT <= tiles) ? SK_ET / SK_TT : tiles - tile0;
+            await_tags(p.sync + (int64_t)tile0 * nchunk, ntile * nchunk, p.sync_tag, p.sync_err);
+        }
+        __syncthreads();
+    }
     // s = sum of the partial matrices in chunk order; columns from k on take part as zeros.  A thread owns up to 4 entries
     // and keeps the loads of 8 chunks of all of them in flight at once: the kernel is a chain of memory latencies otherwise.
     {
@@ -120,7 +178,8 @@ __global__ __launch_bounds__(256) void smallk_expand_kernel(float *__restrict__ 
 #pragma unroll
             for (int i = 0; i < PER; ++i)
 #pragma unroll
-                for (int u = 0; u < 8; ++u) l[i][u] = ptr[i][(int64_t)((c0 + u < nchunk) ? c0 + u : nchunk - 1) * stride];
+                for (int u = 0; u < 8; ++u)   // device scope: possibly written by another die during this launch
+                    l[i][u] = __hip_atomic_load(ptr[i] + (int64_t)((c0 + u < nchunk) ? c0 + u : nchunk - 1) * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
             for (int i = 0; i < PER; ++i)
 #pragma unroll
@@ -141,11 +200,16 @@ __global__ __launch_bounds__(256) void smallk_expand_kernel(float *__restrict__ 
     for (int tt = 0; tt < SK_ET; ++tt) acc[tt] = 0.0f;
     for (int mc = 0; mc < k; mc += 16) {
         float b[16];
+        if (mc == 0) {
 #pragma unroll
-        for (int m = 0; m < 16; ++m) {  // branch-free: a column from k on reads a valid address and becomes 0
-            const float v = HASH ? sq5_unit(sq5_tail(sq5_first((uint32_t)c, (uint32_t)(mc + m), seed)))
-                                 : coef[(int64_t)c * k + ((mc + m < k) ? mc + m : k - 1)];
-            b[m] = (mc + m < k) ? v : 0.0f;
+            for (int m = 0; m < 16; ++m) b[m] = b0[m];
+        } else {
+#pragma unroll
+            for (int m = 0; m < 16; ++m) {
+                const float v = HASH ? sq5_unit(sq5_tail(sq5_first((uint32_t)c, (uint32_t)(mc + m), seed)))
+                                     : coef[(int64_t)c * k + ((mc + m < k) ? mc + m : k - 1)];
+                b[m] = (mc + m < k) ? v : 0.0f;
+            }
         }
         // mc <= 48 and m <= 15: always inside the 64 columns of s
 #pragma unroll
@@ -165,6 +229,31 @@ __global__ __launch_bounds__(256) void smallk_expand_kernel(float *__restrict__ 
 #pragma unroll
     for (int tt = 0; tt < SK_ET; ++tt)
         if (t0 + tt < T) out[(int64_t)(t0 + tt) * ld_out + c] = acc[tt] + bv;
+}
+
+template <bool HASH> __global__ __launch_bounds__(256) void smallk_expand_kernel(SkExpand p) { smallk_expand_block<HASH>(p, blockIdx.x, blockIdx.y); }
+
+// Both in one launch: the contracting blocks first, each publishing a tag when its partial sums are in memory, then the
+// expanding blocks, each waiting for the tags of its 16 tokens' tiles.  At a few tokens the two launches are most of the
+// time of the call.
+struct SkFused {
+    SkContract c;
+    SkExpand e;
+    unsigned long long *slots;
+    int c_tiles, c_blocks, e_colblocks;
+};
+
+template <bool CHASH> __global__ __launch_bounds__(256) void smallk_fused_kernel(SkFused p)
+{
+    const int b = blockIdx.x;
+    if (b < p.c_blocks) {
+        const int bx = b % p.c_tiles, by = b / p.c_tiles;
+        smallk_contract_block<CHASH>(p.c, bx, by);
+        publish_tag(p.slots + (int64_t)bx * p.e.nchunk + by, p.e.sync_tag);
+    } else {
+        const int e = b - p.c_blocks;
+        smallk_expand_block<!CHASH>(p.e, e % p.e_colblocks, e / p.e_colblocks);
+    }
 }
 
 // dC[o, m] = sum_t dy[t, o] * z[t, m].  Block = 256 output rows x one chunk of 16 coefficients; z goes through LDS in tiles
@@ -213,48 +302,78 @@ static bool smallk_wanted(const rdb_linear_desc *d)
     return d->algo == RDB_ALGO_FACTORED || (d->tokens <= 1024 && d->k * (d->in_f + d->out_f) < d->in_f * d->out_f);
 }
 
-// scratch: one partial [tokens x k] fp32 matrix per 256-chunk of the longer of in_f and out_f
+// scratch: one partial [tokens x k] fp32 matrix per 256-chunk of the longer of in_f and out_f, then the tag slots of the
+// one-launch form (one per token tile and chunk) and a word for a waiting block that gave up
+static int64_t partial_bytes(const rdb_linear_desc *d)
+{
+    const int64_t longer = d->in_f > d->out_f ? d->in_f : d->out_f;
+    return (cdiv(longer, 256) * d->tokens * d->k * (int64_t)sizeof(float) + 7) / 8 * 8;
+}
 int64_t linear_smallk_workspace(const rdb_linear_desc *d)
 {
     if (!smallk_ok(d)) return 0;
     const int64_t longer = d->in_f > d->out_f ? d->in_f : d->out_f;
-    return cdiv(longer, 256) * d->tokens * d->k * (int64_t)sizeof(float);
+    return partial_bytes(d) + cdiv(d->tokens, SK_TT) * cdiv(longer, 256) * 8 + 8;
 }
 
-static bool ws_ok(const rdb_linear_desc *d, const void *ws, int64_t bytes) { return ws && bytes >= linear_smallk_workspace(d) && ((uintptr_t)ws & 3) == 0; }
+static bool ws_ok(const rdb_linear_desc *d, const void *ws, int64_t bytes) { return ws && bytes >= linear_smallk_workspace(d) && ((uintptr_t)ws & 7) == 0; }
+
+static unsigned long long next_tag()
+{
+    static std::atomic<unsigned long long> counter{[] {
+        std::random_device rd;
+        return ((unsigned long long)rd() << 32) ^ (unsigned long long)rd() ^ ((unsigned long long)getpid() << 17);
+    }()};
+    unsigned long long v = counter.fetch_add(1) + 1;
+    return v ? v : counter.fetch_add(1) + 1;
+}
+
+// Contraction over J (the rows of src) then expansion to `cols` columns: one launch when an expanding block's tags fit one
+// wave's lanes (J <= 8192), two otherwise.
+template <bool CHASH>
+static int contract_expand(float *out, int64_t ld_out, int cols, const float *src, int64_t ld_src, int J, const float *coef, const float *bias,
+                           const rdb_linear_desc *d, void *workspace, hipStream_t s)
+{
+    const int T = (int)d->tokens, k = (int)d->k;
+    const int nchunk = (int)cdiv(J, 256), tiles = (int)cdiv(T, SK_TT);
+    SkFused f;
+    f.c = {(float *)workspace, src, ld_src, coef, T, J, k, d->seed};
+    f.e = {out, ld_out, (const float *)workspace, nchunk, coef, bias, T, cols, k, d->seed, nullptr, 0, nullptr};
+    f.slots = reinterpret_cast<unsigned long long *>(static_cast<char *>(workspace) + partial_bytes(d));
+    f.c_tiles = tiles;
+    f.c_blocks = tiles * nchunk;
+    f.e_colblocks = (int)cdiv(cols, 256);
+    const int e_blocks = f.e_colblocks * (int)cdiv(T, SK_ET);
+    if (nchunk * (SK_ET / SK_TT) <= 64) {
+        f.e.sync = f.slots;
+        f.e.sync_tag = next_tag();
+        f.e.sync_err = reinterpret_cast<unsigned int *>(f.slots + (int64_t)tiles * nchunk);
+        smallk_fused_kernel<CHASH><<<f.c_blocks + e_blocks, 256, 0, s>>>(f);
+        return check_launch("smallk_fused_kernel");
+    }
+    smallk_contract_kernel<CHASH><<<dim3((unsigned)tiles, nchunk), 256, 0, s>>>(f.c);
+    if (int rc = check_launch("smallk_contract_kernel")) return rc;
+    smallk_expand_kernel<!CHASH><<<dim3((unsigned)f.e_colblocks, (unsigned)cdiv(T, SK_ET)), 256, 0, s>>>(f.e);
+    return check_launch("smallk_expand_kernel");
+}
 
 // The three entry points return RDB_E_UNSUPPORTED, without setting an error, when the request does not fit.
 int linear_fwd_smallk(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
                       const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
     if (!smallk_ok(d) || scale_bias || !smallk_wanted(d) || !ws_ok(d, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
-    const int T = (int)d->tokens, k = (int)d->k;
-    float *z = (float *)workspace;
-    const int nchunk = (int)cdiv(d->in_f, 256);
-    smallk_contract_kernel<true><<<dim3((unsigned)cdiv(T, SK_TT), nchunk), 256, 0, s>>>(z, (const float *)x, ldx, nullptr, T, (int)d->in_f, k,
-                                                                                        d->seed);
-    int rc = check_launch("smallk_contract_kernel<hash>");
-    if (rc) return rc;
-    dim3 grid((unsigned)cdiv(d->out_f, 256), (unsigned)cdiv(T, SK_ET));
-    smallk_expand_kernel<false><<<grid, 256, 0, s>>>((float *)y, ldy, z, nchunk, (const float *)coef, (const float *)bias, T, (int)d->out_f, k,
-                                                     d->seed);
-    return check_launch("smallk_expand_kernel<coef>");
+    // z = x . N^T (hashed), y = z . C^T + bias
+    return contract_expand<true>((float *)y, ldy, (int)d->out_f, (const float *)x, ldx, (int)d->in_f, (const float *)coef, (const float *)bias, d,
+                                 workspace, s);
 }
 
 int linear_dx_smallk(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias, const rdb_linear_desc *d,
                      void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
     if (!smallk_ok(d) || scale_bias || !smallk_wanted(d) || !ws_ok(d, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
-    const int T = (int)d->tokens, k = (int)d->k;
-    float *t = (float *)workspace;
-    const int nchunk = (int)cdiv(d->out_f, 256);
-    smallk_contract_kernel<false><<<dim3((unsigned)cdiv(T, SK_TT), nchunk), 256, 0, s>>>(t, (const float *)dy, lddy, (const float *)coef, T,
-                                                                                         (int)d->out_f, k, d->seed);
-    int rc = check_launch("smallk_contract_kernel<coef>");
-    if (rc) return rc;
-    dim3 grid((unsigned)cdiv(d->in_f, 256), (unsigned)cdiv(T, SK_ET));
-    smallk_expand_kernel<true><<<grid, 256, 0, s>>>((float *)dx, lddx, t, nchunk, nullptr, nullptr, T, (int)d->in_f, k, d->seed);
-    return check_launch("smallk_expand_kernel<hash>");
+    // t = dy . C, dx = t . N (hashed)
+    return contract_expand<false>((float *)dx, lddx, (int)d->in_f, (const float *)dy, lddy, (int)d->out_f, (const float *)coef, nullptr, d,
+                                  workspace, s);
 }
 
 // dcoef is overwritten (no zero fill needed).
@@ -267,8 +386,8 @@ int linear_dcoef_smallk(float *dcoef, const void *dy, int64_t lddy, const void *
     const int T = (int)d->tokens, k = (int)d->k;
     float *z = (float *)workspace;
     const int nchunk = (int)cdiv(d->in_f, 256);
-    smallk_contract_kernel<true><<<dim3((unsigned)cdiv(T, SK_TT), nchunk), 256, 0, s>>>(z, (const float *)x, ldx, nullptr, T, (int)d->in_f, k,
-                                                                                        d->seed);
+    const SkContract c = {z, (const float *)x, ldx, nullptr, T, (int)d->in_f, k, d->seed};
+    smallk_contract_kernel<true><<<dim3((unsigned)cdiv(T, SK_TT), nchunk), 256, 0, s>>>(c);
     int rc = check_launch("smallk_contract_kernel<hash>");
     if (rc) return rc;
     dim3 grid((unsigned)cdiv(d->out_f, 256), (unsigned)cdiv(k, 16));

@@ -199,6 +199,23 @@ def test_small_k_fp32_regime(hip, oracle, batch, matrix):
         assert torch.equal(y2, hip.linear_fwd(x.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED))  # reproducible
 
 
+def test_small_k_fp32_long_contraction_runs_in_two_launches(hip, oracle):
+    """More than 8192 input features: an expanding block would wait for more tags than a wave has lanes, so the contraction and
+    the expansion run as two launches; same arithmetic, same tolerance."""
+    from randumb_amd._lib import RDB_ALGO_FACTORED
+
+    print("case small-k long contraction", flush=True)
+    T, in_f, out_f, k, seed = 3, 8448, 64, 8, 21
+    g = torch.Generator().manual_seed(6)
+    x, dy = torch.randn(T, in_f, generator=g), torch.randn(T, out_f, generator=g)
+    C = torch.randn(out_f, k, generator=g) * 0.1
+    y = hip.linear_fwd(x.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    dx = hip.linear_bwd_dx(dy.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    want_dx, _, _ = oracle.linear_bwd(x.numpy(), dy.numpy(), C.numpy(), in_f, out_f, seed)
+    assert rel_l2(cpu(y), oracle.linear_fwd(x.numpy(), C.numpy(), in_f, out_f, seed)) < F32_TOL
+    assert rel_l2(cpu(dx), want_dx) < F32_TOL
+
+
 def test_small_k_fp32_ragged_shapes(hip, oracle):
     """The fp32 small-k kernels on sizes that divide nothing: 5 tokens, 77 -> 130, k = 23, with bias."""
     from randumb_amd._lib import RDB_ALGO_FACTORED

@@ -113,9 +113,10 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     w_one = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_PROJECTED, ctypes.byref(desc(16384, 4096, 14336, 256)))
     assert w_big >= w_one >= 16384 * 256 * 2 and (w_big - 16384 * 256 * 2) % (14336 * 256 * 4) == 0
     assert L.rdb_linear_projection_layout(ctypes.byref(big), info) == -5 and b"4 states" in L.rdb_last_error_string()
-    # fp32, small k: one partial [tokens x k] matrix per 256 values of the longer side
+    # fp32, small k: one partial [tokens x k] matrix per 256 values of the longer side, a 64-bit tag slot per tile of 8 tokens
+    # and chunk, and a word for a block that gave up waiting
     f32 = desc(16, 4096, 4096, 16, act=_lib.RDB_F32, coef=_lib.RDB_F32)
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(f32)) == 16 * 16 * 16 * 4
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(f32)) == 16 * 16 * 16 * 4 + 2 * 16 * 8 + 8
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(16, 4096, 4096, 128, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 0
 
     bad = ctypes.byref(desc(64, 100, 32, 16))
