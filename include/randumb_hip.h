@@ -221,7 +221,7 @@ int rdb_linear_projection_chunks(const rdb_linear_desc *desc, int64_t *chunk_tok
 
 /* Where the pieces lie inside the state, for tools and tests that want to look at z (no reference counterpart: the
  * reference keeps x).  Returns 0 and fills info[0..7], or RDB_E_UNSUPPORTED:
- *   info[0] byte offset of z for the forward product    info[1] 1: fragment order, rows = tokens; 0: row-major [tokens x k]
+ *   info[0] byte offset of z for the forward product    info[1] 1 (fragment order, rows = tokens)
  *   info[2] byte offset of z transposed (fragment order, rows = coefficients)
  *   info[3] byte offset of C transposed (fragment order, rows = coefficients); valid when the state's first 32-bit word is 1
  *   info[4] k rounded up to 64   info[5] tokens rounded up to 32   info[6] tokens rounded up to 64   info[7] out_f rounded up to 64

@@ -24,15 +24,14 @@ __host__ __device__ inline int64_t frag_index(int64_t row, int64_t kk, int64_t k
 // Where the pieces of a layer's projection state lie in the caller's buffer (a pure function of the layer's sizes).
 //   header : 256 bytes; word 0 = 1 when the transposed coefficients below are present; word 1 != 0: a launch that waits for its
 //            own earlier blocks gave up waiting (never seen; the results of that launch are then undefined)
-//   zf     : z = x . N^T for the forward product: fragment order [tokens32 / 32][kpad / 16] when k <= 256 (rows = tokens),
-//            row-major [tokens x k] otherwise
+//   zf     : z = x . N^T for the forward product: fragment order [tokens32 / 32][kpad / 16], rows = tokens
 //   ztf    : z transposed, fragment order, rows = coefficients: [kpad / 32][tokens64 / 16]   (operand of dC = dy^T . z)
 //   ctf    : C transposed, fragment order, rows = coefficients: [kpad / 32][out64 / 16]      (operand of t = dy . C)
 //   sync   : one 64-bit slot per projection tile (256 tokens x 32 coefficients): the tag of the launch that wrote the tile last,
 //            for the forward launch whose later blocks consume what its earlier blocks project
 // kpad, tokens64, out64: rounded up to 64; tokens32: to 32.
 struct ProjLayout {
-    bool ok, frag_fwd;
+    bool ok, fits_regs;   // fits_regs: k <= 256, the forward product keeps a token's whole contraction in registers
     int kpad;
     int64_t tok32, tok64, out64;
     int64_t zf_off, ztf_off, ctf_off, sync_off, bytes;
@@ -53,10 +52,10 @@ inline ProjLayout proj_layout(const rdb_linear_desc *d)
     // every piece is addressed with 32-bit byte offsets through a buffer descriptor
     if (L.tok64 * L.kpad >= (1ll << 29) || L.out64 * L.kpad >= (1ll << 29) || d->tokens * d->k >= (1ll << 29) || d->out_f * d->k >= (1ll << 29))
         return L;
-    L.frag_fwd = d->k <= PROJ_FRAG_KMAX;
+    L.fits_regs = d->k <= PROJ_FRAG_KMAX;
     auto up = [](int64_t n) { return (n + 255) / 256 * 256; };
     L.zf_off = 256;
-    L.ztf_off = L.zf_off + up((L.frag_fwd ? L.tok32 * L.kpad : d->tokens * d->k) * 2);
+    L.ztf_off = L.zf_off + up(L.tok32 * L.kpad * 2);
     L.ctf_off = L.ztf_off + up(L.tok64 * L.kpad * 2);
     L.sync_off = L.ctf_off + up(L.out64 * L.kpad * 2);
     L.bytes = L.sync_off + up(cdiv(d->tokens, 256) * (L.kpad / 32) * 8);

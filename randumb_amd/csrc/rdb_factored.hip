@@ -30,13 +30,13 @@ constexpr int KZ_BM = 32, KZ_BT = 256;
 struct ZParams {
     const bf16_t *x;
     const bf16_t *coef;  // NULL, or C [out_f x k] to transpose into ctf on the side
-    bf16_t *zf;          // z for the forward product: fragment order (frag_fwd) or row-major [tokens x k]
+    bf16_t *zf;          // z for the forward product: fragment order, rows = tokens
     bf16_t *ztf;         // z transposed in fragment order, rows = coefficients
     bf16_t *ctf;         // C transposed in fragment order, rows = coefficients
     uint32_t *flag;      // header word 0 of the state: 1 when ctf has been written by this launch
     int64_t ldx;
     int tokens, in_f, out_f, k;
-    int kpad, tok32, tok64, out64, frag_fwd;
+    int kpad, tok32, tok64, out64;
     int tiles_m, tiles_t;
     uint32_t seed;
     unsigned long long *sync;   // NULL, or slots [tiles_t][tiles_m]: a block sets its slot to sync_tag when its tile is in memory
@@ -181,7 +181,7 @@ __device__ __forceinline__ void z_block(const ZParams &p, unsigned char *smem_ra
     }
     __syncthreads();
     constexpr int PIECES = KZ_BM * KZ_BT / 8;
-    if (p.frag_fwd) {
+    {
         // rows = tokens, k = coefficients: a piece is 8 coefficients of one token, neighbouring lanes take neighbouring tokens
         // device scope (written through): blocks of this very launch on other dies may be waiting for the tile
         const int ksteps = p.kpad >> 4;
@@ -194,13 +194,6 @@ __device__ __forceinline__ void z_block(const ZParams &p, unsigned char *smem_ra
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, *reinterpret_cast<const f32x4 *>(lds + b * LD + a)), rs_zf,
                                                        (int)((((gb >> 5) * ksteps + (ga >> 4)) * 512 + (((ga >> 3) & 1) * 32 + (gb & 31)) * 8) * 2), 0,
                                                        SCOPE_DEVICE);
-        }
-    } else {
-#pragma unroll
-        for (int q = 0; q < PIECES / KZ_THREADS; ++q) {
-            const int idx = q * KZ_THREADS + t, b = idx / (KZ_BM / 8), a = (idx % (KZ_BM / 8)) * 8;
-            if (tok0 + b < p.tokens && m0 + a < p.k)
-                store_stream(reinterpret_cast<f32x4 *>(p.zf + (int64_t)(tok0 + b) * p.k + m0 + a), *reinterpret_cast<const f32x4 *>(lds + b * LD + a));
         }
     }
     {
@@ -228,17 +221,17 @@ __global__ __launch_bounds__(KZ_THREADS, 1) void factored_z_kernel(ZParams p)
 }
 
 // ----------------------------------------------------------------------------------------------- y = z . C^T
-// tile: 128 output features (engine rows "a") x 128 tokens (engine rows "b"), contraction over k; two blocks per CU, so
-// one block's load latency and store phase overlap the other's matrix work (k is short: a block has few stages)
+// Any k (the kernel for k > 256).  tile: 128 output features (rows "a", C staged through LDS) x 128 tokens (rows "b", z taken
+// from its fragment-ordered copy straight into registers), contraction over k; two blocks per CU.
 constexpr int KY_BO = 128, KY_BT = 128;
 
 struct YParams {
-    const bf16_t *z;
+    const bf16_t *z;   // fragment order, rows = tokens (padded to tok32), k padded to kpad
     const bf16_t *coef;
     const bf16_t *bias;
     bf16_t *y;
     int64_t ldy;
-    int tokens, out_f, k;
+    int tokens, out_f, k, kpad, tok32;
     int tiles_o, tiles_t;
 };
 
@@ -249,6 +242,7 @@ __global__ __launch_bounds__(256, 2) void factored_y_kernel(YParams p)
     // work item = (token tile, output tile), output tile fastest: neighbours share the z tile, a die shares C
     const int w = xcd_work_item(blockIdx.x, p.tiles_o * p.tiles_t);
     if (w >= p.tiles_o * p.tiles_t) return;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, wm = wave >> 1, wn = wave & 1;
     const int o0 = (w % p.tiles_o) * KY_BO, tok0 = (w / p.tiles_o) * KY_BT;
     f32x16 acc[KY_BO / 64][KY_BT / 64];
 #pragma unroll
@@ -256,8 +250,9 @@ __global__ __launch_bounds__(256, 2) void factored_y_kernel(YParams p)
 #pragma unroll
         for (int ni = 0; ni < KY_BT / 64; ++ni) acc[mi][ni] = zero16();
     GlobalOperand<KY_BO, F_BK, K_CONT> opc = {p.coef, (int64_t)p.k, o0, p.out_f, p.k, (int64_t)p.out_f * p.k};
-    GlobalOperand<KY_BT, F_BK, K_CONT> opz = {p.z, (int64_t)p.k, tok0, p.tokens, p.k, (int64_t)p.tokens * p.k};
-    gemm_mainloop<KY_BO, KY_BT, F_BK, 1, 1>(acc, lds, opc, opz, 0, (p.k + F_BK - 1) / F_BK);
+    FragSource fz;   // this wave's 64 tokens; row blocks past tok32 fail the bounds check and read as zeros
+    fz.init(p.z, (int64_t)p.tok32 * p.kpad, p.kpad >> 4, (tok0 + wn * 64) >> 5, lane);
+    direct_mainloop<KY_BO / 64, KY_BT / 64, F_BK / 16, true, 2, 2, 2>(acc, lds, opc, fz, 0, (p.k + F_BK - 1) / F_BK, wm * 64, lane);
     store_tile_bf16<KY_BO, KY_BT>(acc, lds, p.y, p.ldy, o0, p.out_f, tok0, p.tokens, 1.0f, p.bias);
 }
 
@@ -346,7 +341,6 @@ static bool fill_z_params(ZParams &p, void *state, const void *x, int64_t ldx, c
     p.tok32 = (int)L.tok32;
     p.tok64 = (int)L.tok64;
     p.out64 = (int)L.out64;
-    p.frag_fwd = L.frag_fwd ? 1 : 0;
     p.seed = d->seed;
     p.tiles_m = L.kpad / KZ_BM;   // every coefficient row block of the padded pieces is written
     p.tiles_t = (int)cdiv(d->tokens, KZ_BT);
@@ -373,7 +367,7 @@ static int fill_ys_params(StParams &q, void *y, int64_t ldy, const void *state, 
                           int num_cus)
 {
     const ProjLayout L = proj_layout(d);
-    if (!L.ok || !L.frag_fwd || d->coef_dtype != RDB_BF16 || ldy % 8 || !aligned16(y) || !aligned16(state) || !aligned16(coef)) return 0;
+    if (!L.ok || !L.fits_regs || d->coef_dtype != RDB_BF16 || ldy % 8 || !aligned16(y) || !aligned16(state) || !aligned16(coef)) return 0;
     if (((uintptr_t)bias & 7) || d->tokens * ldy >= (1ll << 29)) return 0;
     q.z = state_piece(state, L.zf_off);
     q.coef = (const bf16_t *)coef;
@@ -415,9 +409,8 @@ int linear_project_fwd(void *y, int64_t ldy, void *state, const void *x, int64_t
     const int y_items = fill_ys_params(p.y, y, ldy, state, coef, bias, d, num_cus);
     if (!y_items || p.z.tiles_m > 64) {
         // check the second call's conditions before the first launch, so that a refusal leaves nothing half done
-        const ProjLayout L = proj_layout(d);
         if (d->coef_dtype != RDB_BF16 || ldy % 8 || !aligned16(y) || !aligned16(coef)) return RDB_E_UNSUPPORTED;
-        if (L.frag_fwd && (((uintptr_t)bias & 7) || d->tokens * ldy >= (1ll << 29))) return RDB_E_UNSUPPORTED;
+        if (((uintptr_t)bias & 7) || d->tokens * ldy >= (1ll << 29)) return RDB_E_UNSUPPORTED;
         if (int rc = linear_project(state, x, ldx, with_ct ? coef : nullptr, d, s)) return rc;
         return linear_fwd_projected(y, ldy, state, coef, bias, d, num_cus, s);
     }
@@ -452,7 +445,7 @@ int linear_fwd_projected(void *y, int64_t ldy, const void *state, const void *co
     const ProjLayout L = proj_layout(d);
     if (!L.ok || d->coef_dtype != RDB_BF16 || ldy % 8 || !aligned16(y) || !aligned16(state) || !aligned16(coef)) return RDB_E_UNSUPPORTED;
     const bf16_t *zf = state_piece(state, L.zf_off);
-    if (L.frag_fwd) {   // the contraction of a token fits in registers; z lies in fragment order
+    if (L.fits_regs) {   // the contraction of a token fits in registers
         StParams q;
         const int items = fill_ys_params(q, y, ldy, state, coef, bias, d, num_cus);
         if (!items) return RDB_E_UNSUPPORTED;
@@ -482,6 +475,8 @@ int linear_fwd_projected(void *y, int64_t ldy, const void *state, const void *co
     p.tokens = (int)d->tokens;
     p.out_f = (int)d->out_f;
     p.k = (int)d->k;
+    p.kpad = L.kpad;
+    p.tok32 = (int)L.tok32;
     p.tiles_o = (int)cdiv(d->out_f, KY_BO);
     p.tiles_t = (int)cdiv(d->tokens, KY_BT);
     return launch_engine(factored_y_kernel, p, p.tiles_o * p.tiles_t, engine_smem<KY_BO, KY_BT, F_BK, K_CONT, K_CONT>(), s, "factored_y_kernel");
@@ -508,7 +503,7 @@ int linear_fwd_factored(void *y, int64_t ldy, const void *x, int64_t ldx, const 
     // check everything before the first launch, so that a refusal leaves nothing half done
     if (d->tokens * ldx >= (1ll << 29) || ldx % 8 || ldy % 8 || !aligned16(x) || !aligned16(coef) || !aligned16(y) || !aligned16(workspace))
         return RDB_E_UNSUPPORTED;
-    if (proj_layout(d).frag_fwd && (((uintptr_t)bias & 7) || d->tokens * ldy >= (1ll << 29))) return RDB_E_UNSUPPORTED;
+    if (((uintptr_t)bias & 7) || d->tokens * ldy >= (1ll << 29)) return RDB_E_UNSUPPORTED;
     return linear_project_fwd(y, ldy, workspace, x, ldx, coef, false, bias, d, num_cus, s);
 }
 

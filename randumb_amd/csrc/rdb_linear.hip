@@ -648,7 +648,7 @@ extern "C" int rdb_linear_projection_layout(const rdb_linear_desc *d, int64_t *i
                                           pl.nchunks, (long long)pl.chunk_tokens, (long long)pl.state_stride);
     const ProjLayout L = proj_layout(d);
     info[0] = L.zf_off;
-    info[1] = L.frag_fwd ? 1 : 0;
+    info[1] = 1;
     info[2] = L.ztf_off;
     info[3] = L.ctf_off;
     info[4] = L.kpad;

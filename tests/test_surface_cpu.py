@@ -63,25 +63,25 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     r = ctypes.byref(d)
     zbytes = 8192 * 256 * 2
 
-    def state_bytes(tokens, out_f, k):
-        # header + z for the forward product (tokens to 32 when k <= 256) + z transposed (tokens to 64) + C transposed (out to 64)
+    def state_bytes(tokens, in_f, out_f, k):
+        # header + z for the forward product (tokens to 32) + z transposed (tokens to 64) + C transposed (out to 64)
         # + a 64-bit slot per projection tile (256 tokens x 32 coefficients)
         up = lambda n, m: -(-n // m) * m
         kpad = up(k, 64)
-        zf = up(tokens, 32) * kpad * 2 if k <= 256 else tokens * k * 2
+        zf = up(tokens, 32) * kpad * 2
         return (256 + up(zf, 256) + up(up(tokens, 64) * kpad * 2, 256) + up(up(out_f, 64) * kpad * 2, 256)
                 + up(-(-tokens // 256) * (kpad // 32) * 8, 256))
 
-    assert state_bytes(8192, 3072, 256) == 256 + 2 * zbytes + 3072 * 256 * 2 + 32 * 8 * 8
-    assert L.rdb_linear_projection_bytes(r) == state_bytes(8192, 3072, 256)
+    assert state_bytes(8192, 768, 3072, 256) == 256 + 2 * zbytes + 3072 * 256 * 2 + 32 * 8 * 8
+    assert L.rdb_linear_projection_bytes(r) == state_bytes(8192, 768, 3072, 256)
     info = (ctypes.c_int64 * 8)()
     assert L.rdb_linear_projection_layout(r, info) == 0
     assert list(info) == [256, 1, 256 + zbytes, 256 + 2 * zbytes, 256, 8192, 8192, 3072]
-    assert L.rdb_linear_projection_bytes(ctypes.byref(desc(1000, 200, 328, 72))) == state_bytes(1000, 328, 72)
-    assert L.rdb_linear_projection_bytes(ctypes.byref(desc(4096, 4096, 14336, 1024))) == state_bytes(4096, 14336, 1024)
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, r) == state_bytes(8192, 3072, 256)
+    assert L.rdb_linear_projection_bytes(ctypes.byref(desc(1000, 200, 328, 72))) == state_bytes(1000, 200, 328, 72)
+    assert L.rdb_linear_projection_bytes(ctypes.byref(desc(4096, 4096, 14336, 1024))) == state_bytes(4096, 4096, 14336, 1024)
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, r) == state_bytes(8192, 768, 3072, 256)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, r) == zbytes
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DCOEF, r) == state_bytes(8192, 3072, 256)
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DCOEF, r) == state_bytes(8192, 768, 3072, 256)
     # whole backward pass: dy.C plus the partial sums of the coefficient gradient, one [out x k] fp32 matrix per token split
     extra = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_PROJECTED, r) - zbytes
     assert extra > 0 and extra % (3072 * 256 * 4) == 0
@@ -102,10 +102,10 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     assert L.rdb_linear_projection_chunks(r, ctypes.byref(ct)) == 1 and ct.value == 8192
     big = desc(65536, 4096, 14336, 256)
     assert L.rdb_linear_projection_chunks(ctypes.byref(big), ctypes.byref(ct)) == 4 and ct.value == 16384   # 2^28 / 14336 = 18724 -> 18688
-    assert L.rdb_linear_projection_bytes(ctypes.byref(big)) == 4 * state_bytes(16384, 14336, 256)
+    assert L.rdb_linear_projection_bytes(ctypes.byref(big)) == 4 * state_bytes(16384, 4096, 14336, 256)
     odd = desc(40000, 4096, 14336, 256)                                                   # 3 chunks of 13568, 13568, 12864
     assert L.rdb_linear_projection_chunks(ctypes.byref(odd), ctypes.byref(ct)) == 3 and ct.value == 13568
-    assert L.rdb_linear_projection_bytes(ctypes.byref(odd)) == 3 * state_bytes(13568, 14336, 256)
+    assert L.rdb_linear_projection_bytes(ctypes.byref(odd)) == 3 * state_bytes(13568, 4096, 14336, 256)
     assert L.rdb_linear_projection_chunks(ctypes.byref(desc(1 << 21, 768, 3072, 256)), ctypes.byref(ct)) == 25 and ct.value % 256 == 0
     assert ct.value * 3072 < (1 << 28) + 256 * 3072
     # chunks after the first add to dcoef: their sums pass through the workspace even when a chunk is a single token range
