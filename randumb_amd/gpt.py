@@ -4,8 +4,9 @@ Mirrors the reference's RT_* classes (modded-nanogpt/gpt_models.py:186-257: RT_n
 RT_CausalSelfAttention, RT_MLP, RT_Block) with the deviations the benchmark configuration states: the four linears of a
 block are qkv (d -> 3d), proj (d -> d), fc (d -> 4d) and mlp-proj (4d -> d), all in matrix-coef form with coefficient
 dimension k and seeds taken in layer order from one generator (0..47 for 12 layers); attention is plain causal
-scaled-dot-product attention (the reference's FlexAttention document mask needs a tracing compiler); embeddings and the
-language-model head are ordinary dense layers.  Everything that is not a random-backed linear is stock PyTorch: this file
+scaled-dot-product attention (the reference's FlexAttention document mask needs a tracing compiler); the token embedding
+and the language-model head are ordinary dense layers unless the configuration asks for the reference's random-backed ones
+(modded-nanogpt/gpt_models.py:303, 310).  Everything that is not a random-backed linear is stock PyTorch: this file
 wires layers, the kernels are reached through SillyLinear.
 """
 from dataclasses import dataclass
@@ -15,7 +16,7 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
-from .SillyLayers import SillyLinear
+from .SillyLayers import SillyEmbedding, SillyLinear
 
 
 def RT_norm(x: torch.Tensor) -> torch.Tensor:
@@ -45,6 +46,9 @@ class RT_GPTConfig:
     n_layer: int = 12
     n_head: int = 12
     n_embd: int = 768
+    # True: the token embedding and the output head are random-backed too, as in the reference's model
+    # (modded-nanogpt/gpt_models.py:303, 310); they then draw the first and the last (k, seed) of the generators
+    random_embedding_and_head: bool = False
 
 
 class RT_CastedLinear(SillyLinear):
@@ -103,12 +107,19 @@ class RT_GPT(nn.Module):
 
     def __init__(self, config: RT_GPTConfig):
         super().__init__()
-        self.wte = nn.Embedding(config.vocab_size, config.n_embd)
+        if config.random_embedding_and_head:
+            self.wte = SillyEmbedding(config.vocab_size, config.n_embd, config.int_dim_gen, config.seed_gen)
+        else:
+            self.wte = nn.Embedding(config.vocab_size, config.n_embd)
         self.h = nn.ModuleList([RT_Block(config) for _ in range(config.n_layer)])
-        self.lm_head = nn.Linear(config.n_embd, config.vocab_size, bias=False)
+        if config.random_embedding_and_head:
+            self.lm_head = RT_CastedLinear(config.n_embd, config.vocab_size, config)
+        else:
+            self.lm_head = nn.Linear(config.n_embd, config.vocab_size, bias=False)
 
     def forward(self, idx: torch.Tensor, target: torch.Tensor) -> torch.Tensor:
-        x = RT_norm(self.wte(idx))
+        x = self.wte(idx)
+        x = RT_norm(x.to(self.h[0].mlp.c_fc.weight_coef.dtype))
         for block in self.h:
             x = block(x)
         logits = self.lm_head(RT_norm(x)).float()

@@ -299,6 +299,37 @@ def test_gpt2_small_full_model_starts_at_ln_vocab(ra):
         assert float(gr.float().abs().max()) > 0.0, i
 
 
+def test_gpt_with_random_embedding_and_head(ra):
+    """The reference's model makes the token embedding and the output head random-backed as well
+    (modded-nanogpt/gpt_models.py:303, 310).  A small model built that way: the embedding draws the first seed, the head the
+    last; the loss starts at ln(vocab) (head weights of standard deviation 0.02 on normalised activations); gradients reach
+    the embedding's and the head's coefficients; the head gives the same logits through the fused kernels and through the
+    tensor-subclass dispatch."""
+    print("case config: GPT with random-backed embedding and head", flush=True)
+    from randumb_amd.gpt import RT_GPT, RT_GPTConfig
+
+    torch.manual_seed(0)
+    cfg = RT_GPTConfig(int_dim_gen=ra.listgen([16] * 10), seed_gen=ra.stepgen(0, 1), vocab_size=384, n_layer=2, n_head=2, n_embd=64,
+                       random_embedding_and_head=True)
+    model = RT_GPT(cfg).to(torch.bfloat16).cuda()
+    assert isinstance(model.wte, ra.SillyEmbedding) and model.wte.weight.seed == 0
+    assert isinstance(model.lm_head, ra.SillyLinear) and model.lm_head.weight.seed == 9
+    g = torch.Generator().manual_seed(3)
+    idx = torch.randint(0, 384, (4, 128), generator=g).cuda()
+    tgt = torch.randint(0, 384, (4, 128), generator=g).cuda()
+    loss = model(idx, tgt)
+    assert torch.isfinite(loss) and abs(float(loss.detach()) - math.log(384)) < 0.05 * math.log(384), float(loss.detach())
+    loss.backward()
+    for name, p in (("wte", model.wte.weight_coef), ("lm_head", model.lm_head.weight_coef)):
+        assert p.grad is not None and bool(torch.isfinite(p.grad.float()).all()) and float(p.grad.float().abs().max()) > 0.0, name
+    x = torch.randn(512, 64, generator=g).bfloat16().cuda()
+    model.lm_head.fused = True
+    y_fused = model.lm_head(x)
+    model.lm_head.fused = False
+    y_disp = model.lm_head(x)
+    assert rel_l2(cpu(y_fused), cpu(y_disp)) < BF16_TOL
+
+
 def _tiny_gpt(dtype, fused):
     from randumb_amd.SillyLayers import SillyLinear, listgen, stepgen
     from randumb_amd.gpt import RT_GPT, RT_GPTConfig
