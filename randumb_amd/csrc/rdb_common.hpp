@@ -148,6 +148,19 @@ __device__ __forceinline__ bool await_tags(const unsigned long long *slots, int 
     return false;
 }
 
+// The same wave calls this once its wait has succeeded.  A launch recorded in a graph runs again with the tag it was recorded
+// with, so the slots must not still hold it then: every consumer of the n slots counts itself in `counter`, and the last of
+// the `consumers` (all of them are past their wait by then) clears the slots.  The counter is set to zero by one of the
+// producers of these slots before it publishes its tag (store it before the call of publish_tag).
+__device__ __forceinline__ void release_tags(unsigned long long *slots, int n, unsigned int *counter, int consumers)
+{
+    const int lane = threadIdx.x & 63;
+    unsigned int old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    old = (unsigned int)__builtin_amdgcn_readfirstlane((int)old);
+    if (old == (unsigned int)(consumers - 1) && lane < n) __hip_atomic_store(slots + lane, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 #ifdef RDB_STAMPS
 #ifndef RDB_STAMP_KERNEL_ID
 #define RDB_STAMP_KERNEL_ID 0

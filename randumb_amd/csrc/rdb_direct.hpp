@@ -27,8 +27,9 @@ __host__ __device__ inline int64_t frag_index(int64_t row, int64_t kk, int64_t k
 //   zf     : z = x . N^T for the forward product: fragment order [tokens32 / 32][kpad / 16], rows = tokens
 //   ztf    : z transposed, fragment order, rows = coefficients: [kpad / 32][tokens64 / 16]   (operand of dC = dy^T . z)
 //   ctf    : C transposed, fragment order, rows = coefficients: [kpad / 32][out64 / 16]      (operand of t = dy . C)
-//   sync   : one 64-bit slot per projection tile (256 tokens x 32 coefficients): the tag of the launch that wrote the tile last,
-//            for the forward launch whose later blocks consume what its earlier blocks project
+//   sync   : per 256 tokens, one 64-bit slot per projection tile (32 coefficients) with the tag of the launch that wrote the tile
+//            last, and one counter of the blocks that have consumed them: for the forward launch whose later blocks consume
+//            what its earlier blocks project
 // kpad, tokens64, out64: rounded up to 64; tokens32: to 32.
 struct ProjLayout {
     bool ok, fits_regs;   // fits_regs: k <= 256, the forward product keeps a token's whole contraction in registers
@@ -58,7 +59,7 @@ inline ProjLayout proj_layout(const rdb_linear_desc *d)
     L.ztf_off = L.zf_off + up(L.tok32 * L.kpad * 2);
     L.ctf_off = L.ztf_off + up(L.tok64 * L.kpad * 2);
     L.sync_off = L.ctf_off + up(L.out64 * L.kpad * 2);
-    L.bytes = L.sync_off + up(cdiv(d->tokens, 256) * (L.kpad / 32) * 8);
+    L.bytes = L.sync_off + up(cdiv(d->tokens, 256) * (L.kpad / 32 + 1) * 8);
     L.ok = true;
     return L;
 }

@@ -39,7 +39,8 @@ struct ZParams {
     int kpad, tok32, tok64, out64;
     int tiles_m, tiles_t;
     uint32_t seed;
-    unsigned long long *sync;   // NULL, or slots [tiles_t][tiles_m]: a block sets its slot to sync_tag when its tile is in memory
+    unsigned long long *sync;   // NULL, or slots [tiles_t][tiles_m + 1]: a block sets its slot to sync_tag when its tile is in memory;
+                                // slot tiles_m of a token tile counts its consumers and is cleared by the block of coefficient tile 0
     unsigned long long sync_tag;
 };
 
@@ -210,7 +211,12 @@ __device__ __forceinline__ void z_block(const ZParams &p, unsigned char *smem_ra
             store_stream(reinterpret_cast<f32x4 *>(p.ztf + ((int64_t)(m0 >> 5) * tsteps + (tok0 >> 4) + ks) * 512 + lane * 8), f.f4);
         }
     }
-    if (p.sync) publish_tag(p.sync + (int64_t)(w / p.tiles_m) * p.tiles_m + (w % p.tiles_m), p.sync_tag);
+    if (p.sync) {
+        unsigned long long *slots = p.sync + (int64_t)(w / p.tiles_m) * (p.tiles_m + 1);
+        if (w % p.tiles_m == 0 && t == 0)
+            __hip_atomic_store(reinterpret_cast<unsigned int *>(slots + p.tiles_m), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        publish_tag(slots + (w % p.tiles_m), p.sync_tag);
+    }
     RDB_STAMP(3);
 }
 

@@ -121,10 +121,13 @@ struct SkExpand {
     const float *bias;   // [cols] or NULL
     int T, cols, k;
     uint32_t seed;
-    // NULL, or slots [token tiles of SK_TT][nchunk] that contracting blocks of the same launch set to sync_tag
-    const unsigned long long *sync;
+    // NULL, or slots [token tiles of SK_TT][nchunk] that contracting blocks of the same launch set to sync_tag; sync_count: one
+    // counter per SK_ET tokens of the expanding blocks that have seen them (sync_consumers of them: the last clears the slots)
+    unsigned long long *sync;
     unsigned long long sync_tag;
     unsigned int *sync_err;
+    unsigned int *sync_count;
+    int sync_consumers;
 };
 
 // bx: block of 256 columns, by: block of SK_ET tokens.
@@ -154,7 +157,8 @@ template <bool HASH> __device__ __forceinline__ void smallk_expand_block(const S
         if (tid < 64) {
             const int tile0 = t0 / SK_TT, tiles = (T + SK_TT - 1) / SK_TT;
             const int ntile = (tile0 + SK_ET / SK_TT <= tiles) ? SK_ET / SK_TT : tiles - tile0;
-            await_tags(p.sync + (int64_t)tile0 * nchunk, ntile * nchunk, p.sync_tag, p.sync_err);
+            unsigned long long *slots = p.sync + (int64_t)tile0 * nchunk;
+            if (await_tags(slots, ntile * nchunk, p.sync_tag, p.sync_err)) release_tags(slots, ntile * nchunk, p.sync_count + by, p.sync_consumers);
         }
         __syncthreads();
     }
@@ -240,6 +244,7 @@ struct SkFused {
     SkContract c;
     SkExpand e;
     unsigned long long *slots;
+    unsigned int *counters;   // one per SK_ET tokens, cleared by the contracting block of the group's first tile and chunk 0
     int c_tiles, c_blocks, e_colblocks;
 };
 
@@ -249,6 +254,8 @@ template <bool CHASH> __global__ __launch_bounds__(256) void smallk_fused_kernel
     if (b < p.c_blocks) {
         const int bx = b % p.c_tiles, by = b / p.c_tiles;
         smallk_contract_block<CHASH>(p.c, bx, by);
+        if (by == 0 && bx % (SK_ET / SK_TT) == 0 && threadIdx.x == 0)
+            __hip_atomic_store(p.counters + bx / (SK_ET / SK_TT), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         publish_tag(p.slots + (int64_t)bx * p.e.nchunk + by, p.e.sync_tag);
     } else {
         const int e = b - p.c_blocks;
@@ -303,7 +310,7 @@ static bool smallk_wanted(const rdb_linear_desc *d)
 }
 
 // scratch: one partial [tokens x k] fp32 matrix per 256-chunk of the longer of in_f and out_f, then the tag slots of the
-// one-launch form (one per token tile and chunk) and a word for a waiting block that gave up
+// one-launch form (one per token tile and chunk), a word for a waiting block that gave up and a counter per 16 tokens
 static int64_t partial_bytes(const rdb_linear_desc *d)
 {
     const int64_t longer = d->in_f > d->out_f ? d->in_f : d->out_f;
@@ -313,7 +320,7 @@ int64_t linear_smallk_workspace(const rdb_linear_desc *d)
 {
     if (!smallk_ok(d)) return 0;
     const int64_t longer = d->in_f > d->out_f ? d->in_f : d->out_f;
-    return partial_bytes(d) + cdiv(d->tokens, SK_TT) * cdiv(longer, 256) * 8 + 8;
+    return partial_bytes(d) + cdiv(d->tokens, SK_TT) * cdiv(longer, 256) * 8 + 8 + cdiv(d->tokens, SK_ET) * 8;
 }
 
 static bool ws_ok(const rdb_linear_desc *d, const void *ws, int64_t bytes) { return ws && bytes >= linear_smallk_workspace(d) && ((uintptr_t)ws & 7) == 0; }
@@ -338,7 +345,7 @@ static int contract_expand(float *out, int64_t ld_out, int cols, const float *sr
     const int nchunk = (int)cdiv(J, 256), tiles = (int)cdiv(T, SK_TT);
     SkFused f;
     f.c = {(float *)workspace, src, ld_src, coef, T, J, k, d->seed};
-    f.e = {out, ld_out, (const float *)workspace, nchunk, coef, bias, T, cols, k, d->seed, nullptr, 0, nullptr};
+    f.e = {out, ld_out, (const float *)workspace, nchunk, coef, bias, T, cols, k, d->seed, nullptr, 0, nullptr, nullptr, 0};
     f.slots = reinterpret_cast<unsigned long long *>(static_cast<char *>(workspace) + partial_bytes(d));
     f.c_tiles = tiles;
     f.c_blocks = tiles * nchunk;
@@ -348,6 +355,9 @@ static int contract_expand(float *out, int64_t ld_out, int cols, const float *sr
         f.e.sync = f.slots;
         f.e.sync_tag = next_tag();
         f.e.sync_err = reinterpret_cast<unsigned int *>(f.slots + (int64_t)tiles * nchunk);
+        f.counters = f.e.sync_err + 2;
+        f.e.sync_count = f.counters;
+        f.e.sync_consumers = f.e_colblocks;
         smallk_fused_kernel<CHASH><<<f.c_blocks + e_blocks, 256, 0, s>>>(f);
         return check_launch("smallk_fused_kernel");
     }

@@ -33,9 +33,9 @@ struct StParams {
     int tokens, out_f, k;
     int tiles_t, splits, units_per_split;
     uint32_t seed;       // noise flavour
-    // ZFRAG only: NULL, or slots [token tile of 256][sync_n] that earlier blocks of the same launch set to sync_tag when the tile's
-    // share of z is in memory
-    const unsigned long long *sync;
+    // ZFRAG only: NULL, or slots [token tile of 256][sync_n + 1] that earlier blocks of the same launch set to sync_tag when the
+    // tile's share of z is in memory (the last slot of a tile counts the blocks that have seen them)
+    unsigned long long *sync;
     unsigned long long sync_tag;
     int sync_n;
     unsigned int *sync_err;
@@ -226,7 +226,11 @@ __device__ __forceinline__ void stationary_block(const StParams &p, unsigned cha
         const __amdgpu_buffer_rsrc_t rs_z = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.z), 0, (int)(padded * 2), 0x00020000);
         if (!NOISE) b.issue(b.unit0);
         if (p.sync) {   // z comes from earlier blocks of this launch
-            if (wave == 0) await_tags(p.sync + (int64_t)(w / p.splits) * p.sync_n, p.sync_n, p.sync_tag, p.sync_err);
+            if (wave == 0) {
+                unsigned long long *slots = p.sync + (int64_t)(w / p.splits) * (p.sync_n + 1);
+                if (await_tags(slots, p.sync_n, p.sync_tag, p.sync_err))
+                    release_tags(slots, p.sync_n, reinterpret_cast<unsigned int *>(slots + p.sync_n), p.splits);
+            }
             __syncthreads();
         }
         const int tile = tok0 >> 5;

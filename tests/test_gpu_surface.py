@@ -336,3 +336,38 @@ def test_step_is_graph_capturable(ra):
         torch.cuda.synchronize()
         assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1]), f"replay {i}"
         assert float((got[2] - want[2]).abs().max()) <= 1e-5 * float(want[2].abs().max()), f"replay {i}"
+
+
+def test_one_launch_forms_replay_in_a_graph_on_new_inputs(ra):
+    """The launches whose later blocks wait for tags of their earlier blocks (projection + forward product in bf16, contraction +
+    expansion in fp32 with small k) carry the tag they were recorded with: replayed from a HIP graph on inputs that changed in
+    between, every replay must wait again and give that input's result (the consumers clear the tags they have seen)."""
+    print("case graph replay of the one-launch forms", flush=True)
+    from randumb_amd import hip
+
+    g = torch.Generator().manual_seed(2)
+    T, in_f, out_f, k, seed = 1024, 256, 512, 64, 3
+    xs = [torch.randn(T, in_f, generator=g).bfloat16().cuda() for _ in range(4)]
+    C = (torch.randn(out_f, k, generator=g) * 0.05).bfloat16().cuda()
+    want = [hip.linear_project_fwd(x, C, seed)[0].clone() for x in xs]
+    x = xs[0].clone()
+    T3, in3, out3, k3 = 16, 4096, 4096, 16
+    x3s = [torch.randn(T3, in3, generator=g).cuda() for _ in range(4)]
+    C3 = (torch.randn(out3, k3, generator=g) * 0.05).cuda()
+    want3 = [hip.linear_fwd(v, C3, in3, out3, in3, 1, seed).clone() for v in x3s]
+    x3 = x3s[0].clone()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y, _state = hip.linear_project_fwd(x, C, seed)
+        y3 = hip.linear_fwd(x3, C3, in3, out3, in3, 1, seed)
+    for i in (1, 2, 3, 0, 2):
+        x.copy_(xs[i])
+        x3.copy_(x3s[i])
+        y.fill_(7.0)
+        y3.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want[i]), f"bf16 forward, input {i}"
+        assert torch.equal(y3, want3[i]), f"fp32 small-k forward, input {i}"

@@ -65,14 +65,14 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
 
     def state_bytes(tokens, in_f, out_f, k):
         # header + z for the forward product (tokens to 32) + z transposed (tokens to 64) + C transposed (out to 64)
-        # + a 64-bit slot per projection tile (256 tokens x 32 coefficients)
+        # + per 256 tokens a 64-bit slot per projection tile (32 coefficients) and one counter
         up = lambda n, m: -(-n // m) * m
         kpad = up(k, 64)
         zf = up(tokens, 32) * kpad * 2
         return (256 + up(zf, 256) + up(up(tokens, 64) * kpad * 2, 256) + up(up(out_f, 64) * kpad * 2, 256)
-                + up(-(-tokens // 256) * (kpad // 32) * 8, 256))
+                + up(-(-tokens // 256) * (kpad // 32 + 1) * 8, 256))
 
-    assert state_bytes(8192, 768, 3072, 256) == 256 + 2 * zbytes + 3072 * 256 * 2 + 32 * 8 * 8
+    assert state_bytes(8192, 768, 3072, 256) == 256 + 2 * zbytes + 3072 * 256 * 2 + 32 * 9 * 8
     assert L.rdb_linear_projection_bytes(r) == state_bytes(8192, 768, 3072, 256)
     info = (ctypes.c_int64 * 8)()
     assert L.rdb_linear_projection_layout(r, info) == 0
@@ -114,9 +114,9 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     assert w_big >= w_one >= 16384 * 256 * 2 and (w_big - 16384 * 256 * 2) % (14336 * 256 * 4) == 0
     assert L.rdb_linear_projection_layout(ctypes.byref(big), info) == -5 and b"4 states" in L.rdb_last_error_string()
     # fp32, small k: one partial [tokens x k] matrix per 256 values of the longer side, a 64-bit tag slot per tile of 8 tokens
-    # and chunk, and a word for a block that gave up waiting
+    # and chunk, a word for a block that gave up waiting, and a counter per 16 tokens
     f32 = desc(16, 4096, 4096, 16, act=_lib.RDB_F32, coef=_lib.RDB_F32)
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(f32)) == 16 * 16 * 16 * 4 + 2 * 16 * 8 + 8
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(f32)) == 16 * 16 * 16 * 4 + 2 * 16 * 8 + 8 + 8
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(16, 4096, 4096, 128, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 0
 
     bad = ctypes.byref(desc(64, 100, 32, 16))
