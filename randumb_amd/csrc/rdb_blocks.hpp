@@ -30,8 +30,7 @@ constexpr int KD_BO = 128, KD_BM = 128;
 
 struct DcParams {
     const bf16_t *dy;
-    const bf16_t *z;     // row-major [tokens x k] (dc_block) ...
-    const bf16_t *ztf;   // ... or transposed in fragment order, rows = coefficients (dc_block_direct)
+    const bf16_t *ztf;   // z transposed in fragment order, rows = coefficients
     int tsteps, kpad;    // of ztf: token k-steps per row block (tokens rounded up to 64, / 16), k rounded up to 64
     float *dcoef;
     float *partial;  // NULL: the token splits add into dcoef (zeroed beforehand) with atomics; else split s stores its sums
@@ -88,29 +87,8 @@ __device__ __forceinline__ void dc_store(const DcParams &p, const f32x16 (&acc)[
     }
 }
 
-// `block`: index of this block among the blocks that run this body.
-__device__ __forceinline__ void dc_block(const DcParams &p, bf16_t *lds, int block)
-{
-    // work item = (token split, output tile, coefficient tile), coefficient tile fastest: neighbours share the dy stream
-    const int total = p.tiles_o * p.tiles_m * p.splits;
-    const int w = xcd_work_item(block, total);
-    if (w >= total) return;
-    const int m0 = (w % p.tiles_m) * KD_BM, o0 = ((w / p.tiles_m) % p.tiles_o) * KD_BO, split = w / (p.tiles_m * p.tiles_o);
-    const int t_begin = split * p.tok_per_split;
-    const int t_end = (t_begin + p.tok_per_split < p.tokens) ? t_begin + p.tok_per_split : p.tokens;
-    f32x16 acc[KD_BO / 64][KD_BM / 64];
-#pragma unroll
-    for (int mi = 0; mi < KD_BO / 64; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < KD_BM / 64; ++ni) acc[mi][ni] = zero16();
-    GlobalOperand<KD_BO, B_BK, M_CONT> opdy = {p.dy, p.lddy, o0, p.out_f, t_end, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
-    GlobalOperand<KD_BM, B_BK, M_CONT> opz = {p.z, (int64_t)p.k, m0, p.k, t_end, (int64_t)p.tokens * p.k};
-    gemm_mainloop<KD_BO, KD_BM, B_BK, 1, 1>(acc, lds, opdy, opz, t_begin, (t_end - t_begin + B_BK - 1) / B_BK);
-    dc_store(p, acc, lds, o0, m0, split);
-    RDB_STAMP(3);
-}
-
-// The same block with z taken from its transposed, fragment-ordered copy: only dy passes through LDS.
+// `block`: index of this block among the blocks that run this body.  z comes from its transposed, fragment-ordered copy
+// straight into registers: only dy passes through LDS.
 __device__ __forceinline__ void dc_block_direct(const DcParams &p, bf16_t *lds, int block)
 {
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, wm = wave >> 1, wn = wave & 1;
@@ -210,10 +188,9 @@ __device__ __forceinline__ void tn_block(const TNParams &p, bf16_t *lds, int blo
 // ----------------------------------------------------------------------------------------------- host side
 // Parameters of the coefficient-gradient blocks for layer d; the token range is split so that tiles x splits is about one
 // block per compute unit.  Returns the number of work items.
-inline int make_dc_params(DcParams &p, float *dcoef, const void *dy, int64_t lddy, const void *z, const rdb_linear_desc *d, int num_cus)
+inline int make_dc_params(DcParams &p, float *dcoef, const void *dy, int64_t lddy, const rdb_linear_desc *d, int num_cus)
 {
     p.dy = (const bf16_t *)dy;
-    p.z = (const bf16_t *)z;
     p.ztf = nullptr;
     p.tsteps = 0;
     p.kpad = 0;

@@ -161,10 +161,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dc_dyc_kernel(BwdAParams p)
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
     if ((int)blockIdx.x < p.dc_blocks) {
-        if (p.dc.ztf)
-            dc_block_direct(p.dc, lds, blockIdx.x);
-        else
-            dc_block(p.dc, lds, blockIdx.x);
+        dc_block_direct(p.dc, lds, blockIdx.x);
     } else {
         if (p.dyc.ctf && *p.dyc.ctf_flag)   // the forward pass left the transposed coefficients in the state
             dyc_block_direct(p.dyc, lds, blockIdx.x - p.dc_blocks);
@@ -237,7 +234,7 @@ int64_t linear_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus, bo
 {
     if (!dx_factored_ok(d)) return 0;
     DcParams dc;
-    make_dc_params(dc, nullptr, nullptr, d->out_f, nullptr, d, num_cus);
+    make_dc_params(dc, nullptr, nullptr, d->out_f, d, num_cus);
     if (dc.splits == 1 && !force_partial) return linear_dx_factored_workspace(d);   // a single token range is stored straight into dcoef
     return align256(linear_dx_factored_workspace(d)) + (int64_t)dc.splits * d->out_f * d->k * (int64_t)sizeof(float);
 }
@@ -331,7 +328,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
     const size_t smem_dyc = engine_smem<K1_BC, K1_BT, X_BK, M_CONT, K_CONT>();
     if (workspace_bytes >= linear_bwd_projected_workspace(d, num_cus, accumulate)) {
         BwdAParams a;
-        const int dc_items = make_dc_params(a.dc, dcoef, dy, lddy, nullptr, d, num_cus);
+        const int dc_items = make_dc_params(a.dc, dcoef, dy, lddy, d, num_cus);
         dc_params_from_state(a.dc, z, d);
         // one token range only: its sums are the result, stored straight into dcoef, and nothing is left to add up
         const bool direct = a.dc.splits == 1 && !accumulate;
@@ -398,7 +395,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
     int rc = launch_engine(dx_dyc_kernel, p1, p1.tiles_c * p1.tiles_t, smem_dyc, s, "dx_dyc_kernel");
     if (rc) return rc;
     BwdParams p;
-    const int dc_items = make_dc_params(p.dc, dcoef, dy, lddy, nullptr, d, num_cus);
+    const int dc_items = make_dc_params(p.dc, dcoef, dy, lddy, d, num_cus);
     dc_params_from_state(p.dc, z, d);
     const int tn_items = make_tn_params(p.tn, dx, lddx, workspace, d);
     p.dc_blocks = xcd_grid_size(dc_items);

@@ -291,14 +291,11 @@ template <int KG, bool BIAS> __global__ __launch_bounds__(ST_THREADS, 1) void fa
 }
 
 // ----------------------------------------------------------------------------------------------- dC = dy^T . z
-// body in rdb_blocks.hpp (dc_block)
+// body in rdb_blocks.hpp (dc_block_direct)
 __global__ __launch_bounds__(256, 1) void factored_dc_kernel(DcParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    if (p.ztf)
-        dc_block_direct(p, reinterpret_cast<bf16_t *>(smem_raw), blockIdx.x);
-    else
-        dc_block(p, reinterpret_cast<bf16_t *>(smem_raw), blockIdx.x);
+    dc_block_direct(p, reinterpret_cast<bf16_t *>(smem_raw), blockIdx.x);
 }
 
 // ----------------------------------------------------------------------------------------------- host side
@@ -315,7 +312,6 @@ static bf16_t *state_piece(const void *state, int64_t off) { return reinterpret_
 void dc_params_from_state(DcParams &p, const void *state, const rdb_linear_desc *d)
 {
     const ProjLayout L = proj_layout(d);
-    p.z = nullptr;
     p.ztf = state_piece(state, L.ztf_off);
     p.tsteps = (int)(L.tok64 / 16);
     p.kpad = L.kpad;
@@ -493,7 +489,7 @@ int linear_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const voi
 {
     if (!factored_shape_ok(d) || d->tokens * lddy >= (1ll << 29) || lddy % 8 || !aligned16(dy) || !aligned16(state)) return RDB_E_UNSUPPORTED;
     DcParams p;
-    const int items = make_dc_params(p, dcoef, dy, lddy, nullptr, d, num_cus);
+    const int items = make_dc_params(p, dcoef, dy, lddy, d, num_cus);
     dc_params_from_state(p, state, d);
     return launch_engine(factored_dc_kernel, p, items, engine_smem<KD_BO, KD_BM, F_BK, M_CONT, M_CONT>(), s,
                          "factored_dc_kernel");
