@@ -164,6 +164,13 @@ def test_more_tokens_than_one_launch_addresses(hip, oracle):
     assert rel_l2(cpu(dC)[osel], want_dC.cpu().numpy()) < BF16_TOL
     rest = np.setdiff1d(np.arange(out_f), osel)[:64]
     assert float(dC[torch.from_numpy(rest).cuda()].abs().max()) == 0.0   # rows whose dy is zero
+    # projection and forward product in one call per chunk: the same y, and a state that gives the same backward pass
+    del dx2, dC2
+    y1, state1 = hip.linear_project_fwd(x, C, seed)
+    assert torch.equal(y1, y)
+    del y1
+    dx1, dC1 = hip.linear_bwd_projected(dy, state1, C, in_f, seed)
+    assert torch.equal(dx1, dx) and torch.equal(dC1, dC)
 
 
 @pytest.mark.parametrize("batch", [1, 16, 256])
