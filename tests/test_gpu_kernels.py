@@ -399,6 +399,26 @@ def test_project_fwd_in_one_call(hip, T, in_f, out_f, k, seed):
     assert torch.equal(y_nb, hip.linear_fwd_projected(want_state, cg, in_f, seed))
 
 
+def test_projected_calls_take_leading_dimensions(hip):
+    """x and dy as column slices of wider matrices (row stride larger than the row): the projected calls read them in place and
+    give the bits they give on contiguous copies."""
+    print("case projected calls on strided activations", flush=True)
+    T, in_f, out_f, k, seed = 700, 264, 520, 136, 4
+    g = torch.Generator().manual_seed(8)
+    xw = torch.randn(T, in_f + 40, generator=g).bfloat16().cuda()
+    dyw = torch.randn(T, out_f + 24, generator=g).bfloat16().cuda()
+    C = (torch.randn(out_f, k, generator=g) * 0.05).bfloat16().cuda()
+    x, dy = xw[:, 16:16 + in_f], dyw[:, 8:8 + out_f]          # 16-byte aligned starts, strides in_f + 40 and out_f + 24
+    assert x.stride(0) == in_f + 40 and dy.stride(0) == out_f + 24
+    y, state = hip.linear_project_fwd(x, C, seed)
+    dx, dC = hip.linear_bwd_projected(dy, state, C, in_f, seed)
+    y_c, state_c = hip.linear_project_fwd(x.contiguous(), C, seed)
+    dx_c, dC_c = hip.linear_bwd_projected(dy.contiguous(), state_c, C, in_f, seed)
+    assert torch.equal(y, y_c) and torch.equal(dx, dx_c) and torch.equal(dC, dC_c)
+    # the separate coefficient gradient adds its token ranges with fp32 atomics: equal up to their order
+    assert rel_l2(cpu(hip.linear_bwd_dcoef_projected(dy, state, k, in_f, seed)), cpu(dC_c)) < 1e-5
+
+
 @pytest.mark.parametrize("T,in_f,out_f,k,seed", BWD_SHAPES)
 def test_linear_bwd_projected_one_call(hip, oracle, T, in_f, out_f, k, seed):
     """dx and dcoef from one call (two launches, dcoef blocks and dx blocks side by side) against the oracle and against

@@ -128,6 +128,12 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     assert L.rdb_linear_bwd_projected(None, 768, None, None, 3072, None, None, r, None, 0, None) == -1
     assert L.rdb_linear_fwd_projected(ctypes.c_void_p(16), 8, ctypes.c_void_p(16), ctypes.c_void_p(16), None, r, None) == -2  # ldy < out_f
     assert L.rdb_linear_project(None, None, 768, None, None, None) == -1
+    assert L.rdb_linear_project_fwd(None, 3072, None, None, 768, None, None, r, None) == -1                 # NULL pointers
+    p16 = ctypes.c_void_p(16)
+    assert L.rdb_linear_project_fwd(p16, 8, p16, p16, 768, p16, None, r, None) == -2                        # ldy < out_f
+    assert L.rdb_linear_project_fwd(p16, 3072, p16, p16, 8, p16, None, r, None) == -2                       # ldx < in_f
+    assert L.rdb_linear_project_fwd(p16, 3072, p16, ctypes.c_void_p(24), 768, p16, None, r, None) == -5     # x not 16-byte aligned
+    assert L.rdb_linear_project_fwd(None, 32, None, None, 100, None, None, bad, None) == -5                 # the form does not apply
 
 
 def test_view_ops_stay_lazy_and_only_change_shape_and_stride():
