@@ -268,6 +268,15 @@ int rdb_linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *d
                              const void *coef, const rdb_linear_desc *desc, void *workspace,
                              int64_t workspace_bytes, void *stream);
 
+/* Tuning switch without a counterpart in the reference.  Layers with k > 256 whose products have enough 256 x 256 output
+ * tiles to give every compute unit one run rdb_linear_fwd_projected / rdb_linear_project_fwd / rdb_linear_bwd_projected on
+ * 256-wide tiles with one persistent block per compute unit; all others on 128-wide tiles.  mode 0: never the 256-wide
+ * kernels; 1 (default): by that rule; 2: whenever k > 256 (for tests on small layers).  Both kinds contract in the same
+ * order: y and dx are the same bit for bit; dcoef is contracted over all tokens in one pass by the 256-wide kernels, where the
+ * 128-wide ones may add partial sums over token ranges (same values up to fp32 rounding).  Process-wide; returns the previous
+ * mode. */
+int rdb_set_big_tiles(int mode);
+
 #ifdef __cplusplus
 }
 #endif

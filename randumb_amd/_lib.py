@@ -44,6 +44,7 @@ EXPORTS = [
     "rdb_linear_fwd_projected",
     "rdb_linear_bwd_dcoef_projected",
     "rdb_linear_bwd_projected",
+    "rdb_set_big_tiles",
 ]
 
 
@@ -122,6 +123,8 @@ def load() -> ctypes.CDLL:
     L.rdb_linear_fwd_projected.argtypes = [vp, i64, vp, vp, vp, dp, vp]
     L.rdb_linear_bwd_dcoef_projected.argtypes = [vp, vp, i64, vp, dp, vp]
     L.rdb_linear_bwd_projected.argtypes = [vp, i64, vp, vp, i64, vp, vp, dp, vp, i64, vp]
+    L.rdb_set_big_tiles.argtypes = [ci]
+    L.rdb_set_big_tiles.restype = ci
     for name in ("rdb_sq5_fill_2d", "rdb_sq5_fill_1d", "rdb_materialize_fwd", "rdb_materialize_bwd", "rdb_scale_bias_bwd",
                  "rdb_embed_fwd", "rdb_embed_bwd", "rdb_linear_fwd", "rdb_linear_bwd_dx", "rdb_linear_bwd_dcoef",
                  "rdb_linear_project", "rdb_linear_project_fwd", "rdb_linear_fwd_projected", "rdb_linear_bwd_dcoef_projected",

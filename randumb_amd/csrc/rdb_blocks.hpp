@@ -211,6 +211,16 @@ inline int make_dc_params(DcParams &p, float *dcoef, const void *dy, int64_t ldd
     return p.tiles_o * p.tiles_m * p.splits;
 }
 
+// The same products on 256-wide tiles, one persistent block per compute unit (rdb_big.hip): whether they apply to a layer's
+// forward product / first backward launch, and the launches.  `dc`: where the coefficient gradient's sums are stored.
+bool big_fwd_applies(const rdb_linear_desc *d, int num_cus);
+bool big_bwd_applies(const rdb_linear_desc *d, int num_cus);
+int linear_fwd_big(void *y, int64_t ldy, const void *state, const void *coef, const void *bias, const rdb_linear_desc *d, int num_cus, hipStream_t s);
+int linear_bwd_big(void *t, float *dc, const void *dy, int64_t lddy, const void *state, const void *coef, const rdb_linear_desc *d, int num_cus,
+                   bool want_t, bool want_dc, hipStream_t s);
+void set_big_tiles_mode(int mode);
+int big_tiles_mode();
+
 inline int make_tn_params(TNParams &p, void *dx, int64_t lddx, const void *t, const rdb_linear_desc *d)
 {
     p.t = (const bf16_t *)t;

@@ -343,16 +343,24 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
         }
         if (tn_stationary_ok(d, lddx)) a.dyc.frag_ksteps = (int)cdiv(d->k, 64) * 4;   // the t.N kernel below keeps t in registers
         a.dc_blocks = xcd_grid_size(dc_items);
-        size_t smem = smem_dc > smem_dyc ? smem_dc : smem_dyc;
-        if (int rl = reserve_lds(reinterpret_cast<const void *>(bwd_dc_dyc_kernel), smem, "bwd_dc_dyc_kernel")) return rl;
-        bwd_dc_dyc_kernel<<<a.dc_blocks + xcd_grid_size(p1.tiles_c * p1.tiles_t), 256, smem, s>>>(a);
-        int rc = check_launch("bwd_dc_dyc_kernel");
+        int rc, red_splits = a.dc.splits;
+        if (big_bwd_applies(d, num_cus) && !a.dyc.frag_ksteps) {
+            // long coefficient dimension and many tiles: both products on 256-wide tiles; a dC tile contracts all tokens, so
+            // there is one set of sums, stored where the first split's would go
+            rc = linear_bwd_big(workspace, a.dc.partial, dy, lddy, z, coef, d, num_cus, true, true, s);
+            red_splits = 1;
+        } else {
+            size_t smem = smem_dc > smem_dyc ? smem_dc : smem_dyc;
+            if (int rl = reserve_lds(reinterpret_cast<const void *>(bwd_dc_dyc_kernel), smem, "bwd_dc_dyc_kernel")) return rl;
+            bwd_dc_dyc_kernel<<<a.dc_blocks + xcd_grid_size(p1.tiles_c * p1.tiles_t), 256, smem, s>>>(a);
+            rc = check_launch("bwd_dc_dyc_kernel");
+        }
         if (rc) return rc;
         RedParams red;
         red.partial = a.dc.partial;
         red.out = dcoef;
         red.n = d->out_f * d->k;
-        red.splits = a.dc.splits;
+        red.splits = red_splits;
         red.accumulate = accumulate ? 1 : 0;
         if (tn_stationary_ok(d, lddx)) {
             BwdBsParams bs;

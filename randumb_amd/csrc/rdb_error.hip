@@ -65,5 +65,5 @@ int check_launch(const char *what)
 
 }  // namespace rdb
 
-extern "C" int rdb_abi_version(void) { return 5; }
+extern "C" int rdb_abi_version(void) { return 6; }
 extern "C" const char *rdb_last_error_string(void) { return rdb::g_err; }

@@ -468,6 +468,7 @@ int linear_fwd_projected(void *y, int64_t ldy, const void *state, const void *co
         default: return launch_stationary(factored_ys_kernel<4, false>, q, items, smem, s, "factored_ys_kernel<4>");
         }
     }
+    if (big_fwd_applies(d, num_cus)) return linear_fwd_big(y, ldy, state, coef, bias, d, num_cus, s);
     YParams p;
     p.z = zf;
     p.coef = (const bf16_t *)coef;

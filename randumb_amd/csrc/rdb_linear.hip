@@ -317,6 +317,10 @@ int64_t linear_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus, bo
 int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias,
                        const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
 
+// rdb_big.hip
+void set_big_tiles_mode(int mode);
+int big_tiles_mode();
+
 // rdb_rbias.hip
 int linear_dx_rbias_add(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *scale_bias, const rdb_linear_desc *d, hipStream_t s);
 
@@ -787,4 +791,11 @@ extern "C" int rdb_linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, co
         if (rc) return rc;
     }
     return RDB_OK;
+}
+
+extern "C" int rdb_set_big_tiles(int mode)
+{
+    const int before = big_tiles_mode();
+    set_big_tiles_mode(mode);
+    return before;
 }

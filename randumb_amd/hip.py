@@ -424,3 +424,11 @@ def linear_bwd_projected(dy: torch.Tensor, state: torch.Tensor, coef: torch.Tens
                                         ws_bytes, _stream(dy.device))
     _lib.check(rc, "rdb_linear_bwd_projected")
     return dx, dcoef
+
+
+def set_big_tiles(mode: int) -> int:
+    """Process-wide switch of the projected entry points' kernels for k > 256: 0 = 128-wide tiles only, 1 = 256-wide tiles
+    (one persistent block per compute unit) when the layer has a tile for every other compute unit at least (default),
+    2 = 256-wide tiles whenever k > 256.  y and dx are the same bit for bit either way, dcoef up to the order of fp32 sums over
+    token ranges.  Returns the previous mode."""
+    return int(_lib.load().rdb_set_big_tiles(int(mode)))

@@ -1,0 +1,102 @@
+"""The 256-wide, persistent kernels of the projected entry points (k > 256) against the 128-wide ones and the CPU oracle.
+
+Both kinds contract in the same order (stage after stage of 64, k-step after k-step of 16, fp32 accumulators of the same matrix
+instruction), so y and dx must be equal bit for bit.  dcoef is equal bit for bit where the 128-wide kernels contract all tokens
+in one range too (few tokens, or many output tiles); where they add up partial sums over token ranges the two differ by fp32
+rounding only (1e-6 of the norm).  The oracle comparison holds the bf16 tolerance of the path (2e-2)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = 2e-2
+
+
+def rel_l2(a, b):
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+@pytest.fixture(scope="module")
+def hip():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from randumb_amd import hip as h
+
+    return h
+
+
+def _inputs(T, in_f, out_f, k, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, in_f, generator=g).bfloat16()
+    dy = torch.randn(T, out_f, generator=g).bfloat16()
+    coef = (torch.randn(out_f, k, generator=g) * (3.0 / k) ** 0.5 * 0.05).bfloat16()
+    bias = torch.randn(out_f, generator=g).bfloat16()
+    return x, dy, coef, bias
+
+
+def _run(hip, mode, x, dy, coef, bias, in_f, out_f, k, seed, with_ct):
+    before = hip.set_big_tiles(mode)
+    try:
+        z = hip.linear_project(x, k, out_f, seed, coef=coef if with_ct else None)
+        y = hip.linear_fwd_projected(z, coef, in_f, seed, bias=bias)
+        dx, dc = hip.linear_bwd_projected(dy, z, coef, in_f, seed)
+        torch.cuda.synchronize()
+    finally:
+        hip.set_big_tiles(before)
+    return y, dx, dc
+
+
+SHAPES = [
+    # tokens, in_f, out_f, k, seed
+    (300, 128, 264, 512, 2),      # one ragged tile in every direction
+    (1000, 200, 520, 328, 5),     # k = 8 mod 16 (padded to 384 in the state), three output tiles, four token tiles
+    (2088, 256, 4104, 1024, 7),   # many tiles: several rounds per block, a half-tile tail round, ragged edges
+    (128, 64, 8, 264, 1),         # a single tile, mostly padding
+]
+
+
+@pytest.mark.parametrize("T,in_f,out_f,k,seed", SHAPES)
+@pytest.mark.parametrize("with_ct", [True, False])
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_big_tiles_equal_the_128_wide_kernels(hip, T, in_f, out_f, k, seed, with_ct, with_bias):
+    print(f"case big tiles T={T} in={in_f} out={out_f} k={k} ct={with_ct} bias={with_bias}", flush=True)
+    x, dy, coef, bias = [t.cuda() for t in _inputs(T, in_f, out_f, k, seed)]
+    b = bias if with_bias else None
+    want = _run(hip, 0, x, dy, coef, b, in_f, out_f, k, seed, with_ct)
+    got = _run(hip, 2, x, dy, coef, b, in_f, out_f, k, seed, with_ct)
+    for name, a, w in zip(("y", "dx"), got, want):
+        assert a.shape == w.shape and torch.equal(a, w), f"{name} differs between the 256-wide and the 128-wide kernels"
+    if T <= 256:   # a single token range in the 128-wide kernels as well
+        assert torch.equal(got[2], want[2])
+    assert got[2].shape == want[2].shape and rel_l2(got[2].cpu().numpy(), want[2].cpu().numpy()) < 1e-6
+    # twice in a row on the same buffers: the same bits (no atomics, no state left behind by the persistent blocks)
+    again = _run(hip, 2, x, dy, coef, b, in_f, out_f, k, seed, with_ct)
+    for a, w in zip(again, got):
+        assert torch.equal(a, w)
+
+
+def test_big_tiles_against_the_oracle(hip, oracle):
+    T, in_f, out_f, k, seed = 520, 136, 528, 384, 11
+    print(f"case big tiles oracle T={T} in={in_f} out={out_f} k={k}", flush=True)
+    x, dy, coef, bias = _inputs(T, in_f, out_f, k, seed)
+    xn, dyn, cn = x.float().numpy(), dy.float().numpy(), coef.float().numpy()
+    want_y = oracle.linear_fwd(xn, cn, in_f, out_f, seed, bias=bias.float().numpy())
+    want_dx, want_dc, _ = oracle.linear_bwd(xn, dyn, cn, in_f, out_f, seed)
+    y, dx, dc = _run(hip, 2, x.cuda(), dy.cuda(), coef.cuda(), bias.cuda(), in_f, out_f, k, seed, True)
+    assert rel_l2(y.float().cpu().numpy(), want_y) < BF16_TOL
+    assert rel_l2(dx.float().cpu().numpy(), want_dx) < BF16_TOL
+    assert rel_l2(dc.float().cpu().numpy(), want_dc) < BF16_TOL
+
+
+def test_big_tiles_run_by_default_on_a_layer_with_many_tiles(hip):
+    """4096 -> 14336 with k = 1024 at 4096 tokens takes the 256-wide kernels without being asked to: same bits as with them off."""
+    T, in_f, out_f, k, seed = 4096, 4096, 14336, 1024, 0
+    print("case big tiles default", flush=True)
+    x, dy, coef, _ = [t.cuda() for t in _inputs(T, in_f, out_f, k, seed)]
+    assert hip.set_big_tiles(1) == 1   # the default mode
+    got = _run(hip, 1, x, dy, coef, None, in_f, out_f, k, seed, True)
+    want = _run(hip, 0, x, dy, coef, None, in_f, out_f, k, seed, True)
+    for a, w in zip(got, want):
+        assert torch.equal(a, w)

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_lib.SO_PATH)
     for name in declared:
         assert hasattr(lib, name), name
-    assert _lib.load().rdb_abi_version() == 5
+    assert _lib.load().rdb_abi_version() == 6
     assert ctypes.sizeof(_lib.LinearDesc) == 7 * 8 + 4 * 4
 
 
