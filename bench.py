@@ -154,6 +154,77 @@ class LayerBuffers:
             self._lib.check(rc, "a call of the step")
 
 
+def make_event_ms(torch):
+    def event_ms(fn, iters):
+        """mean duration of fn over `iters` back-to-back calls, HIP events on the launch stream"""
+        for _ in range(max(3, min(iters, 50))):
+            fn()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters
+
+    return event_ms
+
+
+def llm_layer_config(event_ms, torch, L, _lib, dev, g, vendor=True):
+    """LLM-sized layer: 4096 -> 14336, k = 1024, 4096 tokens, bf16, forward + backward through the C ABI, every buffer
+    allocated beforehand.  The headline of this entry is on the flops the kernels execute."""
+    vp = ctypes.c_void_p
+    stream = vp(torch.cuda.current_stream().cuda_stream)
+    Tl, in_f, out_f, k = 4096, 4096, 14336, 1024
+    x = torch.randn(Tl, in_f, generator=g).bfloat16().to(dev)
+    dy = torch.randn(Tl, out_f, generator=g).bfloat16().to(dev)
+    C = (torch.randn(out_f, k, generator=g) / 64.0 * (3.0 / k) ** 0.5).bfloat16().to(dev)
+    y = torch.empty(Tl, out_f, dtype=torch.bfloat16, device=dev)
+    dx = torch.empty(Tl, in_f, dtype=torch.bfloat16, device=dev)
+    dC = torch.empty(out_f, k, dtype=torch.float32, device=dev)
+    d = _lib.LinearDesc()
+    d.tokens, d.in_f, d.out_f, d.k, d.coef_rows, d.sO, d.sI, d.seed = Tl, in_f, out_f, k, out_f, in_f, 1, 0
+    d.act_dtype, d.coef_dtype, d.algo = _lib.RDB_BF16, _lib.RDB_BF16, _lib.RDB_ALGO_AUTO
+    r = ctypes.byref(d)
+    state = torch.empty(L.rdb_linear_projection_bytes(r), dtype=torch.uint8, device=dev)
+    wsb = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_PROJECTED, r)
+    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
+    px, pdy, pC, py, pdx, pdC, pst, pws = (vp(t.data_ptr()) for t in (x, dy, C, y, dx, dC, state, ws))
+
+    def llm_fwd():
+        _lib.check(L.rdb_linear_project(pst, px, in_f, pC, r, stream), "rdb_linear_project")
+        _lib.check(L.rdb_linear_fwd_projected(py, out_f, pst, pC, None, r, stream), "rdb_linear_fwd_projected")
+
+    def llm_bwd():
+        _lib.check(L.rdb_linear_bwd_projected(pdx, in_f, pdC, pdy, out_f, pst, pC, r, pws, wsb, stream), "rdb_linear_bwd_projected")
+
+    # 50 warm-up and 50 timed calls each (about 25 ms of continuous work per figure: the clocks have settled)
+    fwd_ms, bwd_ms = event_ms(llm_fwd, 50), event_ms(llm_bwd, 50)
+    proj_ms = event_ms(lambda: L.rdb_linear_project(pst, px, in_f, pC, r, stream), 50)
+    ms = fwd_ms + bwd_ms
+    F = 6.0 * Tl * in_f * out_f + 6.0 * out_f * in_f * k
+    executed = 4.0 * Tl * k * (in_f + out_f) + 2.0 * Tl * k * out_f
+    res = {
+        "fwd_ms": round(fwd_ms, 4), "bwd_ms": round(bwd_ms, 4), "fwd_bwd_ms": round(ms, 4),
+        "calls_ms": {"rdb_linear_project": round(proj_ms, 4), "rdb_linear_fwd_projected": round(fwd_ms - proj_ms, 4),
+                     "rdb_linear_bwd_projected": round(bwd_ms, 4)},
+        "kernels": "forward product and first backward launch on 256-wide tiles, one persistent block per compute unit",
+        "executed_TFLOPs": round(executed / ms / 1e9, 1), "executed_frac_of_mfma_peak": round(executed / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
+        "prescribed_gflop": round(F / 1e9, 1), "executed_gflop": round(executed / 1e9, 1),
+        "prescribed_TFLOPs_equivalent": round(F / ms / 1e9, 1),
+        "note": "all buffers preallocated; the factored form executes 4.1x fewer flops than the prescribed algorithm at this shape, "
+                "so only the executed figure is a utilisation"}
+    if vendor:
+        zz = torch.randn(Tl, k, device=dev).bfloat16()
+        res["vendor_gemm_on_the_factored_shapes_ms"] = {
+            "y = z.C^T": round(event_ms(lambda: torch.matmul(zz, C.t(), out=y), 50), 4),
+            "t = dy.C": round(event_ms(lambda: torch.matmul(dy, C, out=zz), 50), 4),
+            "dC = dy^T.z": round(event_ms(lambda: torch.matmul(dy.t(), zz), 50), 4)}
+    return res
+
+
 def other_configs(event_ms, torch, L, _lib, dev):
     """The other configurations, timed for the record (they are parity-test cases, not the metric)."""
     from randumb_amd import hip
@@ -186,48 +257,7 @@ def other_configs(event_ms, torch, L, _lib, dev):
                                "actual_HBM_GBps": round(actual / ms / 1e6, 2)}
     out["in4096_out4096_k16_fp32_matrix_coef"] = small
 
-    # ---- LLM-sized layer: 4096 -> 14336, k = 1024, 4096 tokens, bf16, forward + backward through the C ABI, every buffer
-    # allocated beforehand.  The headline of this entry is on the flops the kernels execute.
-    Tl, in_f, out_f, k = 4096, 4096, 14336, 1024
-    x = torch.randn(Tl, in_f, generator=g).bfloat16().to(dev)
-    dy = torch.randn(Tl, out_f, generator=g).bfloat16().to(dev)
-    C = (torch.randn(out_f, k, generator=g) / 64.0 * (3.0 / k) ** 0.5).bfloat16().to(dev)
-    y = torch.empty(Tl, out_f, dtype=torch.bfloat16, device=dev)
-    dx = torch.empty(Tl, in_f, dtype=torch.bfloat16, device=dev)
-    dC = torch.empty(out_f, k, dtype=torch.float32, device=dev)
-    d = _lib.LinearDesc()
-    d.tokens, d.in_f, d.out_f, d.k, d.coef_rows, d.sO, d.sI, d.seed = Tl, in_f, out_f, k, out_f, in_f, 1, 0
-    d.act_dtype, d.coef_dtype, d.algo = _lib.RDB_BF16, _lib.RDB_BF16, _lib.RDB_ALGO_AUTO
-    r = ctypes.byref(d)
-    state = torch.empty(L.rdb_linear_projection_bytes(r), dtype=torch.uint8, device=dev)
-    wsb = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_PROJECTED, r)
-    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
-    px, pdy, pC, py, pdx, pdC, pst, pws = (vp(t.data_ptr()) for t in (x, dy, C, y, dx, dC, state, ws))
-
-    def llm_fwd():
-        _lib.check(L.rdb_linear_project(pst, px, in_f, pC, r, stream), "rdb_linear_project")
-        _lib.check(L.rdb_linear_fwd_projected(py, out_f, pst, pC, None, r, stream), "rdb_linear_fwd_projected")
-
-    def llm_bwd():
-        _lib.check(L.rdb_linear_bwd_projected(pdx, in_f, pdC, pdy, out_f, pst, pC, r, pws, wsb, stream), "rdb_linear_bwd_projected")
-
-    fwd_ms, bwd_ms = event_ms(llm_fwd, 10), event_ms(llm_bwd, 10)
-    ms = fwd_ms + bwd_ms
-    F = 6.0 * Tl * in_f * out_f + 6.0 * out_f * in_f * k
-    executed = 4.0 * Tl * k * (in_f + out_f) + 2.0 * Tl * k * out_f
-    zz = torch.randn(Tl, k, device=dev).bfloat16()
-    vendor = {"y = z.C^T": round(event_ms(lambda: torch.matmul(zz, C.t(), out=y), 10), 4),
-              "t = dy.C": round(event_ms(lambda: torch.matmul(dy, C, out=zz), 10), 4),
-              "dC = dy^T.z": round(event_ms(lambda: torch.matmul(dy.t(), zz), 10), 4)}
-    out["in4096_out14336_k1024_T4096_bf16"] = {
-        "fwd_ms": round(fwd_ms, 4), "bwd_ms": round(bwd_ms, 4), "fwd_bwd_ms": round(ms, 4),
-        "executed_TFLOPs": round(executed / ms / 1e9, 1), "executed_frac_of_mfma_peak": round(executed / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
-        "prescribed_gflop": round(F / 1e9, 1), "executed_gflop": round(executed / 1e9, 1),
-        "prescribed_TFLOPs_equivalent": round(F / ms / 1e9, 1),
-        "vendor_gemm_on_the_factored_shapes_ms": vendor,
-        "note": "all buffers preallocated; the factored form executes 4.1x fewer flops than the prescribed algorithm at this shape, "
-                "so only the executed figure is a utilisation"}
-    del x, dy, C, y, dx, dC, state, ws, zz
+    out["in4096_out14336_k1024_T4096_bf16"] = llm_layer_config(event_ms, torch, L, _lib, dev, g)
 
     # ---- the reference's own (vector-coef, 1-D) form at the headline shape: W = Noise . c with ONE coefficient vector of length
     # k needs k hashes per weight element (604 M per regeneration here): the PRNG-bound regime.  Its data flow is the
@@ -299,6 +329,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="time eager calls only (profiling runs: one kernel record per launch)")
     ap.add_argument("--vector-coef-only", action="store_true",
                     help="run only the vector-coef (reference form) materialise kernels a few times and exit (counter runs)")
+    ap.add_argument("--llm-layer-only", action="store_true",
+                    help="run only the 4096 -> 14336, k = 1024 layer (projection, forward, backward through the C ABI) and exit "
+                         "(profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch plain device copies of 256 MiB (a known 256 MiB read + 256 MiB written per launch) so that "
                          "hardware byte counters collected over this run can be scaled")
@@ -326,12 +359,6 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"ran": "vector-coef materialize_fwd / materialize_bwd, 768x3072, k=256, 5 times each"}))
         return
-    main_set = LayerBuffers(L, _lib, torch, dev, g)
-    sets = [main_set] + [LayerBuffers(L, _lib, torch, dev, g, share_inputs_of=main_set) for _ in range(2)]
-    set_mb = sum(t.numel() * t.element_size() for t in (main_set.x, main_set.dy, main_set.y, main_set.dx, main_set.dC, main_set.ws,
-                                                       main_set.state, main_set.C)) / 1e6
-    step = main_set.step
-
     if args.copy_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
         dst = torch.empty_like(src)
@@ -339,6 +366,14 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.llm_layer_only:
+        print(json.dumps({"in4096_out14336_k1024_T4096_bf16": llm_layer_config(make_event_ms(torch), torch, L, _lib, dev, g, vendor=False)}))
+        return
+    main_set = LayerBuffers(L, _lib, torch, dev, g)
+    sets = [main_set] + [LayerBuffers(L, _lib, torch, dev, g, share_inputs_of=main_set) for _ in range(2)]
+    set_mb = sum(t.numel() * t.element_size() for t in (main_set.x, main_set.dy, main_set.y, main_set.dx, main_set.dC, main_set.ws,
+                                                       main_set.state, main_set.C)) / 1e6
+    step = main_set.step
 
     # ---- the timed region of the contract: W warm-up steps, then exactly K steps between two synchronisations.
     # A step is five short kernel launches; issued one by one from Python the host needs longer per step than the GPU, so
@@ -392,19 +427,7 @@ def main():
     torch.cuda.synchronize()
     ms_rotating = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    def event_ms(fn, iters):
-        """mean duration of fn over `iters` back-to-back calls, HIP events on the launch stream"""
-        for _ in range(max(3, min(iters, 50))):
-            fn()
-        torch.cuda.synchronize()
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(iters):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / iters
+    event_ms = make_event_ms(torch)
 
     ms_events_all = event_ms(step, args.steps)
     # spread of single steps, each between its own pair of events (as triton's do_bench reports: median, 20th, 80th percentile)

@@ -16,6 +16,18 @@ namespace rdb {
 
 constexpr int BG = 256;   // tile edge
 
+// Work item w of the forward product -> (output tile, token tile).  Neighbouring items run at the same time on one die: they
+// are numbered so that 32 of them cover 8 output tiles x 4 token tiles (6 MB of operands, which a die's L2 holds) rather
+// than 32 x 1 (16.5 MB): groups of 4 token tiles, walked through output tile by output tile.
+constexpr int BY_GROUP_T = 4;
+__device__ __forceinline__ void big_y_decode(int w, int tiles_o, int tiles_t, int &to, int &tt)
+{
+    const int per_group = BY_GROUP_T * tiles_o, group = w / per_group, in_group = w - group * per_group;
+    const int first_t = group * BY_GROUP_T, gsize = tiles_t - first_t < BY_GROUP_T ? tiles_t - first_t : BY_GROUP_T;
+    to = in_group / gsize;
+    tt = first_t + in_group - to * gsize;
+}
+
 // 0: never use these kernels, 1: when the layer has enough tiles (default), 2: whenever the shapes allow (tests)
 static std::atomic<int> g_big_mode{1};
 void set_big_tiles_mode(int mode) { g_big_mode.store(mode < 0 ? 0 : mode > 2 ? 2 : mode); }
@@ -66,23 +78,27 @@ template <bool BIAS> __global__ __launch_bounds__(256, 1) void big_y_kernel(BigY
         return -1;
     };
     PA pa;
-    auto init_a = [&](int w) { pa = PA{p.coef, (int64_t)p.k, (w % p.tiles_o) * BG, p.out_f, p.k, (int64_t)p.out_f * p.k}; };
+    auto init_a = [&](int to) { pa = PA{p.coef, (int64_t)p.k, to * BG, p.out_f, p.k, (int64_t)p.out_f * p.k}; };
     int w = next();
     if (w >= 0) {
         PB pb;
         BigRegs<PA, PB> regs;
         auto request = [&](int w) {
-            init_a(w);
+            int to, tt;
+            big_y_decode(w, p.tiles_o, p.tiles_t, to, tt);
+            init_a(to);
             pb.src = p.zf;
             pb.ksteps = p.kpad >> 4;
             pb.nrb = p.tok32 >> 5;
-            pb.rb0 = (w / p.tiles_o) * (BG / 32);
+            pb.rb0 = tt * (BG / 32);
             pb.klim_steps = p.kpad >> 4;
             big_prefetch(regs, pa, pb, 0);
         };
         request(w);
         while (true) {
-            const int o0 = (w % p.tiles_o) * BG, tok0 = (w / p.tiles_o) * BG;
+            int to, tt;
+            big_y_decode(w, p.tiles_o, p.tiles_t, to, tt);
+            const int o0 = to * BG, tok0 = tt * BG;
             f32x16 acc[BG / 64][BG / 64];
             RDB_STAMP(0);
             big_zero<BG, BG>(acc);
@@ -107,10 +123,12 @@ template <bool BIAS> __global__ __launch_bounds__(256, 1) void big_y_kernel(BigY
     w = xcd_work_item(full_rounds * nblk + ((int)blockIdx.x >> 1), total);
     if (w >= total) return;
     {
-        const int o0 = (w % p.tiles_o) * BG, tok0 = (w / p.tiles_o) * BG + ((int)blockIdx.x & 1) * BY_HALF;
+        int to, tt;
+        big_y_decode(w, p.tiles_o, p.tiles_t, to, tt);
+        const int o0 = to * BG, tok0 = tt * BG + ((int)blockIdx.x & 1) * BY_HALF;
         PH pb;
         BigRegs<PA, PH> regs;
-        init_a(w);
+        init_a(to);
         pb.src = p.zf;
         pb.ksteps = p.kpad >> 4;
         pb.nrb = p.tok32 >> 5;
