@@ -327,20 +327,23 @@ int linear_fwd_big(void *y, int64_t ldy, const void *state, const void *coef, co
 }
 
 // First launch of the backward pass: t (row-major, for the t . N kernel of the tile engine) and dC.  `dc`: where the
-// coefficient gradient's sums go (dcoef, or the area a reduction adds to dcoef).  want_t / want_dc: which of the two.
+// coefficient gradient's sums go (dcoef, or the area a reduction adds to dcoef).  want_t / want_dc: which of the two
+// (t alone needs no state, dC alone no coefficients).
 int linear_bwd_big(void *t, float *dc, const void *dy, int64_t lddy, const void *state, const void *coef, const rdb_linear_desc *d, int num_cus,
                    bool want_t, bool want_dc, hipStream_t s)
 {
     const ProjLayout L = proj_layout(d);
-    if (!L.ok || d->coef_dtype != RDB_BF16 || d->tokens * lddy >= (1ll << 29) || lddy % 8) return RDB_E_UNSUPPORTED;
+    if (!L.ok || d->tokens * lddy >= (1ll << 29) || lddy % 8) return RDB_E_UNSUPPORTED;
+    if ((want_t && (d->coef_dtype != RDB_BF16 || !coef || !t)) || (want_dc && (!state || !dc))) return RDB_E_UNSUPPORTED;
     if (!big_aligned16(dy) || !big_aligned16(state) || !big_aligned16(coef) || !big_aligned16(t) || !big_aligned16(dc)) return RDB_E_UNSUPPORTED;
     BigBwdParams p;
     p.dy = (const bf16_t *)dy;
     p.lddy = lddy;
     p.coef = (const bf16_t *)coef;
-    p.ctf = reinterpret_cast<const bf16_t *>(static_cast<const char *>(state) + L.ctf_off);
+    // without a state (the input gradient called on its own) C is staged from its row-major form
+    p.ctf = state ? reinterpret_cast<const bf16_t *>(static_cast<const char *>(state) + L.ctf_off) : nullptr;
     p.ctf_flag = static_cast<const uint32_t *>(state);
-    p.ztf = reinterpret_cast<const bf16_t *>(static_cast<const char *>(state) + L.ztf_off);
+    p.ztf = state ? reinterpret_cast<const bf16_t *>(static_cast<const char *>(state) + L.ztf_off) : nullptr;
     p.t = (bf16_t *)t;
     p.dc = dc;
     p.tokens = (int)d->tokens;

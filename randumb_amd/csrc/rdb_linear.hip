@@ -320,6 +320,9 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
 // rdb_big.hip
 void set_big_tiles_mode(int mode);
 int big_tiles_mode();
+bool big_bwd_applies(const rdb_linear_desc *d, int num_cus);
+int linear_bwd_big(void *t, float *dc, const void *dy, int64_t lddy, const void *state, const void *coef, const rdb_linear_desc *d, int num_cus,
+                   bool want_t, bool want_dc, hipStream_t s);
 
 // rdb_rbias.hip
 int linear_dx_rbias_add(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *scale_bias, const rdb_linear_desc *d, hipStream_t s);
@@ -746,6 +749,11 @@ extern "C" int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int6
         return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dcoef_projected: dy and z must be 16-byte aligned, lddy a multiple of 8 and below "
                                             "twice out_f");
     hipStream_t s = (hipStream_t)stream;
+    if (pl.nchunks == 1 && big_bwd_applies(d, num_compute_units())) {
+        // many 256 x 256 tiles of dcoef: each contracts all tokens and is stored once, nothing to clear or add
+        rc = linear_bwd_big(nullptr, dcoef, dy, lddy, z, nullptr, d, num_compute_units(), false, true, s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
     rc = fill_zero(dcoef, d->coef_rows * d->k, s);
     if (rc) return rc;
     for (int c = 0; c < pl.nchunks; ++c) {   // every chunk adds its share with atomics

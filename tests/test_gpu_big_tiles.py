@@ -42,9 +42,14 @@ def _run(hip, mode, x, dy, coef, bias, in_f, out_f, k, seed, with_ct):
         z = hip.linear_project(x, k, out_f, seed, coef=coef if with_ct else None)
         y = hip.linear_fwd_projected(z, coef, in_f, seed, bias=bias)
         dx, dc = hip.linear_bwd_projected(dy, z, coef, in_f, seed)
+        dc_alone = hip.linear_bwd_dcoef_projected(dy, z, k, in_f, seed)   # the coefficient gradient's own entry point
         torch.cuda.synchronize()
     finally:
         hip.set_big_tiles(before)
+    # one pass over all tokens on the 256-wide tiles, fp32 atomics over token ranges on the 128-wide ones
+    assert rel_l2(dc_alone.cpu().numpy(), dc.cpu().numpy()) < 1e-6
+    if mode == 2:
+        assert torch.equal(dc_alone, dc)
     return y, dx, dc
 
 
