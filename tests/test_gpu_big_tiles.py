@@ -105,3 +105,70 @@ def test_big_tiles_run_by_default_on_a_layer_with_many_tiles(hip):
     want = _run(hip, 0, x, dy, coef, None, in_f, out_f, k, seed, True)
     for a, w in zip(got, want):
         assert torch.equal(a, w)
+
+
+def test_big_tiles_random_shapes(hip):
+    """Sixteen random layers with k > 256 (sizes in multiples of 8, tokens any number, ragged against every tile edge), with
+    the transposed coefficients in the state or not, with the ordered-sum workspace or the smaller one."""
+    rng = np.random.default_rng(31)
+    for case in range(16):
+        T = int(rng.integers(1, 160)) * 8 - int(rng.integers(0, 8))
+        in_f, out_f = (int(rng.integers(1, 100)) * 8 for _ in range(2))
+        k = int(rng.integers(33, 130)) * 8                      # 264 .. 1032
+        seed = int(rng.integers(0, 2**32))
+        print(f"case big tiles random {case}: T={T} in={in_f} out={out_f} k={k} seed={seed}", flush=True)
+        x, dy, coef, bias = [t.cuda() for t in _inputs(T, in_f, out_f, k, case)]
+        b = bias if case % 2 else None
+        outs = {}
+        for mode in (0, 2):
+            before = hip.set_big_tiles(mode)
+            try:
+                z = hip.linear_project(x, k, out_f, seed, coef=coef if case % 3 else None)
+                y = hip.linear_fwd_projected(z, coef, in_f, seed, bias=b)
+                dx, dc = hip.linear_bwd_projected(dy, z, coef, in_f, seed, ordered_sums=case % 4 != 0)
+                torch.cuda.synchronize()
+            finally:
+                hip.set_big_tiles(before)
+            outs[mode] = (y, dx, dc)
+        assert torch.equal(outs[2][0], outs[0][0]) and torch.equal(outs[2][1], outs[0][1]), case
+        assert rel_l2(outs[2][2].cpu().numpy(), outs[0][2].cpu().numpy()) < 1e-5, case   # atomics / token ranges in the 128-wide kernels
+
+
+def test_big_tiles_take_leading_dimensions(hip):
+    """dy as a column slice of a wider matrix and y, dx written into wider matrices: same bits as on contiguous buffers."""
+    import ctypes
+
+    from randumb_amd import _lib
+    from randumb_amd.hip import RDB_OP_LINEAR_BWD_PROJECTED, _p, _proj_desc, _stream
+
+    print("case big tiles on strided activations", flush=True)
+    T, in_f, out_f, k, seed = 700, 264, 520, 520, 4
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(T, in_f, generator=g).bfloat16().cuda()
+    dyw = torch.randn(T, out_f + 24, generator=g).bfloat16().cuda()
+    C = (torch.randn(out_f, k, generator=g) * 0.05).bfloat16().cuda()
+    dy = dyw[:, 8:8 + out_f]
+    L = _lib.load()
+    before = hip.set_big_tiles(2)
+    try:
+        z = hip.linear_project(x, k, out_f, seed, coef=C)
+        y_c = hip.linear_fwd_projected(z, C, in_f, seed)
+        dx_c, dC_c = hip.linear_bwd_projected(dy.contiguous(), z, C, in_f, seed)
+        d = _proj_desc(T, in_f, out_f, k, seed)
+        yw = torch.full((T, out_f + 40), 7.0, dtype=torch.bfloat16, device="cuda")
+        dxw = torch.full((T, in_f + 16), 7.0, dtype=torch.bfloat16, device="cuda")
+        dC = torch.empty(out_f, k, dtype=torch.float32, device="cuda")
+        y, dx = yw[:, 16:16 + out_f], dxw[:, 8:8 + in_f]
+        n = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_PROJECTED, ctypes.byref(d))
+        ws = torch.empty(max(n, 16), dtype=torch.uint8, device="cuda")
+        st = _stream(x.device)
+        _lib.check(L.rdb_linear_fwd_projected(_p(y), y.stride(0), _p(z), _p(C), None, ctypes.byref(d), st), "rdb_linear_fwd_projected")
+        _lib.check(L.rdb_linear_bwd_projected(_p(dx), dx.stride(0), _p(dC), _p(dy), dy.stride(0), _p(z), _p(C), ctypes.byref(d), _p(ws), n, st),
+                   "rdb_linear_bwd_projected")
+        torch.cuda.synchronize()
+    finally:
+        hip.set_big_tiles(before)
+    assert torch.equal(y, y_c) and torch.equal(dx, dx_c) and torch.equal(dC, dC_c)
+    # nothing outside the slices was written
+    assert bool((yw[:, :16] == 7).all()) and bool((yw[:, 16 + out_f:] == 7).all())
+    assert bool((dxw[:, :8] == 7).all()) and bool((dxw[:, 8 + in_f:] == 7).all())
