@@ -164,18 +164,20 @@ struct BigBwdParams {
     int osteps, tsteps;           // k-steps per row block of ctf (out_f rounded up to 64, / 16) and of ztf (tokens likewise)
     int t_tiles_m, t_tiles_t;     // t tiles: 256 coefficients x 128 tokens; 0 tiles: the launch computes dC only
     int c_tiles_o, c_tiles_m;     // dC tiles: 256 output features x 256 coefficients; 0 tiles: t only
+    int t_first;                  // the t tiles come first in the list (they are the longer ones), else the dC tiles
 };
 
 // t tiles of one block.  CT: C^T from its fragment-ordered copy; otherwise C itself, staged as an M_CONT operand.
-template <bool CT> __device__ __forceinline__ void big_t_items(const BigBwdParams &p, bf16_t *lds, int &r, int n1, int n1v)
+template <bool CT> __device__ __forceinline__ void big_t_items(const BigBwdParams &p, bf16_t *lds, int &r, int base, int n1)
 {
+    const int n1v = (n1 + 7) / 8 * 8;
     typedef typename std::conditional<CT, FragOperand<BG, 64>, GlobalOperand<BG, 64, M_CONT>>::type PA;   // rows = coefficients
     typedef GlobalOperand<BT_TOK, 64, K_CONT> PB;                                                          // dy: rows = tokens
     const int nblk = gridDim.x, nstage = (p.out_f + 63) / 64;
     auto next = [&]() {
         for (;; ++r) {
-            const int v = big_item(blockIdx.x, r, nblk);
-            if (v >= n1v) return -1;   // r stays at the first round that is not a t tile
+            const int v = big_item(blockIdx.x, r, nblk) - base;
+            if (v >= n1v) return -1;   // r stays at the first round past the t tiles
             const int w = xcd_work_item(v, n1);
             if (w < n1) { ++r; return w; }
         }
@@ -214,17 +216,16 @@ template <bool CT> __device__ __forceinline__ void big_t_items(const BigBwdParam
     }
 }
 
-// dC tiles of one block; r: the block's first round that is not a t tile.
-__device__ __forceinline__ void big_dc_items(const BigBwdParams &p, bf16_t *lds, int r, int n1v, int n2)
+// dC tiles of one block, from the block's round r on; `base`: index of the first dC tile in the launch's list.
+__device__ __forceinline__ void big_dc_items(const BigBwdParams &p, bf16_t *lds, int &r, int base, int n2)
 {
     typedef GlobalOperand<BG, 64, M_CONT> PA;   // dy: rows = output features, contraction = tokens
     typedef FragOperand<BG, 64> PB;             // z^T: rows = coefficients
     const int nblk = gridDim.x, nstage = (p.tokens + 63) / 64, n2v = (n2 + 7) / 8 * 8;
     auto next = [&]() {
         for (;; ++r) {
-            const int v = big_item(blockIdx.x, r, nblk) - n1v;
+            const int v = big_item(blockIdx.x, r, nblk) - base;
             if (v >= n2v) return -1;
-            if (v < 0) continue;   // a t tile of another block's round (the rows alternate direction)
             const int w = xcd_work_item(v, n2);
             if (w < n2) { ++r; return w; }
         }
@@ -258,19 +259,30 @@ __device__ __forceinline__ void big_dc_items(const BigBwdParams &p, bf16_t *lds,
     }
 }
 
-// The t tiles (the longer ones when out_f > tokens / 2 ... whichever: the list is t tiles first, dC tiles after them) are dealt
-// out to the blocks in rows of alternating direction (big_item), so the blocks with a t tile get fewer dC tiles.
+// The launch's list holds the tiles of the longer kind first (a t tile contracts out_f with half-size stages, a dC tile the
+// tokens) and is dealt out to the blocks in rows of alternating direction (big_item): the blocks that got a long tile in
+// one row get the later, shorter ones of the next.  A block's rounds walk through the list in order, so it finishes its
+// tiles of the first kind before it starts on the second.
 __global__ __launch_bounds__(256, 1) void big_bwd_kernel(BigBwdParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
-    const int n1 = p.t_tiles_m * p.t_tiles_t, n1v = (n1 + 7) / 8 * 8, n2 = p.c_tiles_o * p.c_tiles_m;
+    const int n1 = p.t_tiles_m * p.t_tiles_t, n1v = (n1 + 7) / 8 * 8, n2 = p.c_tiles_o * p.c_tiles_m, n2v = (n2 + 7) / 8 * 8;
+    const bool ct = n1 && p.ctf && *p.ctf_flag;
     int r = 0;
-    if (n1) {
-        if (p.ctf && *p.ctf_flag) big_t_items<true>(p, lds, r, n1, n1v);
-        else big_t_items<false>(p, lds, r, n1, n1v);
+    if (p.t_first) {
+        if (n1) {
+            if (ct) big_t_items<true>(p, lds, r, 0, n1);
+            else big_t_items<false>(p, lds, r, 0, n1);
+        }
+        if (n2) big_dc_items(p, lds, r, n1v, n2);
+    } else {
+        if (n2) big_dc_items(p, lds, r, 0, n2);
+        if (n1) {
+            if (ct) big_t_items<true>(p, lds, r, n2v, n1);
+            else big_t_items<false>(p, lds, r, n2v, n1);
+        }
     }
-    if (n2) big_dc_items(p, lds, r, n1v, n2);
 }
 
 // ----------------------------------------------------------------------------------------------- host side
@@ -360,7 +372,8 @@ int linear_bwd_big(void *t, float *dc, const void *dy, int64_t lddy, const void 
     typedef FragTile<BG, 64> TF;
     typedef OperandTile<BT_TOK, 64, K_CONT> TD;
     constexpr size_t smem_dc = big_smem<BG, BG, TM, TF>(), smem_t = big_smem<BG, BT_TOK, TM, TD>();
-    const int items = (p.t_tiles_m * p.t_tiles_t + 7) / 8 * 8 + p.c_tiles_o * p.c_tiles_m;
+    p.t_first = d->out_f >= 2 * d->tokens;   // stages of 64 at half the matrix work against stages of 64 over the tokens
+    const int items = (p.t_tiles_m * p.t_tiles_t + 7) / 8 * 8 + (p.c_tiles_o * p.c_tiles_m + 7) / 8 * 8;
     return launch_big(big_bwd_kernel, p, items, num_cus, smem_dc > smem_t ? smem_dc : smem_t, s, "big_bwd_kernel");
 }
 
