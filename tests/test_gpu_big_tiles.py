@@ -172,3 +172,32 @@ def test_big_tiles_take_leading_dimensions(hip):
     # nothing outside the slices was written
     assert bool((yw[:, :16] == 7).all()) and bool((yw[:, 16 + out_f:] == 7).all())
     assert bool((dxw[:, :8] == 7).all()) and bool((dxw[:, 8 + in_f:] == 7).all())
+
+
+def test_big_tiles_through_the_layer(hip):
+    """SillyLinear in matrix-coef form with k = 512: forward, backward and the gradients of input and coefficients are the
+    same with the 256-wide kernels as with the 128-wide ones (autograd function, custom ops and C ABI in between)."""
+    import randumb_amd as rten
+
+    print("case big tiles through SillyLinear", flush=True)
+    torch.manual_seed(3)
+    outs = {}
+    for mode in (0, 2):
+        before = hip.set_big_tiles(mode)
+        try:
+            assert hip.linear_projection_preferred(300, 1032, 2056, 512)   # the projected kernels are what the layer runs
+            layer = rten.SillyLinear(1032, 2056, [512, 512], [9, 10], bias=False, matrix_coef=True).to(torch.bfloat16).cuda()
+            with torch.no_grad():
+                g = torch.Generator().manual_seed(5)
+                layer.weight_coef.copy_((torch.randn(2056, 512, generator=g) * 0.02).bfloat16())
+                layer.weight_scale_bias.zero_()
+            x = torch.randn(300, 1032, generator=torch.Generator().manual_seed(6)).bfloat16().cuda().requires_grad_(True)
+            y = layer(x)
+            (y.float() ** 2).sum().backward()
+            torch.cuda.synchronize()
+            outs[mode] = (y.detach(), x.grad.detach(), layer.weight_coef.grad.detach())
+        finally:
+            hip.set_big_tiles(before)
+    assert torch.equal(outs[2][0], outs[0][0]) and torch.equal(outs[2][1], outs[0][1])
+    assert rel_l2(outs[2][2].float().cpu().numpy(), outs[0][2].float().cpu().numpy()) < 1e-2   # bf16 gradients of fp32 sums in two orders
+    assert float(outs[2][2].float().abs().sum()) > 0
