@@ -29,6 +29,20 @@ def test_library_exports_every_declared_symbol():
     assert ctypes.sizeof(_lib.LinearDesc) == 7 * 8 + 4 * 4
 
 
+def test_big_tiles_switch_without_a_gpu():
+    """rdb_set_big_tiles returns the previous mode, clamps to 0..2 and starts at 1 (the 256-wide kernels by the tile-count rule)."""
+    from randumb_amd import _lib
+
+    L = _lib.load()
+    first = L.rdb_set_big_tiles(0)
+    try:
+        assert first == 1
+        assert L.rdb_set_big_tiles(7) == 0 and L.rdb_set_big_tiles(-3) == 2 and L.rdb_set_big_tiles(2) == 0
+    finally:
+        L.rdb_set_big_tiles(first)
+    assert L.rdb_set_big_tiles(first) == first
+
+
 def test_argument_errors_come_back_as_codes_without_a_gpu():
     from randumb_amd import _lib
 
