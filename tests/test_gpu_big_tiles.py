@@ -201,3 +201,33 @@ def test_big_tiles_through_the_layer(hip):
     assert torch.equal(outs[2][0], outs[0][0]) and torch.equal(outs[2][1], outs[0][1])
     assert rel_l2(outs[2][2].float().cpu().numpy(), outs[0][2].float().cpu().numpy()) < 1e-2   # bf16 gradients of fp32 sums in two orders
     assert float(outs[2][2].float().abs().sum()) > 0
+
+
+def test_big_tiles_on_chunked_tokens(hip):
+    """40000 tokens x 14336 output features hold more elements than one launch addresses: the projected calls run the layer
+    in chunks of tokens, the later chunks adding to dcoef.  Same y and dx bit for bit on both kinds of kernels, same dcoef up to
+    the order of fp32 sums, and the same dcoef bit for bit on a second run."""
+    T, in_f, out_f, k, seed = 40000, 256, 14336, 512, 3
+    print(f"case big tiles chunked T={T} in={in_f} out={out_f} k={k}", flush=True)
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(T, in_f, generator=g).bfloat16().cuda()
+    dy = (torch.randn(T, 64, generator=g).bfloat16().cuda()).repeat(1, out_f // 64)   # cheap to make, still different per column block
+    dy = dy * torch.linspace(0.5, 1.5, out_f, device="cuda").bfloat16()
+    coef = (torch.randn(out_f, k, generator=g) * 0.01).bfloat16().cuda()
+    outs = {}
+    for mode in (0, 2, 2):
+        before = hip.set_big_tiles(mode)
+        try:
+            z = hip.linear_project(x, k, out_f, seed, coef=coef)
+            y = hip.linear_fwd_projected(z, coef, in_f, seed)
+            dx, dc = hip.linear_bwd_projected(dy, z, coef, in_f, seed)
+            torch.cuda.synchronize()
+        finally:
+            hip.set_big_tiles(before)
+        if mode in outs:   # second run on the 256-wide kernels
+            assert torch.equal(outs[mode][2], dc) and torch.equal(outs[mode][0], y)
+        outs[mode] = (y, dx, dc)
+        del z
+    assert torch.equal(outs[2][0], outs[0][0]) and torch.equal(outs[2][1], outs[0][1])
+    assert rel_l2(outs[2][2].cpu().numpy(), outs[0][2].cpu().numpy()) < 1e-5
+    assert float(outs[2][2].abs().sum()) > 0
