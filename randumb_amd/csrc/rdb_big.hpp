@@ -101,7 +101,7 @@ template <class PA, class PB> __device__ __forceinline__ void big_prefetch(BigRe
 }
 
 // One stage of 4 k-steps, entered right after the barrier that completed LDS buffer `cur`.  The last k-step of a stage is not
-// multiplied inside its own stage: its fragments (pa_f[1], pb_f[1] on entry) wait in registers across the barrier and their
+// multiplied inside its own stage: its fragments (fa[1], fb[1] on entry) wait in registers across the barrier and their
 // MFMAs run here first, while this stage's first fragments come in from LDS.  With one wave per SIMD nothing else would cover
 // that wait.  Between the MFMAs, as in pipeline_stage: the registers ra / rb (a later stage) go to the idle buffer `oth` and
 // are refilled with stages next_a / next_b.
