@@ -110,7 +110,7 @@ template <bool BIAS> __global__ __launch_bounds__(256, 1) void big_y_kernel(BigY
             if (wn >= 0) request(wn);   // on its way while this tile leaves
             __builtin_amdgcn_sched_barrier(0);
             RDB_STAMP(2);
-            big_store_bf16<BG, BG, BIAS>(acc, lds, p.y, p.ldy, p.y_elems, o0, p.out_f, tok0, p.tokens, bias, opaque_tid());
+            big_store_bf16<BG, BG, BIAS, true>(acc, lds, p.y, p.ldy, p.y_elems, o0, p.out_f, tok0, p.tokens, bias, opaque_tid());
             RDB_STAMP(3);
 #ifdef RDB_STAMPS
             ++rdb_stamp_seq;
@@ -143,7 +143,7 @@ template <bool BIAS> __global__ __launch_bounds__(256, 1) void big_y_kernel(BigY
         BigBias<BG> bias;
         if (BIAS) big_load_bias<BG>(bias, p.bias, o0, p.out_f);
         RDB_STAMP(2);
-        big_store_bf16<BG, BY_HALF, BIAS>(acc, lds, p.y, p.ldy, p.y_elems, o0, p.out_f, tok0, p.tokens, bias, opaque_tid());
+        big_store_bf16<BG, BY_HALF, BIAS, true>(acc, lds, p.y, p.ldy, p.y_elems, o0, p.out_f, tok0, p.tokens, bias, opaque_tid());
         RDB_STAMP(3);
     }
 }

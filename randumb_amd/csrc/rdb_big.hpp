@@ -247,7 +247,7 @@ template <int BM> __device__ __forceinline__ void big_load_bias(BigBias<BM> &bw,
                 __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(rs, (a0 + wm * MI * 32 + mi * 32 + 8 * jq + 4 * g) * 2, 0, 0));
 }
 
-template <int BM, int BN, bool BIAS>
+template <int BM, int BN, bool BIAS, bool STREAM = false>
 __device__ __forceinline__ void big_store_bf16(f32x16 (&acc)[BM / 64][BN / 64], bf16_t *__restrict__ lds, bf16_t *__restrict__ out, int64_t ld,
                                                int64_t out_elems, int a0, int na, int b0, int nb, const BigBias<BM> &bw, int t)
 {
@@ -291,7 +291,7 @@ __device__ __forceinline__ void big_store_bf16(f32x16 (&acc)[BM / 64][BN / 64], 
         for (int q = 0; q < GROUP; ++q) {
             const int b = (p0 + q) * (256 / (BM / 8)) + bq;
             const uint32_t off = (a_ok && b0 + b < nb) ? (uint32_t)(((int64_t)(b0 + b) * ld + a0 + a) * 2) : BUFFER_OOB;
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v[q]), rs, (int)off, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v[q]), rs, (int)off, 0, STREAM ? 2 : 0);
         }
         __builtin_amdgcn_sched_barrier(0);
     }
