@@ -298,8 +298,10 @@ bool big_fwd_applies(const rdb_linear_desc *d, int num_cus)
 bool big_bwd_applies(const rdb_linear_desc *d, int num_cus)
 {
     const ProjLayout L = proj_layout(d);
-    // every dC tile contracts all tokens (no partial sums over token ranges), so the tiles alone must fill the chip
-    return L.ok && !L.fits_regs && enough_tiles(cdiv(d->out_f, BG) * cdiv(d->k, BG), num_cus);
+    // every dC tile contracts all tokens (no partial sums over token ranges), so the tiles alone must fill the chip; and the t
+    // tiles, each of which contracts all of out_f, must not be so few that a handful of blocks is left with all of that work
+    return L.ok && !L.fits_regs && enough_tiles(cdiv(d->out_f, BG) * cdiv(d->k, BG), num_cus) &&
+           enough_tiles(2 * cdiv(d->k, BG) * cdiv(d->tokens, BT_TOK), num_cus);
 }
 
 template <class K, class P> static int launch_big(K kernel, const P &p, int items, int num_cus, size_t smem, hipStream_t s, const char *name)
