@@ -225,6 +225,27 @@ def llm_layer_config(event_ms, torch, L, _lib, dev, g, vendor=True):
     return res
 
 
+def gpt_step_config(event_ms, torch, dev, g):
+    """GPT-2 small with random-backed linears: 12 layers, d = 768, 12 heads, vocab 50304, k = 256, seeds 0..47, bf16, batch
+    8 x 1024 random token ids; one training step (forward + backward).  Attention, norms, embedding, head and loss are stock
+    PyTorch; the 48 linears run the projected kernels."""
+    from randumb_amd.SillyLayers import listgen, stepgen
+    from randumb_amd.gpt import RT_GPT, RT_GPTConfig
+
+    torch.manual_seed(0)
+    model = RT_GPT(RT_GPTConfig(int_dim_gen=listgen([256] * 48), seed_gen=stepgen(0, 1))).to(torch.bfloat16).to(dev)
+    idx = torch.randint(0, 50304, (8, 1024), generator=g).to(dev)
+    tgt = torch.randint(0, 50304, (8, 1024), generator=g).to(dev)
+
+    def gpt_step():
+        model.zero_grad(set_to_none=True)
+        model(idx, tgt).backward()
+
+    ms = event_ms(gpt_step, 5)
+    return {"fwd_bwd_ms": round(ms, 2), "tokens_per_s": round(8192 / ms * 1e3, 0),
+            "note": "random-backed qkv/proj/fc/mlp-proj; attention, norms, embedding, head and loss are stock PyTorch"}
+
+
 def other_configs(event_ms, torch, L, _lib, dev):
     """The other configurations, timed for the record (they are parity-test cases, not the metric)."""
     from randumb_amd import hip
@@ -297,25 +318,7 @@ def other_configs(event_ms, torch, L, _lib, dev):
                 "256-token tile instead"}
     del dW, xh, dyh
 
-    # ---- GPT-2 small with random-backed linears: 12 layers, d = 768, 12 heads, vocab 50304, k = 256, seeds 0..47, bf16,
-    # batch 8 x 1024 random token ids; one training step (forward + backward).  Attention, norms, embedding, head and loss
-    # are stock PyTorch; the 48 linears run the projected kernels.
-    from randumb_amd.SillyLayers import listgen, stepgen
-    from randumb_amd.gpt import RT_GPT, RT_GPTConfig
-
-    torch.manual_seed(0)
-    model = RT_GPT(RT_GPTConfig(int_dim_gen=listgen([256] * 48), seed_gen=stepgen(0, 1))).to(torch.bfloat16).to(dev)
-    idx = torch.randint(0, 50304, (8, 1024), generator=g).to(dev)
-    tgt = torch.randint(0, 50304, (8, 1024), generator=g).to(dev)
-
-    def gpt_step():
-        model.zero_grad(set_to_none=True)
-        model(idx, tgt).backward()
-
-    ms = event_ms(gpt_step, 5)
-    out["gpt2_small_12L_k256_seeds0to47_bf16_8x1024"] = {"fwd_bwd_ms": round(ms, 2), "tokens_per_s": round(8192 / ms * 1e3, 0),
-                                                        "note": "random-backed qkv/proj/fc/mlp-proj; attention, norms, embedding, "
-                                                                "head and loss are stock PyTorch"}
+    out["gpt2_small_12L_k256_seeds0to47_bf16_8x1024"] = gpt_step_config(event_ms, torch, dev, g)
     return out
 
 
@@ -332,6 +335,8 @@ def main():
     ap.add_argument("--llm-layer-only", action="store_true",
                     help="run only the 4096 -> 14336, k = 1024 layer (projection, forward, backward through the C ABI) and exit "
                          "(profiling runs)")
+    ap.add_argument("--gpt-only", action="store_true",
+                    help="run only the GPT-2 small training step with random-backed linears and exit (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch plain device copies of 256 MiB (a known 256 MiB read + 256 MiB written per launch) so that "
                          "hardware byte counters collected over this run can be scaled")
@@ -366,6 +371,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.gpt_only:
+        print(json.dumps({"gpt2_small_12L_k256_seeds0to47_bf16_8x1024": gpt_step_config(make_event_ms(torch), torch, dev, g)}))
+        return
     if args.llm_layer_only:
         print(json.dumps({"in4096_out14336_k1024_T4096_bf16": llm_layer_config(make_event_ms(torch), torch, L, _lib, dev, g, vendor=False)}))
         return
