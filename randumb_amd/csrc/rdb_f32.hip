@@ -1,0 +1,402 @@
+// Fused linear layer, matrix-coef + fp32, any coefficient dimension and many tokens: the factored algorithm on the fp32
+// matrix cores (v_mfma_f32_32x32x2_f32).
+//
+//   forward  z = x . N^T [T x k],  y = z . C^T (+ bias)
+//   dx       t = dy . C  [T x k],  dx = t . N
+//   dcoef    z as above,           dC = dy^T . z     (token ranges summed in a fixed order: bit-reproducible)
+//
+// N[m, i] = noise(PRIME*i + m) is hashed into the pipeline's LDS tiles and never stored; W = C . N is never formed.  All
+// five products run on one kernel template that differs in where its two operands come from (a row-major matrix read along
+// or across its rows, or the hash).  Everything is fp32: operands, products and sums.
+// Replaces materialize() + dense product (src/rten_cpp/RandumbTensor.py:942-946) and MmBackward's dW followed by
+// materialize_bwd (RandumbTensor.py:979-990, 304-359) for fp32 layers beyond the few-token regime of rdb_smallk.hip.
+#include "rdb_gemm.hpp"
+
+namespace rdb {
+
+constexpr int FG_BN = 128;        // B rows (output columns) per block
+constexpr int FG_BK = 16;         // contraction values per stage
+constexpr int FG_THREADS = 256;   // four waves, 2 x 2
+
+// Where an operand's tile [rows x FG_BK] comes from.  In LDS every tile is [FG_BK][rows + 4]: an MFMA operand is 32
+// consecutive floats of each of two contraction values.
+enum FgSource {
+    FG_KCONT = 0,    // src[row * ld + kk]: a row-major matrix whose rows are the tile's rows
+    FG_MCONT = 1,    // src[kk * ld + row]: a row-major matrix whose rows are contraction values
+    FG_NOISE_M = 2,  // 2-D noise (feature kk, coefficient row): the rows are coefficients, the contraction runs over features
+    FG_NOISE_I = 3   // 2-D noise (feature row, coefficient kk): the rows are features, the contraction runs over coefficients
+};
+
+struct FgParams {
+    const float *a;   // A operand's matrix (FG_KCONT / FG_MCONT)
+    int64_t lda;
+    const float *b;   // B operand's matrix; not used by the noise sources
+    int64_t ldb;
+    float *out;       // [M x N], leading dimension ldo; split s of the contraction writes out + s * split_stride
+    int64_t ldo, split_stride;
+    const float *bias;   // [N] or NULL
+    int M, N, K;
+    int kchunk;          // contraction values per split (a multiple of FG_BK); K when there is one split
+    int64_t a_bytes, b_bytes;   // extent of the matrices, for the bounds check of the loads (< 2^31)
+    uint32_t seed;
+};
+
+// One operand's way from its source into LDS: load(stage) requests / hashes the stage's values into registers, store() puts
+// them into a tile.  Rows past `rows` and contraction values past `kend` are zeros.
+template <int ROWS, int SRC> struct FgOperand {
+    static constexpr int LD = ROWS + 4, TILE = FG_BK * LD, NV = ROWS * FG_BK / FG_THREADS / 4;   // float4 per thread and stage
+    static_assert(NV >= 1, "a stage is at least one float4 per thread");
+    __amdgpu_buffer_rsrc_t rs;
+    uint32_t off[NV];   // byte offset of the thread's pieces at stage 0 (BUFFER_OOB: a row past the end)
+    uint32_t step;      // bytes per stage
+    uint32_t first;     // noise: first-round value of the thread's first element at stage 0
+    int kk0, kend, k_begin, row_ok;
+    f32x4 r[NV];
+
+    __device__ __forceinline__ void init(const float *src, int64_t ld, int64_t bytes, int row0, int rows, int k_begin_, int kend_, uint32_t seed)
+    {
+        const int t = threadIdx.x;
+        k_begin = k_begin_;
+        kend = kend_;
+        if (SRC == FG_KCONT) {
+            rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(src), 0, (int)bytes, 0x00020000);
+            step = FG_BK * 4;
+#pragma unroll
+            for (int h = 0; h < NV; ++h) {
+                const int idx = h * FG_THREADS + t, row = idx >> 2, kq = idx & 3;
+                off[h] = row0 + row < rows ? (uint32_t)(((int64_t)(row0 + row) * ld + k_begin + kq * 4) * 4) : BUFFER_OOB;
+            }
+            kk0 = (t & 3) * 4;
+        } else if (SRC == FG_MCONT) {
+            rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(src), 0, (int)bytes, 0x00020000);
+            step = (uint32_t)(FG_BK * ld * 4);
+#pragma unroll
+            for (int h = 0; h < NV; ++h) {
+                const int idx = h * FG_THREADS + t, kk = idx / (ROWS / 4), r4 = (idx % (ROWS / 4)) * 4;
+                off[h] = row0 + r4 < rows ? (uint32_t)(((int64_t)(k_begin + kk) * ld + row0 + r4) * 4) : BUFFER_OOB;
+            }
+            kk0 = t / (ROWS / 4);
+        } else {
+            const int row = t % ROWS;
+            kk0 = t / ROWS;
+            row_ok = row0 + row < rows;
+            first = SRC == FG_NOISE_M ? sq5_first((uint32_t)(k_begin + kk0), (uint32_t)(row0 + row), seed)
+                                      : sq5_first((uint32_t)(row0 + row), (uint32_t)(k_begin + kk0), seed);
+        }
+    }
+    __device__ __forceinline__ void load(int stage)
+    {
+        if (SRC == FG_KCONT) {
+            // a thread's four values are consecutive contraction values: all inside or all outside (K is a multiple of 4)
+            const bool in = k_begin + stage * FG_BK + kk0 < kend;
+#pragma unroll
+            for (int h = 0; h < NV; ++h)
+                r[h] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, in ? (int)(off[h] + (uint32_t)stage * step) : (int)BUFFER_OOB, 0, 0));
+        } else if (SRC == FG_MCONT) {
+#pragma unroll
+            for (int h = 0; h < NV; ++h) {
+                const bool in = k_begin + stage * FG_BK + kk0 + h * (FG_THREADS / (ROWS / 4)) < kend;
+                r[h] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, in ? (int)(off[h] + (uint32_t)stage * step) : (int)BUFFER_OOB, 0, 0));
+            }
+        } else {
+            // element j of the thread: contraction value kk0 + j * (FG_THREADS / ROWS) of the stage, one add apart in the first round
+            constexpr int KSTEP = FG_THREADS / ROWS;
+            const uint32_t inc = SRC == FG_NOISE_M ? PN1 : SQ5_N1;
+            uint32_t f = first + (uint32_t)(stage * FG_BK) * inc;
+#pragma unroll
+            for (int j = 0; j < NV * 4; ++j, f += (uint32_t)KSTEP * inc) {
+                const bool in = row_ok && k_begin + stage * FG_BK + kk0 + j * KSTEP < kend;
+                r[j >> 2][j & 3] = in ? sq5_unit(sq5_tail(f)) : 0.0f;
+            }
+        }
+    }
+    __device__ __forceinline__ void store(float *__restrict__ tile) const
+    {
+        const int t = threadIdx.x;
+        if (SRC == FG_KCONT) {
+#pragma unroll
+            for (int h = 0; h < NV; ++h) {
+                const int idx = h * FG_THREADS + t, row = idx >> 2, kq = idx & 3;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) tile[(kq * 4 + j) * LD + row] = r[h][j];
+            }
+        } else if (SRC == FG_MCONT) {
+#pragma unroll
+            for (int h = 0; h < NV; ++h) {
+                const int idx = h * FG_THREADS + t, kk = idx / (ROWS / 4), r4 = (idx % (ROWS / 4)) * 4;
+                *reinterpret_cast<f32x4 *>(tile + kk * LD + r4) = r[h];
+            }
+        } else {
+            constexpr int KSTEP = FG_THREADS / ROWS;
+            const int row = t % ROWS;
+#pragma unroll
+            for (int j = 0; j < NV * 4; ++j) tile[(kk0 + j * KSTEP) * LD + row] = r[j >> 2][j & 3];
+        }
+    }
+};
+
+// out[M x N] (+)= A . B^T over one split of the contraction.  Block: BM x 128 of the output, four waves as 2 x 2, a wave owns
+// (BM / 2) x 64 in BM / 64 x 2 accumulator tiles.  Two LDS buffers, one barrier per stage: while a stage is multiplied the
+// next one is on its way from memory (or being hashed) in registers.
+template <int BM, int ASRC, int BSRC, bool BIAS> __global__ __launch_bounds__(FG_THREADS, 2) void f32_gemm_kernel(FgParams p)
+{
+    typedef FgOperand<BM, ASRC> PA;
+    typedef FgOperand<FG_BN, BSRC> PB;
+    constexpr int MI = BM / 64, NI = 2, STAGE = PA::TILE + PB::TILE;
+    __shared__ __align__(16) float lds[2 * STAGE];
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * FG_BN;
+    const int k_begin = blockIdx.z * p.kchunk, kend = min(p.K, k_begin + p.kchunk);
+    const int nstage = (kend - k_begin + FG_BK - 1) / FG_BK;
+    PA pa;
+    PB pb;
+    pa.init(p.a, p.lda, p.a_bytes, m0, p.M, k_begin, kend, p.seed);
+    pb.init(p.b, p.ldb, p.b_bytes, n0, p.N, k_begin, kend, p.seed);
+    f32x16 acc[MI][NI];
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.0f;
+    pa.load(0);
+    pb.load(0);
+    for (int s = 0; s < nstage; ++s) {
+        float *As = lds + (s & 1) * STAGE, *Bs = As + PA::TILE;
+        pa.store(As);
+        pb.store(Bs);
+        __syncthreads();   // also: every wave is done reading the other buffer (the stage before this one)
+        if (s + 1 < nstage) {
+            pa.load(s + 1);
+            pb.load(s + 1);
+        }
+        const float *ap = As + g * PA::LD + wm * (BM / 2) + r, *bp = Bs + g * PB::LD + wn * 64 + r;
+#pragma unroll
+        for (int ks = 0; ks < FG_BK / 2; ++ks) {
+            float fa[MI], fb[NI];
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi) fa[mi] = ap[ks * 2 * PA::LD + mi * 32];
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) fb[ni] = bp[ks * 2 * PB::LD + ni * 32];
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi], fb[ni], acc[mi][ni], 0, 0, 0);
+        }
+    }
+    // accumulator j of lane (r, g): row 8 (j / 4) + 4 g + j % 4 of the A side, column r of the B side
+    float *out = p.out + (int64_t)blockIdx.z * p.split_stride;
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) {
+        const int n = n0 + wn * 64 + ni * 32 + r;
+        if (n >= p.N) continue;
+        const float bv = BIAS ? p.bias[n] : 0.0f;
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int m = m0 + wm * (BM / 2) + mi * 32 + 8 * (j >> 2) + 4 * g + (j & 3);
+                if (m < p.M) out[(int64_t)m * p.ldo + n] = acc[mi][ni][j] + bv;
+            }
+    }
+}
+
+// out[i] = part[0][i] + part[1][i] + ... in split order, four values per thread
+__global__ __launch_bounds__(256) void f32_sum_splits_kernel(float *__restrict__ out, const float *__restrict__ part, int64_t n4, int64_t stride, int splits)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    f32x4 v = *reinterpret_cast<const f32x4 *>(part + i * 4);
+    for (int s = 1; s < splits; ++s) v += *reinterpret_cast<const f32x4 *>(part + s * stride + i * 4);
+    *reinterpret_cast<f32x4 *>(out + i * 4) = v;
+}
+
+// ----------------------------------------------------------------------------------------------- host side
+static bool fg_aligned16(const void *q) { return ((uintptr_t)q & 15) == 0; }
+static int64_t up256(int64_t n) { return (n + 255) / 256 * 256; }
+
+// The shapes these kernels take: matrix-coef fp32, every extent a multiple of 4 (16-byte pieces), matrices below 2^31 bytes.
+static bool fg_ok(const rdb_linear_desc *d)
+{
+    return d->act_dtype == RDB_F32 && d->coef_dtype == RDB_F32 && d->coef_rows != 0 && d->k > 0 && d->tokens > 0 && d->in_f > 0 && d->out_f > 0 &&
+           d->k % 4 == 0 && d->in_f % 4 == 0 && d->out_f % 4 == 0 && d->tokens * d->k < (1ll << 29) && d->out_f * d->k < (1ll << 29) &&
+           d->in_f < (1 << 30) && d->out_f < (1 << 30);
+}
+static bool fg_wanted(const rdb_linear_desc *d) { return d->algo == RDB_ALGO_FACTORED || d->k * (d->in_f + d->out_f) < d->in_f * d->out_f; }
+
+// Token ranges of the coefficient gradient: enough blocks for about two per compute unit, ranges of at least 256 tokens.
+static int dc_splits(const rdb_linear_desc *d, int num_cus)
+{
+    const int64_t tiles = cdiv(d->out_f, 128) * cdiv(d->k, FG_BN);
+    int64_t s = cdiv(2 * (int64_t)num_cus, tiles);
+    const int64_t most = cdiv(d->tokens, 256);
+    if (s > most) s = most;
+    if (s > 64) s = 64;
+    return s < 1 ? 1 : (int)s;
+}
+
+// Ranges of the contraction of z = x . N^T and t = dy . C when their [tokens x k] output has too few tiles to give every
+// compute unit a block: each range leaves a partial matrix, added up in range order afterwards.  At least 128 values a range.
+static int zt_splits(const rdb_linear_desc *d, int64_t K, int num_cus)
+{
+    const int64_t tiles = cdiv(d->tokens, 64) * cdiv(d->k, FG_BN);
+    if (tiles >= num_cus) return 1;
+    int64_t s = cdiv(num_cus, tiles);
+    if (s > K / 128) s = K / 128;
+    if (s > 32) s = 32;
+    return s < 1 ? 1 : (int)s;
+}
+
+// scratch: z or t [tokens x k] and its partial matrices; for the coefficient gradient also one [out_f x k] matrix per token range
+int64_t linear_f32_workspace(int op, const rdb_linear_desc *d, int num_cus)
+{
+    rdb_linear_desc dd = *d;
+    if (op == RDB_OP_LINEAR_BWD_DCOEF) dd.coef_dtype = RDB_F32;   // reads no coefficients
+    if (!fg_ok(&dd)) return 0;
+    const int64_t zt = up256(d->tokens * d->k * 4);
+    auto with_parts = [&](int64_t K) { const int s = zt_splits(d, K, num_cus); return zt * (s > 1 ? 1 + s : 1); };
+    if (op == RDB_OP_LINEAR_FWD) return with_parts(d->in_f);
+    if (op == RDB_OP_LINEAR_BWD_DX) return with_parts(d->out_f);
+    if (op != RDB_OP_LINEAR_BWD_DCOEF) return 0;
+    const int s = dc_splits(d, num_cus);
+    return with_parts(d->in_f) + (s > 1 ? (int64_t)s * up256(d->out_f * d->k * 4) : 0);
+}
+
+struct FgProduct {
+    const float *a;
+    int64_t lda, a_elems;
+    const float *b;
+    int64_t ldb, b_elems;
+    float *out;
+    int64_t ldo;
+    const float *bias;
+    int64_t M, N, K;
+    int64_t kchunk;         // contraction values per range (a multiple of FG_BK); 0: one range
+    int64_t split_stride;   // floats between the ranges' outputs
+    uint32_t seed;
+};
+
+template <int ASRC, int BSRC> static int fg_launch(const FgProduct &q, int num_cus, hipStream_t s, const char *name)
+{
+    if (q.a_elems >= (1ll << 29) || q.b_elems >= (1ll << 29) || q.M >= (1ll << 30) || q.N >= (1ll << 30) || q.K >= (1ll << 30)) return RDB_E_UNSUPPORTED;
+    FgParams p = {};
+    p.a = q.a;
+    p.lda = q.lda;
+    p.b = q.b;
+    p.ldb = q.ldb;
+    p.out = q.out;
+    p.ldo = q.ldo;
+    p.split_stride = q.split_stride;
+    p.bias = q.bias;
+    p.M = (int)q.M;
+    p.N = (int)q.N;
+    p.K = (int)q.K;
+    p.kchunk = (int)(q.kchunk > 0 ? q.kchunk : cdiv(q.K, FG_BK) * FG_BK);
+    p.a_bytes = q.a_elems * 4;
+    p.b_bytes = q.b_elems * 4;
+    p.seed = q.seed;
+    const int splits = (int)cdiv(q.K, p.kchunk);
+    // 128-row tiles when they give every compute unit a block, 64-row tiles otherwise
+    const int64_t tiles128 = cdiv(q.M, 128) * cdiv(q.N, FG_BN) * splits;
+    if (tiles128 >= num_cus) {
+        const dim3 grid((unsigned)cdiv(q.N, FG_BN), (unsigned)cdiv(q.M, 128), (unsigned)splits);
+        if (q.bias) f32_gemm_kernel<128, ASRC, BSRC, true><<<grid, FG_THREADS, 0, s>>>(p);
+        else f32_gemm_kernel<128, ASRC, BSRC, false><<<grid, FG_THREADS, 0, s>>>(p);
+    } else {
+        const dim3 grid((unsigned)cdiv(q.N, FG_BN), (unsigned)cdiv(q.M, 64), (unsigned)splits);
+        if (q.bias) f32_gemm_kernel<64, ASRC, BSRC, true><<<grid, FG_THREADS, 0, s>>>(p);
+        else f32_gemm_kernel<64, ASRC, BSRC, false><<<grid, FG_THREADS, 0, s>>>(p);
+    }
+    return check_launch(name);
+}
+
+static bool fg_ws_ok(int op, const rdb_linear_desc *d, int num_cus, const void *ws, int64_t bytes)
+{
+    return ws && fg_aligned16(ws) && bytes >= linear_f32_workspace(op, d, num_cus);
+}
+
+static int fg_sum(float *out, const float *part, int64_t n, int64_t stride, int splits, hipStream_t s)
+{
+    f32_sum_splits_kernel<<<(unsigned)cdiv(n / 4, 256), 256, 0, s>>>(out, part, n / 4, stride, splits);
+    return check_launch("f32_sum_splits_kernel");
+}
+
+// A product whose dense output [M x N] (ldo = N) may be computed in `splits` ranges of the contraction: the ranges' partial
+// matrices go to `part` (stride floats apart) and are added up into q.out in range order.
+template <int ASRC, int BSRC> static int fg_launch_ranges(FgProduct q, int splits, float *part, int64_t stride, int num_cus, hipStream_t s, const char *name)
+{
+    const int kchunk = (int)(cdiv(cdiv(q.K, splits), FG_BK) * FG_BK);
+    splits = (int)cdiv(q.K, kchunk);   // the ranges that hold something
+    if (splits <= 1) {
+        q.kchunk = 0;
+        q.split_stride = 0;
+        return fg_launch<ASRC, BSRC>(q, num_cus, s, name);
+    }
+    float *out = q.out;
+    q.out = part;
+    q.kchunk = kchunk;
+    q.split_stride = stride;
+    if (int rc = fg_launch<ASRC, BSRC>(q, num_cus, s, name)) return rc;
+    return fg_sum(out, part, q.M * q.N, stride, splits, s);
+}
+
+// z[T x k] = src[T x in_f] . N^T; the partial matrices of its ranges follow z in the workspace
+static int fg_project(float *z, const float *x, int64_t ldx, const rdb_linear_desc *d, int num_cus, hipStream_t s)
+{
+    FgProduct q = {x, ldx, (d->tokens - 1) * ldx + d->in_f, nullptr, 0, 0, z, d->k, nullptr, d->tokens, d->k, d->in_f, 0, 0, d->seed};
+    const int64_t zt = up256(d->tokens * d->k * 4) / 4;
+    return fg_launch_ranges<FG_KCONT, FG_NOISE_M>(q, zt_splits(d, d->in_f, num_cus), z + zt, zt, num_cus, s, "f32_gemm_kernel (z = x . N^T)");
+}
+
+// The three entry points return RDB_E_UNSUPPORTED, without setting an error, when the request does not fit.
+int linear_fwd_f32(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
+                   const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s)
+{
+    if (!fg_ok(d) || scale_bias || !fg_wanted(d) || !fg_ws_ok(RDB_OP_LINEAR_FWD, d, num_cus, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    if (ldx % 4 || ldy % 4 || !fg_aligned16(x) || !fg_aligned16(coef) || d->tokens * ldx >= (1ll << 29) || d->tokens * ldy >= (1ll << 29))
+        return RDB_E_UNSUPPORTED;
+    float *z = (float *)workspace;
+    if (int rc = fg_project(z, (const float *)x, ldx, d, num_cus, s)) return rc;
+    FgProduct q = {z, d->k, d->tokens * d->k, (const float *)coef, d->k, d->out_f * d->k, (float *)y, ldy, (const float *)bias,
+                   d->tokens, d->out_f, d->k, 0, 0, d->seed};
+    return fg_launch<FG_KCONT, FG_KCONT>(q, num_cus, s, "f32_gemm_kernel (y = z . C^T)");
+}
+
+int linear_dx_f32(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias, const rdb_linear_desc *d,
+                  int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s)
+{
+    if (!fg_ok(d) || scale_bias || !fg_wanted(d) || !fg_ws_ok(RDB_OP_LINEAR_BWD_DX, d, num_cus, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    if (lddx % 4 || lddy % 4 || !fg_aligned16(dy) || !fg_aligned16(coef) || d->tokens * lddx >= (1ll << 29) || d->tokens * lddy >= (1ll << 29))
+        return RDB_E_UNSUPPORTED;
+    float *t = (float *)workspace;
+    // t[T x k] = dy[T x out_f] . C: the B side's rows are coefficients, read across the rows of C
+    FgProduct q1 = {(const float *)dy, lddy, (d->tokens - 1) * lddy + d->out_f, (const float *)coef, d->k, d->out_f * d->k, t, d->k, nullptr,
+                    d->tokens, d->k, d->out_f, 0, 0, d->seed};
+    const int64_t zt = up256(d->tokens * d->k * 4) / 4;
+    if (int rc = fg_launch_ranges<FG_KCONT, FG_MCONT>(q1, zt_splits(d, d->out_f, num_cus), t + zt, zt, num_cus, s, "f32_gemm_kernel (t = dy . C)")) return rc;
+    // dx[T x in_f] = t . N: the B side's rows are input features, hashed
+    FgProduct q2 = {t, d->k, d->tokens * d->k, nullptr, 0, 0, (float *)dx, lddx, nullptr, d->tokens, d->in_f, d->k, 0, 0, d->seed};
+    return fg_launch<FG_KCONT, FG_NOISE_I>(q2, num_cus, s, "f32_gemm_kernel (dx = t . N)");
+}
+
+// dcoef is overwritten (no zero fill needed).
+int linear_dcoef_f32(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus, void *workspace,
+                     int64_t workspace_bytes, hipStream_t s)
+{
+    rdb_linear_desc dd = *d;
+    dd.coef_dtype = RDB_F32;   // no coefficients are read here
+    if (!fg_ok(&dd) || !fg_wanted(&dd) || !fg_ws_ok(RDB_OP_LINEAR_BWD_DCOEF, &dd, num_cus, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    if (ldx % 4 || lddy % 4 || !fg_aligned16(x) || !fg_aligned16(dy) || !fg_aligned16(dcoef) || d->tokens * ldx >= (1ll << 29) ||
+        d->tokens * lddy >= (1ll << 29))
+        return RDB_E_UNSUPPORTED;
+    float *z = (float *)workspace;
+    if (int rc = fg_project(z, (const float *)x, ldx, &dd, num_cus, s)) return rc;
+    // dC[out_f x k] = dy^T . z: both sides are read across their rows (the contraction runs over the tokens)
+    const int zs = zt_splits(&dd, d->in_f, num_cus);
+    float *part = reinterpret_cast<float *>(static_cast<char *>(workspace) + up256(d->tokens * d->k * 4) * (zs > 1 ? 1 + zs : 1));
+    FgProduct q = {(const float *)dy, lddy, (d->tokens - 1) * lddy + d->out_f, z, d->k, d->tokens * d->k, dcoef, d->k, nullptr,
+                   d->out_f, d->k, d->tokens, 0, 0, d->seed};
+    return fg_launch_ranges<FG_MCONT, FG_MCONT>(q, dc_splits(&dd, num_cus), part, up256(d->out_f * d->k * 4) / 4, num_cus, s, "f32_gemm_kernel (dC = dy^T . z)");
+}
+
+}  // namespace rdb

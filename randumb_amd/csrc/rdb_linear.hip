@@ -309,6 +309,14 @@ int linear_dx_smallk(void *dx, int64_t lddx, const void *dy, int64_t lddy, const
 int linear_dcoef_smallk(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, void *workspace,
                         int64_t workspace_bytes, hipStream_t s);
 
+// rdb_f32.hip
+int64_t linear_f32_workspace(int op, const rdb_linear_desc *d, int num_cus);
+int linear_fwd_f32(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
+                   const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
+int linear_dx_f32(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias, const rdb_linear_desc *d,
+                  int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
+int linear_dcoef_f32(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus, void *workspace,
+                     int64_t workspace_bytes, hipStream_t s);
 // rdb_dx.hip
 int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z, const void *coef,
                          const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, bool accumulate, hipStream_t s);
@@ -384,7 +392,10 @@ extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
     if (d->act_dtype == RDB_F32) {  // fp32: the small-k kernels, whose scratch is one [tokens x k] fp32 matrix
         rdb_linear_desc dd = *d;
         if (op == RDB_OP_LINEAR_BWD_DCOEF) dd.coef_dtype = RDB_F32;
-        return (op == RDB_OP_LINEAR_FWD || op == RDB_OP_LINEAR_BWD_DX || op == RDB_OP_LINEAR_BWD_DCOEF) ? linear_smallk_workspace(&dd) : 0;
+        if (op != RDB_OP_LINEAR_FWD && op != RDB_OP_LINEAR_BWD_DX && op != RDB_OP_LINEAR_BWD_DCOEF) return 0;
+        // or the matrix-core kernels of rdb_f32.hip: a [tokens x k] matrix, and the coefficient gradient's token-range sums
+        const int64_t a = linear_smallk_workspace(&dd), b = linear_f32_workspace(op, &dd, num_compute_units());
+        return a > b ? a : b;
     }
     if (op == RDB_OP_LINEAR_BWD_DX) return linear_dx_factored_workspace(d);
     if (op == RDB_OP_LINEAR_BWD_PROJECTED) return bwd_projected_workspace(d);
@@ -407,10 +418,12 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
         if (rc != RDB_E_UNSUPPORTED) return rc;
         rc = linear_fwd_smallk(y, ldy, x, ldx, coef, scale_bias, bias, d, workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
+        rc = linear_fwd_f32(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), workspace, workspace_bytes, s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
         if (d->algo == RDB_ALGO_FACTORED)
             return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd: the factored algorithm needs matrix-coef, no scale_bias, a workspace of "
                                                 "rdb_linear_workspace_bytes() bytes and either bf16 (activations and coef; sizes that are "
-                                                "multiples of 8; aligned rows) or fp32 with k <= 64 and tokens <= 4096");
+                                                "multiples of 8; aligned rows) or fp32 (sizes that are multiples of 4; aligned rows)");
     }
     if (d->algo != RDB_ALGO_TILE) {
         rc = linear_fwd_strip(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), s);
@@ -460,10 +473,12 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
         if (rc != RDB_E_UNSUPPORTED) return rc;
         rc = linear_dx_smallk(dx, lddx, dy, lddy, coef, scale_bias, d, workspace, workspace_bytes, (hipStream_t)stream);
         if (rc != RDB_E_UNSUPPORTED) return rc;
+        rc = linear_dx_f32(dx, lddx, dy, lddy, coef, scale_bias, d, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
         if (d->algo == RDB_ALGO_FACTORED)
             return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dx: the factored algorithm needs matrix-coef, a workspace of "
                                                 "rdb_linear_workspace_bytes() bytes and either bf16 (activations and coef; sizes that are "
-                                                "multiples of 8; aligned rows) or fp32 with k <= 64 and tokens <= 4096");
+                                                "multiples of 8; aligned rows) or fp32 (sizes that are multiples of 4; aligned rows)");
     }
     if (d->algo != RDB_ALGO_TILE) {  // forms W chunks on chip, with the block's noise columns hashed once
         rc = linear_dx_nstrip(dx, lddx, dy, lddy, coef, scale_bias, d, (hipStream_t)stream);
@@ -515,11 +530,13 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
         if (rc != RDB_E_UNSUPPORTED) return rc;
         rc = linear_dcoef_smallk(dcoef, dy, lddy, x, ldx, d, workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
+        rc = linear_dcoef_f32(dcoef, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
     }
     if (d->algo == RDB_ALGO_FACTORED)
         return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dcoef: the factored algorithm needs matrix-coef, no scale_bias gradient, a "
                                             "workspace of rdb_linear_workspace_bytes() bytes and either bf16 activations (sizes that are "
-                                            "multiples of 8; aligned rows) or fp32 with k <= 64 and tokens <= 4096");
+                                            "multiples of 8; aligned rows) or fp32 (sizes that are multiples of 4; aligned rows)");
     if (d->algo != RDB_ALGO_TILE) {
         rc = linear_dcoef_fast(dcoef, d_scale_bias, dy, lddy, x, ldx, d, num_compute_units(), s);
         if (rc != RDB_E_UNSUPPORTED) return rc;

@@ -1,0 +1,130 @@
+"""fp32 matrix-coef layers on the fp32 matrix cores (the factored algorithm, any k, many tokens) against the CPU oracle, at the
+fp32 tolerance of the path (rel-L2 1e-5), and against the general kernel.
+
+Asking for RDB_ALGO_FACTORED makes the library refuse rather than fall back to the general kernel, so a call that succeeds
+with k > 64 (beyond the vector-ALU kernels for few tokens) ran these kernels."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 1e-5
+
+
+def rel_l2(a, b):
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+@pytest.fixture(scope="module")
+def hip():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from randumb_amd import hip as h
+
+    return h
+
+
+def _inputs(T, in_f, out_f, k, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, in_f, generator=g)
+    dy = torch.randn(T, out_f, generator=g)
+    coef = torch.randn(out_f, k, generator=g) * (3.0 / k) ** 0.5 * 0.05
+    bias = torch.randn(out_f, generator=g)
+    return x, dy, coef, bias
+
+
+SHAPES = [
+    # tokens, in_f, out_f, k, seed
+    (512, 768, 1024, 128, 3),     # whole tiles
+    (300, 260, 516, 68, 1337),    # ragged in every extent (multiples of 4)
+    (64, 1024, 1024, 256, 5),     # few tokens: 64-row tiles
+    (4500, 128, 256, 32, 9),      # small k, more tokens than the vector-ALU kernels take
+    (4, 8, 12, 68, 1),            # smaller than one tile
+    (2100, 516, 132, 100, 77),    # the coefficient gradient in several token ranges, ragged last range
+]
+
+
+@pytest.mark.parametrize("T,in_f,out_f,k,seed", SHAPES)
+def test_against_the_oracle(hip, oracle, T, in_f, out_f, k, seed):
+    from randumb_amd._lib import RDB_ALGO_FACTORED
+
+    print(f"case f32 matrix cores T={T} in={in_f} out={out_f} k={k}", flush=True)
+    x, dy, coef, bias = _inputs(T, in_f, out_f, k, seed)
+    xn, dyn, cn = x.numpy(), dy.numpy(), coef.numpy()
+    want_y = oracle.linear_fwd(xn, cn, in_f, out_f, seed, bias=bias.numpy())
+    want_dx, want_dc, _ = oracle.linear_bwd(xn, dyn, cn, in_f, out_f, seed)
+    xc, dyc, cc = x.cuda(), dy.cuda(), coef.cuda()
+    y = hip.linear_fwd(xc, cc, in_f, out_f, in_f, 1, seed, bias=bias.cuda(), algo=RDB_ALGO_FACTORED)
+    assert y.dtype == torch.float32 and y.shape == (T, out_f)
+    assert rel_l2(y.cpu().numpy(), want_y) < F32_TOL
+    dx = hip.linear_bwd_dx(dyc, cc, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    assert rel_l2(dx.cpu().numpy(), want_dx) < F32_TOL
+    dc, _ = hip.linear_bwd_dcoef(dyc, xc, k, out_f, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    assert dc.shape == coef.shape and rel_l2(dc.cpu().numpy(), want_dc) < F32_TOL
+    # the same calls again give the same bits (token ranges are added in a fixed order)
+    dc2, _ = hip.linear_bwd_dcoef(dyc, xc, k, out_f, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    assert torch.equal(dc, dc2)
+
+
+def test_default_choice_and_the_general_kernel_agree(hip):
+    """AUTO at a shape where the factored form is cheaper, against the kernel that forms W tiles (RDB_ALGO_TILE)."""
+    from randumb_amd._lib import RDB_ALGO_TILE
+
+    T, in_f, out_f, k, seed = 2048, 384, 640, 96, 21
+    x, dy, coef, bias = _inputs(T, in_f, out_f, k, seed)
+    xc, dyc, cc, bc = x.cuda(), dy.cuda(), coef.cuda(), bias.cuda()
+    y = hip.linear_fwd(xc, cc, in_f, out_f, in_f, 1, seed, bias=bc)
+    y_t = hip.linear_fwd(xc, cc, in_f, out_f, in_f, 1, seed, bias=bc, algo=RDB_ALGO_TILE)
+    assert rel_l2(y.cpu().numpy(), y_t.cpu().numpy()) < F32_TOL
+    dx = hip.linear_bwd_dx(dyc, cc, in_f, out_f, in_f, 1, seed)
+    dx_t = hip.linear_bwd_dx(dyc, cc, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_TILE)
+    assert rel_l2(dx.cpu().numpy(), dx_t.cpu().numpy()) < F32_TOL
+    dc, _ = hip.linear_bwd_dcoef(dyc, xc, k, out_f, in_f, out_f, in_f, 1, seed)
+    dc_t, _ = hip.linear_bwd_dcoef(dyc, xc, k, out_f, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_TILE)
+    assert rel_l2(dc.cpu().numpy(), dc_t.cpu().numpy()) < F32_TOL
+
+
+def test_strided_activations(hip, oracle):
+    """x, dy, y's producers as column slices of wider matrices (leading dimension larger than the row)."""
+    from randumb_amd._lib import RDB_ALGO_FACTORED
+
+    T, in_f, out_f, k, seed = 260, 200, 328, 72, 13
+    x, dy, coef, _ = _inputs(T, in_f, out_f, k, seed)
+    wide_x = torch.zeros(T, in_f + 24).cuda()
+    wide_x[:, 8:8 + in_f] = x.cuda()
+    wide_dy = torch.zeros(T, out_f + 12).cuda()
+    wide_dy[:, 4:4 + out_f] = dy.cuda()
+    xs, dys, cc = wide_x[:, 8:8 + in_f], wide_dy[:, 4:4 + out_f], coef.cuda()
+    assert not xs.is_contiguous() and not dys.is_contiguous()
+    want_y = oracle.linear_fwd(x.numpy(), coef.numpy(), in_f, out_f, seed)
+    want_dx, want_dc, _ = oracle.linear_bwd(x.numpy(), dy.numpy(), coef.numpy(), in_f, out_f, seed)
+    y = hip.linear_fwd(xs, cc, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    assert rel_l2(y.cpu().numpy(), want_y) < F32_TOL
+    dx = hip.linear_bwd_dx(dys, cc, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    assert rel_l2(dx.cpu().numpy(), want_dx) < F32_TOL
+    dc, _ = hip.linear_bwd_dcoef(dys, xs, k, out_f, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    assert rel_l2(dc.cpu().numpy(), want_dc) < F32_TOL
+
+
+def test_layer_level_fp32(hip, oracle):
+    """SillyLinear(matrix_coef=True) in fp32 at a GPT-like slice: forward, input gradient and coefficient gradient through autograd."""
+    from randumb_amd.SillyLayers import SillyLinear
+
+    T, in_f, out_f, k, seed = 1536, 256, 1024, 128, 4
+    lin = SillyLinear(in_f, out_f, [k], [seed], bias=False, device="cuda", dtype=torch.float32, matrix_coef=True)
+    g = torch.Generator().manual_seed(2)
+    with torch.no_grad():
+        lin.weight_coef.copy_((torch.randn(out_f, k, generator=g) * 0.01).cuda())
+    x = torch.randn(T, in_f, generator=g)
+    dy = torch.randn(T, out_f, generator=g)
+    xc = x.cuda().requires_grad_(True)
+    y = lin(xc)
+    y.backward(dy.cuda())
+    cn = lin.weight_coef.detach().cpu().numpy()
+    want_y = oracle.linear_fwd(x.numpy(), cn, in_f, out_f, seed)
+    want_dx, want_dc, _ = oracle.linear_bwd(x.numpy(), dy.numpy(), cn, in_f, out_f, seed)
+    assert rel_l2(y.detach().cpu().numpy(), want_y) < F32_TOL
+    assert rel_l2(xc.grad.cpu().numpy(), want_dx) < F32_TOL
+    assert rel_l2(lin.weight_coef.grad.cpu().numpy(), want_dc) < F32_TOL
