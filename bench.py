@@ -50,6 +50,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+MFMA_F32_PEAK_TFLOPS = 157.3    # MI355X dense fp32 matrix
 HBM_PEAK_TBPS = 8.0
 T, IN_F, OUT_F, K, SEED = 8192, 768, 3072, 256, 0
 
@@ -225,6 +226,61 @@ def llm_layer_config(event_ms, torch, L, _lib, dev, g, vendor=True):
     return res
 
 
+def f32_layer_config(event_ms, torch, L, _lib, dev, g, compare=True):
+    """The headline layer in fp32 (768 -> 3072, k = 256, 8192 tokens): the three one-call entry points on the fp32 matrix cores,
+    every buffer allocated beforehand.  Fractions are on the flops the kernels execute (each call forms its own z or t),
+    against the fp32 matrix peak."""
+    vp = ctypes.c_void_p
+    stream = vp(torch.cuda.current_stream().cuda_stream)
+    Tl, in_f, out_f, k = T, IN_F, OUT_F, K
+    x = torch.randn(Tl, in_f, generator=g).to(dev)
+    dy = torch.randn(Tl, out_f, generator=g).to(dev)
+    C = (torch.randn(out_f, k, generator=g) * (3 * 0.02**2 / k) ** 0.5).to(dev)
+    y = torch.empty(Tl, out_f, device=dev)
+    dx = torch.empty(Tl, in_f, device=dev)
+    dC = torch.empty(out_f, k, device=dev)
+    px, pdy, pC, py, pdx, pdC = (vp(t.data_ptr()) for t in (x, dy, C, y, dx, dC))
+
+    def calls(algo):
+        d = _lib.LinearDesc()
+        d.tokens, d.in_f, d.out_f, d.k, d.coef_rows, d.sO, d.sI, d.seed = Tl, in_f, out_f, k, out_f, in_f, 1, SEED
+        d.act_dtype, d.coef_dtype, d.algo = _lib.RDB_F32, _lib.RDB_F32, algo
+        r = ctypes.byref(d)
+        n = max(L.rdb_linear_workspace_bytes(op, r) for op in (_lib.RDB_OP_LINEAR_FWD, _lib.RDB_OP_LINEAR_BWD_DX, _lib.RDB_OP_LINEAR_BWD_DCOEF))
+        ws = torch.empty(max(n, 16), dtype=torch.uint8, device=dev)
+        pws = vp(ws.data_ptr())
+        keep = (d, ws)
+        return (lambda: _lib.check(L.rdb_linear_fwd(py, out_f, px, in_f, pC, None, None, r, pws, n, stream), "rdb_linear_fwd"),
+                lambda: _lib.check(L.rdb_linear_bwd_dx(pdx, in_f, pdy, out_f, pC, None, r, pws, n, stream), "rdb_linear_bwd_dx"),
+                lambda: _lib.check(L.rdb_linear_bwd_dcoef(pdC, None, pdy, out_f, px, in_f, r, pws, n, stream), "rdb_linear_bwd_dcoef"), keep)
+
+    fwd, bdx, bdc, keep = calls(_lib.RDB_ALGO_AUTO)
+    t_fwd, t_dx, t_dc = event_ms(fwd, 50), event_ms(bdx, 50), event_ms(bdc, 50)
+    proj = 2.0 * Tl * k * in_f   # z = x.N^T or dx = t.N
+    prod = 2.0 * Tl * k * out_f  # y = z.C^T, t = dy.C, dC = dy^T.z
+    ms = t_fwd + t_dx + t_dc
+    executed = 3 * (proj + prod)
+    res = {
+        "calls_ms": {"rdb_linear_fwd": round(t_fwd, 4), "rdb_linear_bwd_dx": round(t_dx, 4), "rdb_linear_bwd_dcoef": round(t_dc, 4)},
+        "fwd_bwd_ms": round(ms, 4), "executed_gflop": round(executed / 1e9, 1), "executed_TFLOPs": round(executed / ms / 1e9, 1),
+        "executed_frac_of_f32_mfma_peak": round(executed / ms / 1e9 / MFMA_F32_PEAK_TFLOPS, 4),
+        "prescribed_TFLOPs_equivalent": round(F_STEP / ms / 1e9, 1),
+        "kernels": "f32_gemm_kernel (v_mfma_f32_32x32x2_f32) for the five products, noise hashed into the operand tiles",
+        "note": "fp32 activations, coefficients and sums; the forward and the coefficient gradient each form z = x.N^T"}
+    del keep
+    if compare:
+        gf, gdx, gdc, keep = calls(_lib.RDB_ALGO_TILE)
+        res["general_kernels_that_form_w_tiles_ms"] = {"fwd": round(event_ms(gf, 5), 4), "dx": round(event_ms(gdx, 5), 4),
+                                                        "dcoef": round(event_ms(gdc, 5), 4)}
+        del keep
+        zz = torch.randn(Tl, k, device=dev)
+        res["vendor_gemm_on_the_factored_shapes_ms"] = {
+            "y = z.C^T": round(event_ms(lambda: torch.matmul(zz, C.t(), out=y), 20), 4),
+            "t = dy.C": round(event_ms(lambda: torch.matmul(dy, C, out=zz), 20), 4),
+            "dC = dy^T.z": round(event_ms(lambda: torch.matmul(dy.t(), zz), 20), 4)}
+    return res
+
+
 def gpt_step_config(event_ms, torch, dev, g):
     """GPT-2 small with random-backed linears: 12 layers, d = 768, 12 heads, vocab 50304, k = 256, seeds 0..47, bf16, batch
     8 x 1024 random token ids; one training step (forward + backward).  Attention, norms, embedding, head and loss are stock
@@ -279,6 +335,7 @@ def other_configs(event_ms, torch, L, _lib, dev):
     out["in4096_out4096_k16_fp32_matrix_coef"] = small
 
     out["in4096_out14336_k1024_T4096_bf16"] = llm_layer_config(event_ms, torch, L, _lib, dev, g)
+    out["in768_out3072_k256_T8192_fp32"] = f32_layer_config(event_ms, torch, L, _lib, dev, g)
 
     # ---- the reference's own (vector-coef, 1-D) form at the headline shape: W = Noise . c with ONE coefficient vector of length
     # k needs k hashes per weight element (604 M per regeneration here): the PRNG-bound regime.  Its data flow is the
@@ -335,6 +392,8 @@ def main():
     ap.add_argument("--llm-layer-only", action="store_true",
                     help="run only the 4096 -> 14336, k = 1024 layer (projection, forward, backward through the C ABI) and exit "
                          "(profiling runs)")
+    ap.add_argument("--f32-layer-only", action="store_true",
+                    help="time only the fp32 form of the headline layer (profiling runs)")
     ap.add_argument("--gpt-only", action="store_true",
                     help="run only the GPT-2 small training step with random-backed linears and exit (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -373,6 +432,9 @@ def main():
         del src, dst
     if args.gpt_only:
         print(json.dumps({"gpt2_small_12L_k256_seeds0to47_bf16_8x1024": gpt_step_config(make_event_ms(torch), torch, dev, g)}))
+        return
+    if args.f32_layer_only:
+        print(json.dumps({"in768_out3072_k256_T8192_fp32": f32_layer_config(make_event_ms(torch), torch, L, _lib, dev, g, compare=False)}))
         return
     if args.llm_layer_only:
         print(json.dumps({"in4096_out14336_k1024_T4096_bf16": llm_layer_config(make_event_ms(torch), torch, L, _lib, dev, g, vendor=False)}))

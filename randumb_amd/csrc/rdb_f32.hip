@@ -99,16 +99,20 @@ template <int ROWS, int SRC> struct FgOperand {
                 r[h] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, in ? (int)(off[h] + (uint32_t)stage * step) : (int)BUFFER_OOB, 0, 0));
             }
         } else {
-            // element j of the thread: contraction value kk0 + j * (FG_THREADS / ROWS) of the stage, one add apart in the first round
-            constexpr int KSTEP = FG_THREADS / ROWS;
-            const uint32_t inc = SRC == FG_NOISE_M ? PN1 : SQ5_N1;
-            uint32_t f = first + (uint32_t)(stage * FG_BK) * inc;
 #pragma unroll
-            for (int j = 0; j < NV * 4; ++j, f += (uint32_t)KSTEP * inc) {
-                const bool in = row_ok && k_begin + stage * FG_BK + kk0 + j * KSTEP < kend;
-                r[j >> 2][j & 3] = in ? sq5_unit(sq5_tail(f)) : 0.0f;
-            }
+            for (int j = 0; j < NV * 4; ++j) hash_piece(stage, j);
         }
+    }
+    // Noise sources: element j of the thread's NV * 4 values of a stage (contraction value kk0 + j * (FG_THREADS / ROWS), one add
+    // apart in the first round).  The main loop calls this between the matrix instructions of the stage before.
+    static constexpr bool HASHED = SRC == FG_NOISE_M || SRC == FG_NOISE_I;
+    __device__ __forceinline__ void hash_piece(int stage, int j)
+    {
+        constexpr int KSTEP = FG_THREADS / ROWS;
+        const uint32_t inc = SRC == FG_NOISE_M ? PN1 : SQ5_N1;
+        const uint32_t f = first + (uint32_t)(stage * FG_BK + j * KSTEP) * inc;
+        const bool in = row_ok && k_begin + stage * FG_BK + kk0 + j * KSTEP < kend;
+        r[j >> 2][j & 3] = in ? sq5_unit(sq5_tail(f)) : 0.0f;
     }
     __device__ __forceinline__ void store(float *__restrict__ tile) const
     {
@@ -166,9 +170,10 @@ template <int BM, int ASRC, int BSRC, bool BIAS> __global__ __launch_bounds__(FG
         pa.store(As);
         pb.store(Bs);
         __syncthreads();   // also: every wave is done reading the other buffer (the stage before this one)
-        if (s + 1 < nstage) {
-            pa.load(s + 1);
-            pb.load(s + 1);
+        const bool more = s + 1 < nstage;
+        if (more) {
+            if (!PA::HASHED) pa.load(s + 1);
+            if (!PB::HASHED) pb.load(s + 1);
         }
         const float *ap = As + g * PA::LD + wm * (BM / 2) + r, *bp = Bs + g * PB::LD + wn * 64 + r;
 #pragma unroll
@@ -182,6 +187,12 @@ template <int BM, int ASRC, int BSRC, bool BIAS> __global__ __launch_bounds__(FG
             for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
                 for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi], fb[ni], acc[mi][ni], 0, 0, 0);
+            // the next stage's noise values are hashed in the shadow of these matrix instructions, a share per k-step
+            if (PB::HASHED && more) {
+                constexpr int PER = (PB::NV * 4 + FG_BK / 2 - 1) / (FG_BK / 2);
+#pragma unroll
+                for (int j = ks * PER; j < (ks + 1) * PER && j < PB::NV * 4; ++j) pb.hash_piece(s + 1, j);
+            }
         }
     }
     // accumulator j of lane (r, g): row 8 (j / 4) + 4 g + j % 4 of the A side, column r of the B side
@@ -224,28 +235,33 @@ static bool fg_ok(const rdb_linear_desc *d)
 }
 static bool fg_wanted(const rdb_linear_desc *d) { return d->algo == RDB_ALGO_FACTORED || d->k * (d->in_f + d->out_f) < d->in_f * d->out_f; }
 
-// Token ranges of the coefficient gradient: enough blocks for about two per compute unit, ranges of at least 256 tokens.
-static int dc_splits(const rdb_linear_desc *d, int num_cus)
+// Tile height and number of contraction ranges of a product [M x N] over K.  Planned for two blocks per compute unit at a
+// time (the hardware takes up to four).  A product with fewer tiles than that is cut into ranges of the contraction (at least
+// min_range values each, at most max_ranges): each range leaves a partial matrix, added up in range order afterwards, so the
+// result does not depend on which block finishes first.  128-row tiles unless even in ranges they would leave half of the
+// compute units without a block; 64-row tiles then.
+struct FgPlan {
+    int bm, ranges;
+};
+static FgPlan fg_plan(int64_t M, int64_t N, int64_t K, int num_cus, int64_t min_range, int max_ranges)
 {
-    const int64_t tiles = cdiv(d->out_f, 128) * cdiv(d->k, FG_BN);
-    int64_t s = cdiv(2 * (int64_t)num_cus, tiles);
-    const int64_t most = cdiv(d->tokens, 256);
-    if (s > most) s = most;
-    if (s > 64) s = 64;
-    return s < 1 ? 1 : (int)s;
+    const int64_t slots = 2 * (int64_t)num_cus;
+    const int64_t t128 = cdiv(M, 128) * cdiv(N, FG_BN), t64 = cdiv(M, 64) * cdiv(N, FG_BN);
+    int64_t cap = K / min_range;
+    if (cap > max_ranges) cap = max_ranges;
+    if (cap < 1) cap = 1;
+    auto ranges = [&](int64_t tiles) {
+        int64_t r = slots / tiles;
+        if (r > cap) r = cap;
+        return r < 1 ? (int64_t)1 : r;
+    };
+    const int64_t r128 = ranges(t128), r64 = ranges(t64);
+    if (t128 * r128 * 2 < slots) return {64, (int)r64};
+    return {128, (int)r128};
 }
-
-// Ranges of the contraction of z = x . N^T and t = dy . C when their [tokens x k] output has too few tiles to give every
-// compute unit a block: each range leaves a partial matrix, added up in range order afterwards.  At least 128 values a range.
-static int zt_splits(const rdb_linear_desc *d, int64_t K, int num_cus)
-{
-    const int64_t tiles = cdiv(d->tokens, 64) * cdiv(d->k, FG_BN);
-    if (tiles >= num_cus) return 1;
-    int64_t s = cdiv(num_cus, tiles);
-    if (s > K / 128) s = K / 128;
-    if (s > 32) s = 32;
-    return s < 1 ? 1 : (int)s;
-}
+// z = x . N^T and t = dy . C, [tokens x k] over K = in_f or out_f; dC = dy^T . z, [out_f x k] over the tokens
+static FgPlan zt_plan(const rdb_linear_desc *d, int64_t K, int num_cus) { return fg_plan(d->tokens, d->k, K, num_cus, 128, 32); }
+static FgPlan dc_plan(const rdb_linear_desc *d, int num_cus) { return fg_plan(d->out_f, d->k, d->tokens, num_cus, 256, 64); }
 
 // scratch: z or t [tokens x k] and its partial matrices; for the coefficient gradient also one [out_f x k] matrix per token range
 int64_t linear_f32_workspace(int op, const rdb_linear_desc *d, int num_cus)
@@ -254,12 +270,12 @@ int64_t linear_f32_workspace(int op, const rdb_linear_desc *d, int num_cus)
     if (op == RDB_OP_LINEAR_BWD_DCOEF) dd.coef_dtype = RDB_F32;   // reads no coefficients
     if (!fg_ok(&dd)) return 0;
     const int64_t zt = up256(d->tokens * d->k * 4);
-    auto with_parts = [&](int64_t K) { const int s = zt_splits(d, K, num_cus); return zt * (s > 1 ? 1 + s : 1); };
+    auto with_parts = [&](int64_t K) { const int r = zt_plan(d, K, num_cus).ranges; return zt * (r > 1 ? 1 + r : 1); };
     if (op == RDB_OP_LINEAR_FWD) return with_parts(d->in_f);
     if (op == RDB_OP_LINEAR_BWD_DX) return with_parts(d->out_f);
     if (op != RDB_OP_LINEAR_BWD_DCOEF) return 0;
-    const int s = dc_splits(d, num_cus);
-    return with_parts(d->in_f) + (s > 1 ? (int64_t)s * up256(d->out_f * d->k * 4) : 0);
+    const int r = dc_plan(d, num_cus).ranges;
+    return with_parts(d->in_f) + (r > 1 ? (int64_t)r * up256(d->out_f * d->k * 4) : 0);
 }
 
 struct FgProduct {
@@ -271,6 +287,7 @@ struct FgProduct {
     int64_t ldo;
     const float *bias;
     int64_t M, N, K;
+    int bm;                 // tile height: 128 or 64
     int64_t kchunk;         // contraction values per range (a multiple of FG_BK); 0: one range
     int64_t split_stride;   // floats between the ranges' outputs
     uint32_t seed;
@@ -296,9 +313,7 @@ template <int ASRC, int BSRC> static int fg_launch(const FgProduct &q, int num_c
     p.b_bytes = q.b_elems * 4;
     p.seed = q.seed;
     const int splits = (int)cdiv(q.K, p.kchunk);
-    // 128-row tiles when they give every compute unit a block, 64-row tiles otherwise
-    const int64_t tiles128 = cdiv(q.M, 128) * cdiv(q.N, FG_BN) * splits;
-    if (tiles128 >= num_cus) {
+    if (q.bm == 128) {
         const dim3 grid((unsigned)cdiv(q.N, FG_BN), (unsigned)cdiv(q.M, 128), (unsigned)splits);
         if (q.bias) f32_gemm_kernel<128, ASRC, BSRC, true><<<grid, FG_THREADS, 0, s>>>(p);
         else f32_gemm_kernel<128, ASRC, BSRC, false><<<grid, FG_THREADS, 0, s>>>(p);
@@ -323,8 +338,10 @@ static int fg_sum(float *out, const float *part, int64_t n, int64_t stride, int 
 
 // A product whose dense output [M x N] (ldo = N) may be computed in `splits` ranges of the contraction: the ranges' partial
 // matrices go to `part` (stride floats apart) and are added up into q.out in range order.
-template <int ASRC, int BSRC> static int fg_launch_ranges(FgProduct q, int splits, float *part, int64_t stride, int num_cus, hipStream_t s, const char *name)
+template <int ASRC, int BSRC> static int fg_launch_ranges(FgProduct q, FgPlan plan, float *part, int64_t stride, int num_cus, hipStream_t s, const char *name)
 {
+    int splits = plan.ranges;
+    q.bm = plan.bm;
     const int kchunk = (int)(cdiv(cdiv(q.K, splits), FG_BK) * FG_BK);
     splits = (int)cdiv(q.K, kchunk);   // the ranges that hold something
     if (splits <= 1) {
@@ -343,9 +360,9 @@ template <int ASRC, int BSRC> static int fg_launch_ranges(FgProduct q, int split
 // z[T x k] = src[T x in_f] . N^T; the partial matrices of its ranges follow z in the workspace
 static int fg_project(float *z, const float *x, int64_t ldx, const rdb_linear_desc *d, int num_cus, hipStream_t s)
 {
-    FgProduct q = {x, ldx, (d->tokens - 1) * ldx + d->in_f, nullptr, 0, 0, z, d->k, nullptr, d->tokens, d->k, d->in_f, 0, 0, d->seed};
+    FgProduct q = {x, ldx, (d->tokens - 1) * ldx + d->in_f, nullptr, 0, 0, z, d->k, nullptr, d->tokens, d->k, d->in_f, 128, 0, 0, d->seed};
     const int64_t zt = up256(d->tokens * d->k * 4) / 4;
-    return fg_launch_ranges<FG_KCONT, FG_NOISE_M>(q, zt_splits(d, d->in_f, num_cus), z + zt, zt, num_cus, s, "f32_gemm_kernel (z = x . N^T)");
+    return fg_launch_ranges<FG_KCONT, FG_NOISE_M>(q, zt_plan(d, d->in_f, num_cus), z + zt, zt, num_cus, s, "f32_gemm_kernel (z = x . N^T)");
 }
 
 // The three entry points return RDB_E_UNSUPPORTED, without setting an error, when the request does not fit.
@@ -358,7 +375,7 @@ int linear_fwd_f32(void *y, int64_t ldy, const void *x, int64_t ldx, const void 
     float *z = (float *)workspace;
     if (int rc = fg_project(z, (const float *)x, ldx, d, num_cus, s)) return rc;
     FgProduct q = {z, d->k, d->tokens * d->k, (const float *)coef, d->k, d->out_f * d->k, (float *)y, ldy, (const float *)bias,
-                   d->tokens, d->out_f, d->k, 0, 0, d->seed};
+                   d->tokens, d->out_f, d->k, fg_plan(d->tokens, d->out_f, d->k, num_cus, d->k, 1).bm, 0, 0, d->seed};
     return fg_launch<FG_KCONT, FG_KCONT>(q, num_cus, s, "f32_gemm_kernel (y = z . C^T)");
 }
 
@@ -371,11 +388,12 @@ int linear_dx_f32(void *dx, int64_t lddx, const void *dy, int64_t lddy, const vo
     float *t = (float *)workspace;
     // t[T x k] = dy[T x out_f] . C: the B side's rows are coefficients, read across the rows of C
     FgProduct q1 = {(const float *)dy, lddy, (d->tokens - 1) * lddy + d->out_f, (const float *)coef, d->k, d->out_f * d->k, t, d->k, nullptr,
-                    d->tokens, d->k, d->out_f, 0, 0, d->seed};
+                    d->tokens, d->k, d->out_f, 128, 0, 0, d->seed};
     const int64_t zt = up256(d->tokens * d->k * 4) / 4;
-    if (int rc = fg_launch_ranges<FG_KCONT, FG_MCONT>(q1, zt_splits(d, d->out_f, num_cus), t + zt, zt, num_cus, s, "f32_gemm_kernel (t = dy . C)")) return rc;
+    if (int rc = fg_launch_ranges<FG_KCONT, FG_MCONT>(q1, zt_plan(d, d->out_f, num_cus), t + zt, zt, num_cus, s, "f32_gemm_kernel (t = dy . C)")) return rc;
     // dx[T x in_f] = t . N: the B side's rows are input features, hashed
-    FgProduct q2 = {t, d->k, d->tokens * d->k, nullptr, 0, 0, (float *)dx, lddx, nullptr, d->tokens, d->in_f, d->k, 0, 0, d->seed};
+    FgProduct q2 = {t, d->k, d->tokens * d->k, nullptr, 0, 0, (float *)dx, lddx, nullptr, d->tokens, d->in_f, d->k,
+                    fg_plan(d->tokens, d->in_f, d->k, num_cus, d->k, 1).bm, 0, 0, d->seed};
     return fg_launch<FG_KCONT, FG_NOISE_I>(q2, num_cus, s, "f32_gemm_kernel (dx = t . N)");
 }
 
@@ -392,11 +410,11 @@ int linear_dcoef_f32(float *dcoef, const void *dy, int64_t lddy, const void *x, 
     float *z = (float *)workspace;
     if (int rc = fg_project(z, (const float *)x, ldx, &dd, num_cus, s)) return rc;
     // dC[out_f x k] = dy^T . z: both sides are read across their rows (the contraction runs over the tokens)
-    const int zs = zt_splits(&dd, d->in_f, num_cus);
+    const int zs = zt_plan(&dd, d->in_f, num_cus).ranges;
     float *part = reinterpret_cast<float *>(static_cast<char *>(workspace) + up256(d->tokens * d->k * 4) * (zs > 1 ? 1 + zs : 1));
     FgProduct q = {(const float *)dy, lddy, (d->tokens - 1) * lddy + d->out_f, z, d->k, d->tokens * d->k, dcoef, d->k, nullptr,
-                   d->out_f, d->k, d->tokens, 0, 0, d->seed};
-    return fg_launch_ranges<FG_MCONT, FG_MCONT>(q, dc_splits(&dd, num_cus), part, up256(d->out_f * d->k * 4) / 4, num_cus, s, "f32_gemm_kernel (dC = dy^T . z)");
+                   d->out_f, d->k, d->tokens, 128, 0, 0, d->seed};
+    return fg_launch_ranges<FG_MCONT, FG_MCONT>(q, dc_plan(&dd, num_cus), part, up256(d->out_f * d->k * 4) / 4, num_cus, s, "f32_gemm_kernel (dC = dy^T . z)");
 }
 
 }  // namespace rdb

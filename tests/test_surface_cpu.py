@@ -130,18 +130,23 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     # fp32, small k: one partial [tokens x k] matrix per 256 values of the longer side, a 64-bit tag slot per tile of 8 tokens
     # and chunk, a word for a block that gave up waiting, and a counter per 16 tokens
     # ... or, for the fp32 matrix-core kernels (any k, sizes that are multiples of 4), z [tokens x k] rounded up to 256 bytes plus
-    # one partial matrix per range of the contraction when the [tokens x k] product has fewer 64 x 128 tiles than compute units
-    # (256 without a GPU): here one tile, 4096 / 128 = 32 ranges.  The query returns the larger of the two.
+    # one partial matrix per range of the contraction when the [tokens x k] product has fewer tiles than two per compute unit
+    # (256 units without a GPU; ranges of at least 128 values, at most 32): here one tile, 4096 / 128 = 32 ranges.  The query
+    # returns the larger of the two.
     f32 = desc(16, 4096, 4096, 16, act=_lib.RDB_F32, coef=_lib.RDB_F32)
     small_k = 16 * 16 * 16 * 4 + 2 * 16 * 8 + 8 + 8
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(f32)) == max(small_k, 1024 * (1 + 32))
     k128 = desc(16, 4096, 4096, 128, act=_lib.RDB_F32, coef=_lib.RDB_F32)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(k128)) == 16 * 128 * 4 * (1 + 32)
-    # enough tiles: no ranges; the coefficient gradient adds one [out_f x k] matrix per range of tokens (here 2 * 256 / 48 -> 11)
+    # 8192 tokens x 256 coefficients are 128 tiles of 128 x 128: four ranges; the coefficient gradient's 48 tiles: ten ranges of
+    # tokens, one [out_f x k] matrix each
     c2 = desc(8192, 768, 3072, 256, act=_lib.RDB_F32, coef=_lib.RDB_F32)
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(c2)) == 8192 * 256 * 4
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(c2)) == 8192 * 256 * 4
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DCOEF, ctypes.byref(c2)) == 8192 * 256 * 4 + 11 * 3072 * 256 * 4
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(c2)) == 8192 * 256 * 4 * (1 + 4)
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(c2)) == 8192 * 256 * 4 * (1 + 4)
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DCOEF, ctypes.byref(c2)) == 8192 * 256 * 4 * (1 + 4) + 10 * 3072 * 256 * 4
+    # enough tiles: no ranges
+    wide = desc(65536, 768, 3072, 256, act=_lib.RDB_F32, coef=_lib.RDB_F32)
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(wide)) == 65536 * 256 * 4
     # extents that are not multiples of 4 stay with the general kernel: no scratch
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(16, 4096, 4094, 128, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 0
 
