@@ -8,7 +8,10 @@ through ``RandumbTensorConstructor``.  Differences, all additive:
 * ``coefs`` may be 2-D (matrix-coef form, one coef row per row of a ``(rows, row_len)`` tensor);
 * ``aten.mm`` / ``aten.addmm`` against a dense CUDA matrix run the fused kernels, which regenerate the weight
   on chip instead of writing it to memory first (the reference materialises and calls a dense product,
-  RandumbTensor.py:942-946).  ``RandumbTensor.FUSED_MM = False`` restores materialise-then-matmul;
+  RandumbTensor.py:942-946).  ``RandumbTensor.FUSED_MM = False`` restores materialise-then-matmul.  Vector-coef tensors
+  (the reference's form: k hashes per weight element) take materialise-then-matmul by default, because a fused product has
+  to regenerate the whole weight for every block of 128 rows of the other matrix; ``RandumbTensor.FUSED_MM_VECTOR = True``
+  gives them the fused kernels too (no transient weight in memory, at the price of that regeneration);
 * ``_to_copy(dtype=...)`` yields a tensor that reports, and materialises to, the requested dtype.
 """
 from __future__ import annotations
@@ -44,6 +47,7 @@ class RandumbTensor(torch.Tensor):
     """
 
     FUSED_MM = True
+    FUSED_MM_VECTOR = False
 
     @staticmethod
     def __new__(cls, data: torch.Tensor, seed: int, shape: Union[tuple, torch.Size], scale_bias: Optional[torch.Tensor],
@@ -132,7 +136,7 @@ class RandumbTensor(torch.Tensor):
 
     # -------------------------------------------------------------------------------------------- fused products
     def _fused_ok(self, other) -> bool:
-        return (type(self).FUSED_MM and self.dim() == 2 and isinstance(other, torch.Tensor)
+        return (type(self).FUSED_MM and (self.coef_rows or type(self).FUSED_MM_VECTOR) and self.dim() == 2 and isinstance(other, torch.Tensor)
                 and not isinstance(other, RandumbTensor) and other.is_cuda and other.dim() == 2
                 and other.dtype in (torch.float32, torch.bfloat16) and other.dtype == self.dtype)
 

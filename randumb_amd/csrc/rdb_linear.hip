@@ -528,10 +528,19 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
     if ((d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) && !d_scale_bias) {
         rc = linear_dcoef_factored(dcoef, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
+        // fp32: the vector-ALU kernel's coefficient gradient grows with the tokens (49 us at 256 tokens, 158 us at 1024 for
+        // 784 -> 512, k = 64; the matrix-core kernels take 39 us at 1028), so beyond 128 tokens the matrix cores come first
+        const bool matrix_cores_first = d->tokens > 128;
+        if (matrix_cores_first) {
+            rc = linear_dcoef_f32(dcoef, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
+            if (rc != RDB_E_UNSUPPORTED) return rc;
+        }
         rc = linear_dcoef_smallk(dcoef, dy, lddy, x, ldx, d, workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
-        rc = linear_dcoef_f32(dcoef, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
-        if (rc != RDB_E_UNSUPPORTED) return rc;
+        if (!matrix_cores_first) {
+            rc = linear_dcoef_f32(dcoef, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
+            if (rc != RDB_E_UNSUPPORTED) return rc;
+        }
     }
     if (d->algo == RDB_ALGO_FACTORED)
         return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dcoef: the factored algorithm needs matrix-coef, no scale_bias gradient, a "

@@ -371,7 +371,11 @@ static int contract_expand(float *out, int64_t ld_out, int cols, const float *sr
 int linear_fwd_smallk(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
                       const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
-    if (!smallk_ok(d) || scale_bias || !smallk_wanted(d) || !ws_ok(d, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    // a layer with a handful of output features (a classifier head) gives the kernel that forms W tiles one column of blocks,
+    // each hashing all of N: the factored form wins there whatever the flop counts say (256 -> 10, k = 64, 128 tokens: 19 us
+    // against 57)
+    const bool few_outputs = d->tokens <= 1024 && d->out_f <= 32;
+    if (!smallk_ok(d) || scale_bias || !(smallk_wanted(d) || few_outputs) || !ws_ok(d, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
     // z = x . N^T (hashed), y = z . C^T + bias
     return contract_expand<true>((float *)y, ldy, (int)d->out_f, (const float *)x, ldx, (int)d->in_f, (const float *)coef, (const float *)bias, d,
                                  workspace, s);

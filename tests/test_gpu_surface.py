@@ -68,15 +68,25 @@ def test_dispatch_semantics(ra, oracle):
     assert (rt.to(torch.bfloat16) + 0).dtype == torch.bfloat16
     x = torch.randn(5, 10).cuda()
     want = cpu(x).astype(np.float64) @ W.T.astype(np.float64)
-    assert rel_l2(cpu(x @ rt.t()), want) < F32_TOL              # fused mat1 @ tensor
-    assert rel_l2(cpu(F.linear(x, rt)), want) < F32_TOL
     z = torch.randn(10, 4).cuda()
-    assert rel_l2(cpu(rt @ z), W.astype(np.float64) @ cpu(z).astype(np.float64)) < F32_TOL   # tensor @ mat2
-    ra.RandumbTensor.FUSED_MM = False
+    # a vector-coef tensor: materialise-then-matmul (the reference's data flow) unless the fused kernels are asked for
+    assert not ra.RandumbTensor.FUSED_MM_VECTOR
+    assert rel_l2(cpu(x @ rt.t()), want) < F32_TOL
+    ra.RandumbTensor.FUSED_MM_VECTOR = True
     try:
-        assert rel_l2(cpu(x @ rt.t()), want) < F32_TOL          # materialise-then-matmul, the reference's data flow
+        assert rt._fused_ok(x)
+        assert rel_l2(cpu(x @ rt.t()), want) < F32_TOL              # fused mat1 @ tensor
+        assert rel_l2(cpu(F.linear(x, rt)), want) < F32_TOL
+        assert rel_l2(cpu(rt @ z), W.astype(np.float64) @ cpu(z).astype(np.float64)) < F32_TOL   # tensor @ mat2
+        ra.RandumbTensor.FUSED_MM = False
+        try:
+            assert not rt._fused_ok(x)
+            assert rel_l2(cpu(x @ rt.t()), want) < F32_TOL
+        finally:
+            ra.RandumbTensor.FUSED_MM = True
     finally:
-        ra.RandumbTensor.FUSED_MM = True
+        ra.RandumbTensor.FUSED_MM_VECTOR = False
+    assert not rt._fused_ok(x)
     # fused random bias
     sb = torch.tensor([0.3]).cuda()
     rtb = ra.CreateRandumbTensor(c, seed, (6, 10), sb, True)
