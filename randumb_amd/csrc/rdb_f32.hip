@@ -233,7 +233,9 @@ static bool fg_ok(const rdb_linear_desc *d)
            d->k % 4 == 0 && d->in_f % 4 == 0 && d->out_f % 4 == 0 && d->tokens * d->k < (1ll << 29) && d->out_f * d->k < (1ll << 29) &&
            d->in_f < (1 << 30) && d->out_f < (1 << 30);
 }
-static bool fg_wanted(const rdb_linear_desc *d) { return d->algo == RDB_ALGO_FACTORED || d->k * (d->in_f + d->out_f) < d->in_f * d->out_f; }
+// Wanted whenever the shapes fit: what AUTO would run instead is the general kernel, which forms W tiles on the vector ALU at a
+// few TFLOP/s, so the factored form on the matrix cores wins also where it is more flops than a product on a stored W.
+static bool fg_wanted(const rdb_linear_desc *) { return true; }
 
 // Tile height and number of contraction ranges of a product [M x N] over K.  Planned for two blocks per compute unit at a
 // time (the hardware takes up to four).  A product with fewer tiles than that is cut into ranges of the contraction (at least

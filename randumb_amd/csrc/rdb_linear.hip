@@ -334,6 +334,7 @@ int linear_bwd_big(void *t, float *dc, const void *dy, int64_t lddy, const void 
 
 // rdb_rbias.hip
 int linear_dx_rbias_add(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *scale_bias, const rdb_linear_desc *d, hipStream_t s);
+int linear_fwd_rbias_add(void *y, int64_t ldy, const void *x, int64_t ldx, const void *scale_bias, const rdb_linear_desc *d, hipStream_t s);
 
 // rdb_dcoef.hip
 int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d,
@@ -432,6 +433,18 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
             return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd: the strip algorithm needs matrix-coef, bf16 activations, in_f %% 8 == 0, "
                                                 "16-byte aligned x rows and a weight strip that fits LDS");
     }
+    if (d->algo == RDB_ALGO_AUTO && scale_bias && d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16) {
+        // W = C.N + s.R where no weight strip fits on chip (a long in_f): the low-rank share through the factored kernels, then
+        // the random-bias share added on top (3072 -> 768, k = 256, 8192 tokens: 3.0 ms for the general kernel below)
+        rdb_linear_desc df = *d;
+        df.algo = RDB_ALGO_FACTORED;
+        rc = linear_fwd_factored(y, ldy, x, ldx, coef, nullptr, bias, &df, num_compute_units(), workspace, workspace_bytes, s);
+        if (rc == RDB_OK) {
+            rc = linear_fwd_rbias_add(y, ldy, x, ldx, scale_bias, d, s);
+            if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd: internal: the random-bias share refused a request the factored share took");
+        }
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
     const int es = d->act_dtype == RDB_BF16 ? 2 : 4;
     LinParams p = {};
     p.w = make_spec(d, coef, scale_bias);
@@ -462,7 +475,9 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
     if (d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) {
         if (scale_bias && d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16 && d->tokens * lddx < (1ll << 29)) {
             // W = C.N + s.R: the low-rank share through the factored kernels, then the random-bias share added on top
-            rc = linear_dx_factored(dx, lddx, dy, lddy, coef, nullptr, d, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
+            rdb_linear_desc df = *d;
+            df.algo = RDB_ALGO_FACTORED;   // also where it is more flops than a product on a stored W: the alternative is the general kernel
+            rc = linear_dx_factored(dx, lddx, dy, lddy, coef, nullptr, &df, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
             if (rc == RDB_OK) {
                 rc = linear_dx_rbias_add(dx, lddx, dy, lddy, scale_bias, d, (hipStream_t)stream);
                 if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dx: internal: the random-bias share refused a request the factored share took");
@@ -486,6 +501,15 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
         if (d->algo == RDB_ALGO_STRIP)
             return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dx: the strip algorithm needs matrix-coef in bf16 with k <= 256, bf16 "
                                                 "activations, no scale_bias, sizes that are multiples of 8 and aligned rows");
+    }
+    if (d->algo == RDB_ALGO_AUTO) {
+        // Nothing above took it (k > 256, say, where no kernel re-forms W for the input gradient on the matrix cores): the
+        // factored form's two products are still far ahead of the general kernel below, also where they are more flops than
+        // one product on a stored W would be (2048 tokens, 1024 -> 1024, k = 512, bf16: 1.06 ms for the general kernel).
+        rdb_linear_desc df = *d;
+        df.algo = RDB_ALGO_FACTORED;
+        rc = linear_dx_factored(dx, lddx, dy, lddy, coef, scale_bias, &df, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
     }
     const int es = d->act_dtype == RDB_BF16 ? 2 : 4;
     LinParams p = {};

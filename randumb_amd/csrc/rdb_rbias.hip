@@ -1,11 +1,12 @@
-// The fused random bias in the fast input-gradient path.
+// The fused random bias beside the factored kernels.
 //
 // With scale_bias the weight is W = C . N + s . R,  R[o, i] = noise1d(o*in_f + i)  (src/rten_cpp/RandumbTensor.py:286-289;
 // it is what the reference's default initialisation starts from: zero coefficients, random bias,
 // src/rten_cpp/SillyLayers.py:122-133, 218-221).  R is a full-rank pseudorandom matrix, so its share of a product is a
 // dense contraction whatever is done about C . N; the low-rank share keeps its factored kernels and this file adds
-//     dx[t, i] += s * sum_o dy[t, o] * R[o, i]
-// on the tile engine with R as a hashed operand: a tile of 64 input features x 256 tokens, R hashed once per block and
+//     dx[t, i] += s * sum_o dy[t, o] * R[o, i]        (input gradient)
+//     y[t, o]  += s * sum_i x[t, i]  * R[o, i]        (forward, where no kernel that forms W strips fits)
+// on the tile engine with R as a hashed operand: a tile of 64 features x 256 tokens, R hashed once per block and
 // stage straight into the pipeline's registers (as 2^31 * noise in bf16, the scale folded into the epilogue), two blocks
 // per compute unit so that one block's hashing runs under the other's matrix work.  R never exists in memory.
 #include "rdb_gemm.hpp"
@@ -42,17 +43,20 @@ template <int ROWS, int BK> struct Noise1DOperand {
     }
 };
 
-struct RBiasDxParams {
-    const bf16_t *dy;
+// dst[t, a] += s * sum_c src[t, c] * noise1d(a * sR + c * sK):  the input gradient has a = input feature, c = output feature
+// (sR = 1, sK = in_f), the forward a = output feature, c = input feature (sR = in_f, sK = 1).
+struct RBiasParams {
+    const bf16_t *dy;           // src [tokens x out_f (contraction)]
     const bf16_t *scale_bias;   // one bf16 value
-    bf16_t *dx;
+    bf16_t *dx;                 // dst [tokens x in_f (columns)]
     int64_t lddy, lddx;
-    int tokens, in_f, out_f;
+    int tokens, in_f, out_f;    // in_f: columns of dst, out_f: contraction length
     int tiles_i, tiles_t;
+    uint32_t sR, sK;
     uint32_t seed;
 };
 
-__global__ __launch_bounds__(256, 2) void rbias_dx_add_kernel(RBiasDxParams p)
+__global__ __launch_bounds__(256, 2) void rbias_add_kernel(RBiasParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
@@ -66,9 +70,9 @@ __global__ __launch_bounds__(256, 2) void rbias_dx_add_kernel(RBiasDxParams p)
     for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = zero16();
-    // "A": 2^31 * R[o, i], rows = i, contraction = o: the noise index o*in_f + i moves by 1 per row and by in_f per k
-    Noise1DOperand<RB_BI, RB_BK> opr = {i0, 1u, (uint32_t)p.in_f, p.seed};
-    // "B": dy[tok][o]; output rows past out_f read as zeros, whatever the hash says there
+    // "A": 2^31 * R, rows = columns of dst: the noise index moves by sR per row and by sK per contraction value
+    Noise1DOperand<RB_BI, RB_BK> opr = {i0, p.sR, p.sK, p.seed};
+    // "B": src[tok][c]; contraction values past the end read as zeros, whatever the hash says there
     GlobalOperand<RB_BT, RB_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
     gemm_mainloop<RB_BI, RB_BT, RB_BK, 1, 2, 1>(acc, lds, opr, opdy, 0, (p.out_f + RB_BK - 1) / RB_BK);
     // dx += s * 2^-31 * acc, through LDS as fp32 so that every lane updates 8 consecutive features of a token's row
@@ -106,30 +110,44 @@ __global__ __launch_bounds__(256, 2) void rbias_dx_add_kernel(RBiasDxParams p)
     }
 }
 
-// dx += s * dy . R on the launch stream, after the kernels that wrote dx.  Returns RDB_E_UNSUPPORTED (without setting an
-// error) when the request does not fit.
-int linear_dx_rbias_add(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *scale_bias, const rdb_linear_desc *d, hipStream_t s)
+static int rbias_add(void *dst, int64_t ld_dst, int64_t cols, const void *src, int64_t ld_src, int64_t contraction, uint32_t sR, uint32_t sK,
+                     const void *scale_bias, const rdb_linear_desc *d, hipStream_t s)
 {
     if (d->act_dtype != RDB_BF16 || d->coef_dtype != RDB_BF16 || d->coef_rows == 0 || !scale_bias) return RDB_E_UNSUPPORTED;
     if (d->in_f % 8 || d->out_f % 8 || d->tokens < 1 || d->in_f < 1 || d->out_f < 1) return RDB_E_UNSUPPORTED;
-    if (lddy % 8 || lddx % 8 || ((uintptr_t)dy & 15) || ((uintptr_t)dx & 15)) return RDB_E_UNSUPPORTED;
-    if (d->tokens * lddy >= (1ll << 29) || d->tokens * lddx >= (1ll << 29)) return RDB_E_UNSUPPORTED;
-    RBiasDxParams p;
-    p.dy = (const bf16_t *)dy;
+    if (ld_src % 8 || ld_dst % 8 || ((uintptr_t)src & 15) || ((uintptr_t)dst & 15)) return RDB_E_UNSUPPORTED;
+    if (d->tokens * ld_src >= (1ll << 29) || d->tokens * ld_dst >= (1ll << 29)) return RDB_E_UNSUPPORTED;
+    RBiasParams p;
+    p.dy = (const bf16_t *)src;
     p.scale_bias = (const bf16_t *)scale_bias;
-    p.dx = (bf16_t *)dx;
-    p.lddy = lddy;
-    p.lddx = lddx;
+    p.dx = (bf16_t *)dst;
+    p.lddy = ld_src;
+    p.lddx = ld_dst;
     p.tokens = (int)d->tokens;
-    p.in_f = (int)d->in_f;
-    p.out_f = (int)d->out_f;
-    p.tiles_i = (int)cdiv(d->in_f, RB_BI);
+    p.in_f = (int)cols;
+    p.out_f = (int)contraction;
+    p.tiles_i = (int)cdiv(cols, RB_BI);
     p.tiles_t = (int)cdiv(d->tokens, RB_BT);
+    p.sR = sR;
+    p.sK = sK;
     p.seed = d->seed;
     size_t smem = engine_smem<RB_BI, RB_BT, RB_BK, K_CONT, K_CONT>();
     const size_t stage = (size_t)RB_BT * (RB_BI + 4) * sizeof(float);
     if (smem < stage) smem = stage;
-    return launch_engine(rbias_dx_add_kernel, p, p.tiles_i * p.tiles_t, smem, s, "rbias_dx_add_kernel");
+    return launch_engine(rbias_add_kernel, p, p.tiles_i * p.tiles_t, smem, s, "rbias_add_kernel");
+}
+
+// dx += s * dy . R on the launch stream, after the kernels that wrote dx.  Returns RDB_E_UNSUPPORTED (without setting an
+// error) when the request does not fit.
+int linear_dx_rbias_add(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *scale_bias, const rdb_linear_desc *d, hipStream_t s)
+{
+    return rbias_add(dx, lddx, d->in_f, dy, lddy, d->out_f, 1u, (uint32_t)d->in_f, scale_bias, d, s);
+}
+
+// y += s * x . R^T on the launch stream, after the kernels that wrote y; same conditions.
+int linear_fwd_rbias_add(void *y, int64_t ldy, const void *x, int64_t ldx, const void *scale_bias, const rdb_linear_desc *d, hipStream_t s)
+{
+    return rbias_add(y, ldy, d->out_f, x, ldx, d->in_f, (uint32_t)d->in_f, 1u, scale_bias, d, s);
 }
 
 }  // namespace rdb

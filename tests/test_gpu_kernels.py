@@ -483,7 +483,12 @@ def test_factored_dx_needs_what_it_says(hip):
         hip.linear_bwd_dcoef(dy, x, 16, 48, 40, 48, 40, 1, 0, want_scale_bias_grad=True, algo=RDB_ALGO_FACTORED)
 
 
-@pytest.mark.parametrize("T,in_f,out_f,k", [(2048, 768, 3072, 256), (200, 72, 136, 40)])
+@pytest.mark.parametrize("T,in_f,out_f,k", [
+    (2048, 768, 3072, 256),
+    (200, 72, 136, 40),
+    (1024, 3072, 768, 256),   # in_f too long for a weight strip on chip: factored forward + the random-bias share added on top
+    (512, 1024, 1024, 512),   # k > 256 and the factored form not the cheaper one in flops: still the one that runs
+])
 def test_default_layer_fast_path_with_scale_bias(hip, oracle, T, in_f, out_f, k):
     """The reference's default layer starts from zero coefficients and a fused random bias (SillyLayers.py:122-133, 218-221):
     W = C.N + s.noise1d.  Forward, input gradient (factored share + hashed random-bias share), coefficient gradient and the
