@@ -8,6 +8,9 @@
 // N[m, i] = noise(PRIME*i + m) is hashed into the pipeline's LDS tiles and never stored; W = C . N is never formed.  All
 // five products run on one kernel template that differs in where its two operands come from (a row-major matrix read along
 // or across its rows, or the hash).  Everything is fp32: operands, products and sums.
+// With scale_bias (W = C . N + s . R, R[o, i] = noise1d(o*in_f + i), full rank: src/rten_cpp/RandumbTensor.py:286-289) the
+// random-bias share is one more product with R as the hashed operand, added on top:  y += s * x . R^T,  dx += s * dy . R,  and
+// the gradient of s is <dy, x . R^T>, summed tile by tile in the epilogue of that product and block by block afterwards.
 // Replaces materialize() + dense product (src/rten_cpp/RandumbTensor.py:942-946) and MmBackward's dW followed by
 // materialize_bwd (RandumbTensor.py:979-990, 304-359) for fp32 layers beyond the few-token regime of rdb_smallk.hip.
 #include "rdb_gemm.hpp"
@@ -24,7 +27,15 @@ enum FgSource {
     FG_KCONT = 0,    // src[row * ld + kk]: a row-major matrix whose rows are the tile's rows
     FG_MCONT = 1,    // src[kk * ld + row]: a row-major matrix whose rows are contraction values
     FG_NOISE_M = 2,  // 2-D noise (feature kk, coefficient row): the rows are coefficients, the contraction runs over features
-    FG_NOISE_I = 3   // 2-D noise (feature row, coefficient kk): the rows are features, the contraction runs over coefficients
+    FG_NOISE_I = 3,  // 2-D noise (feature row, coefficient kk): the rows are features, the contraction runs over coefficients
+    FG_NOISE_1D = 4  // 1-D noise at index row * sR + kk * sK: the random-bias matrix R, read along or across its rows
+};
+// What a block does with its accumulators.
+enum FgEpilogue {
+    FG_STORE = 0,       // out = acc
+    FG_STORE_BIAS = 1,  // out = acc + bias[column]
+    FG_ADD_SCALED = 2,  // out += scale[0] * acc
+    FG_DOT = 3          // dot_part[block] = sum over the tile of acc * dotm (nothing is stored to out)
 };
 
 struct FgParams {
@@ -39,6 +50,11 @@ struct FgParams {
     int kchunk;          // contraction values per split (a multiple of FG_BK); K when there is one split
     int64_t a_bytes, b_bytes;   // extent of the matrices, for the bounds check of the loads (< 2^31)
     uint32_t seed;
+    uint32_t nsR, nsK;          // FG_NOISE_1D: index steps per row and per contraction value
+    const float *scale;         // FG_ADD_SCALED: one device value
+    const float *dotm;          // FG_DOT: [M x N] matrix, leading dimension lddot
+    int64_t lddot;
+    float *dot_part;            // FG_DOT: one value per block, in block order (x fastest, then y)
 };
 
 // One operand's way from its source into LDS: load(stage) requests / hashes the stage's values into registers, store() puts
@@ -53,7 +69,9 @@ template <int ROWS, int SRC> struct FgOperand {
     int kk0, kend, k_begin, row_ok;
     f32x4 r[NV];
 
-    __device__ __forceinline__ void init(const float *src, int64_t ld, int64_t bytes, int row0, int rows, int k_begin_, int kend_, uint32_t seed)
+    uint32_t inc;       // noise: first-round step per contraction value
+    __device__ __forceinline__ void init(const float *src, int64_t ld, int64_t bytes, int row0, int rows, int k_begin_, int kend_, uint32_t seed,
+                                         uint32_t sR, uint32_t sK)
     {
         const int t = threadIdx.x;
         k_begin = k_begin_;
@@ -80,8 +98,14 @@ template <int ROWS, int SRC> struct FgOperand {
             const int row = t % ROWS;
             kk0 = t / ROWS;
             row_ok = row0 + row < rows;
-            first = SRC == FG_NOISE_M ? sq5_first((uint32_t)(k_begin + kk0), (uint32_t)(row0 + row), seed)
-                                      : sq5_first((uint32_t)(row0 + row), (uint32_t)(k_begin + kk0), seed);
+            if (SRC == FG_NOISE_1D) {
+                first = ((uint32_t)(row0 + row) * sR + (uint32_t)(k_begin + kk0) * sK) * SQ5_N1 + seed;
+                inc = sK * SQ5_N1;
+            } else {
+                first = SRC == FG_NOISE_M ? sq5_first((uint32_t)(k_begin + kk0), (uint32_t)(row0 + row), seed)
+                                          : sq5_first((uint32_t)(row0 + row), (uint32_t)(k_begin + kk0), seed);
+                inc = SRC == FG_NOISE_M ? PN1 : SQ5_N1;
+            }
         }
     }
     __device__ __forceinline__ void load(int stage)
@@ -105,11 +129,10 @@ template <int ROWS, int SRC> struct FgOperand {
     }
     // Noise sources: element j of the thread's NV * 4 values of a stage (contraction value kk0 + j * (FG_THREADS / ROWS), one add
     // apart in the first round).  The main loop calls this between the matrix instructions of the stage before.
-    static constexpr bool HASHED = SRC == FG_NOISE_M || SRC == FG_NOISE_I;
+    static constexpr bool HASHED = SRC == FG_NOISE_M || SRC == FG_NOISE_I || SRC == FG_NOISE_1D;
     __device__ __forceinline__ void hash_piece(int stage, int j)
     {
         constexpr int KSTEP = FG_THREADS / ROWS;
-        const uint32_t inc = SRC == FG_NOISE_M ? PN1 : SQ5_N1;
         const uint32_t f = first + (uint32_t)(stage * FG_BK + j * KSTEP) * inc;
         const bool in = row_ok && k_begin + stage * FG_BK + kk0 + j * KSTEP < kend;
         r[j >> 2][j & 3] = in ? sq5_unit(sq5_tail(f)) : 0.0f;
@@ -142,7 +165,7 @@ template <int ROWS, int SRC> struct FgOperand {
 // out[M x N] (+)= A . B^T over one split of the contraction.  Block: BM x 128 of the output, four waves as 2 x 2, a wave owns
 // (BM / 2) x 64 in BM / 64 x 2 accumulator tiles.  Two LDS buffers, one barrier per stage: while a stage is multiplied the
 // next one is on its way from memory (or being hashed) in registers.
-template <int BM, int ASRC, int BSRC, bool BIAS> __global__ __launch_bounds__(FG_THREADS, 2) void f32_gemm_kernel(FgParams p)
+template <int BM, int ASRC, int BSRC, int EPI> __global__ __launch_bounds__(FG_THREADS, 2) void f32_gemm_kernel(FgParams p)
 {
     typedef FgOperand<BM, ASRC> PA;
     typedef FgOperand<FG_BN, BSRC> PB;
@@ -154,8 +177,8 @@ template <int BM, int ASRC, int BSRC, bool BIAS> __global__ __launch_bounds__(FG
     const int nstage = (kend - k_begin + FG_BK - 1) / FG_BK;
     PA pa;
     PB pb;
-    pa.init(p.a, p.lda, p.a_bytes, m0, p.M, k_begin, kend, p.seed);
-    pb.init(p.b, p.ldb, p.b_bytes, n0, p.N, k_begin, kend, p.seed);
+    pa.init(p.a, p.lda, p.a_bytes, m0, p.M, k_begin, kend, p.seed, p.nsR, p.nsK);
+    pb.init(p.b, p.ldb, p.b_bytes, n0, p.N, k_begin, kend, p.seed, p.nsR, p.nsK);
     f32x16 acc[MI][NI];
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
@@ -197,19 +220,48 @@ template <int BM, int ASRC, int BSRC, bool BIAS> __global__ __launch_bounds__(FG
     }
     // accumulator j of lane (r, g): row 8 (j / 4) + 4 g + j % 4 of the A side, column r of the B side
     float *out = p.out + (int64_t)blockIdx.z * p.split_stride;
+    const float scale = EPI == FG_ADD_SCALED ? p.scale[0] : 0.0f;
+    float dot = 0.0f;
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni) {
         const int n = n0 + wn * 64 + ni * 32 + r;
         if (n >= p.N) continue;
-        const float bv = BIAS ? p.bias[n] : 0.0f;
+        const float bv = EPI == FG_STORE_BIAS ? p.bias[n] : 0.0f;
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
                 const int m = m0 + wm * (BM / 2) + mi * 32 + 8 * (j >> 2) + 4 * g + (j & 3);
-                if (m < p.M) out[(int64_t)m * p.ldo + n] = acc[mi][ni][j] + bv;
+                if (m >= p.M) continue;
+                if (EPI == FG_DOT) dot = fmaf(acc[mi][ni][j], p.dotm[(int64_t)m * p.lddot + n], dot);
+                else if (EPI == FG_ADD_SCALED) out[(int64_t)m * p.ldo + n] = fmaf(scale, acc[mi][ni][j], out[(int64_t)m * p.ldo + n]);
+                else out[(int64_t)m * p.ldo + n] = acc[mi][ni][j] + bv;
             }
     }
+    if (EPI == FG_DOT) {
+        // lanes, then waves, in a fixed order
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) dot += __shfl_xor(dot, o);
+        __syncthreads();   // the stage buffers are free
+        if (lane == 0) lds[wave] = dot;
+        __syncthreads();
+        if (t == 0) p.dot_part[(int64_t)blockIdx.y * gridDim.x + blockIdx.x] = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+    }
+}
+
+// out[0] = part[0] + part[1] + ... : one block, every thread a strided share in index order, then the shares in thread order
+__global__ __launch_bounds__(256) void f32_sum_scalars_kernel(float *__restrict__ out, const float *__restrict__ part, int n)
+{
+    __shared__ float sh[256];
+    float v = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 256) v += part[i];
+    sh[threadIdx.x] = v;
+    __syncthreads();
+    for (int w = 128; w >= 1; w >>= 1) {
+        if ((int)threadIdx.x < w) sh[threadIdx.x] += sh[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = sh[0];
 }
 
 // out[i] = part[0][i] + part[1][i] + ... in split order, four values per thread
@@ -277,7 +329,8 @@ int64_t linear_f32_workspace(int op, const rdb_linear_desc *d, int num_cus)
     if (op == RDB_OP_LINEAR_BWD_DX) return with_parts(d->out_f);
     if (op != RDB_OP_LINEAR_BWD_DCOEF) return 0;
     const int r = dc_plan(d, num_cus).ranges;
-    return with_parts(d->in_f) + (r > 1 ? (int64_t)r * up256(d->out_f * d->k * 4) : 0);
+    // ... and, for the gradient of the random bias's scale, one value per 64 x 128 tile of [tokens x out_f]
+    return with_parts(d->in_f) + (r > 1 ? (int64_t)r * up256(d->out_f * d->k * 4) : 0) + up256(cdiv(d->tokens, 64) * cdiv(d->out_f, FG_BN) * 4);
 }
 
 struct FgProduct {
@@ -293,6 +346,12 @@ struct FgProduct {
     int64_t kchunk;         // contraction values per range (a multiple of FG_BK); 0: one range
     int64_t split_stride;   // floats between the ranges' outputs
     uint32_t seed;
+    // the random-bias products (FG_NOISE_1D on the B side): index steps, and what the epilogue does
+    uint32_t nsR, nsK;
+    const float *scale;     // out += scale[0] * product
+    const float *dotm;      // or: dot_part[block] = <product tile, dotm tile>
+    int64_t lddot;
+    float *dot_part;
 };
 
 template <int ASRC, int BSRC> static int fg_launch(const FgProduct &q, int num_cus, hipStream_t s, const char *name)
@@ -314,15 +373,28 @@ template <int ASRC, int BSRC> static int fg_launch(const FgProduct &q, int num_c
     p.a_bytes = q.a_elems * 4;
     p.b_bytes = q.b_elems * 4;
     p.seed = q.seed;
+    p.nsR = q.nsR;
+    p.nsK = q.nsK;
+    p.scale = q.scale;
+    p.dotm = q.dotm;
+    p.lddot = q.lddot;
+    p.dot_part = q.dot_part;
     const int splits = (int)cdiv(q.K, p.kchunk);
-    if (q.bm == 128) {
-        const dim3 grid((unsigned)cdiv(q.N, FG_BN), (unsigned)cdiv(q.M, 128), (unsigned)splits);
-        if (q.bias) f32_gemm_kernel<128, ASRC, BSRC, true><<<grid, FG_THREADS, 0, s>>>(p);
-        else f32_gemm_kernel<128, ASRC, BSRC, false><<<grid, FG_THREADS, 0, s>>>(p);
+    const dim3 grid((unsigned)cdiv(q.N, FG_BN), (unsigned)cdiv(q.M, q.bm), (unsigned)splits);
+    if (BSRC == FG_NOISE_1D) {   // the random-bias products: added on top of an output, or reduced against a matrix
+        if (q.bm == 128) {
+            if (q.dotm) f32_gemm_kernel<128, ASRC, BSRC, FG_DOT><<<grid, FG_THREADS, 0, s>>>(p);
+            else f32_gemm_kernel<128, ASRC, BSRC, FG_ADD_SCALED><<<grid, FG_THREADS, 0, s>>>(p);
+        } else {
+            if (q.dotm) f32_gemm_kernel<64, ASRC, BSRC, FG_DOT><<<grid, FG_THREADS, 0, s>>>(p);
+            else f32_gemm_kernel<64, ASRC, BSRC, FG_ADD_SCALED><<<grid, FG_THREADS, 0, s>>>(p);
+        }
+    } else if (q.bm == 128) {
+        if (q.bias) f32_gemm_kernel<128, ASRC, BSRC, FG_STORE_BIAS><<<grid, FG_THREADS, 0, s>>>(p);
+        else f32_gemm_kernel<128, ASRC, BSRC, FG_STORE><<<grid, FG_THREADS, 0, s>>>(p);
     } else {
-        const dim3 grid((unsigned)cdiv(q.N, FG_BN), (unsigned)cdiv(q.M, 64), (unsigned)splits);
-        if (q.bias) f32_gemm_kernel<64, ASRC, BSRC, true><<<grid, FG_THREADS, 0, s>>>(p);
-        else f32_gemm_kernel<64, ASRC, BSRC, false><<<grid, FG_THREADS, 0, s>>>(p);
+        if (q.bias) f32_gemm_kernel<64, ASRC, BSRC, FG_STORE_BIAS><<<grid, FG_THREADS, 0, s>>>(p);
+        else f32_gemm_kernel<64, ASRC, BSRC, FG_STORE><<<grid, FG_THREADS, 0, s>>>(p);
     }
     return check_launch(name);
 }
@@ -371,20 +443,26 @@ static int fg_project(float *z, const float *x, int64_t ldx, const rdb_linear_de
 int linear_fwd_f32(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
                    const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
-    if (!fg_ok(d) || scale_bias || !fg_wanted(d) || !fg_ws_ok(RDB_OP_LINEAR_FWD, d, num_cus, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    if (!fg_ok(d) || !fg_wanted(d) || !fg_ws_ok(RDB_OP_LINEAR_FWD, d, num_cus, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
     if (ldx % 4 || ldy % 4 || !fg_aligned16(x) || !fg_aligned16(coef) || d->tokens * ldx >= (1ll << 29) || d->tokens * ldy >= (1ll << 29))
         return RDB_E_UNSUPPORTED;
     float *z = (float *)workspace;
     if (int rc = fg_project(z, (const float *)x, ldx, d, num_cus, s)) return rc;
     FgProduct q = {z, d->k, d->tokens * d->k, (const float *)coef, d->k, d->out_f * d->k, (float *)y, ldy, (const float *)bias,
                    d->tokens, d->out_f, d->k, fg_plan(d->tokens, d->out_f, d->k, num_cus, d->k, 1).bm, 0, 0, d->seed};
-    return fg_launch<FG_KCONT, FG_KCONT>(q, num_cus, s, "f32_gemm_kernel (y = z . C^T)");
+    if (int rc = fg_launch<FG_KCONT, FG_KCONT>(q, num_cus, s, "f32_gemm_kernel (y = z . C^T)")) return rc;
+    if (!scale_bias) return RDB_OK;
+    // y += s * x . R^T: the B side's rows are output features, index o * in_f + i
+    FgProduct qr = {(const float *)x, ldx, (d->tokens - 1) * ldx + d->in_f, nullptr, 0, 0, (float *)y, ldy, nullptr, d->tokens, d->out_f, d->in_f,
+                    fg_plan(d->tokens, d->out_f, d->in_f, num_cus, d->in_f, 1).bm, 0, 0, d->seed, (uint32_t)d->in_f, 1u, (const float *)scale_bias,
+                    nullptr, 0, nullptr};
+    return fg_launch<FG_KCONT, FG_NOISE_1D>(qr, num_cus, s, "f32_gemm_kernel (y += s x . R^T)");
 }
 
 int linear_dx_f32(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias, const rdb_linear_desc *d,
                   int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
-    if (!fg_ok(d) || scale_bias || !fg_wanted(d) || !fg_ws_ok(RDB_OP_LINEAR_BWD_DX, d, num_cus, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    if (!fg_ok(d) || !fg_wanted(d) || !fg_ws_ok(RDB_OP_LINEAR_BWD_DX, d, num_cus, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
     if (lddx % 4 || lddy % 4 || !fg_aligned16(dy) || !fg_aligned16(coef) || d->tokens * lddx >= (1ll << 29) || d->tokens * lddy >= (1ll << 29))
         return RDB_E_UNSUPPORTED;
     float *t = (float *)workspace;
@@ -396,12 +474,19 @@ int linear_dx_f32(void *dx, int64_t lddx, const void *dy, int64_t lddy, const vo
     // dx[T x in_f] = t . N: the B side's rows are input features, hashed
     FgProduct q2 = {t, d->k, d->tokens * d->k, nullptr, 0, 0, (float *)dx, lddx, nullptr, d->tokens, d->in_f, d->k,
                     fg_plan(d->tokens, d->in_f, d->k, num_cus, d->k, 1).bm, 0, 0, d->seed};
-    return fg_launch<FG_KCONT, FG_NOISE_I>(q2, num_cus, s, "f32_gemm_kernel (dx = t . N)");
+    if (int rc = fg_launch<FG_KCONT, FG_NOISE_I>(q2, num_cus, s, "f32_gemm_kernel (dx = t . N)")) return rc;
+    if (!scale_bias) return RDB_OK;
+    // dx += s * dy . R: the B side's rows are input features, index o * in_f + i
+    FgProduct qr = {(const float *)dy, lddy, (d->tokens - 1) * lddy + d->out_f, nullptr, 0, 0, (float *)dx, lddx, nullptr, d->tokens, d->in_f, d->out_f,
+                    fg_plan(d->tokens, d->in_f, d->out_f, num_cus, d->out_f, 1).bm, 0, 0, d->seed, 1u, (uint32_t)d->in_f, (const float *)scale_bias,
+                    nullptr, 0, nullptr};
+    return fg_launch<FG_KCONT, FG_NOISE_1D>(qr, num_cus, s, "f32_gemm_kernel (dx += s dy . R)");
 }
 
 // dcoef is overwritten (no zero fill needed).
-int linear_dcoef_f32(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus, void *workspace,
-                     int64_t workspace_bytes, hipStream_t s)
+// d_scale_bias: NULL, or where the gradient of the random bias's scale goes: <dy, x . R^T>.
+int linear_dcoef_f32(float *dcoef, float *d_scale_bias, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus,
+                     void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
     rdb_linear_desc dd = *d;
     dd.coef_dtype = RDB_F32;   // no coefficients are read here
@@ -416,7 +501,18 @@ int linear_dcoef_f32(float *dcoef, const void *dy, int64_t lddy, const void *x, 
     float *part = reinterpret_cast<float *>(static_cast<char *>(workspace) + up256(d->tokens * d->k * 4) * (zs > 1 ? 1 + zs : 1));
     FgProduct q = {(const float *)dy, lddy, (d->tokens - 1) * lddy + d->out_f, z, d->k, d->tokens * d->k, dcoef, d->k, nullptr,
                    d->out_f, d->k, d->tokens, 128, 0, 0, d->seed};
-    return fg_launch_ranges<FG_MCONT, FG_MCONT>(q, dc_plan(&dd, num_cus), part, up256(d->out_f * d->k * 4) / 4, num_cus, s, "f32_gemm_kernel (dC = dy^T . z)");
+    const FgPlan dcp = dc_plan(&dd, num_cus);
+    if (int rc = fg_launch_ranges<FG_MCONT, FG_MCONT>(q, dcp, part, up256(d->out_f * d->k * 4) / 4, num_cus, s, "f32_gemm_kernel (dC = dy^T . z)")) return rc;
+    if (!d_scale_bias) return RDB_OK;
+    // <dy, x . R^T>: the random-bias product once more, each block reducing its tile against dy's; then the blocks in order
+    float *dots = part + (dcp.ranges > 1 ? (int64_t)dcp.ranges * (up256(d->out_f * d->k * 4) / 4) : 0);
+    FgProduct qr = {(const float *)x, ldx, (d->tokens - 1) * ldx + d->in_f, nullptr, 0, 0, nullptr, 0, nullptr, d->tokens, d->out_f, d->in_f,
+                    fg_plan(d->tokens, d->out_f, d->in_f, num_cus, d->in_f, 1).bm, 0, 0, d->seed, (uint32_t)d->in_f, 1u, nullptr,
+                    (const float *)dy, lddy, dots};
+    if (int rc = fg_launch<FG_KCONT, FG_NOISE_1D>(qr, num_cus, s, "f32_gemm_kernel (<dy, x . R^T>)")) return rc;
+    const int nblocks = (int)(cdiv(d->tokens, qr.bm) * cdiv(d->out_f, FG_BN));
+    f32_sum_scalars_kernel<<<1, 256, 0, s>>>(d_scale_bias, dots, nblocks);
+    return check_launch("f32_sum_scalars_kernel");
 }
 
 }  // namespace rdb

@@ -315,8 +315,8 @@ int linear_fwd_f32(void *y, int64_t ldy, const void *x, int64_t ldx, const void 
                    const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
 int linear_dx_f32(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias, const rdb_linear_desc *d,
                   int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
-int linear_dcoef_f32(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus, void *workspace,
-                     int64_t workspace_bytes, hipStream_t s);
+int linear_dcoef_f32(float *dcoef, float *d_scale_bias, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus,
+                     void *workspace, int64_t workspace_bytes, hipStream_t s);
 // rdb_dx.hip
 int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z, const void *coef,
                          const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, bool accumulate, hipStream_t s);
@@ -549,6 +549,11 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
     if (d->tokens == 0 || d->in_f == 0 || d->out_f == 0 || (ncoef == 0 && !d_scale_bias)) return RDB_OK;
     if (!dy || !x) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef: dy or x is NULL");
     if (lddy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dcoef: leading dimension smaller than the row");
+    if ((d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) && d_scale_bias) {
+        // fp32: the matrix-core kernels also return the gradient of the random bias's scale
+        rc = linear_dcoef_f32(dcoef, d_scale_bias, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
     if ((d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) && !d_scale_bias) {
         rc = linear_dcoef_factored(dcoef, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
@@ -556,13 +561,13 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
         // 784 -> 512, k = 64; the matrix-core kernels take 39 us at 1028), so beyond 128 tokens the matrix cores come first
         const bool matrix_cores_first = d->tokens > 128;
         if (matrix_cores_first) {
-            rc = linear_dcoef_f32(dcoef, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
+            rc = linear_dcoef_f32(dcoef, nullptr, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
             if (rc != RDB_E_UNSUPPORTED) return rc;
         }
         rc = linear_dcoef_smallk(dcoef, dy, lddy, x, ldx, d, workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
         if (!matrix_cores_first) {
-            rc = linear_dcoef_f32(dcoef, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
+            rc = linear_dcoef_f32(dcoef, nullptr, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
             if (rc != RDB_E_UNSUPPORTED) return rc;
         }
     }

@@ -128,3 +128,28 @@ def test_layer_level_fp32(hip, oracle):
     assert rel_l2(y.detach().cpu().numpy(), want_y) < F32_TOL
     assert rel_l2(xc.grad.cpu().numpy(), want_dx) < F32_TOL
     assert rel_l2(lin.weight_coef.grad.cpu().numpy(), want_dc) < F32_TOL
+
+
+@pytest.mark.parametrize("T,in_f,out_f,k", [(1024, 768, 1024, 128), (200, 72, 136, 40), (1100, 1024, 260, 68)])
+def test_fused_random_bias_in_fp32(hip, oracle, T, in_f, out_f, k):
+    """W = C.N + s.noise1d (the reference's default layer, SillyLayers.py:122-133, 218-221) in fp32: forward, input gradient,
+    coefficient gradient and the gradient of s against the oracle, with C != 0 and with C = 0; the gradient of s twice (same bits)."""
+    print(f"case f32 random bias T={T} in={in_f} out={out_f} k={k}", flush=True)
+    x, dy, coef, bias = _inputs(T, in_f, out_f, k, 31)
+    sbv = 0.0625
+    sb = torch.tensor([sbv])
+    for c in (coef, torch.zeros_like(coef)):
+        xn, dyn, cn = x.numpy(), dy.numpy(), c.numpy()
+        want_y = oracle.linear_fwd(xn, cn, in_f, out_f, 9, bias=bias.numpy(), scale_bias=sbv)
+        want_dx, want_dc, dW = oracle.linear_bwd(xn, dyn, cn, in_f, out_f, 9, scale_bias=sbv)
+        want_ds = float(oracle.scale_bias_bwd(dW.astype(np.float32), 9)[0])
+        xg, dyg, cg, sg = x.cuda(), dy.cuda(), c.cuda(), sb.cuda()
+        y = hip.linear_fwd(xg, cg, in_f, out_f, in_f, 1, 9, scale_bias=sg, bias=bias.cuda())
+        dx = hip.linear_bwd_dx(dyg, cg, in_f, out_f, in_f, 1, 9, scale_bias=sg)
+        dc, ds = hip.linear_bwd_dcoef(dyg, xg, k, out_f, in_f, out_f, in_f, 1, 9, want_scale_bias_grad=True)
+        assert rel_l2(y.cpu().numpy(), want_y) < F32_TOL
+        assert rel_l2(dx.cpu().numpy(), want_dx) < F32_TOL
+        assert rel_l2(dc.cpu().numpy(), want_dc) < F32_TOL
+        assert abs(float(ds) - want_ds) < 1e-4 * max(abs(want_ds), float(np.linalg.norm(dW)))
+        _, ds2 = hip.linear_bwd_dcoef(dyg, xg, k, out_f, in_f, out_f, in_f, 1, 9, want_scale_bias_grad=True)
+        assert torch.equal(ds, ds2)

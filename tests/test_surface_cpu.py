@@ -143,7 +143,8 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     c2 = desc(8192, 768, 3072, 256, act=_lib.RDB_F32, coef=_lib.RDB_F32)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(c2)) == 8192 * 256 * 4 * (1 + 4)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(c2)) == 8192 * 256 * 4 * (1 + 4)
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DCOEF, ctypes.byref(c2)) == 8192 * 256 * 4 * (1 + 4) + 10 * 3072 * 256 * 4
+    # ... and a value per 64 x 128 tile of [tokens x out_f] for the gradient of the random bias's scale
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DCOEF, ctypes.byref(c2)) == 8192 * 256 * 4 * (1 + 4) + 10 * 3072 * 256 * 4 + 128 * 24 * 4
     # enough tiles: no ranges
     wide = desc(65536, 768, 3072, 256, act=_lib.RDB_F32, coef=_lib.RDB_F32)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(wide)) == 65536 * 256 * 4
