@@ -285,8 +285,8 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
     if (!workspace || workspace_bytes < linear_dx_factored_workspace(d) || ((uintptr_t)workspace & 15)) return RDB_E_UNSUPPORTED;
     if (d->tokens * lddy >= (1ll << 29)) return RDB_E_UNSUPPORTED;
     if (lddy % 8 || lddx % 8 || ((uintptr_t)dy & 15) || ((uintptr_t)coef & 15) || ((uintptr_t)dx & 15)) return RDB_E_UNSUPPORTED;
-    // only worth it when the factored form is cheaper than forming the weight
-    if (d->algo == RDB_ALGO_AUTO && d->k * (d->in_f + d->out_f) >= d->in_f * d->out_f) return RDB_E_UNSUPPORTED;
+    // AUTO: up to 16 times the flops of one product on a stored W (the same bound as the forward's: see cheaper_factored there)
+    if (d->algo == RDB_ALGO_AUTO && d->k * (d->in_f + d->out_f) >= 16 * d->in_f * d->out_f) return RDB_E_UNSUPPORTED;
 
     DyCParams p1;
     make_dyc_params(p1, dy, lddy, coef, workspace, d);

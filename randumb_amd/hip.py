@@ -279,9 +279,10 @@ def linear_projection_supported(tokens: int, in_f: int, out_f: int, k: int) -> b
 
 
 def linear_projection_preferred(tokens: int, in_f: int, out_f: int, k: int) -> bool:
-    """Whether the projected form is also the cheaper one: the factored products need 2*tokens*k*(in_f + out_f) flops per
-    direction, forming the weight 2*tokens*in_f*out_f (+ its generation)."""
-    return k * (in_f + out_f) < in_f * out_f and linear_projection_supported(tokens, in_f, out_f, k)
+    """Whether the projected form is also the faster one.  The factored products need 2*tokens*k*(in_f + out_f) flops per
+    direction, a product on a stored weight 2*tokens*in_f*out_f; the kernels that form the weight on chip instead lose
+    against the factored ones up to at least 8 times that (measured), so the bound is 16 times, as in the library."""
+    return k * (in_f + out_f) < 16 * in_f * out_f and linear_projection_supported(tokens, in_f, out_f, k)
 
 
 def linear_project(x: torch.Tensor, k: int, out_f: int, seed: int, coef: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -288,7 +288,7 @@ def test_materialised_weight_has_the_target_std(oracle):
 
 def test_projected_form_is_chosen_only_where_it_runs_and_pays():
     """ops.linear takes the projected form only for layers whose activations fit the kernels' addressing and for which the
-    factored products are cheaper than forming the weight; everything else goes to rten::linear_fwd (whose backward cannot
+    factored products are faster than forming the weight on chip; everything else goes to rten::linear_fwd (whose backward cannot
     be refused late, in the backward pass)."""
     from randumb_amd import hip
 
@@ -297,7 +297,9 @@ def test_projected_form_is_chosen_only_where_it_runs_and_pays():
     assert hip.linear_projection_bytes(65536, 4096, 14336, 256) > 0
     assert hip.linear_projection_supported(65536, 4096, 14336, 256) and hip.linear_projection_preferred(65536, 4096, 14336, 256)
     assert hip.linear_projection_supported(1 << 17, 4096, 64, 8)
-    # k >= in*out/(in+out): forming the weight is cheaper (768 -> 384 at k = 256 is exactly on the boundary)
-    assert hip.linear_projection_supported(512, 768, 384, 256) and not hip.linear_projection_preferred(512, 768, 384, 256)
+    # preferred up to k (in + out) = 16 in out: beyond the point where its flops equal those of a product on a stored weight
+    # (768 -> 384 at k = 256), because the alternative is a kernel that forms the weight on chip
+    assert hip.linear_projection_supported(512, 768, 384, 256) and hip.linear_projection_preferred(512, 768, 384, 256)
     assert hip.linear_projection_preferred(512, 768, 512, 256)
-    assert not hip.linear_projection_preferred(64, 8, 8, 8)
+    assert hip.linear_projection_preferred(64, 8, 8, 8)           # ratio 2
+    assert hip.linear_projection_supported(64, 8, 8, 64) and not hip.linear_projection_preferred(64, 8, 8, 64)   # ratio 16
