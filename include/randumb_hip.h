@@ -143,10 +143,12 @@ enum {
                              y = (x.N^T).C^T, dx = (dy.C).N, dcoef = dy^T.(x.N^T); the [tokens x k] intermediate lives
                              in the caller's workspace.  bf16 activations and coef: matrix-core kernels; fp32 with
                              k <= 64 and at most 1024 tokens (the GEMV-like regime; up to 4096 when asked for by this
-                             value): vector-ALU kernels; fp32 otherwise, with k, in_f, out_f and the leading dimensions
-                             multiples of 4 and 16-byte aligned pointers: fp32 matrix-core kernels (operands, products
-                             and sums in fp32, the noise hashed into the operand tiles).  Both fp32 forms add partial
-                             sums in a fixed order: bit-reproducible.
+                             value): vector-ALU kernels; fp32 otherwise: fp32 matrix-core kernels (operands, products
+                             and sums in fp32, the noise hashed into the operand tiles; any sizes and alignments, 16
+                             bytes at a time where sizes, leading dimensions and pointers are multiples of 4 elements
+                             / 16 bytes; also with scale_bias, whose share is one more product with the random-bias
+                             matrix hashed as an operand, and with its gradient).  Both fp32 forms add partial sums in
+                             a fixed order: bit-reproducible.
                              With scale_bias (W = C.N + s.R, R the fused random bias, full rank) the input gradient adds
                              s * dy.R on top with R hashed into the matrix pipeline; forward and dcoef then need the
                              kernels that form W (RDB_ALGO_AUTO picks them). */

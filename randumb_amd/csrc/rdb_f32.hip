@@ -20,6 +20,7 @@ namespace rdb {
 constexpr int FG_BN = 128;        // B rows (output columns) per block
 constexpr int FG_BK = 16;         // contraction values per stage
 constexpr int FG_THREADS = 256;   // four waves, 2 x 2
+constexpr uint32_t FG_OOB = 0x80000000u;   // a byte offset past the end of any matrix these kernels take (below 2^31 bytes)
 
 // Where an operand's tile [rows x FG_BK] comes from.  In LDS every tile is [FG_BK][rows + 4]: an MFMA operand is 32
 // consecutive floats of each of two contraction values.
@@ -59,14 +60,18 @@ struct FgParams {
 
 // One operand's way from its source into LDS: load(stage) requests / hashes the stage's values into registers, store() puts
 // them into a tile.  Rows past `rows` and contraction values past `kend` are zeros.
-template <int ROWS, int SRC> struct FgOperand {
+// VEC: the matrix is read in 16-byte pieces (16-byte aligned base, leading dimension a multiple of 4, and the extent that
+// runs along a piece a multiple of 4, so that a piece lies inside or outside as a whole); otherwise value by value.
+template <int ROWS, int SRC, bool VEC> struct FgOperand {
     static constexpr int LD = ROWS + 4, TILE = FG_BK * LD, NV = ROWS * FG_BK / FG_THREADS / 4;   // float4 per thread and stage
     static_assert(NV >= 1, "a stage is at least one float4 per thread");
     __amdgpu_buffer_rsrc_t rs;
-    uint32_t off[NV];   // byte offset of the thread's pieces at stage 0 (BUFFER_OOB: a row past the end)
+    uint32_t off[NV];   // byte offset of the thread's pieces at stage 0
+    bool ok[NV];        // ... and whether the piece's (first) row exists
     uint32_t step;      // bytes per stage
     uint32_t first;     // noise: first-round value of the thread's first element at stage 0
     int kk0, kend, k_begin, row_ok;
+    int rows_left[NV];  // FG_MCONT without VEC: how many of the piece's four rows exist
     f32x4 r[NV];
 
     uint32_t inc;       // noise: first-round step per contraction value
@@ -82,7 +87,8 @@ template <int ROWS, int SRC> struct FgOperand {
 #pragma unroll
             for (int h = 0; h < NV; ++h) {
                 const int idx = h * FG_THREADS + t, row = idx >> 2, kq = idx & 3;
-                off[h] = row0 + row < rows ? (uint32_t)(((int64_t)(row0 + row) * ld + k_begin + kq * 4) * 4) : BUFFER_OOB;
+                ok[h] = row0 + row < rows;
+                off[h] = ok[h] ? (uint32_t)(((int64_t)(row0 + row) * ld + k_begin + kq * 4) * 4) : 0u;
             }
             kk0 = (t & 3) * 4;
         } else if (SRC == FG_MCONT) {
@@ -91,7 +97,9 @@ template <int ROWS, int SRC> struct FgOperand {
 #pragma unroll
             for (int h = 0; h < NV; ++h) {
                 const int idx = h * FG_THREADS + t, kk = idx / (ROWS / 4), r4 = (idx % (ROWS / 4)) * 4;
-                off[h] = row0 + r4 < rows ? (uint32_t)(((int64_t)(k_begin + kk) * ld + row0 + r4) * 4) : BUFFER_OOB;
+                ok[h] = row0 + r4 < rows;
+                off[h] = ok[h] ? (uint32_t)(((int64_t)(k_begin + kk) * ld + row0 + r4) * 4) : 0u;
+                rows_left[h] = rows - (row0 + r4);
             }
             kk0 = t / (ROWS / 4);
         } else {
@@ -111,16 +119,31 @@ template <int ROWS, int SRC> struct FgOperand {
     __device__ __forceinline__ void load(int stage)
     {
         if (SRC == FG_KCONT) {
-            // a thread's four values are consecutive contraction values: all inside or all outside (K is a multiple of 4)
-            const bool in = k_begin + stage * FG_BK + kk0 < kend;
+            // a thread's four values are consecutive contraction values
+            const int kk = k_begin + stage * FG_BK + kk0;
 #pragma unroll
-            for (int h = 0; h < NV; ++h)
-                r[h] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, in ? (int)(off[h] + (uint32_t)stage * step) : (int)BUFFER_OOB, 0, 0));
+            for (int h = 0; h < NV; ++h) {
+                const uint32_t o = off[h] + (uint32_t)stage * step;
+                if (VEC) {   // all inside or all outside
+                    r[h] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (ok[h] && kk < kend) ? (int)o : (int)FG_OOB, 0, 0));
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        r[h][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, (ok[h] && kk + j < kend) ? (int)(o + 4 * j) : (int)FG_OOB, 0, 0));
+                }
+            }
         } else if (SRC == FG_MCONT) {
 #pragma unroll
             for (int h = 0; h < NV; ++h) {
-                const bool in = k_begin + stage * FG_BK + kk0 + h * (FG_THREADS / (ROWS / 4)) < kend;
-                r[h] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, in ? (int)(off[h] + (uint32_t)stage * step) : (int)BUFFER_OOB, 0, 0));
+                const bool in = ok[h] && k_begin + stage * FG_BK + kk0 + h * (FG_THREADS / (ROWS / 4)) < kend;
+                const uint32_t o = off[h] + (uint32_t)stage * step;
+                if (VEC) {
+                    r[h] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, in ? (int)o : (int)FG_OOB, 0, 0));
+                } else {   // a thread's four values are consecutive rows: rows_left of them exist
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        r[h][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, (in && j < rows_left[h]) ? (int)(o + 4 * j) : (int)FG_OOB, 0, 0));
+                }
             }
         } else {
 #pragma unroll
@@ -165,10 +188,10 @@ template <int ROWS, int SRC> struct FgOperand {
 // out[M x N] (+)= A . B^T over one split of the contraction.  Block: BM x 128 of the output, four waves as 2 x 2, a wave owns
 // (BM / 2) x 64 in BM / 64 x 2 accumulator tiles.  Two LDS buffers, one barrier per stage: while a stage is multiplied the
 // next one is on its way from memory (or being hashed) in registers.
-template <int BM, int ASRC, int BSRC, int EPI> __global__ __launch_bounds__(FG_THREADS, 2) void f32_gemm_kernel(FgParams p)
+template <int BM, int ASRC, int BSRC, int EPI, bool VEC> __global__ __launch_bounds__(FG_THREADS, 2) void f32_gemm_kernel(FgParams p)
 {
-    typedef FgOperand<BM, ASRC> PA;
-    typedef FgOperand<FG_BN, BSRC> PB;
+    typedef FgOperand<BM, ASRC, VEC> PA;
+    typedef FgOperand<FG_BN, BSRC, VEC> PB;
     constexpr int MI = BM / 64, NI = 2, STAGE = PA::TILE + PB::TILE;
     __shared__ __align__(16) float lds[2 * STAGE];
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
@@ -264,26 +287,33 @@ __global__ __launch_bounds__(256) void f32_sum_scalars_kernel(float *__restrict_
     if (threadIdx.x == 0) out[0] = sh[0];
 }
 
-// out[i] = part[0][i] + part[1][i] + ... in split order, four values per thread
-__global__ __launch_bounds__(256) void f32_sum_splits_kernel(float *__restrict__ out, const float *__restrict__ part, int64_t n4, int64_t stride, int splits)
+// out[i] = part[0][i] + part[1][i] + ... in split order, four values per thread (n4 groups of four, then the n % 4 last values
+// one thread each)
+__global__ __launch_bounds__(256) void f32_sum_splits_kernel(float *__restrict__ out, const float *__restrict__ part, int64_t n, int64_t stride, int splits, int vec)
 {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n4) return;
-    f32x4 v = *reinterpret_cast<const f32x4 *>(part + i * 4);
-    for (int s = 1; s < splits; ++s) v += *reinterpret_cast<const f32x4 *>(part + s * stride + i * 4);
-    *reinterpret_cast<f32x4 *>(out + i * 4) = v;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x, n4 = vec ? n / 4 : 0;
+    if (i < n4) {
+        f32x4 v = *reinterpret_cast<const f32x4 *>(part + i * 4);
+        for (int s = 1; s < splits; ++s) v += *reinterpret_cast<const f32x4 *>(part + s * stride + i * 4);
+        *reinterpret_cast<f32x4 *>(out + i * 4) = v;
+    } else if (n4 * 4 + (i - n4) < n) {
+        const int64_t e = n4 * 4 + (i - n4);
+        float v = part[e];
+        for (int s = 1; s < splits; ++s) v += part[s * stride + e];
+        out[e] = v;
+    }
 }
 
 // ----------------------------------------------------------------------------------------------- host side
 static bool fg_aligned16(const void *q) { return ((uintptr_t)q & 15) == 0; }
 static int64_t up256(int64_t n) { return (n + 255) / 256 * 256; }
 
-// The shapes these kernels take: matrix-coef fp32, every extent a multiple of 4 (16-byte pieces), matrices below 2^31 bytes.
+// The shapes these kernels take: matrix-coef fp32, matrices below 2^31 bytes.  Extents, leading dimensions and pointers that are
+// multiples of 4 elements / 16 bytes get the kernels that read 16 bytes at a time, everything else the value-by-value ones.
 static bool fg_ok(const rdb_linear_desc *d)
 {
     return d->act_dtype == RDB_F32 && d->coef_dtype == RDB_F32 && d->coef_rows != 0 && d->k > 0 && d->tokens > 0 && d->in_f > 0 && d->out_f > 0 &&
-           d->k % 4 == 0 && d->in_f % 4 == 0 && d->out_f % 4 == 0 && d->tokens * d->k < (1ll << 29) && d->out_f * d->k < (1ll << 29) &&
-           d->in_f < (1 << 30) && d->out_f < (1 << 30);
+           d->tokens * d->k < (1ll << 29) && d->out_f * d->k < (1ll << 29) && d->in_f < (1 << 30) && d->out_f < (1 << 30);
 }
 // Wanted whenever the shapes fit: what AUTO would run instead is the general kernel, which forms W tiles on the vector ALU at a
 // few TFLOP/s, so the factored form on the matrix cores wins also where it is more flops than a product on a stored W.
@@ -354,6 +384,11 @@ struct FgProduct {
     float *dot_part;
 };
 
+#define FG_LAUNCH(BM_, EPI_)                                                                      \
+    do {                                                                                          \
+        if (vec) f32_gemm_kernel<BM_, ASRC, BSRC, EPI_, true><<<grid, FG_THREADS, 0, s>>>(p);     \
+        else f32_gemm_kernel<BM_, ASRC, BSRC, EPI_, false><<<grid, FG_THREADS, 0, s>>>(p);        \
+    } while (0)
 template <int ASRC, int BSRC> static int fg_launch(const FgProduct &q, int num_cus, hipStream_t s, const char *name)
 {
     if (q.a_elems >= (1ll << 29) || q.b_elems >= (1ll << 29) || q.M >= (1ll << 30) || q.N >= (1ll << 30) || q.K >= (1ll << 30)) return RDB_E_UNSUPPORTED;
@@ -380,21 +415,28 @@ template <int ASRC, int BSRC> static int fg_launch(const FgProduct &q, int num_c
     p.lddot = q.lddot;
     p.dot_part = q.dot_part;
     const int splits = (int)cdiv(q.K, p.kchunk);
+    // 16-byte pieces when both matrices allow them: aligned bases and leading dimensions, and the extent along a piece a multiple of 4
+    // (along the rows of a matrix: the contraction; across them: the rows of the tile)
+    auto vec_ok = [&](int src, const float *m, int64_t ld, int64_t rows) {
+        if (src != FG_KCONT && src != FG_MCONT) return true;
+        return fg_aligned16(m) && ld % 4 == 0 && (src == FG_KCONT ? q.K % 4 == 0 : rows % 4 == 0);
+    };
+    const bool vec = vec_ok(ASRC, q.a, q.lda, q.M) && vec_ok(BSRC, q.b, q.ldb, q.N);
     const dim3 grid((unsigned)cdiv(q.N, FG_BN), (unsigned)cdiv(q.M, q.bm), (unsigned)splits);
     if (BSRC == FG_NOISE_1D) {   // the random-bias products: added on top of an output, or reduced against a matrix
         if (q.bm == 128) {
-            if (q.dotm) f32_gemm_kernel<128, ASRC, BSRC, FG_DOT><<<grid, FG_THREADS, 0, s>>>(p);
-            else f32_gemm_kernel<128, ASRC, BSRC, FG_ADD_SCALED><<<grid, FG_THREADS, 0, s>>>(p);
+            if (q.dotm) FG_LAUNCH(128, FG_DOT);
+            else FG_LAUNCH(128, FG_ADD_SCALED);
         } else {
-            if (q.dotm) f32_gemm_kernel<64, ASRC, BSRC, FG_DOT><<<grid, FG_THREADS, 0, s>>>(p);
-            else f32_gemm_kernel<64, ASRC, BSRC, FG_ADD_SCALED><<<grid, FG_THREADS, 0, s>>>(p);
+            if (q.dotm) FG_LAUNCH(64, FG_DOT);
+            else FG_LAUNCH(64, FG_ADD_SCALED);
         }
     } else if (q.bm == 128) {
-        if (q.bias) f32_gemm_kernel<128, ASRC, BSRC, FG_STORE_BIAS><<<grid, FG_THREADS, 0, s>>>(p);
-        else f32_gemm_kernel<128, ASRC, BSRC, FG_STORE><<<grid, FG_THREADS, 0, s>>>(p);
+        if (q.bias) FG_LAUNCH(128, FG_STORE_BIAS);
+        else FG_LAUNCH(128, FG_STORE);
     } else {
-        if (q.bias) f32_gemm_kernel<64, ASRC, BSRC, FG_STORE_BIAS><<<grid, FG_THREADS, 0, s>>>(p);
-        else f32_gemm_kernel<64, ASRC, BSRC, FG_STORE><<<grid, FG_THREADS, 0, s>>>(p);
+        if (q.bias) FG_LAUNCH(64, FG_STORE_BIAS);
+        else FG_LAUNCH(64, FG_STORE);
     }
     return check_launch(name);
 }
@@ -406,7 +448,8 @@ static bool fg_ws_ok(int op, const rdb_linear_desc *d, int num_cus, const void *
 
 static int fg_sum(float *out, const float *part, int64_t n, int64_t stride, int splits, hipStream_t s)
 {
-    f32_sum_splits_kernel<<<(unsigned)cdiv(n / 4, 256), 256, 0, s>>>(out, part, n / 4, stride, splits);
+    const int vec = fg_aligned16(out) ? 1 : 0;   // the partial matrices are 256-byte aligned
+    f32_sum_splits_kernel<<<(unsigned)cdiv(vec ? n / 4 + n % 4 : n, 256), 256, 0, s>>>(out, part, n, stride, splits, vec);
     return check_launch("f32_sum_splits_kernel");
 }
 
@@ -444,8 +487,7 @@ int linear_fwd_f32(void *y, int64_t ldy, const void *x, int64_t ldx, const void 
                    const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
     if (!fg_ok(d) || !fg_wanted(d) || !fg_ws_ok(RDB_OP_LINEAR_FWD, d, num_cus, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
-    if (ldx % 4 || ldy % 4 || !fg_aligned16(x) || !fg_aligned16(coef) || d->tokens * ldx >= (1ll << 29) || d->tokens * ldy >= (1ll << 29))
-        return RDB_E_UNSUPPORTED;
+    if (d->tokens * ldx >= (1ll << 29) || d->tokens * ldy >= (1ll << 29)) return RDB_E_UNSUPPORTED;
     float *z = (float *)workspace;
     if (int rc = fg_project(z, (const float *)x, ldx, d, num_cus, s)) return rc;
     FgProduct q = {z, d->k, d->tokens * d->k, (const float *)coef, d->k, d->out_f * d->k, (float *)y, ldy, (const float *)bias,
@@ -463,8 +505,7 @@ int linear_dx_f32(void *dx, int64_t lddx, const void *dy, int64_t lddy, const vo
                   int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
     if (!fg_ok(d) || !fg_wanted(d) || !fg_ws_ok(RDB_OP_LINEAR_BWD_DX, d, num_cus, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
-    if (lddx % 4 || lddy % 4 || !fg_aligned16(dy) || !fg_aligned16(coef) || d->tokens * lddx >= (1ll << 29) || d->tokens * lddy >= (1ll << 29))
-        return RDB_E_UNSUPPORTED;
+    if (d->tokens * lddx >= (1ll << 29) || d->tokens * lddy >= (1ll << 29)) return RDB_E_UNSUPPORTED;
     float *t = (float *)workspace;
     // t[T x k] = dy[T x out_f] . C: the B side's rows are coefficients, read across the rows of C
     FgProduct q1 = {(const float *)dy, lddy, (d->tokens - 1) * lddy + d->out_f, (const float *)coef, d->k, d->out_f * d->k, t, d->k, nullptr,
@@ -491,9 +532,7 @@ int linear_dcoef_f32(float *dcoef, float *d_scale_bias, const void *dy, int64_t 
     rdb_linear_desc dd = *d;
     dd.coef_dtype = RDB_F32;   // no coefficients are read here
     if (!fg_ok(&dd) || !fg_wanted(&dd) || !fg_ws_ok(RDB_OP_LINEAR_BWD_DCOEF, &dd, num_cus, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
-    if (ldx % 4 || lddy % 4 || !fg_aligned16(x) || !fg_aligned16(dy) || !fg_aligned16(dcoef) || d->tokens * ldx >= (1ll << 29) ||
-        d->tokens * lddy >= (1ll << 29))
-        return RDB_E_UNSUPPORTED;
+    if (d->tokens * ldx >= (1ll << 29) || d->tokens * lddy >= (1ll << 29)) return RDB_E_UNSUPPORTED;
     float *z = (float *)workspace;
     if (int rc = fg_project(z, (const float *)x, ldx, &dd, num_cus, s)) return rc;
     // dC[out_f x k] = dy^T . z: both sides are read across their rows (the contraction runs over the tokens)

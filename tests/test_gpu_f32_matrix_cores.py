@@ -43,6 +43,9 @@ SHAPES = [
     (4500, 128, 256, 32, 9),      # small k, more tokens than the vector-ALU kernels take
     (4, 8, 12, 68, 1),            # smaller than one tile
     (2100, 516, 132, 100, 77),    # the coefficient gradient in several token ranges, ragged last range
+    (333, 777, 555, 99, 8),       # no extent a multiple of 4: operands read value by value
+    (130, 1001, 999, 102, 12),
+    (7, 5, 3, 2, 3),
 ]
 
 
@@ -108,6 +111,29 @@ def test_strided_activations(hip, oracle):
     assert rel_l2(dc.cpu().numpy(), want_dc) < F32_TOL
 
 
+def test_unaligned_views(hip, oracle):
+    """Activations that start one element into a wider, odd-width matrix: neither the base nor the leading dimension is a
+    multiple of 16 bytes."""
+    from randumb_amd._lib import RDB_ALGO_FACTORED
+
+    T, in_f, out_f, k, seed = 150, 96, 200, 72, 17
+    x, dy, coef, bias = _inputs(T, in_f, out_f, k, seed)
+    wide_x = torch.zeros(T, in_f + 3).cuda()
+    wide_x[:, 1:1 + in_f] = x.cuda()
+    wide_dy = torch.zeros(T, out_f + 5).cuda()
+    wide_dy[:, 1:1 + out_f] = dy.cuda()
+    xs, dys, cc = wide_x[:, 1:1 + in_f], wide_dy[:, 1:1 + out_f], coef.cuda()
+    assert xs.data_ptr() % 16 and dys.data_ptr() % 16 and xs.stride(0) % 4 and dys.stride(0) % 4
+    want_y = oracle.linear_fwd(x.numpy(), coef.numpy(), in_f, out_f, seed, bias=bias.numpy())
+    want_dx, want_dc, _ = oracle.linear_bwd(x.numpy(), dy.numpy(), coef.numpy(), in_f, out_f, seed)
+    y = hip.linear_fwd(xs, cc, in_f, out_f, in_f, 1, seed, bias=bias.cuda(), algo=RDB_ALGO_FACTORED)
+    assert rel_l2(y.cpu().numpy(), want_y) < F32_TOL
+    dx = hip.linear_bwd_dx(dys, cc, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    assert rel_l2(dx.cpu().numpy(), want_dx) < F32_TOL
+    dc, _ = hip.linear_bwd_dcoef(dys, xs, k, out_f, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+    assert rel_l2(dc.cpu().numpy(), want_dc) < F32_TOL
+
+
 def test_layer_level_fp32(hip, oracle):
     """SillyLinear(matrix_coef=True) in fp32 at a GPT-like slice: forward, input gradient and coefficient gradient through autograd."""
     from randumb_amd.SillyLayers import SillyLinear
@@ -130,7 +156,7 @@ def test_layer_level_fp32(hip, oracle):
     assert rel_l2(lin.weight_coef.grad.cpu().numpy(), want_dc) < F32_TOL
 
 
-@pytest.mark.parametrize("T,in_f,out_f,k", [(1024, 768, 1024, 128), (200, 72, 136, 40), (1100, 1024, 260, 68)])
+@pytest.mark.parametrize("T,in_f,out_f,k", [(1024, 768, 1024, 128), (200, 72, 136, 40), (1100, 1024, 260, 68), (333, 77, 55, 9)])
 def test_fused_random_bias_in_fp32(hip, oracle, T, in_f, out_f, k):
     """W = C.N + s.noise1d (the reference's default layer, SillyLayers.py:122-133, 218-221) in fp32: forward, input gradient,
     coefficient gradient and the gradient of s against the oracle, with C != 0 and with C = 0; the gradient of s twice (same bits)."""

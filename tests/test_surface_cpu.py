@@ -148,8 +148,10 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     # enough tiles: no ranges
     wide = desc(65536, 768, 3072, 256, act=_lib.RDB_F32, coef=_lib.RDB_F32)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(wide)) == 65536 * 256 * 4
-    # extents that are not multiples of 4 stay with the general kernel: no scratch
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(16, 4096, 4094, 128, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 0
+    # extents that are not multiples of 4 run on the same kernels (operands read value by value): same scratch
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(16, 4096, 4094, 128, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 16 * 128 * 4 * (1 + 32)
+    # vector-coef: the general kernel, no scratch
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(16, 4096, 4096, 128, rows=0, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 0
 
     bad = ctypes.byref(desc(64, 100, 32, 16))
     assert L.rdb_linear_project(None, None, 100, None, bad, None) == -5  # RDB_E_UNSUPPORTED
