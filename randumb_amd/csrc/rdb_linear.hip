@@ -538,6 +538,30 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
     const int64_t ncoef = (d->coef_rows ? d->coef_rows : 1) * d->k;
     if (ncoef > 0 && !dcoef) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef: dcoef is NULL");
     hipStream_t s = (hipStream_t)stream;
+    const bool empty = d->tokens == 0 || d->in_f == 0 || d->out_f == 0 || (ncoef == 0 && !d_scale_bias);
+    if (!empty) {
+        if (!dy || !x) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef: dy or x is NULL");
+        if (lddy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dcoef: leading dimension smaller than the row");
+    }
+    if (!empty && d->act_dtype == RDB_F32 && (d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED)) {
+        // The fp32 factored kernels overwrite their outputs: nothing to clear first.  The matrix-core kernels also return the
+        // gradient of the random bias's scale.  Without it: the vector-ALU kernel's coefficient gradient grows with the tokens
+        // (49 us at 256 tokens, 158 us at 1024 for 784 -> 512, k = 64; the matrix-core kernels take 39 us at 1028), so beyond
+        // 128 tokens the matrix cores come first.
+        const bool matrix_cores_first = d_scale_bias || d->tokens > 128;
+        if (matrix_cores_first) {
+            rc = linear_dcoef_f32(dcoef, d_scale_bias, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
+            if (rc != RDB_E_UNSUPPORTED) return rc;
+        }
+        if (!d_scale_bias) {
+            rc = linear_dcoef_smallk(dcoef, dy, lddy, x, ldx, d, workspace, workspace_bytes, s);
+            if (rc != RDB_E_UNSUPPORTED) return rc;
+            if (!matrix_cores_first) {
+                rc = linear_dcoef_f32(dcoef, nullptr, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
+                if (rc != RDB_E_UNSUPPORTED) return rc;
+            }
+        }
+    }
     if (ncoef > 0) {
         rc = fill_zero(dcoef, ncoef, s);
         if (rc) return rc;
@@ -546,30 +570,10 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
         rc = fill_zero(d_scale_bias, 1, s);
         if (rc) return rc;
     }
-    if (d->tokens == 0 || d->in_f == 0 || d->out_f == 0 || (ncoef == 0 && !d_scale_bias)) return RDB_OK;
-    if (!dy || !x) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef: dy or x is NULL");
-    if (lddy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dcoef: leading dimension smaller than the row");
-    if ((d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) && d_scale_bias) {
-        // fp32: the matrix-core kernels also return the gradient of the random bias's scale
-        rc = linear_dcoef_f32(dcoef, d_scale_bias, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
-        if (rc != RDB_E_UNSUPPORTED) return rc;
-    }
+    if (empty) return RDB_OK;
     if ((d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) && !d_scale_bias) {
         rc = linear_dcoef_factored(dcoef, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
-        // fp32: the vector-ALU kernel's coefficient gradient grows with the tokens (49 us at 256 tokens, 158 us at 1024 for
-        // 784 -> 512, k = 64; the matrix-core kernels take 39 us at 1028), so beyond 128 tokens the matrix cores come first
-        const bool matrix_cores_first = d->tokens > 128;
-        if (matrix_cores_first) {
-            rc = linear_dcoef_f32(dcoef, nullptr, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
-            if (rc != RDB_E_UNSUPPORTED) return rc;
-        }
-        rc = linear_dcoef_smallk(dcoef, dy, lddy, x, ldx, d, workspace, workspace_bytes, s);
-        if (rc != RDB_E_UNSUPPORTED) return rc;
-        if (!matrix_cores_first) {
-            rc = linear_dcoef_f32(dcoef, nullptr, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
-            if (rc != RDB_E_UNSUPPORTED) return rc;
-        }
     }
     if (d->algo == RDB_ALGO_FACTORED)
         return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dcoef: the factored algorithm needs matrix-coef, no scale_bias gradient, a "
