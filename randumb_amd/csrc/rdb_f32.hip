@@ -7,7 +7,9 @@
 //
 // N[m, i] = noise(PRIME*i + m) is hashed into the pipeline's LDS tiles and never stored; W = C . N is never formed.  All
 // five products run on one kernel template that differs in where its two operands come from (a row-major matrix read along
-// or across its rows, or the hash).  Everything is fp32: operands, products and sums.
+// or across its rows, or the hash).  Everything is fp32: operands, products and sums.  (bf16 layers whose sizes keep them off
+// the bf16 kernels, which want multiples of 8, run here too: bf16 matrices are read value by value and widened, z and t stay
+// fp32, y and dx are rounded to bf16 once.)
 // With scale_bias (W = C . N + s . R, R[o, i] = noise1d(o*in_f + i), full rank: src/rten_cpp/RandumbTensor.py:286-289) the
 // random-bias share is one more product with R as the hashed operand, added on top:  y += s * x . R^T,  dx += s * dy . R,  and
 // the gradient of s is <dy, x . R^T>, summed tile by tile in the epilogue of that product and block by block afterwards.
@@ -51,6 +53,9 @@ struct FgParams {
     int kchunk;          // contraction values per split (a multiple of FG_BK); K when there is one split
     int64_t a_bytes, b_bytes;   // extent of the matrices, for the bounds check of the loads (< 2^31)
     uint32_t seed;
+    int a_es, b_es;             // bytes per element of the A and B matrices: 4, or 2 (bf16; only the value-by-value kernels)
+    int out_bf16;               // out, bias and dotm are bf16 (the activations' dtype)
+    int scale_bf16;             // scale is bf16 (the coefficients' dtype)
     uint32_t nsR, nsK;          // FG_NOISE_1D: index steps per row and per contraction value
     const float *scale;         // FG_ADD_SCALED: one device value
     const float *dotm;          // FG_DOT: [M x N] matrix, leading dimension lddot
@@ -75,30 +80,40 @@ template <int ROWS, int SRC, bool VEC> struct FgOperand {
     f32x4 r[NV];
 
     uint32_t inc;       // noise: first-round step per contraction value
+    int es;             // bytes per element of the matrix (2: bf16, value by value only)
+    __device__ __forceinline__ float load1(uint32_t o, bool in, int j) const
+    {
+        if (es == 2) {
+            const unsigned short h = __builtin_amdgcn_raw_buffer_load_b16(rs, in ? (int)(o + 2 * j) : (int)FG_OOB, 0, 0);
+            return bf16_to_f32(h);
+        }
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, in ? (int)(o + 4 * j) : (int)FG_OOB, 0, 0));
+    }
     __device__ __forceinline__ void init(const float *src, int64_t ld, int64_t bytes, int row0, int rows, int k_begin_, int kend_, uint32_t seed,
-                                         uint32_t sR, uint32_t sK)
+                                         uint32_t sR, uint32_t sK, int es_)
     {
         const int t = threadIdx.x;
         k_begin = k_begin_;
         kend = kend_;
+        es = es_;
         if (SRC == FG_KCONT) {
             rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(src), 0, (int)bytes, 0x00020000);
-            step = FG_BK * 4;
+            step = (uint32_t)(FG_BK * es);
 #pragma unroll
             for (int h = 0; h < NV; ++h) {
                 const int idx = h * FG_THREADS + t, row = idx >> 2, kq = idx & 3;
                 ok[h] = row0 + row < rows;
-                off[h] = ok[h] ? (uint32_t)(((int64_t)(row0 + row) * ld + k_begin + kq * 4) * 4) : 0u;
+                off[h] = ok[h] ? (uint32_t)(((int64_t)(row0 + row) * ld + k_begin + kq * 4) * es) : 0u;
             }
             kk0 = (t & 3) * 4;
         } else if (SRC == FG_MCONT) {
             rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(src), 0, (int)bytes, 0x00020000);
-            step = (uint32_t)(FG_BK * ld * 4);
+            step = (uint32_t)(FG_BK * ld * es);
 #pragma unroll
             for (int h = 0; h < NV; ++h) {
                 const int idx = h * FG_THREADS + t, kk = idx / (ROWS / 4), r4 = (idx % (ROWS / 4)) * 4;
                 ok[h] = row0 + r4 < rows;
-                off[h] = ok[h] ? (uint32_t)(((int64_t)(k_begin + kk) * ld + row0 + r4) * 4) : 0u;
+                off[h] = ok[h] ? (uint32_t)(((int64_t)(k_begin + kk) * ld + row0 + r4) * es) : 0u;
                 rows_left[h] = rows - (row0 + r4);
             }
             kk0 = t / (ROWS / 4);
@@ -128,8 +143,7 @@ template <int ROWS, int SRC, bool VEC> struct FgOperand {
                     r[h] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (ok[h] && kk < kend) ? (int)o : (int)FG_OOB, 0, 0));
                 } else {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        r[h][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, (ok[h] && kk + j < kend) ? (int)(o + 4 * j) : (int)FG_OOB, 0, 0));
+                    for (int j = 0; j < 4; ++j) r[h][j] = load1(o, ok[h] && kk + j < kend, j);
                 }
             }
         } else if (SRC == FG_MCONT) {
@@ -141,8 +155,7 @@ template <int ROWS, int SRC, bool VEC> struct FgOperand {
                     r[h] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, in ? (int)o : (int)FG_OOB, 0, 0));
                 } else {   // a thread's four values are consecutive rows: rows_left of them exist
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        r[h][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, (in && j < rows_left[h]) ? (int)(o + 4 * j) : (int)FG_OOB, 0, 0));
+                    for (int j = 0; j < 4; ++j) r[h][j] = load1(o, in && j < rows_left[h], j);
                 }
             }
         } else {
@@ -200,8 +213,8 @@ template <int BM, int ASRC, int BSRC, int EPI, bool VEC> __global__ __launch_bou
     const int nstage = (kend - k_begin + FG_BK - 1) / FG_BK;
     PA pa;
     PB pb;
-    pa.init(p.a, p.lda, p.a_bytes, m0, p.M, k_begin, kend, p.seed, p.nsR, p.nsK);
-    pb.init(p.b, p.ldb, p.b_bytes, n0, p.N, k_begin, kend, p.seed, p.nsR, p.nsK);
+    pa.init(p.a, p.lda, p.a_bytes, m0, p.M, k_begin, kend, p.seed, p.nsR, p.nsK, p.a_es);
+    pb.init(p.b, p.ldb, p.b_bytes, n0, p.N, k_begin, kend, p.seed, p.nsR, p.nsK, p.b_es);
     f32x16 acc[MI][NI];
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
@@ -243,22 +256,30 @@ template <int BM, int ASRC, int BSRC, int EPI, bool VEC> __global__ __launch_bou
     }
     // accumulator j of lane (r, g): row 8 (j / 4) + 4 g + j % 4 of the A side, column r of the B side
     float *out = p.out + (int64_t)blockIdx.z * p.split_stride;
-    const float scale = EPI == FG_ADD_SCALED ? p.scale[0] : 0.0f;
+    bf16_t *out16 = reinterpret_cast<bf16_t *>(p.out);   // bf16 outputs are never the ranges' partial matrices
+    const bool o16 = p.out_bf16 != 0;
+    const float scale = EPI != FG_ADD_SCALED ? 0.0f : p.scale_bf16 ? bf16_to_f32(reinterpret_cast<const bf16_t *>(p.scale)[0]) : p.scale[0];
     float dot = 0.0f;
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni) {
         const int n = n0 + wn * 64 + ni * 32 + r;
         if (n >= p.N) continue;
-        const float bv = EPI == FG_STORE_BIAS ? p.bias[n] : 0.0f;
+        const float bv = EPI != FG_STORE_BIAS ? 0.0f : o16 ? bf16_to_f32(reinterpret_cast<const bf16_t *>(p.bias)[n]) : p.bias[n];
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
             for (int j = 0; j < 16; ++j) {
                 const int m = m0 + wm * (BM / 2) + mi * 32 + 8 * (j >> 2) + 4 * g + (j & 3);
                 if (m >= p.M) continue;
-                if (EPI == FG_DOT) dot = fmaf(acc[mi][ni][j], p.dotm[(int64_t)m * p.lddot + n], dot);
-                else if (EPI == FG_ADD_SCALED) out[(int64_t)m * p.ldo + n] = fmaf(scale, acc[mi][ni][j], out[(int64_t)m * p.ldo + n]);
-                else out[(int64_t)m * p.ldo + n] = acc[mi][ni][j] + bv;
+                const float a = acc[mi][ni][j];
+                if (EPI == FG_DOT) {
+                    const int64_t e = (int64_t)m * p.lddot + n;
+                    dot = fmaf(a, o16 ? bf16_to_f32(reinterpret_cast<const bf16_t *>(p.dotm)[e]) : p.dotm[e], dot);
+                } else {
+                    const int64_t e = (int64_t)m * p.ldo + n;
+                    if (o16) out16[e] = f32_to_bf16(EPI == FG_ADD_SCALED ? fmaf(scale, a, bf16_to_f32(out16[e])) : a + bv);
+                    else out[e] = EPI == FG_ADD_SCALED ? fmaf(scale, a, out[e]) : a + bv;
+                }
             }
     }
     if (EPI == FG_DOT) {
@@ -312,9 +333,11 @@ static int64_t up256(int64_t n) { return (n + 255) / 256 * 256; }
 // multiples of 4 elements / 16 bytes get the kernels that read 16 bytes at a time, everything else the value-by-value ones.
 static bool fg_ok(const rdb_linear_desc *d)
 {
-    return d->act_dtype == RDB_F32 && d->coef_dtype == RDB_F32 && d->coef_rows != 0 && d->k > 0 && d->tokens > 0 && d->in_f > 0 && d->out_f > 0 &&
+    const bool f32 = d->act_dtype == RDB_F32 && d->coef_dtype == RDB_F32, b16 = d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16;
+    return (f32 || b16) && d->coef_rows != 0 && d->k > 0 && d->tokens > 0 && d->in_f > 0 && d->out_f > 0 &&
            d->tokens * d->k < (1ll << 29) && d->out_f * d->k < (1ll << 29) && d->in_f < (1 << 30) && d->out_f < (1 << 30);
 }
+static int fg_es(int dtype) { return dtype == RDB_BF16 ? 2 : 4; }
 // Wanted whenever the shapes fit: what AUTO would run instead is the general kernel, which forms W tiles on the vector ALU at a
 // few TFLOP/s, so the factored form on the matrix cores wins also where it is more flops than a product on a stored W.
 static bool fg_wanted(const rdb_linear_desc *) { return true; }
@@ -351,7 +374,7 @@ static FgPlan dc_plan(const rdb_linear_desc *d, int num_cus) { return fg_plan(d-
 int64_t linear_f32_workspace(int op, const rdb_linear_desc *d, int num_cus)
 {
     rdb_linear_desc dd = *d;
-    if (op == RDB_OP_LINEAR_BWD_DCOEF) dd.coef_dtype = RDB_F32;   // reads no coefficients
+    if (op == RDB_OP_LINEAR_BWD_DCOEF) dd.coef_dtype = dd.act_dtype;   // reads no coefficients
     if (!fg_ok(&dd)) return 0;
     const int64_t zt = up256(d->tokens * d->k * 4);
     auto with_parts = [&](int64_t K) { const int r = zt_plan(d, K, num_cus).ranges; return zt * (r > 1 ? 1 + r : 1); };
@@ -382,6 +405,8 @@ struct FgProduct {
     const float *dotm;      // or: dot_part[block] = <product tile, dotm tile>
     int64_t lddot;
     float *dot_part;
+    // bytes per element of the A and B matrices (2: bf16), and whether out / bias / dotm and scale are bf16
+    int a_es = 4, b_es = 4, out_bf16 = 0, scale_bf16 = 0;
 };
 
 #define FG_LAUNCH(BM_, EPI_)                                                                      \
@@ -405,8 +430,12 @@ template <int ASRC, int BSRC> static int fg_launch(const FgProduct &q, int num_c
     p.N = (int)q.N;
     p.K = (int)q.K;
     p.kchunk = (int)(q.kchunk > 0 ? q.kchunk : cdiv(q.K, FG_BK) * FG_BK);
-    p.a_bytes = q.a_elems * 4;
-    p.b_bytes = q.b_elems * 4;
+    p.a_bytes = q.a_elems * q.a_es;
+    p.b_bytes = q.b_elems * q.b_es;
+    p.a_es = q.a_es;
+    p.b_es = q.b_es;
+    p.out_bf16 = q.out_bf16;
+    p.scale_bf16 = q.scale_bf16;
     p.seed = q.seed;
     p.nsR = q.nsR;
     p.nsK = q.nsK;
@@ -421,7 +450,7 @@ template <int ASRC, int BSRC> static int fg_launch(const FgProduct &q, int num_c
         if (src != FG_KCONT && src != FG_MCONT) return true;
         return fg_aligned16(m) && ld % 4 == 0 && (src == FG_KCONT ? q.K % 4 == 0 : rows % 4 == 0);
     };
-    const bool vec = vec_ok(ASRC, q.a, q.lda, q.M) && vec_ok(BSRC, q.b, q.ldb, q.N);
+    const bool vec = vec_ok(ASRC, q.a, q.lda, q.M) && vec_ok(BSRC, q.b, q.ldb, q.N) && q.a_es == 4 && q.b_es == 4;   // bf16: value by value
     const dim3 grid((unsigned)cdiv(q.N, FG_BN), (unsigned)cdiv(q.M, q.bm), (unsigned)splits);
     if (BSRC == FG_NOISE_1D) {   // the random-bias products: added on top of an output, or reduced against a matrix
         if (q.bm == 128) {
@@ -478,6 +507,7 @@ template <int ASRC, int BSRC> static int fg_launch_ranges(FgProduct q, FgPlan pl
 static int fg_project(float *z, const float *x, int64_t ldx, const rdb_linear_desc *d, int num_cus, hipStream_t s)
 {
     FgProduct q = {x, ldx, (d->tokens - 1) * ldx + d->in_f, nullptr, 0, 0, z, d->k, nullptr, d->tokens, d->k, d->in_f, 128, 0, 0, d->seed};
+    q.a_es = fg_es(d->act_dtype);
     const int64_t zt = up256(d->tokens * d->k * 4) / 4;
     return fg_launch_ranges<FG_KCONT, FG_NOISE_M>(q, zt_plan(d, d->in_f, num_cus), z + zt, zt, num_cus, s, "f32_gemm_kernel (z = x . N^T)");
 }
@@ -492,12 +522,18 @@ int linear_fwd_f32(void *y, int64_t ldy, const void *x, int64_t ldx, const void 
     if (int rc = fg_project(z, (const float *)x, ldx, d, num_cus, s)) return rc;
     FgProduct q = {z, d->k, d->tokens * d->k, (const float *)coef, d->k, d->out_f * d->k, (float *)y, ldy, (const float *)bias,
                    d->tokens, d->out_f, d->k, fg_plan(d->tokens, d->out_f, d->k, num_cus, d->k, 1).bm, 0, 0, d->seed};
+    const int b16 = d->act_dtype == RDB_BF16;
+    q.b_es = fg_es(d->coef_dtype);
+    q.out_bf16 = b16;
     if (int rc = fg_launch<FG_KCONT, FG_KCONT>(q, num_cus, s, "f32_gemm_kernel (y = z . C^T)")) return rc;
     if (!scale_bias) return RDB_OK;
     // y += s * x . R^T: the B side's rows are output features, index o * in_f + i
     FgProduct qr = {(const float *)x, ldx, (d->tokens - 1) * ldx + d->in_f, nullptr, 0, 0, (float *)y, ldy, nullptr, d->tokens, d->out_f, d->in_f,
                     fg_plan(d->tokens, d->out_f, d->in_f, num_cus, d->in_f, 1).bm, 0, 0, d->seed, (uint32_t)d->in_f, 1u, (const float *)scale_bias,
                     nullptr, 0, nullptr};
+    qr.a_es = fg_es(d->act_dtype);
+    qr.out_bf16 = b16;
+    qr.scale_bf16 = d->coef_dtype == RDB_BF16;
     return fg_launch<FG_KCONT, FG_NOISE_1D>(qr, num_cus, s, "f32_gemm_kernel (y += s x . R^T)");
 }
 
@@ -510,17 +546,24 @@ int linear_dx_f32(void *dx, int64_t lddx, const void *dy, int64_t lddy, const vo
     // t[T x k] = dy[T x out_f] . C: the B side's rows are coefficients, read across the rows of C
     FgProduct q1 = {(const float *)dy, lddy, (d->tokens - 1) * lddy + d->out_f, (const float *)coef, d->k, d->out_f * d->k, t, d->k, nullptr,
                     d->tokens, d->k, d->out_f, 128, 0, 0, d->seed};
+    const int b16 = d->act_dtype == RDB_BF16;
+    q1.a_es = fg_es(d->act_dtype);
+    q1.b_es = fg_es(d->coef_dtype);
     const int64_t zt = up256(d->tokens * d->k * 4) / 4;
     if (int rc = fg_launch_ranges<FG_KCONT, FG_MCONT>(q1, zt_plan(d, d->out_f, num_cus), t + zt, zt, num_cus, s, "f32_gemm_kernel (t = dy . C)")) return rc;
     // dx[T x in_f] = t . N: the B side's rows are input features, hashed
     FgProduct q2 = {t, d->k, d->tokens * d->k, nullptr, 0, 0, (float *)dx, lddx, nullptr, d->tokens, d->in_f, d->k,
                     fg_plan(d->tokens, d->in_f, d->k, num_cus, d->k, 1).bm, 0, 0, d->seed};
+    q2.out_bf16 = b16;
     if (int rc = fg_launch<FG_KCONT, FG_NOISE_I>(q2, num_cus, s, "f32_gemm_kernel (dx = t . N)")) return rc;
     if (!scale_bias) return RDB_OK;
     // dx += s * dy . R: the B side's rows are input features, index o * in_f + i
     FgProduct qr = {(const float *)dy, lddy, (d->tokens - 1) * lddy + d->out_f, nullptr, 0, 0, (float *)dx, lddx, nullptr, d->tokens, d->in_f, d->out_f,
                     fg_plan(d->tokens, d->in_f, d->out_f, num_cus, d->out_f, 1).bm, 0, 0, d->seed, 1u, (uint32_t)d->in_f, (const float *)scale_bias,
                     nullptr, 0, nullptr};
+    qr.a_es = fg_es(d->act_dtype);
+    qr.out_bf16 = b16;
+    qr.scale_bf16 = d->coef_dtype == RDB_BF16;
     return fg_launch<FG_KCONT, FG_NOISE_1D>(qr, num_cus, s, "f32_gemm_kernel (dx += s dy . R)");
 }
 
@@ -530,7 +573,7 @@ int linear_dcoef_f32(float *dcoef, float *d_scale_bias, const void *dy, int64_t 
                      void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
     rdb_linear_desc dd = *d;
-    dd.coef_dtype = RDB_F32;   // no coefficients are read here
+    dd.coef_dtype = dd.act_dtype;   // no coefficients are read here
     if (!fg_ok(&dd) || !fg_wanted(&dd) || !fg_ws_ok(RDB_OP_LINEAR_BWD_DCOEF, &dd, num_cus, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
     if (d->tokens * ldx >= (1ll << 29) || d->tokens * lddy >= (1ll << 29)) return RDB_E_UNSUPPORTED;
     float *z = (float *)workspace;
@@ -541,6 +584,7 @@ int linear_dcoef_f32(float *dcoef, float *d_scale_bias, const void *dy, int64_t 
     FgProduct q = {(const float *)dy, lddy, (d->tokens - 1) * lddy + d->out_f, z, d->k, d->tokens * d->k, dcoef, d->k, nullptr,
                    d->out_f, d->k, d->tokens, 128, 0, 0, d->seed};
     const FgPlan dcp = dc_plan(&dd, num_cus);
+    q.a_es = fg_es(d->act_dtype);
     if (int rc = fg_launch_ranges<FG_MCONT, FG_MCONT>(q, dcp, part, up256(d->out_f * d->k * 4) / 4, num_cus, s, "f32_gemm_kernel (dC = dy^T . z)")) return rc;
     if (!d_scale_bias) return RDB_OK;
     // <dy, x . R^T>: the random-bias product once more, each block reducing its tile against dy's; then the blocks in order
@@ -548,6 +592,8 @@ int linear_dcoef_f32(float *dcoef, float *d_scale_bias, const void *dy, int64_t 
     FgProduct qr = {(const float *)x, ldx, (d->tokens - 1) * ldx + d->in_f, nullptr, 0, 0, nullptr, 0, nullptr, d->tokens, d->out_f, d->in_f,
                     fg_plan(d->tokens, d->out_f, d->in_f, num_cus, d->in_f, 1).bm, 0, 0, d->seed, (uint32_t)d->in_f, 1u, nullptr,
                     (const float *)dy, lddy, dots};
+    qr.a_es = fg_es(d->act_dtype);
+    qr.out_bf16 = d->act_dtype == RDB_BF16;   // dy, the matrix the product is reduced against
     if (int rc = fg_launch<FG_KCONT, FG_NOISE_1D>(qr, num_cus, s, "f32_gemm_kernel (<dy, x . R^T>)")) return rc;
     const int nblocks = (int)(cdiv(d->tokens, qr.bm) * cdiv(d->out_f, FG_BN));
     f32_sum_scalars_kernel<<<1, 256, 0, s>>>(d_scale_bias, dots, nblocks);

@@ -398,6 +398,14 @@ extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
         const int64_t a = linear_smallk_workspace(&dd), b = linear_f32_workspace(op, &dd, num_compute_units());
         return a > b ? a : b;
     }
+    if (d->act_dtype == RDB_BF16 && d->coef_rows != 0 && (d->in_f % 8 || d->out_f % 8 || d->k % 8) &&
+        (op == RDB_OP_LINEAR_FWD || op == RDB_OP_LINEAR_BWD_DX || op == RDB_OP_LINEAR_BWD_DCOEF)) {
+        // bf16 layers the bf16 factored kernels do not take (sizes that are not multiples of 8): the fp32 matrix-core kernels
+        // with bf16 matrices read value by value
+        rdb_linear_desc dd = *d;
+        if (op == RDB_OP_LINEAR_BWD_DCOEF) dd.coef_dtype = RDB_BF16;
+        return linear_f32_workspace(op, &dd, num_compute_units());
+    }
     if (op == RDB_OP_LINEAR_BWD_DX) return linear_dx_factored_workspace(d);
     if (op == RDB_OP_LINEAR_BWD_PROJECTED) return bwd_projected_workspace(d);
     if (op == RDB_OP_LINEAR_FWD) return d->coef_dtype == RDB_BF16 ? linear_projection_bytes(d) : 0;
@@ -419,8 +427,10 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
         if (rc != RDB_E_UNSUPPORTED) return rc;
         rc = linear_fwd_smallk(y, ldy, x, ldx, coef, scale_bias, bias, d, workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
-        rc = linear_fwd_f32(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), workspace, workspace_bytes, s);
-        if (rc != RDB_E_UNSUPPORTED) return rc;
+        if (d->act_dtype == RDB_F32) {
+            rc = linear_fwd_f32(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), workspace, workspace_bytes, s);
+            if (rc != RDB_E_UNSUPPORTED) return rc;
+        }
         if (d->algo == RDB_ALGO_FACTORED)
             return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd: the factored algorithm needs matrix-coef, no scale_bias, a workspace of "
                                                 "rdb_linear_workspace_bytes() bytes and either bf16 (activations and coef; sizes that are "
@@ -443,6 +453,11 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
             rc = linear_fwd_rbias_add(y, ldy, x, ldx, scale_bias, d, s);
             if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd: internal: the random-bias share refused a request the factored share took");
         }
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
+    if (d->algo == RDB_ALGO_AUTO && d->act_dtype == RDB_BF16) {
+        // bf16 sizes that kept every kernel above away (not multiples of 8): the fp32 matrix cores, reading bf16 value by value
+        rc = linear_fwd_f32(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
     }
     const int es = d->act_dtype == RDB_BF16 ? 2 : 4;
@@ -488,8 +503,10 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
         if (rc != RDB_E_UNSUPPORTED) return rc;
         rc = linear_dx_smallk(dx, lddx, dy, lddy, coef, scale_bias, d, workspace, workspace_bytes, (hipStream_t)stream);
         if (rc != RDB_E_UNSUPPORTED) return rc;
-        rc = linear_dx_f32(dx, lddx, dy, lddy, coef, scale_bias, d, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
-        if (rc != RDB_E_UNSUPPORTED) return rc;
+        if (d->act_dtype == RDB_F32) {
+            rc = linear_dx_f32(dx, lddx, dy, lddy, coef, scale_bias, d, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
+            if (rc != RDB_E_UNSUPPORTED) return rc;
+        }
         if (d->algo == RDB_ALGO_FACTORED)
             return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dx: the factored algorithm needs matrix-coef, a workspace of "
                                                 "rdb_linear_workspace_bytes() bytes and either bf16 (activations and coef; sizes that are "
@@ -510,6 +527,10 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
         df.algo = RDB_ALGO_FACTORED;
         rc = linear_dx_factored(dx, lddx, dy, lddy, coef, scale_bias, &df, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
         if (rc != RDB_E_UNSUPPORTED) return rc;
+        if (d->act_dtype == RDB_BF16) {   // sizes that are not multiples of 8: the fp32 matrix cores, reading bf16 value by value
+            rc = linear_dx_f32(dx, lddx, dy, lddy, coef, scale_bias, d, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
+            if (rc != RDB_E_UNSUPPORTED) return rc;
+        }
     }
     const int es = d->act_dtype == RDB_BF16 ? 2 : 4;
     LinParams p = {};
@@ -581,6 +602,11 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
                                             "multiples of 8; aligned rows) or fp32 (sizes that are multiples of 4; aligned rows)");
     if (d->algo != RDB_ALGO_TILE) {
         rc = linear_dcoef_fast(dcoef, d_scale_bias, dy, lddy, x, ldx, d, num_compute_units(), s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
+    if (d->algo == RDB_ALGO_AUTO && d->act_dtype == RDB_BF16) {
+        // sizes that are not multiples of 8: the fp32 matrix cores, reading bf16 value by value (they overwrite what was cleared)
+        rc = linear_dcoef_f32(dcoef, d_scale_bias, dy, lddy, x, ldx, d, num_compute_units(), workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
     }
     const int es = d->act_dtype == RDB_BF16 ? 2 : 4;

@@ -150,6 +150,9 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(wide)) == 65536 * 256 * 4
     # extents that are not multiples of 4 run on the same kernels (operands read value by value): same scratch
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(16, 4096, 4094, 128, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 16 * 128 * 4 * (1 + 32)
+    # bf16 sizes that are not multiples of 8 run on these kernels too (bf16 read value by value, z and t kept in fp32)
+    odd16 = desc(16, 4096, 4094, 128)
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(odd16)) == 16 * 128 * 4 * (1 + 32)
     # vector-coef: the general kernel, no scratch
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(16, 4096, 4096, 128, rows=0, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 0
 
