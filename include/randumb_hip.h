@@ -148,7 +148,8 @@ enum {
                              bytes at a time where sizes, leading dimensions and pointers are multiples of 4 elements
                              / 16 bytes; also with scale_bias, whose share is one more product with the random-bias
                              matrix hashed as an operand, and with its gradient).  Both fp32 forms add partial sums in
-                             a fixed order: bit-reproducible.
+                             a fixed order: bit-reproducible.  bf16 layers whose sizes are not multiples of 8 run on
+                             the fp32 matrix-core kernels too, their bf16 matrices read value by value.
                              With scale_bias (W = C.N + s.R, R the fused random bias, full rank) the input gradient adds
                              s * dy.R on top with R hashed into the matrix pipeline; forward and dcoef then need the
                              kernels that form W (RDB_ALGO_AUTO picks them). */
