@@ -208,7 +208,7 @@ template <int BM, int ASRC, int BSRC, int EPI, bool VEC> __global__ __launch_bou
     constexpr int MI = BM / 64, NI = 2, STAGE = PA::TILE + PB::TILE;
     __shared__ __align__(16) float lds[2 * STAGE];
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * FG_BN;
+    const int m0 = blockIdx.x * BM, n0 = blockIdx.y * FG_BN;   // the long extent (tokens, as a rule) on the grid's x
     const int k_begin = blockIdx.z * p.kchunk, kend = min(p.K, k_begin + p.kchunk);
     const int nstage = (kend - k_begin + FG_BK - 1) / FG_BK;
     PA pa;
@@ -451,7 +451,8 @@ template <int ASRC, int BSRC> static int fg_launch(const FgProduct &q, int num_c
         return fg_aligned16(m) && ld % 4 == 0 && (src == FG_KCONT ? q.K % 4 == 0 : rows % 4 == 0);
     };
     const bool vec = vec_ok(ASRC, q.a, q.lda, q.M) && vec_ok(BSRC, q.b, q.ldb, q.N) && q.a_es == 4 && q.b_es == 4;   // bf16: value by value
-    const dim3 grid((unsigned)cdiv(q.N, FG_BN), (unsigned)cdiv(q.M, q.bm), (unsigned)splits);
+    if (cdiv(q.N, FG_BN) > 65535) return RDB_E_UNSUPPORTED;   // the grid's y
+    const dim3 grid((unsigned)cdiv(q.M, q.bm), (unsigned)cdiv(q.N, FG_BN), (unsigned)splits);
     if (BSRC == FG_NOISE_1D) {   // the random-bias products: added on top of an output, or reduced against a matrix
         if (q.bm == 128) {
             if (q.dotm) FG_LAUNCH(128, FG_DOT);
