@@ -79,7 +79,10 @@ int rdb_materialize_fwd(float *out, const void *coef, int coef_dtype, int64_t co
  *   matrix-coef: Nw = coef_rows*row_len, dcoef[o*k+m] = sum_i noise(PRIME*i + m) * dW[o*row_len+i].
  * The reduction is a fixed tree (no atomics): results are bitwise reproducible run to run.
  * workspace: device scratch of at least rdb_materialize_bwd_workspace_bytes(...) bytes (may be NULL
- * when that returns 0). */
+ * when that returns 0).  Matrix-coef tensors of some millions of multiply-adds or more run as the matrix
+ * product dW . N^T on the fp32 matrix cores with the noise hashed as an operand (rdb_materialize_fwd: C . N
+ * likewise); the workspace then holds the sums over ranges of the row, added up in range order; with less
+ * workspace than the query asks for the vector-ALU kernel runs instead. */
 int rdb_materialize_bwd(float *dcoef, const void *dW, int dw_dtype, int64_t coef_rows, int64_t k,
                         int64_t row_len, int64_t Nw, uint32_t seed, void *workspace,
                         int64_t workspace_bytes, void *stream);

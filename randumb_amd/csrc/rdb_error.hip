@@ -63,6 +63,20 @@ int check_launch(const char *what)
     return set_error((int)e, "%s: %s", what, hipGetErrorString(e));
 }
 
+// Compute units of the current device; 256 when there is none (size queries without a GPU).
+int num_compute_units()
+{
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 }  // namespace rdb
 
 extern "C" int rdb_abi_version(void) { return 6; }

@@ -38,7 +38,8 @@ enum FgEpilogue {
     FG_STORE = 0,       // out = acc
     FG_STORE_BIAS = 1,  // out = acc + bias[column]
     FG_ADD_SCALED = 2,  // out += scale[0] * acc
-    FG_DOT = 3          // dot_part[block] = sum over the tile of acc * dotm (nothing is stored to out)
+    FG_DOT = 3,         // dot_part[block] = sum over the tile of acc * dotm (nothing is stored to out)
+    FG_STORE_RBIAS = 4  // out = acc + scale[0] * noise1d(row * nsR + column * nsK): materialising W = C . N + s . R
 };
 
 struct FgParams {
@@ -252,13 +253,19 @@ template <int BM, int ASRC, int BSRC, int EPI, bool VEC> __global__ __launch_bou
 #pragma unroll
                 for (int j = ks * PER; j < (ks + 1) * PER && j < PB::NV * 4; ++j) pb.hash_piece(s + 1, j);
             }
+            if (PA::HASHED && more) {
+                constexpr int PER = (PA::NV * 4 + FG_BK / 2 - 1) / (FG_BK / 2);
+#pragma unroll
+                for (int j = ks * PER; j < (ks + 1) * PER && j < PA::NV * 4; ++j) pa.hash_piece(s + 1, j);
+            }
         }
     }
     // accumulator j of lane (r, g): row 8 (j / 4) + 4 g + j % 4 of the A side, column r of the B side
     float *out = p.out + (int64_t)blockIdx.z * p.split_stride;
     bf16_t *out16 = reinterpret_cast<bf16_t *>(p.out);   // bf16 outputs are never the ranges' partial matrices
     const bool o16 = p.out_bf16 != 0;
-    const float scale = EPI != FG_ADD_SCALED ? 0.0f : p.scale_bf16 ? bf16_to_f32(reinterpret_cast<const bf16_t *>(p.scale)[0]) : p.scale[0];
+    const float scale = (EPI != FG_ADD_SCALED && EPI != FG_STORE_RBIAS) ? 0.0f
+                        : p.scale_bf16 ? bf16_to_f32(reinterpret_cast<const bf16_t *>(p.scale)[0]) : p.scale[0];
     float dot = 0.0f;
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni) {
@@ -277,7 +284,8 @@ template <int BM, int ASRC, int BSRC, int EPI, bool VEC> __global__ __launch_bou
                     dot = fmaf(a, o16 ? bf16_to_f32(reinterpret_cast<const bf16_t *>(p.dotm)[e]) : p.dotm[e], dot);
                 } else {
                     const int64_t e = (int64_t)m * p.ldo + n;
-                    if (o16) out16[e] = f32_to_bf16(EPI == FG_ADD_SCALED ? fmaf(scale, a, bf16_to_f32(out16[e])) : a + bv);
+                    if (EPI == FG_STORE_RBIAS) out[e] = fmaf(scale, noise1d((uint32_t)m * p.nsR + (uint32_t)n * p.nsK, p.seed), a);
+                    else if (o16) out16[e] = f32_to_bf16(EPI == FG_ADD_SCALED ? fmaf(scale, a, bf16_to_f32(out16[e])) : a + bv);
                     else out[e] = EPI == FG_ADD_SCALED ? fmaf(scale, a, out[e]) : a + bv;
                 }
             }
@@ -461,6 +469,9 @@ template <int ASRC, int BSRC> static int fg_launch(const FgProduct &q, int num_c
             if (q.dotm) FG_LAUNCH(64, FG_DOT);
             else FG_LAUNCH(64, FG_ADD_SCALED);
         }
+    } else if (q.scale) {        // materialising W with its random-bias share
+        if (q.bm == 128) FG_LAUNCH(128, FG_STORE_RBIAS);
+        else FG_LAUNCH(64, FG_STORE_RBIAS);
     } else if (q.bm == 128) {
         if (q.bias) FG_LAUNCH(128, FG_STORE_BIAS);
         else FG_LAUNCH(128, FG_STORE);
@@ -599,6 +610,63 @@ int linear_dcoef_f32(float *dcoef, float *d_scale_bias, const void *dy, int64_t 
     const int nblocks = (int)(cdiv(d->tokens, qr.bm) * cdiv(d->out_f, FG_BN));
     f32_sum_scalars_kernel<<<1, 256, 0, s>>>(d_scale_bias, dots, nblocks);
     return check_launch("f32_sum_scalars_kernel");
+}
+
+// ----------------------------------------------------------------------------------------------- materialise on the matrix cores
+// W = C . N (+ s . R) written to memory as fp32, matrix-coef, the (coef_rows, row_len) base tensor or its transpose
+// (src/rten_cpp/RandumbTensor.py:235-290), and its adjoint dcoef = dW . N^T (RandumbTensor.py:304-359): the same products as
+// the factored layer's, with the other operand being C or dW.  Worth it from some tens of millions of multiply-adds on; below
+// that the caller's vector-ALU kernels are as fast.
+constexpr int64_t FG_MATERIALIZE_MIN_MACS = (int64_t)1 << 26, FG_COEF_GRAD_MIN_MACS = (int64_t)1 << 23;
+
+static bool fg_mat_ok(int64_t coef_rows, int64_t k, int64_t row_len, int64_t min_macs)
+{
+    return coef_rows > 0 && k > 0 && row_len > 0 && coef_rows * k < (1ll << 29) && coef_rows * row_len < (1ll << 29) && row_len < (1 << 30) &&
+           coef_rows * k * row_len >= min_macs;
+}
+
+int materialize_mat_f32(float *out, const void *coef, int coef_dtype, int64_t coef_rows, int64_t k, int64_t row_len, bool transposed, uint32_t seed,
+                        const void *scale_bias, int num_cus, hipStream_t s)
+{
+    if (!fg_mat_ok(coef_rows, k, row_len, FG_MATERIALIZE_MIN_MACS)) return RDB_E_UNSUPPORTED;
+    const float *C = (const float *)coef;
+    if (!transposed) {
+        // W[o, i] = sum_m C[o, m] noise(i, m): rows = o from C, columns = i hashed; the random bias at index o * row_len + i
+        FgProduct q = {C, k, coef_rows * k, nullptr, 0, 0, out, row_len, nullptr, coef_rows, row_len, k,
+                       fg_plan(coef_rows, row_len, k, num_cus, k, 1).bm, 0, 0, seed, (uint32_t)row_len, 1u, (const float *)scale_bias, nullptr, 0, nullptr};
+        q.a_es = fg_es(coef_dtype);
+        q.scale_bf16 = coef_dtype == RDB_BF16;
+        return fg_launch<FG_KCONT, FG_NOISE_I>(q, num_cus, s, "f32_gemm_kernel (W = C . N)");
+    }
+    // W^T[i, o]: rows = i hashed, columns = o from C; the random bias at index o * row_len + i
+    FgProduct q = {nullptr, 0, 0, C, k, coef_rows * k, out, coef_rows, nullptr, row_len, coef_rows, k,
+                   fg_plan(row_len, coef_rows, k, num_cus, k, 1).bm, 0, 0, seed, 1u, (uint32_t)row_len, (const float *)scale_bias, nullptr, 0, nullptr};
+    q.b_es = fg_es(coef_dtype);
+    q.scale_bf16 = coef_dtype == RDB_BF16;
+    return fg_launch<FG_NOISE_I, FG_KCONT>(q, num_cus, s, "f32_gemm_kernel (W^T = N^T . C^T)");
+}
+
+static FgPlan mat_bwd_plan(int64_t coef_rows, int64_t k, int64_t row_len, int num_cus) { return fg_plan(coef_rows, k, row_len, num_cus, 256, 64); }
+
+// scratch of the adjoint: one [coef_rows x k] matrix per range of the row (none with a single range)
+int64_t coef_grad_mat_f32_workspace(int64_t coef_rows, int64_t k, int64_t row_len, int num_cus)
+{
+    if (!fg_mat_ok(coef_rows, k, row_len, FG_COEF_GRAD_MIN_MACS)) return 0;
+    const int r = mat_bwd_plan(coef_rows, k, row_len, num_cus).ranges;
+    return r > 1 ? (int64_t)r * up256(coef_rows * k * 4) : 0;
+}
+
+// dcoef[o, m] = sum_i dW[o, i] noise(i, m); dcoef is overwritten
+int coef_grad_mat_f32(float *dcoef, const void *dW, int dw_dtype, int64_t coef_rows, int64_t k, int64_t row_len, uint32_t seed, void *workspace,
+                      int64_t workspace_bytes, int num_cus, hipStream_t s)
+{
+    if (!fg_mat_ok(coef_rows, k, row_len, FG_COEF_GRAD_MIN_MACS)) return RDB_E_UNSUPPORTED;
+    const int64_t need = coef_grad_mat_f32_workspace(coef_rows, k, row_len, num_cus);
+    if (need > 0 && (!workspace || !fg_aligned16(workspace) || workspace_bytes < need)) return RDB_E_UNSUPPORTED;
+    FgProduct q = {(const float *)dW, row_len, coef_rows * row_len, nullptr, 0, 0, dcoef, k, nullptr, coef_rows, k, row_len, 128, 0, 0, seed};
+    q.a_es = fg_es(dw_dtype);
+    return fg_launch_ranges<FG_KCONT, FG_NOISE_M>(q, mat_bwd_plan(coef_rows, k, row_len, num_cus), (float *)workspace, up256(coef_rows * k * 4) / 4, num_cus,
+                                                  s, "f32_gemm_kernel (dcoef = dW . N^T)");
 }
 
 }  // namespace rdb

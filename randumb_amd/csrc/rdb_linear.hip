@@ -309,6 +309,9 @@ int linear_dx_smallk(void *dx, int64_t lddx, const void *dy, int64_t lddy, const
 int linear_dcoef_smallk(float *dcoef, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, void *workspace,
                         int64_t workspace_bytes, hipStream_t s);
 
+// rdb_error.hip
+int num_compute_units();   // of the current device (256 when there is none)
+
 // rdb_f32.hip
 int64_t linear_f32_workspace(int op, const rdb_linear_desc *d, int num_cus);
 int linear_fwd_f32(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
@@ -341,18 +344,6 @@ int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, co
                       int num_cus, hipStream_t s);
 
 // Compute units of the current device (cached per device id).
-static int num_compute_units()
-{
-    static int cached[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev] = n;
-    }
-    return cached[dev];
-}
 
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 

@@ -282,6 +282,14 @@ static void split_plan(int64_t Nw, int64_t k, int64_t *splits, int64_t *span)
     *splits = cdiv(Nw, sp) > 0 ? cdiv(Nw, sp) : 1;
 }
 
+// rdb_error.hip, rdb_f32.hip
+int num_compute_units();
+int materialize_mat_f32(float *out, const void *coef, int coef_dtype, int64_t coef_rows, int64_t k, int64_t row_len, bool transposed, uint32_t seed,
+                        const void *scale_bias, int num_cus, hipStream_t s);
+int64_t coef_grad_mat_f32_workspace(int64_t coef_rows, int64_t k, int64_t row_len, int num_cus);
+int coef_grad_mat_f32(float *dcoef, const void *dW, int dw_dtype, int64_t coef_rows, int64_t k, int64_t row_len, uint32_t seed, void *workspace,
+                      int64_t workspace_bytes, int num_cus, hipStream_t s);
+
 }  // namespace rdb
 
 using namespace rdb;
@@ -331,6 +339,9 @@ extern "C" int rdb_materialize_fwd(float *out, const void *coef, int coef_dtype,
     const bool base = (P == coef_rows && Q == row_len && sP == row_len && sQ == 1);
     const bool transposed = (P == row_len && Q == coef_rows && sP == 1 && sQ == row_len);
     if (base || transposed) {
+        // from some tens of millions of multiply-adds on: C . N on the fp32 matrix cores, the noise hashed as an operand
+        const int rc = materialize_mat_f32(out, coef, coef_dtype, coef_rows, k, row_len, transposed, seed, scale_bias, num_compute_units(), s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
         dim3 grid((unsigned)cdiv(row_len, MT_I), (unsigned)cdiv(coef_rows, MT_O));
         materialize_mat_tiled_kernel<<<grid, NT, 0, s>>>(out, coef, coef_dtype, coef_rows, k, row_len, base ? row_len : 1,
                                                          base ? 1 : coef_rows, seed, scale_bias);
@@ -343,8 +354,8 @@ extern "C" int rdb_materialize_fwd(float *out, const void *coef, int coef_dtype,
 
 extern "C" int64_t rdb_materialize_bwd_workspace_bytes(int64_t coef_rows, int64_t k, int64_t row_len, int64_t Nw)
 {
-    (void)row_len;
-    if (coef_rows != 0 || k <= 0 || Nw <= 0) return 0;
+    if (coef_rows != 0) return coef_grad_mat_f32_workspace(coef_rows, k, row_len, num_compute_units());   // matrix-coef: the ranges' sums
+    if (k <= 0 || Nw <= 0) return 0;
     int64_t splits, span;
     split_plan(Nw, k, &splits, &span);
     return splits > 1 ? splits * k * (int64_t)sizeof(float) : 0;
@@ -395,6 +406,10 @@ extern "C" int rdb_materialize_bwd(float *dcoef, const void *dW, int dw_dtype, i
         return set_error(RDB_E_SHAPE, "rdb_materialize_bwd: Nw=%lld is not rows*row_len=%lld*%lld", (long long)Nw,
                          (long long)coef_rows, (long long)row_len);
     if (!dW && Nw > 0) return set_error(RDB_E_NULL, "rdb_materialize_bwd: dW is NULL");
+    {   // large enough: dW . N^T on the fp32 matrix cores
+        const int rc = coef_grad_mat_f32(dcoef, dW, dw_dtype, coef_rows, k, row_len, seed, workspace, workspace_bytes, num_compute_units(), s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
     dim3 grid((unsigned)cdiv(k, GB_M), (unsigned)cdiv(coef_rows, GB_O));
     coef_grad_mat_kernel<<<grid, NT, 0, s>>>(dcoef, dW, dw_dtype, coef_rows, k, row_len, seed);
     return check_launch("coef_grad_mat_kernel");

@@ -179,3 +179,26 @@ def test_fused_random_bias_in_fp32(hip, oracle, T, in_f, out_f, k):
         assert abs(float(ds) - want_ds) < 1e-4 * max(abs(want_ds), float(np.linalg.norm(dW)))
         _, ds2 = hip.linear_bwd_dcoef(dyg, xg, k, out_f, in_f, out_f, in_f, 1, 9, want_scale_bias_grad=True)
         assert torch.equal(ds, ds2)
+
+
+@pytest.mark.parametrize("rows,row_len,k", [(512, 768, 256), (300, 1001, 230), (2048, 260, 132)])
+def test_materialise_on_the_matrix_cores(hip, oracle, rows, row_len, k):
+    """Matrix-coef W = C.N (+ s.noise1d) written to memory, its transposed view, and the adjoint dcoef = dW.N^T, at sizes the
+    matrix-core kernels take (some tens of millions of multiply-adds on), against the oracle."""
+    print(f"case materialise on the matrix cores rows={rows} row_len={row_len} k={k}", flush=True)
+    g = torch.Generator().manual_seed(rows + k)
+    C = torch.randn(rows, k, generator=g) * 0.05
+    sb = torch.tensor([0.3])
+    for s_ in (None, sb):
+        sbv = None if s_ is None else 0.3
+        W = oracle.materialize_fwd(C.numpy(), (rows, row_len), (row_len, 1), 7, scale_bias=sbv, row_len=row_len)
+        got = hip.materialize_fwd(C.cuda(), (rows, row_len), (row_len, 1), 7, None if s_ is None else s_.cuda(), s_ is not None, row_len)
+        assert got.shape == (rows, row_len) and rel_l2(got.cpu().numpy(), W) < F32_TOL
+        got_t = hip.materialize_fwd(C.cuda(), (row_len, rows), (1, row_len), 7, None if s_ is None else s_.cuda(), s_ is not None, row_len)
+        assert got_t.shape == (row_len, rows) and rel_l2(got_t.cpu().numpy(), W.T) < F32_TOL
+    dW = torch.randn(rows, row_len, generator=g)
+    want = oracle.materialize_bwd(dW.numpy(), k, 7, coef_rows=rows)
+    got = hip.materialize_bwd(dW.cuda(), k, 7, rows)
+    assert got.shape == (rows, k) and rel_l2(got.cpu().numpy(), want) < F32_TOL
+    got2 = hip.materialize_bwd(dW.cuda(), k, 7, rows)
+    assert torch.equal(got, got2)

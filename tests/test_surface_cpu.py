@@ -57,7 +57,9 @@ def test_argument_errors_come_back_as_codes_without_a_gpu():
     assert L.rdb_linear_fwd(None, 6, None, 8, None, None, None, ctypes.byref(d), None, 0, None) == -2  # coef_rows != out_f
     assert L.rdb_linear_fwd(None, 6, None, 8, None, None, None, None, None, 0, None) == -1
     assert L.rdb_materialize_bwd_workspace_bytes(0, 256, 0, 2359296) > 0
-    assert L.rdb_materialize_bwd_workspace_bytes(3072, 256, 768, 2359296) == 0
+    # matrix-coef, large enough for the matrix-core kernels: one [rows x k] matrix per range of the row (here 768 / 256 = 3)
+    assert L.rdb_materialize_bwd_workspace_bytes(3072, 256, 768, 2359296) == 3 * 3072 * 256 * 4
+    assert L.rdb_materialize_bwd_workspace_bytes(10, 64, 256, 2560) == 0
 
 
 def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
