@@ -262,6 +262,45 @@ def _(dy, state, coefs, in_features, seed):
     return [dy.new_empty([dy.shape[0], in_features]), dy.new_empty([coefs.shape[0], coefs.shape[1]], dtype=torch.float32)]
 
 
+def _tracing() -> bool:
+    return torch.compiler.is_compiling()
+
+
+def _dense(t: Optional[Tensor]) -> Optional[Tensor]:
+    """A pseudorandom tensor (a random-backed bias) as the dense tensor the library reads; the operator wrappers get this from
+    the tensor subclass's dispatch, the direct calls have to ask for it."""
+    return t.get_materialized() if t is not None and hasattr(t, "get_materialized") else t
+
+
+class _EagerLinear(torch.autograd.Function):
+    """``rten::linear_fwd`` and its registered backward, without the operator wrappers: what ``linear`` runs eagerly."""
+
+    @staticmethod
+    def forward(ctx, x, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias, bias):
+        ctx.save_for_backward(x, coefs, scale_bias)
+        ctx.meta = (in_features, out_features, stride_o, stride_i, seed)
+        ctx.bias_dtype = None if bias is None else bias.dtype
+        return hip.linear_fwd(x, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias, _dense(bias))
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, coefs, scale_bias = ctx.saved_tensors
+        in_f, out_f, sO, sI, seed = ctx.meta
+        dy = dy.contiguous()
+        dx = dcoefs = dsb = dbias = None
+        if ctx.needs_input_grad[0]:
+            dx = hip.linear_bwd_dx(dy, coefs, in_f, out_f, sO, sI, seed, scale_bias)
+        want_sb = scale_bias is not None and ctx.needs_input_grad[7]
+        if ctx.needs_input_grad[1] or want_sb:
+            dc, ds = hip.linear_bwd_dcoef(dy, x, coefs.shape[-1], 0 if coefs.dim() == 1 else coefs.shape[0], in_f, out_f, sO, sI, seed, want_sb)
+            dcoefs = dc.to(coefs.dtype)
+            if want_sb:
+                dsb = ds.to(scale_bias.dtype)
+        if ctx.bias_dtype is not None and ctx.needs_input_grad[8]:
+            dbias = dy.sum(0).to(ctx.bias_dtype)
+        return dx, dcoefs, None, None, None, None, None, dsb, dbias
+
+
 class _ProjectedLinear(torch.autograd.Function):
     """``y = x @ W.T (+ bias)`` for a matrix-coef weight in bf16.  The forward pass computes the projection state
     (``z = x @ Noise.T`` and the transposed coefficients) once and saves it for the backward pass in place of ``x``; the
@@ -269,7 +308,9 @@ class _ProjectedLinear(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, coefs, in_features, out_features, seed, bias):
-        y, state = linear_project_fwd(x, coefs, seed, bias)
+        # eagerly: straight to the library (the operator wrappers of torch.library cost more host time than the layer's
+        # kernels take); under torch.compile: through the registered operators, which it can trace
+        y, state = linear_project_fwd(x, coefs, seed, bias) if _tracing() else hip.linear_project_fwd(x, coefs, seed, _dense(bias))
         ctx.save_for_backward(state, coefs)
         ctx.meta = (in_features, out_features, seed)
         ctx.bias_dtype = None if bias is None else bias.dtype
@@ -281,13 +322,17 @@ class _ProjectedLinear(torch.autograd.Function):
         in_f, out_f, seed = ctx.meta
         dy = dy.contiguous()
         dx = dcoefs = dbias = None
+        direct = not _tracing()
         if ctx.needs_input_grad[0] and ctx.needs_input_grad[1]:
-            dx, dc = linear_bwd_projected(dy, state, coefs, in_f, seed)
+            dx, dc = hip.linear_bwd_projected(dy, state, coefs, in_f, seed) if direct else linear_bwd_projected(dy, state, coefs, in_f, seed)
             dcoefs = dc.to(coefs.dtype)
         elif ctx.needs_input_grad[0]:
-            dx = linear_bwd_dx(dy, coefs, in_f, out_f, in_f, 1, seed, None)
+            dx = (hip.linear_bwd_dx(dy, coefs, in_f, out_f, in_f, 1, seed, None) if direct
+                  else linear_bwd_dx(dy, coefs, in_f, out_f, in_f, 1, seed, None))
         elif ctx.needs_input_grad[1]:
-            dcoefs = linear_bwd_dcoef_projected(dy, state, coefs.shape[1], in_f, seed).to(coefs.dtype)
+            dc = (hip.linear_bwd_dcoef_projected(dy, state, coefs.shape[1], in_f, seed) if direct
+                  else linear_bwd_dcoef_projected(dy, state, coefs.shape[1], in_f, seed))
+            dcoefs = dc.to(coefs.dtype)
         if ctx.bias_dtype is not None and ctx.needs_input_grad[5]:
             dbias = dy.sum(0).to(ctx.bias_dtype)
         return dx, dcoefs, None, None, None, dbias
@@ -302,6 +347,8 @@ def linear(x: Tensor, coefs: Tensor, in_features: int, out_features: int, stride
             and (bias is None or bias.dtype == torch.bfloat16)
             and hip.linear_projection_preferred(x.shape[0], in_features, out_features, coefs.shape[1])):
         return _ProjectedLinear.apply(x, coefs, in_features, out_features, seed, bias)
+    if x.is_cuda and not _tracing():
+        return _EagerLinear.apply(x, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias, bias)
     return linear_fwd(x, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias, bias)
 
 
