@@ -142,20 +142,12 @@ enum {
                            strip must fit LDS).  dx: the workgroup keeps the noise columns of its 128 input features in
                            LDS and re-forms W in chunks of 64 output rows on the matrix cores (bf16 coef, k <= 256, no
                            scale_bias).  dcoef: dW tiles are formed and contracted with regenerated noise on chip. */
-    RDB_ALGO_FACTORED = 3 /* matrix-coef only: use W = C.N associatively so that no weight tile is formed at all:
-                             y = (x.N^T).C^T, dx = (dy.C).N, dcoef = dy^T.(x.N^T); the [tokens x k] intermediate lives
-                             in the caller's workspace.  bf16 activations and coef: matrix-core kernels; fp32 with
-                             k <= 64 and at most 1024 tokens (the GEMV-like regime; up to 4096 when asked for by this
-                             value): vector-ALU kernels; fp32 otherwise: fp32 matrix-core kernels (operands, products
-                             and sums in fp32, the noise hashed into the operand tiles; any sizes and alignments, 16
-                             bytes at a time where sizes, leading dimensions and pointers are multiples of 4 elements
-                             / 16 bytes; also with scale_bias, whose share is one more product with the random-bias
-                             matrix hashed as an operand, and with its gradient).  Both fp32 forms add partial sums in
-                             a fixed order: bit-reproducible.  bf16 layers whose sizes are not multiples of 8 run on
-                             the fp32 matrix-core kernels too, their bf16 matrices read value by value.
-                             With scale_bias (W = C.N + s.R, R the fused random bias, full rank) the input gradient adds
-                             s * dy.R on top with R hashed into the matrix pipeline; forward and dcoef then need the
-                             kernels that form W (RDB_ALGO_AUTO picks them). */
+    RDB_ALGO_FACTORED = 3 /* matrix-coef only: use W = C.N associatively so that no weight tile is formed:
+                             y = (x.N^T).C^T, dx = (dy.C).N, dcoef = dy^T.(x.N^T); the [tokens x k] intermediate lives in
+                             the caller's workspace.  bf16 activations and coef (sizes multiples of 8): bf16 matrix cores;
+                             fp32, or bf16 with other sizes: fp32 matrix cores, or the vector ALU for k <= 64 and few
+                             tokens; partial sums are added in a fixed order.  With scale_bias the full-rank share s.R is
+                             one more product with R hashed as an operand. */
 };
 
 enum { RDB_OP_LINEAR_FWD = 0, RDB_OP_LINEAR_BWD_DX = 1, RDB_OP_LINEAR_BWD_DCOEF = 2, RDB_OP_LINEAR_BWD_PROJECTED = 3 };
@@ -192,8 +184,10 @@ int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t lddy, cons
  * materialize_bwd (+ scale_bias_bwd) (R.py:979-990): dW is contracted with the regenerated noise tile
  * as it is produced and never written to memory.
  * dcoef (fp32, [k] or [out_f x k]) and, when d_scale_bias != NULL, d_scale_bias (fp32 [1]) are
- * OVERWRITTEN.  Partial sums from different tiles are combined with fp32 atomics (order-dependent in
- * the last bits, like the reference's relaxed atomics, R.py:359). */
+ * OVERWRITTEN.  fp32 activations: partial sums are added in a fixed order, the result is the same bit for
+ * bit from run to run.  bf16 activations: partial sums from different tiles are combined with fp32 atomics
+ * (order-dependent in the last bits, like the reference's relaxed atomics, R.py:359);
+ * rdb_linear_bwd_projected is the bf16 entry point with ordered sums. */
 int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const void *dy, int64_t lddy, const void *x,
                          int64_t ldx, const rdb_linear_desc *desc, void *workspace, int64_t workspace_bytes,
                          void *stream);
@@ -286,6 +280,32 @@ int rdb_linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *d
  * 128-wide ones may add partial sums over token ranges (same values up to fp32 rounding).  Process-wide; returns the previous
  * mode. */
 int rdb_set_big_tiles(int mode);
+
+/* ------------------------------------------------------------------------------- one-launch forms and their bounded waits
+ * No counterpart in the reference (its kernels are one launch per product).  rdb_linear_project_fwd / rdb_linear_fwd with
+ * bf16 and k <= 256, and rdb_linear_fwd / rdb_linear_bwd_dx with fp32, k <= 64 and few tokens, run producer and consumer
+ * blocks in ONE launch: consumers wait for per-tile tags that the producers publish.  The hardware is seen to hand out a
+ * launch's blocks in index order, so a consumer never keeps the producers it waits for off the chip; this is observed, not
+ * documented, so the wait is bounded (2^17 polls, a fraction of a second).  A block whose wait runs out does NOT compute: it
+ * fills its share of the output (y or dx) with NaN, adds one to a per-device counter inside the library and leaves; for the
+ * projected form it also sets bit 1 of the state's second 32-bit word.  The counter only ever grows.
+ *
+ * rdb_set_one_launch: mode 0 = never the one-launch forms (producers and consumers as separate launches: same results bit
+ * for bit), 1 (default) = where they apply.  Process-wide; returns the previous mode.
+ * rdb_sync_giveups_async: enqueues on `stream` a copy of the current device's counter to host_count (pinned host memory
+ * if the copy is to be asynchronous); does not wait.  rdb_sync_giveups: the same, and waits for `stream`.
+ * A caller that finds the counter changed must treat the outputs written since it last looked as invalid, and the
+ * projection states and recorded graphs of those launches as unusable; switching to mode 0 avoids a repeat. */
+int rdb_set_one_launch(int mode);
+int rdb_sync_giveups_async(uint32_t *host_count, void *stream);
+int rdb_sync_giveups(uint32_t *count, void *stream);
+
+/* Test hook, no counterpart in the reference: runs ONLY the consumer blocks of a one-launch forward on `scratch` (bf16
+ * layers: a projection state of rdb_linear_projection_bytes; fp32 layers: a forward workspace of rdb_linear_workspace_bytes)
+ * with a tag that nobody publishes and a wait of `polls` polls, so that every block's wait runs out: y becomes NaN
+ * throughout, the counter above grows by the number of blocks, every kernel ends normally. */
+int rdb_selftest_sync_giveup(void *y, int64_t ldy, void *scratch, int64_t scratch_bytes, const void *coef,
+                             const rdb_linear_desc *desc, int polls, void *stream);
 
 #ifdef __cplusplus
 }

@@ -45,7 +45,13 @@ EXPORTS = [
     "rdb_linear_bwd_dcoef_projected",
     "rdb_linear_bwd_projected",
     "rdb_set_big_tiles",
+    "rdb_set_one_launch",
+    "rdb_sync_giveups_async",
+    "rdb_sync_giveups",
+    "rdb_selftest_sync_giveup",
 ]
+
+ABI_VERSION = 7   # what this binding was written against (rdb_abi_version)
 
 
 class LinearDesc(ctypes.Structure):
@@ -87,6 +93,12 @@ def load() -> ctypes.CDLL:
     i64, u32, vp, ci = ctypes.c_int64, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_int
     L.rdb_abi_version.restype = ci
     L.rdb_abi_version.argtypes = []
+    # a library built from other sources may export the same names with other argument lists: calling those with this
+    # binding's arguments would hand the kernels shifted pointers
+    found = int(L.rdb_abi_version())
+    if found != ABI_VERSION:
+        raise RandumbHipError(f"{SO_PATH} has ABI version {found}, this package binds version {ABI_VERSION}: rebuild it with "
+                              "`make -C randumb_amd/csrc`")
     L.rdb_last_error_string.restype = ctypes.c_char_p
     L.rdb_last_error_string.argtypes = []
     L.rdb_sq5_fill_2d.argtypes = [vp, i64, i64, u32, vp]
@@ -125,6 +137,14 @@ def load() -> ctypes.CDLL:
     L.rdb_linear_bwd_projected.argtypes = [vp, i64, vp, vp, i64, vp, vp, dp, vp, i64, vp]
     L.rdb_set_big_tiles.argtypes = [ci]
     L.rdb_set_big_tiles.restype = ci
+    L.rdb_set_one_launch.argtypes = [ci]
+    L.rdb_set_one_launch.restype = ci
+    L.rdb_sync_giveups_async.argtypes = [vp, vp]
+    L.rdb_sync_giveups_async.restype = ci
+    L.rdb_sync_giveups.argtypes = [vp, vp]
+    L.rdb_sync_giveups.restype = ci
+    L.rdb_selftest_sync_giveup.argtypes = [vp, i64, vp, i64, vp, dp, ci, vp]
+    L.rdb_selftest_sync_giveup.restype = ci
     for name in ("rdb_sq5_fill_2d", "rdb_sq5_fill_1d", "rdb_materialize_fwd", "rdb_materialize_bwd", "rdb_scale_bias_bwd",
                  "rdb_embed_fwd", "rdb_embed_bwd", "rdb_linear_fwd", "rdb_linear_bwd_dx", "rdb_linear_bwd_dcoef",
                  "rdb_linear_project", "rdb_linear_project_fwd", "rdb_linear_fwd_projected", "rdb_linear_bwd_dcoef_projected",

@@ -116,14 +116,29 @@ template <class V> __device__ __forceinline__ void store_stream(V *dst, const V 
 // Blocks of one launch that consume what earlier blocks of the same launch produce: a producer publishes a 64-bit tag, unique
 // to the launch, in a slot of its own when its output is in memory; a consumer polls the slots it depends on.  Hardware
 // queues hand out the blocks of a launch in index order (per die), so a consumer that only waits for blocks with lower
-// indices cannot starve them.  The wait is bounded all the same: after SYNC_SPIN_LIMIT polls (a fraction of a second) the
-// consumer gives up, records it in *err and goes on with whatever is there.
+// indices cannot starve them.  That order is what the hardware is seen to do, not something its documentation promises, so
+// the wait is bounded: after `polls` polls (SYNC_SPIN_LIMIT: a fraction of a second) the consumer gives up.  A block that
+// gives up never computes on what happens to be in memory: it counts itself in the library's per-device give-up counter
+// (which the host reads: rdb_sync_giveups), sets bit 1 of *err when the caller has such a word, and its caller fills the
+// block's share of the output with NaN and leaves.
 //
 // The dies' L2 caches are not coherent with each other, and the fences that make them so (write back / invalidate a whole
 // L2) cost microseconds per block.  So the data that passes from producer to consumer goes around them instead: stored and
 // loaded with device scope (SCOPE_DEVICE below: write-through, and read from memory), as the tags are.
 constexpr int SYNC_SPIN_LIMIT = 1 << 17;
 constexpr int SCOPE_DEVICE = 16;   // cache-policy argument of the raw buffer loads and stores: sc1
+
+// What a waiting block needs besides its slots: how long to wait and where to report that it gave up.
+struct SyncWait {
+    unsigned int *err;       // NULL, or a word of the caller's state: bit 1 is set by a block that gave up
+    unsigned int *giveups;   // the library's counter of such blocks on this device
+    int polls;               // bound of the wait
+};
+
+// Device address of the give-up counter of the current device (rdb_error.hip); one per device, zero when the library loads.
+int sync_giveups_ptr(unsigned int **out);
+// 1: the one-launch forms run where they apply; 0: producers and consumers always as separate launches (rdb_set_one_launch).
+int one_launch_mode();
 
 // All threads of the block call this after their last store (with SCOPE_DEVICE) of the block's output.
 __device__ __forceinline__ void publish_tag(unsigned long long *slot, unsigned long long tag)
@@ -133,18 +148,21 @@ __device__ __forceinline__ void publish_tag(unsigned long long *slot, unsigned l
     if (threadIdx.x == 0) __hip_atomic_store(slot, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// One wave calls this: lanes 0 .. n - 1 (n <= 64) poll slots[0 .. n - 1].  Returns false after the spin limit.  Loads of the
-// producers' data that follow must use SCOPE_DEVICE.
-__device__ __forceinline__ bool await_tags(const unsigned long long *slots, int n, unsigned long long tag, unsigned int *err)
+// One wave calls this: lanes 0 .. n - 1 (n <= 64) poll slots[0 .. n - 1].  Returns false after the poll limit: the caller must
+// then poison its output instead of computing it.  Loads of the producers' data that follow must use SCOPE_DEVICE.
+__device__ __forceinline__ bool await_tags(const unsigned long long *slots, int n, unsigned long long tag, const SyncWait &w)
 {
     const int lane = threadIdx.x & 63;
     const unsigned long long *mine = slots + (lane < n ? lane : 0);
-    for (int it = 0; it < SYNC_SPIN_LIMIT; ++it) {
+    for (int it = 0; it < w.polls; ++it) {
         const unsigned long long v = __hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (__all(v == tag)) return true;
         __builtin_amdgcn_s_sleep(20);
     }
-    if (lane == 0) atomicOr(err, 2u);
+    if (lane == 0) {
+        if (w.err) atomicOr(w.err, 2u);
+        atomicAdd(w.giveups, 1u);
+    }
     return false;
 }
 

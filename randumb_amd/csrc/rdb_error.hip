@@ -77,7 +77,61 @@ int num_compute_units()
     return cached[dev];
 }
 
+// ----------------------------------------------------------------------------------------------- waits that gave up
+// Counter of blocks that gave up waiting for blocks of their own launch (rdb_common.hpp: await_tags); every device that runs
+// the library holds its own copy, zero when the library is loaded there.  In host code the name is only a handle: the
+// address is asked for once per device, with that device current, and kept.
+static __device__ unsigned int rdb_sync_giveup_count;
+
+int sync_giveups_ptr(unsigned int **out)
+{
+    static unsigned int *ptrs[64] = {nullptr};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return set_error((int)e, "give-up counter: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= 64) return set_error(RDB_E_UNSUPPORTED, "give-up counter: device index %d outside 0..63", dev);
+    unsigned int *p = __atomic_load_n(&ptrs[dev], __ATOMIC_ACQUIRE);
+    if (!p) {
+        void *v = nullptr;
+        e = hipGetSymbolAddress(&v, HIP_SYMBOL(rdb_sync_giveup_count));
+        if (e != hipSuccess || !v) return set_error(e != hipSuccess ? (int)e : RDB_E_UNSUPPORTED, "give-up counter: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        p = static_cast<unsigned int *>(v);
+        __atomic_store_n(&ptrs[dev], p, __ATOMIC_RELEASE);   // every thread that gets here asks for the same address
+    }
+    *out = p;
+    return RDB_OK;
+}
+
+static int g_one_launch = 1;
+int one_launch_mode() { return __atomic_load_n(&g_one_launch, __ATOMIC_RELAXED); }
+
 }  // namespace rdb
 
-extern "C" int rdb_abi_version(void) { return 6; }
+extern "C" int rdb_abi_version(void) { return 7; }
+
+extern "C" int rdb_set_one_launch(int mode)
+{
+    return __atomic_exchange_n(&rdb::g_one_launch, mode ? 1 : 0, __ATOMIC_RELAXED);
+}
+
+extern "C" int rdb_sync_giveups_async(uint32_t *host_count, void *stream)
+{
+    if (!host_count) return rdb::set_error(RDB_E_NULL, "rdb_sync_giveups_async: host_count is NULL");
+    unsigned int *p = nullptr;
+    if (int rc = rdb::sync_giveups_ptr(&p)) return rc;
+    hipError_t e = hipMemcpyAsync(host_count, p, sizeof(uint32_t), hipMemcpyDeviceToHost, (hipStream_t)stream);
+    if (e != hipSuccess) return rdb::set_error((int)e, "rdb_sync_giveups_async: hipMemcpyAsync: %s", hipGetErrorString(e));
+    return RDB_OK;
+}
+
+extern "C" int rdb_sync_giveups(uint32_t *count, void *stream)
+{
+    if (!count) return rdb::set_error(RDB_E_NULL, "rdb_sync_giveups: count is NULL");
+    unsigned int *p = nullptr;
+    if (int rc = rdb::sync_giveups_ptr(&p)) return rc;
+    hipError_t e = hipMemcpyAsync(count, p, sizeof(uint32_t), hipMemcpyDeviceToHost, (hipStream_t)stream);
+    if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
+    if (e != hipSuccess) return rdb::set_error((int)e, "rdb_sync_giveups: %s", hipGetErrorString(e));
+    return RDB_OK;
+}
 extern "C" const char *rdb_last_error_string(void) { return rdb::g_err; }

@@ -93,6 +93,11 @@ __device__ __forceinline__ void z_block(const ZParams &p, unsigned char *smem_ra
         return;
     }
     const int m0 = (w % p.tiles_m) * KZ_BM, tok0 = (w / p.tiles_m) * KZ_BT;
+    // A replay of a recorded launch carries the tag it was recorded with.  The consumers clear the slots when all of them are
+    // past their wait; should one of them have given up in an earlier replay, a slot may still hold the tag: take it back
+    // before this tile is touched.
+    if (p.sync && t == 0)
+        __hip_atomic_store(p.sync + (int64_t)(w / p.tiles_m) * (p.tiles_m + 1) + w % p.tiles_m, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     RDB_STAMP(0);
     typedef OperandTile<KZ_BM, F_BK, K_CONT> TN;   // noise tile: rows = coefficients, contraction = input features
     typedef OperandTile<KZ_BT, F_BK, K_CONT> TX;   // x tile: rows = tokens
@@ -413,7 +418,7 @@ int linear_project_fwd(void *y, int64_t ldy, void *state, const void *x, int64_t
     ZYParams p;
     if (!fill_z_params(p.z, state, x, ldx, with_ct ? coef : nullptr, d)) return RDB_E_UNSUPPORTED;
     const int y_items = fill_ys_params(p.y, y, ldy, state, coef, bias, d, num_cus);
-    if (!y_items || p.z.tiles_m > 64) {
+    if (!y_items || p.z.tiles_m > 64 || !one_launch_mode()) {
         // check the second call's conditions before the first launch, so that a refusal leaves nothing half done
         if (d->coef_dtype != RDB_BF16 || ldy % 8 || !aligned16(y) || !aligned16(coef)) return RDB_E_UNSUPPORTED;
         if (((uintptr_t)bias & 7) || d->tokens * ldy >= (1ll << 29)) return RDB_E_UNSUPPORTED;
@@ -426,7 +431,9 @@ int linear_project_fwd(void *y, int64_t ldy, void *state, const void *x, int64_t
     p.y.sync = p.z.sync;
     p.y.sync_tag = p.z.sync_tag;
     p.y.sync_n = p.z.tiles_m;
-    p.y.sync_err = reinterpret_cast<unsigned int *>(state) + 1;
+    p.y.sync_wait.err = reinterpret_cast<unsigned int *>(state) + 1;
+    p.y.sync_wait.polls = SYNC_SPIN_LIMIT;
+    if (int rc = sync_giveups_ptr(&p.y.sync_wait.giveups)) return rc;
     p.z_blocks = xcd_grid_size(p.z.tiles_m * p.z.tiles_t);
     const int kg = (int)cdiv(d->k, 64);
     if (bias) {
@@ -442,6 +449,30 @@ int linear_project_fwd(void *y, int64_t ldy, void *state, const void *x, int64_t
     case 2: return launch_zy<2, false>(p, y_items, s);
     case 3: return launch_zy<3, false>(p, y_items, s);
     default: return launch_zy<4, false>(p, y_items, s);
+    }
+}
+
+// Test hook: only the multiplying blocks of the one-launch forward, waiting (at most `polls` polls each) for a tag that
+// nobody publishes on `state`.  Every block gives up, fills its share of y with NaN and reports to the give-up counter.
+int selftest_giveup_factored(void *y, int64_t ldy, void *state, const void *coef, const rdb_linear_desc *d, int num_cus, int polls, hipStream_t s)
+{
+    StParams q;
+    const int items = fill_ys_params(q, y, ldy, state, coef, nullptr, d, num_cus);
+    const ProjLayout L = proj_layout(d);
+    if (!items || L.kpad / KZ_BM > 64) return RDB_E_UNSUPPORTED;
+    q.sync = reinterpret_cast<unsigned long long *>(static_cast<char *>(state) + L.sync_off);
+    q.sync_tag = next_sync_tag();
+    q.sync_n = L.kpad / KZ_BM;
+    q.sync_wait.err = reinterpret_cast<unsigned int *>(state) + 1;
+    q.sync_wait.polls = polls;
+    if (int rc = sync_giveups_ptr(&q.sync_wait.giveups)) return rc;
+    const int kg = (int)cdiv(d->k, 64);
+    const size_t smem = stationary_smem(kg);
+    switch (kg) {
+    case 1: return launch_stationary(factored_ys_kernel<1, false>, q, items, smem, s, "factored_ys_kernel<1> (self-test)");
+    case 2: return launch_stationary(factored_ys_kernel<2, false>, q, items, smem, s, "factored_ys_kernel<2> (self-test)");
+    case 3: return launch_stationary(factored_ys_kernel<3, false>, q, items, smem, s, "factored_ys_kernel<3> (self-test)");
+    default: return launch_stationary(factored_ys_kernel<4, false>, q, items, smem, s, "factored_ys_kernel<4> (self-test)");
     }
 }
 

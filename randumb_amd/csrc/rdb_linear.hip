@@ -877,6 +877,34 @@ extern "C" int rdb_linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, co
     return RDB_OK;
 }
 
+// rdb_factored.hip, rdb_smallk.hip
+namespace rdb {
+int selftest_giveup_factored(void *y, int64_t ldy, void *state, const void *coef, const rdb_linear_desc *d, int num_cus, int polls, hipStream_t s);
+int selftest_giveup_smallk(void *y, int64_t ldy, const void *coef, const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, int polls,
+                           hipStream_t s);
+}
+
+extern "C" int rdb_selftest_sync_giveup(void *y, int64_t ldy, void *scratch, int64_t scratch_bytes, const void *coef, const rdb_linear_desc *d,
+                                        int polls, void *stream)
+{
+    int rc = check_desc("rdb_selftest_sync_giveup", d);
+    if (rc) return rc;
+    if (!y || !scratch || !coef) return set_error(RDB_E_NULL, "rdb_selftest_sync_giveup: y, scratch or coef is NULL");
+    if (polls < 1 || polls > SYNC_SPIN_LIMIT) return set_error(RDB_E_SHAPE, "rdb_selftest_sync_giveup: polls must be 1 .. %d", SYNC_SPIN_LIMIT);
+    if (ldy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_selftest_sync_giveup: leading dimension smaller than the row");
+    if (d->act_dtype == RDB_BF16) {
+        const ChunkPlan pl = chunk_plan(d);
+        if (pl.nchunks != 1 || scratch_bytes < pl.state_stride) rc = RDB_E_UNSUPPORTED;
+        else rc = selftest_giveup_factored(y, ldy, scratch, coef, d, num_compute_units(), polls, (hipStream_t)stream);
+    } else {
+        rc = selftest_giveup_smallk(y, ldy, coef, d, scratch, scratch_bytes, polls, (hipStream_t)stream);
+    }
+    if (rc == RDB_E_UNSUPPORTED)
+        return set_error(RDB_E_UNSUPPORTED, "rdb_selftest_sync_giveup: needs a layer whose forward has a one-launch form (bf16 matrix-coef, k <= 256, "
+                                            "or fp32 matrix-coef, k <= 64, in_f <= 8192) and its scratch (projection state / forward workspace)");
+    return rc;
+}
+
 extern "C" int rdb_set_big_tiles(int mode)
 {
     const int before = big_tiles_mode();

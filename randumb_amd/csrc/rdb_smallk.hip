@@ -125,7 +125,7 @@ struct SkExpand {
     // counter per SK_ET tokens of the expanding blocks that have seen them (sync_consumers of them: the last clears the slots)
     unsigned long long *sync;
     unsigned long long sync_tag;
-    unsigned int *sync_err;
+    SyncWait sync_wait;
     unsigned int *sync_count;
     int sync_consumers;
 };
@@ -154,13 +154,22 @@ template <bool HASH> __device__ __forceinline__ void smallk_expand_block(const S
         }
     }
     if (p.sync) {   // the partial sums of these tokens come from earlier blocks of this launch
+        __shared__ int verdict;
         if (tid < 64) {
             const int tile0 = t0 / SK_TT, tiles = (T + SK_TT - 1) / SK_TT;
             const int ntile = (tile0 + SK_ET / SK_TT <= tiles) ? SK_ET / SK_TT : tiles - tile0;
             unsigned long long *slots = p.sync + (int64_t)tile0 * nchunk;
-            if (await_tags(slots, ntile * nchunk, p.sync_tag, p.sync_err)) release_tags(slots, ntile * nchunk, p.sync_count + by, p.sync_consumers);
+            const bool there = await_tags(slots, ntile * nchunk, p.sync_tag, p.sync_wait);
+            if (there) release_tags(slots, ntile * nchunk, p.sync_count + by, p.sync_consumers);
+            if (tid == 0) verdict = there ? 1 : 0;
         }
         __syncthreads();
+        if (verdict == 0) {   // gave up: the block's share of the output becomes NaN, never a sum of whatever is in memory
+            if (c < cols)
+                for (int tt = 0; tt < SK_ET; ++tt)
+                    if (t0 + tt < T) out[(int64_t)(t0 + tt) * ld_out + c] = __uint_as_float(0x7fc00000u);
+            return;
+        }
     }
     // s = sum of the partial matrices in chunk order; columns from k on take part as zeros.  A thread owns up to 4 entries
     // and keeps the loads of 8 chunks of all of them in flight at once: the kernel is a chain of memory latencies otherwise.
@@ -253,6 +262,9 @@ template <bool CHASH> __global__ __launch_bounds__(256) void smallk_fused_kernel
     const int b = blockIdx.x;
     if (b < p.c_blocks) {
         const int bx = b % p.c_tiles, by = b / p.c_tiles;
+        // a replayed launch carries the tag it was recorded with: should a consumer of an earlier replay have given up, the slot
+        // may still hold it (the consumers clear the slots only when all of them got past their wait)
+        if (threadIdx.x == 0) __hip_atomic_store(p.slots + (int64_t)bx * p.e.nchunk + by, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         smallk_contract_block<CHASH>(p.c, bx, by);
         if (by == 0 && bx % (SK_ET / SK_TT) == 0 && threadIdx.x == 0)
             __hip_atomic_store(p.counters + bx / (SK_ET / SK_TT), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -310,7 +322,8 @@ static bool smallk_wanted(const rdb_linear_desc *d)
 }
 
 // scratch: one partial [tokens x k] fp32 matrix per 256-chunk of the longer of in_f and out_f, then the tag slots of the
-// one-launch form (one per token tile and chunk), a word for a waiting block that gave up and a counter per 16 tokens
+// one-launch form (one per token tile and chunk), 8 bytes not in use and a counter per 16 tokens (a waiting block that gives
+// up reports to the library's per-device counter: the scratch may be the caller's and gone by the time anybody looks)
 static int64_t partial_bytes(const rdb_linear_desc *d)
 {
     const int64_t longer = d->in_f > d->out_f ? d->in_f : d->out_f;
@@ -345,17 +358,17 @@ static int contract_expand(float *out, int64_t ld_out, int cols, const float *sr
     const int nchunk = (int)cdiv(J, 256), tiles = (int)cdiv(T, SK_TT);
     SkFused f;
     f.c = {(float *)workspace, src, ld_src, coef, T, J, k, d->seed};
-    f.e = {out, ld_out, (const float *)workspace, nchunk, coef, bias, T, cols, k, d->seed, nullptr, 0, nullptr, nullptr, 0};
+    f.e = {out, ld_out, (const float *)workspace, nchunk, coef, bias, T, cols, k, d->seed, nullptr, 0, {nullptr, nullptr, SYNC_SPIN_LIMIT}, nullptr, 0};
     f.slots = reinterpret_cast<unsigned long long *>(static_cast<char *>(workspace) + partial_bytes(d));
     f.c_tiles = tiles;
     f.c_blocks = tiles * nchunk;
     f.e_colblocks = (int)cdiv(cols, 256);
     const int e_blocks = f.e_colblocks * (int)cdiv(T, SK_ET);
-    if (nchunk * (SK_ET / SK_TT) <= 64) {
+    if (nchunk * (SK_ET / SK_TT) <= 64 && one_launch_mode()) {
         f.e.sync = f.slots;
         f.e.sync_tag = next_tag();
-        f.e.sync_err = reinterpret_cast<unsigned int *>(f.slots + (int64_t)tiles * nchunk);
-        f.counters = f.e.sync_err + 2;
+        if (int rc = sync_giveups_ptr(&f.e.sync_wait.giveups)) return rc;
+        f.counters = reinterpret_cast<unsigned int *>(f.slots + (int64_t)tiles * nchunk) + 2;
         f.e.sync_count = f.counters;
         f.e.sync_consumers = f.e_colblocks;
         smallk_fused_kernel<CHASH><<<f.c_blocks + e_blocks, 256, 0, s>>>(f);
@@ -365,6 +378,25 @@ static int contract_expand(float *out, int64_t ld_out, int cols, const float *sr
     if (int rc = check_launch("smallk_contract_kernel")) return rc;
     smallk_expand_kernel<!CHASH><<<dim3((unsigned)f.e_colblocks, (unsigned)cdiv(T, SK_ET)), 256, 0, s>>>(f.e);
     return check_launch("smallk_expand_kernel");
+}
+
+// Test hook: only the expanding blocks of the one-launch form, waiting (at most `polls` polls each) for a tag that nobody
+// publishes.  Every block gives up, fills its share of y with NaN and reports to the give-up counter.
+int selftest_giveup_smallk(void *y, int64_t ldy, const void *coef, const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, int polls,
+                           hipStream_t s)
+{
+    if (!smallk_ok(d) || !ws_ok(d, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    const int T = (int)d->tokens, k = (int)d->k, nchunk = (int)cdiv(d->in_f, 256), tiles = (int)cdiv(T, SK_TT);
+    if (nchunk * (SK_ET / SK_TT) > 64) return RDB_E_UNSUPPORTED;
+    SkExpand e = {(float *)y, ldy, (const float *)workspace, nchunk, (const float *)coef, nullptr, T, (int)d->out_f, k, d->seed, nullptr, 0,
+                  {nullptr, nullptr, polls}, nullptr, 0};
+    e.sync = reinterpret_cast<unsigned long long *>(static_cast<char *>(workspace) + partial_bytes(d));
+    e.sync_tag = next_tag();
+    if (int rc = sync_giveups_ptr(&e.sync_wait.giveups)) return rc;
+    e.sync_count = reinterpret_cast<unsigned int *>(e.sync + (int64_t)tiles * nchunk) + 2;
+    e.sync_consumers = (int)cdiv(d->out_f, 256);
+    smallk_expand_kernel<false><<<dim3((unsigned)cdiv(d->out_f, 256), (unsigned)cdiv(T, SK_ET)), 256, 0, s>>>(e);
+    return check_launch("smallk_expand_kernel (self-test)");
 }
 
 // The three entry points return RDB_E_UNSUPPORTED, without setting an error, when the request does not fit.

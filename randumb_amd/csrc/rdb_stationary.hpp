@@ -38,7 +38,7 @@ struct StParams {
     unsigned long long *sync;
     unsigned long long sync_tag;
     int sync_n;
-    unsigned int *sync_err;
+    SyncWait sync_wait;
 };
 
 // KG: k rounded up to groups of 64 (compile time: the k loop is one straight line of code).  NOISE: the right operand's
@@ -226,12 +226,28 @@ __device__ __forceinline__ void stationary_block(const StParams &p, unsigned cha
         const __amdgpu_buffer_rsrc_t rs_z = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t *>(p.z), 0, (int)(padded * 2), 0x00020000);
         if (!NOISE) b.issue(b.unit0);
         if (p.sync) {   // z comes from earlier blocks of this launch
+            // the verdict of the waiting wave reaches the others through a word of LDS that nothing else touches: the padding
+            // at the end of the last row of the last wave's epilogue patch
+            volatile int *verdict = reinterpret_cast<volatile int *>(b.Cs + 2 * ST_BO * B::ldk + ST_BT * ST_STG_LD) - 1;
             if (wave == 0) {
                 unsigned long long *slots = p.sync + (int64_t)(w / p.splits) * (p.sync_n + 1);
-                if (await_tags(slots, p.sync_n, p.sync_tag, p.sync_err))
-                    release_tags(slots, p.sync_n, reinterpret_cast<unsigned int *>(slots + p.sync_n), p.splits);
+                const bool there = await_tags(slots, p.sync_n, p.sync_tag, p.sync_wait);
+                if (there) release_tags(slots, p.sync_n, reinterpret_cast<unsigned int *>(slots + p.sync_n), p.splits);
+                if (b.lane == 0) *verdict = there ? 1 : 0;
             }
             __syncthreads();
+            if (*verdict == 0) {
+                // gave up: z of these tokens is not known to be in memory.  The block's share of y becomes NaN (a result
+                // nobody can mistake for one) and the block leaves; the host learns of it from the give-up counter.
+                const i32x4 nan8 = {0x7fc07fc0, 0x7fc07fc0, 0x7fc07fc0, 0x7fc07fc0};
+                const int o_begin = b.unit0 * ST_BO, o_end = min(p.out_f, (b.unit0 + b.nunits) * ST_BO);
+                const int pieces = (o_end - o_begin) / 8;   // out_f is a multiple of 8
+                for (int e = t; e < ST_BT * pieces; e += ST_THREADS) {
+                    const int tok = (w / p.splits) * ST_BT + e / pieces, o = o_begin + (e % pieces) * 8;
+                    if (tok < p.tokens) __builtin_amdgcn_raw_buffer_store_b128(nan8, b.rs_y, (int)(((int64_t)tok * p.ldy + o) * 2), 0, 0);
+                }
+                return;
+            }
         }
         const int tile = tok0 >> 5;
         if (p.sync) {   // written by other dies during this launch: read around this die's L2
@@ -326,7 +342,7 @@ inline int make_stationary_grid(StParams &q, int64_t tokens, int64_t out_f, int 
     q.sync = nullptr;   // the left operand comes from an earlier launch unless the caller says otherwise afterwards
     q.sync_tag = 0;
     q.sync_n = 0;
-    q.sync_err = nullptr;
+    q.sync_wait = {nullptr, nullptr, SYNC_SPIN_LIMIT};
     q.tiles_t = (int)cdiv(tokens, ST_BT);
     const int units = (int)cdiv(out_f, ST_BO);
     int splits = (int)cdiv(num_cus, q.tiles_t);

@@ -5,6 +5,7 @@ raises ``NotImplementedError`` exactly as the reference's CPU registrations do
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional, Sequence
 
 import torch
@@ -50,6 +51,102 @@ def _seed(seed: int) -> int:
     if not 0 <= seed < 2**32:
         raise ValueError(f"seed must fit in 32 unsigned bits, got {seed}")
     return seed
+
+
+# ------------------------------------------------------------------------------------------------ waits that gave up
+class SyncWatch:
+    """Host side of the one-launch kernels' bounded waits.  A block that gives up waiting for blocks of its own launch fills
+    its share of the output with NaN and adds one to a counter on the device; this object looks at that counter without ever
+    making the hot loop wait: every ``every`` calls of an entry point that may run such a kernel it enqueues a 4-byte copy of
+    the counter into pinned host memory behind the work already on the stream, and looks at the copy once the stream has got
+    there.  A changed counter switches the library to separate launches (``rdb_set_one_launch(0)``) and raises."""
+
+    def __init__(self, lib=None, host_word=None, event_factory=None, every: int = 64):
+        self._lib = lib
+        self._host = host_word
+        self._event_factory = event_factory
+        self.every = every
+        self.calls = 0
+        self.seen = 0
+        self.pending = None
+
+    def _library(self):
+        return self._lib if self._lib is not None else _lib.load()
+
+    def _host_word(self):
+        if self._host is None:
+            self._host = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        return self._host
+
+    def _enqueue(self, stream) -> None:
+        L = self._library()
+        _lib.check(L.rdb_sync_giveups_async(ctypes.c_void_p(self._host_word().data_ptr()), stream), "rdb_sync_giveups_async")
+        ev = self._event_factory() if self._event_factory is not None else torch.cuda.Event()
+        ev.record()
+        self.pending = ev
+
+    def _judge(self) -> None:
+        self.pending = None
+        count = int(self._host_word()[0]) & 0xFFFFFFFF
+        if count != self.seen:
+            new, self.seen = (count - self.seen) & 0xFFFFFFFF, count
+            self._library().rdb_set_one_launch(0)
+            raise _lib.RandumbHipError(
+                f"{new} block(s) of a one-launch kernel gave up waiting for blocks of their own launch: the outputs they stood "
+                "for were filled with NaN, and projection states and recorded graphs of those launches must not be used again. "
+                "The library now runs producers and consumers as separate launches (rdb_set_one_launch(0)).")
+
+    def tick(self, stream) -> None:
+        """Called by the entry points that may run a one-launch kernel; never waits for the device."""
+        self.calls += 1
+        if self.pending is not None and self.pending.query():
+            self._judge()
+        if self.pending is None and self.calls % self.every == 0:
+            self._enqueue(stream)
+
+    def check(self, stream) -> None:
+        """Waits for the work on ``stream`` and raises if any block gave up since the last look."""
+        if self.pending is None:
+            self._enqueue(stream)
+        self.pending.synchronize()
+        self._judge()
+
+
+_watches: dict = {}
+
+
+def _watch(device) -> SyncWatch:
+    key = torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device()
+    w = _watches.get(key)
+    if w is None:
+        w = _watches[key] = SyncWatch()
+    return w
+
+
+def sync_check(device="cuda") -> None:
+    """Waits for the current stream of ``device`` and raises ``RandumbHipError`` if a block of a one-launch kernel has given
+    up its bounded wait since the last look (a training loop may call this once per optimizer step; the entry points look by
+    themselves, without waiting, every 64 calls)."""
+    dev = torch.device(device)
+    with torch.cuda.device(dev):
+        _watch(dev).check(_stream(dev))
+
+
+def set_one_launch(mode: int) -> int:
+    """Process-wide: 0 = producers and consumers of the factored forward (and of the fp32 small-k products) always as
+    separate launches, 1 = in one launch where that applies (default).  Same results bit for bit.  Returns the previous mode."""
+    return int(_lib.load().rdb_set_one_launch(int(mode)))
+
+
+def selftest_sync_giveup(y: torch.Tensor, scratch: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int, polls: int = 64) -> None:
+    """Test hook: runs only the consumer blocks of the one-launch forward of the layer ``coef`` (out_f, k) on ``scratch`` with
+    a tag nobody publishes; every block gives up after ``polls`` polls, ``y`` becomes NaN and the give-up counter grows."""
+    _need_gpu("selftest_sync_giveup", y, scratch, coef)
+    d = _desc(y.shape[0], in_f, coef.shape[0], coef, in_f, 1, seed, y.dtype, RDB_ALGO_AUTO)
+    with torch.cuda.device(y.device):
+        rc = _lib.load().rdb_selftest_sync_giveup(_p(y), y.stride(0), _p(scratch), scratch.numel() * scratch.element_size(), _p(coef),
+                                                  ctypes.byref(d), int(polls), _stream(y.device))
+    _lib.check(rc, "rdb_selftest_sync_giveup")
 
 
 # ------------------------------------------------------------------------------------------------ probes
@@ -209,9 +306,10 @@ def linear_fwd(x: torch.Tensor, coef: torch.Tensor, in_f: int, out_f: int, sO: i
     with torch.cuda.device(x.device):
         ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_FWD, ctypes.byref(d))
         ws = _workspace(ws_bytes, x.device)
-        rc = L.rdb_linear_fwd(_p(y), y.stride(0), _p(x), x.stride(0), _p(c), _p(sb), _p(b), ctypes.byref(d), _p(ws), ws_bytes,
-                              _stream(x.device))
-    _lib.check(rc, "rdb_linear_fwd")
+        st = _stream(x.device)
+        rc = L.rdb_linear_fwd(_p(y), y.stride(0), _p(x), x.stride(0), _p(c), _p(sb), _p(b), ctypes.byref(d), _p(ws), ws_bytes, st)
+        _lib.check(rc, "rdb_linear_fwd")
+        _watch(x.device).tick(st)
     return y
 
 
@@ -228,9 +326,10 @@ def linear_bwd_dx(dy: torch.Tensor, coef: torch.Tensor, in_f: int, out_f: int, s
     with torch.cuda.device(dy.device):
         ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX, ctypes.byref(d))
         ws = _workspace(ws_bytes, dy.device)
-        rc = L.rdb_linear_bwd_dx(_p(dx), dx.stride(0), _p(dy), dy.stride(0), _p(c), _p(sb), ctypes.byref(d), _p(ws), ws_bytes,
-                                 _stream(dy.device))
-    _lib.check(rc, "rdb_linear_bwd_dx")
+        st = _stream(dy.device)
+        rc = L.rdb_linear_bwd_dx(_p(dx), dx.stride(0), _p(dy), dy.stride(0), _p(c), _p(sb), ctypes.byref(d), _p(ws), ws_bytes, st)
+        _lib.check(rc, "rdb_linear_bwd_dx")
+        _watch(dy.device).tick(st)
     return dx
 
 
@@ -279,10 +378,17 @@ def linear_projection_supported(tokens: int, in_f: int, out_f: int, k: int) -> b
 
 
 def linear_projection_preferred(tokens: int, in_f: int, out_f: int, k: int) -> bool:
-    """Whether the projected form is also the faster one.  The factored products need 2*tokens*k*(in_f + out_f) flops per
-    direction, a product on a stored weight 2*tokens*in_f*out_f; the kernels that form the weight on chip instead lose
-    against the factored ones up to at least 8 times that (measured), so the bound is 16 times, as in the library."""
-    return k * (in_f + out_f) < 16 * in_f * out_f and linear_projection_supported(tokens, in_f, out_f, k)
+    """Whether a training step should save the projection state in place of ``x``.  Two conditions.  Speed: the factored
+    products need 2*tokens*k*(in_f + out_f) flops per direction, a product on a stored weight 2*tokens*in_f*out_f; the kernels
+    that form the weight on chip instead lose against the factored ones up to at least 8 times that (measured), so the bound
+    is 16 times, as in the library.  Memory: the state holds z twice (two element orders), 2 * 2 * k bytes per token with k
+    rounded up to 64, where the reference's autograd saves the 2 * in_f bytes of x (src/rten_cpp/RandumbTensor.py:942-946);
+    the state may cost up to twice that, i.e. k rounded up to 64 must not exceed in_f (768 -> 3072, k = 256: 1024 against
+    1536 bytes per token).  Layers that fail the second test still run the factored kernels, through ``rdb_linear_fwd`` and a
+    transient workspace, with x saved."""
+    kpad = -(-k // 64) * 64
+    return (k * (in_f + out_f) < 16 * in_f * out_f and kpad <= in_f
+            and linear_projection_supported(tokens, in_f, out_f, k))
 
 
 def linear_project(x: torch.Tensor, k: int, out_f: int, seed: int, coef: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -329,8 +435,10 @@ def linear_project_fwd(x: torch.Tensor, coef: torch.Tensor, seed: int, bias: Opt
     b = None if bias is None else bias.to(torch.bfloat16).contiguous()
     y = torch.empty((x.shape[0], out_f), dtype=torch.bfloat16, device=x.device)
     with torch.cuda.device(x.device):
-        rc = L.rdb_linear_project_fwd(_p(y), y.stride(0), _p(state), _p(x), x.stride(0), _p(c), _p(b), ctypes.byref(d), _stream(x.device))
-    _lib.check(rc, "rdb_linear_project_fwd")
+        st = _stream(x.device)
+        rc = L.rdb_linear_project_fwd(_p(y), y.stride(0), _p(state), _p(x), x.stride(0), _p(c), _p(b), ctypes.byref(d), st)
+        _lib.check(rc, "rdb_linear_project_fwd")
+        _watch(x.device).tick(st)
     return y, state
 
 
@@ -404,6 +512,23 @@ def linear_bwd_dcoef_projected(dy: torch.Tensor, state: torch.Tensor, k: int, in
     return dcoef
 
 
+# The backward kernels read C transposed from the copy the forward pass left in the state and never look at the values
+# behind ``coef`` for dy.C: a caller that changes coef between the two passes (an optimizer step before a delayed backward,
+# a state kept across steps) gets the gradient of the old coefficients with no error.  autograd's version counters catch that
+# for tensors it saved; RANDUMB_CHECK_STATE=1 (or this flag) makes every linear_bwd_projected compare the copy with coef
+# first, at the price of a device synchronisation.
+CHECK_STATE_COEF = os.environ.get("RANDUMB_CHECK_STATE", "0") not in ("", "0")
+
+
+def check_state_coef(state: torch.Tensor, coef: torch.Tensor, in_f: int) -> None:
+    """Raises if the transposed coefficients inside ``state`` are not the values of ``coef`` (out_f, k)."""
+    out_f, k = coef.shape
+    got = projection_unpack(state, in_f, out_f, k)["coef_t"]
+    if got is not None and not torch.equal(got, coef.to(torch.bfloat16).t()):
+        raise _lib.RandumbHipError("linear_bwd_projected: the coefficients have changed since the forward pass wrote this projection "
+                                   "state; its copy of them is what the backward kernels would read")
+
+
 def linear_bwd_projected(dy: torch.Tensor, state: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int, ordered_sums: bool = True):
     """Whole backward pass of a matrix-coef bf16 layer from the projection state: ``(dx, dcoef)`` with ``dx = dy @ W`` in
     bf16 and ``dcoef = dy.T @ z`` in fp32, in two kernel launches.  ``ordered_sums`` gives the library room for the partial
@@ -414,6 +539,8 @@ def linear_bwd_projected(dy: torch.Tensor, state: torch.Tensor, coef: torch.Tens
     out_f, k = c.shape
     d = _proj_desc(dy.shape[0], in_f, out_f, k, seed, c.dtype)
     _check_state(state, d, "linear_bwd_projected")
+    if CHECK_STATE_COEF:
+        check_state_coef(state, c, in_f)
     z = state
     dx = torch.empty((dy.shape[0], in_f), dtype=dy.dtype, device=dy.device)
     dcoef = torch.empty((out_f, k), dtype=torch.float32, device=dy.device)

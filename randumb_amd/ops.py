@@ -303,8 +303,11 @@ class _EagerLinear(torch.autograd.Function):
 
 class _ProjectedLinear(torch.autograd.Function):
     """``y = x @ W.T (+ bias)`` for a matrix-coef weight in bf16.  The forward pass computes the projection state
-    (``z = x @ Noise.T`` and the transposed coefficients) once and saves it for the backward pass in place of ``x``; the
-    reference's autograd saves ``x`` and materialises ``W`` again (RandumbTensor.py:942-946, 979-990)."""
+    (``z = x @ Noise.T`` in the two element orders its consumers read, and the transposed coefficients) once and saves it for
+    the backward pass in place of ``x``; the reference's autograd saves ``x`` and materialises ``W`` again
+    (RandumbTensor.py:942-946, 979-990).  Per token the state holds 4 bytes per coefficient (k rounded up to 64) where x holds
+    2 per input feature, plus once per layer a copy of the coefficients; ``linear`` takes this function only while that is at
+    most twice the size of x (``hip.linear_projection_preferred``)."""
 
     @staticmethod
     def forward(ctx, x, coefs, in_features, out_features, seed, bias):

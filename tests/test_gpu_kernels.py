@@ -399,6 +399,62 @@ def test_project_fwd_in_one_call(hip, T, in_f, out_f, k, seed):
     assert torch.equal(y_nb, hip.linear_fwd_projected(want_state, cg, in_f, seed))
 
 
+def test_a_wait_that_gives_up_is_loud(hip):
+    """Only the consumer blocks of the one-launch forward run, on a tag nobody publishes and with a wait of 32 polls: every
+    block gives up, every kernel ends normally, y is NaN throughout (never a product of whatever lay in memory), the state says
+    so, the host-side watch raises and switches the library to separate launches; with the switch back on, the next one-launch
+    call on the same state gives the bits of the two separate calls again.  bf16 (projection state) and fp32 small k (workspace)."""
+    from randumb_amd import _lib
+
+    print("case bounded wait gives up: bf16", flush=True)
+    T, in_f, out_f, k, seed = 1000, 264, 520, 136, 4
+    x, _, coef = _inputs(T, in_f, out_f, k, True, torch.bfloat16, seed)
+    xg, cg = x.cuda(), coef.cuda()
+    hip.sync_check()   # whatever earlier tests left is looked at here
+    want_y, state = hip.linear_project_fwd(xg, cg, seed)
+    y = torch.zeros_like(want_y)
+    hip.selftest_sync_giveup(y, state, cg, in_f, seed, polls=32)
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(y.float()).all()), "a block that gave up stored something other than NaN"
+    assert int(state.view(-1)[:8].view(torch.int32)[1]) == 2
+    with pytest.raises(_lib.RandumbHipError, match="gave up"):
+        hip.sync_check()
+    assert hip.set_one_launch(1) == 0, "the watch did not switch the one-launch forms off"
+    hip.sync_check()   # nothing new: no error
+    y2, state2 = hip.linear_project_fwd(xg, cg, seed)
+    assert torch.equal(y2, want_y) and int(state2.view(-1)[:8].view(torch.int32)[1]) == 0
+    want_state = hip.linear_project(xg, k, out_f, seed, coef=cg)
+    assert torch.equal(hip.linear_fwd_projected(want_state, cg, in_f, seed), want_y)
+    # separate launches give the same bits
+    assert hip.set_one_launch(0) == 1
+    try:
+        y3, _ = hip.linear_project_fwd(xg, cg, seed)
+        assert torch.equal(y3, want_y)
+    finally:
+        hip.set_one_launch(1)
+
+    print("case bounded wait gives up: fp32 small k", flush=True)
+    T, in_f, out_f, k, seed = 37, 1000, 520, 16, 9
+    x, _, coef = _inputs(T, in_f, out_f, k, True, torch.float32, seed)
+    xg, cg = x.cuda(), coef.cuda()
+    want = hip.linear_fwd(xg, cg, in_f, out_f, in_f, 1, seed)
+    d = hip._desc(T, in_f, out_f, cg, in_f, 1, seed, torch.float32, 0)
+    import ctypes
+    ws = torch.zeros(int(_lib.load().rdb_linear_workspace_bytes(0, ctypes.byref(d))), dtype=torch.uint8, device="cuda")
+    y = torch.zeros(T, out_f, device="cuda")
+    hip.selftest_sync_giveup(y, ws, cg, in_f, seed, polls=32)
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(y).all())
+    with pytest.raises(_lib.RandumbHipError, match="gave up"):
+        hip.sync_check()
+    hip.set_one_launch(0)
+    try:
+        two = hip.linear_fwd(xg, cg, in_f, out_f, in_f, 1, seed)
+    finally:
+        hip.set_one_launch(1)
+    assert torch.equal(two, want) and torch.equal(hip.linear_fwd(xg, cg, in_f, out_f, in_f, 1, seed), want)
+
+
 def test_projected_calls_take_leading_dimensions(hip):
     """x and dy as column slices of wider matrices (row stride larger than the row): the projected calls read them in place and
     give the bits they give on contiguous copies."""

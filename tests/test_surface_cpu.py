@@ -25,8 +25,97 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_lib.SO_PATH)
     for name in declared:
         assert hasattr(lib, name), name
-    assert _lib.load().rdb_abi_version() == 6
+    assert _lib.load().rdb_abi_version() == _lib.ABI_VERSION == 7
     assert ctypes.sizeof(_lib.LinearDesc) == 7 * 8 + 4 * 4
+
+
+def test_loader_refuses_a_library_of_another_abi_version(monkeypatch):
+    """A library that exports the same names with another ABI version is refused at load, not called with shifted arguments."""
+    from randumb_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "ABI_VERSION", 6)
+    with pytest.raises(_lib.RandumbHipError, match="ABI version 7"):
+        _lib.load()
+    monkeypatch.setattr(_lib, "ABI_VERSION", 7)
+    assert _lib.load().rdb_abi_version() == 7
+
+
+def test_one_launch_switch_without_a_gpu():
+    """rdb_set_one_launch returns the previous mode and starts at 1; the counter queries refuse a NULL destination."""
+    from randumb_amd import _lib
+
+    L = _lib.load()
+    assert L.rdb_set_one_launch(0) == 1 and L.rdb_set_one_launch(5) == 0 and L.rdb_set_one_launch(1) == 1
+    assert L.rdb_sync_giveups_async(None, None) == -1 and L.rdb_sync_giveups(None, None) == -1
+
+
+def test_sync_watch_host_logic():
+    """The host side of the one-launch kernels' bounded waits, with the library and the device stubbed out: the counter is
+    copied every `every` calls, looked at only when the copy has arrived, and a change switches the library to separate
+    launches and raises once (a later unchanged counter does not raise again)."""
+    from randumb_amd import _lib, hip
+
+    class FakeEvent:
+        done = False
+
+        def record(self):
+            pass
+
+        def query(self):
+            return self.done
+
+        def synchronize(self):
+            self.done = True
+
+    class FakeLib:
+        counter = 0
+        one_launch = 1
+        copies = 0
+
+        def __init__(self, host):
+            self.host = host
+
+        def rdb_sync_giveups_async(self, dst, stream):
+            self.copies += 1
+            self.host[0] = self.counter
+            return 0
+
+        def rdb_set_one_launch(self, mode):
+            old, self.one_launch = self.one_launch, mode
+            return old
+
+    host = torch.zeros(1, dtype=torch.int32)
+    lib = FakeLib(host)
+    events = []
+
+    def make_event():
+        events.append(FakeEvent())
+        return events[-1]
+
+    w = hip.SyncWatch(lib=lib, host_word=host, event_factory=make_event, every=4)
+    for _ in range(3):
+        w.tick(None)
+    assert lib.copies == 0 and w.pending is None
+    w.tick(None)                      # 4th call: a copy is enqueued, nothing is waited for
+    assert lib.copies == 1 and w.pending is events[0]
+    for _ in range(10):
+        w.tick(None)                  # the copy has not arrived: no look, no second copy
+    assert lib.copies == 1 and lib.one_launch == 1
+    events[0].done = True
+    w.tick(None)                      # arrived, counter unchanged: fine
+    assert w.pending is None and lib.one_launch == 1
+    lib.counter = 3                   # three blocks give up
+    w.tick(None)                      # call 16: next copy
+    assert lib.copies == 2
+    events[1].done = True
+    with pytest.raises(_lib.RandumbHipError, match="3 block"):
+        w.tick(None)
+    assert lib.one_launch == 0 and w.seen == 3
+    w.check(None)                     # an explicit look waits for the copy; the counter has not moved since: no error
+    lib.counter = 4
+    with pytest.raises(_lib.RandumbHipError, match="1 block"):
+        w.check(None)
 
 
 def test_big_tiles_switch_without_a_gpu():
@@ -308,5 +397,9 @@ def test_projected_form_is_chosen_only_where_it_runs_and_pays():
     # (768 -> 384 at k = 256), because the alternative is a kernel that forms the weight on chip
     assert hip.linear_projection_supported(512, 768, 384, 256) and hip.linear_projection_preferred(512, 768, 384, 256)
     assert hip.linear_projection_preferred(512, 768, 512, 256)
-    assert hip.linear_projection_preferred(64, 8, 8, 8)           # ratio 2
+    assert hip.linear_projection_preferred(64, 64, 64, 64)        # ratio 2
     assert hip.linear_projection_supported(64, 8, 8, 64) and not hip.linear_projection_preferred(64, 8, 8, 64)   # ratio 16
+    # ... and only while the state costs at most twice the memory of the x it is saved in place of: k (rounded up to 64) <= in_f
+    assert hip.linear_projection_preferred(4096, 4096, 14336, 1024) and hip.linear_projection_preferred(300, 1032, 2056, 512)
+    assert hip.linear_projection_supported(512, 256, 1024, 512) and not hip.linear_projection_preferred(512, 256, 1024, 512)
+    assert not hip.linear_projection_preferred(64, 8, 8, 8)
