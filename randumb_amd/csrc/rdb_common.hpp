@@ -137,6 +137,8 @@ struct SyncWait {
 
 // Device address of the give-up counter of the current device (rdb_error.hip); one per device, zero when the library loads.
 int sync_giveups_ptr(unsigned int **out);
+// The tag of a launch (never 0).
+unsigned long long next_sync_tag();
 // 1: the one-launch forms run where they apply; 0: producers and consumers always as separate launches (rdb_set_one_launch).
 int one_launch_mode();
 

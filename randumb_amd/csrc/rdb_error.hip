@@ -1,6 +1,10 @@
 // Error bookkeeping and library identification for librandumb_hip.
 #include <stdarg.h>
 #include <stdio.h>
+#include <unistd.h>
+
+#include <atomic>
+#include <random>
 
 #include "rdb_common.hpp"
 
@@ -100,6 +104,18 @@ int sync_giveups_ptr(unsigned int **out)
     }
     *out = p;
     return RDB_OK;
+}
+
+// A tag no other launch of any process is likely ever to have written where a launch's slots lie: a counter that starts at a
+// random 64-bit value.
+unsigned long long next_sync_tag()
+{
+    static std::atomic<unsigned long long> counter{[] {
+        std::random_device rd;
+        return ((unsigned long long)rd() << 32) ^ (unsigned long long)rd() ^ ((unsigned long long)getpid() << 17);
+    }()};
+    unsigned long long v = counter.fetch_add(1) + 1;
+    return v ? v : counter.fetch_add(1) + 1;
 }
 
 static int g_one_launch = 1;

@@ -13,9 +13,6 @@
 #include "rdb_blocks.hpp"
 #include "rdb_stationary.hpp"
 #include <algorithm>
-#include <atomic>
-#include <random>
-#include <unistd.h>
 
 namespace rdb {
 
@@ -388,18 +385,6 @@ static int fill_ys_params(StParams &q, void *y, int64_t ldy, const void *state, 
     q.k = (int)d->k;
     q.seed = 0;
     return make_stationary_grid(q, d->tokens, d->out_f, num_cus);
-}
-
-// A tag no other launch of any process is likely ever to have written where this launch's slots lie: a counter that starts
-// at a random 64-bit value.
-static unsigned long long next_sync_tag()
-{
-    static std::atomic<unsigned long long> counter{[] {
-        std::random_device rd;
-        return ((unsigned long long)rd() << 32) ^ (unsigned long long)rd() ^ ((unsigned long long)getpid() << 17);
-    }()};
-    unsigned long long v = counter.fetch_add(1) + 1;
-    return v ? v : counter.fetch_add(1) + 1;
 }
 
 template <int KG, bool BIAS> static int launch_zy(const ZYParams &p, int y_items, hipStream_t s)

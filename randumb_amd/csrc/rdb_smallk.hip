@@ -10,9 +10,6 @@
 // Replaces materialize() + dense product (src/rten_cpp/RandumbTensor.py:942-946) and MmBackward's dW followed by
 // materialize_bwd (RandumbTensor.py:979-990, 304-359) in the regime where a stored-W product would be bound by reading W.
 #include "rdb_common.hpp"
-#include <atomic>
-#include <random>
-#include <unistd.h>
 
 namespace rdb {
 
@@ -338,16 +335,6 @@ int64_t linear_smallk_workspace(const rdb_linear_desc *d)
 
 static bool ws_ok(const rdb_linear_desc *d, const void *ws, int64_t bytes) { return ws && bytes >= linear_smallk_workspace(d) && ((uintptr_t)ws & 7) == 0; }
 
-static unsigned long long next_tag()
-{
-    static std::atomic<unsigned long long> counter{[] {
-        std::random_device rd;
-        return ((unsigned long long)rd() << 32) ^ (unsigned long long)rd() ^ ((unsigned long long)getpid() << 17);
-    }()};
-    unsigned long long v = counter.fetch_add(1) + 1;
-    return v ? v : counter.fetch_add(1) + 1;
-}
-
 // Contraction over J (the rows of src) then expansion to `cols` columns: one launch when an expanding block's tags fit one
 // wave's lanes (J <= 8192), two otherwise.
 template <bool CHASH>
@@ -366,7 +353,7 @@ static int contract_expand(float *out, int64_t ld_out, int cols, const float *sr
     const int e_blocks = f.e_colblocks * (int)cdiv(T, SK_ET);
     if (nchunk * (SK_ET / SK_TT) <= 64 && one_launch_mode()) {
         f.e.sync = f.slots;
-        f.e.sync_tag = next_tag();
+        f.e.sync_tag = next_sync_tag();
         if (int rc = sync_giveups_ptr(&f.e.sync_wait.giveups)) return rc;
         f.counters = reinterpret_cast<unsigned int *>(f.slots + (int64_t)tiles * nchunk) + 2;
         f.e.sync_count = f.counters;
@@ -391,7 +378,7 @@ int selftest_giveup_smallk(void *y, int64_t ldy, const void *coef, const rdb_lin
     SkExpand e = {(float *)y, ldy, (const float *)workspace, nchunk, (const float *)coef, nullptr, T, (int)d->out_f, k, d->seed, nullptr, 0,
                   {nullptr, nullptr, polls}, nullptr, 0};
     e.sync = reinterpret_cast<unsigned long long *>(static_cast<char *>(workspace) + partial_bytes(d));
-    e.sync_tag = next_tag();
+    e.sync_tag = next_sync_tag();
     if (int rc = sync_giveups_ptr(&e.sync_wait.giveups)) return rc;
     e.sync_count = reinterpret_cast<unsigned int *>(e.sync + (int64_t)tiles * nchunk) + 2;
     e.sync_consumers = (int)cdiv(d->out_f, 256);
