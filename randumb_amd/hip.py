@@ -373,8 +373,20 @@ def linear_projection_bytes(tokens: int, in_f: int, out_f: int, k: int) -> int:
 
 def linear_projection_supported(tokens: int, in_f: int, out_f: int, k: int) -> bool:
     """Whether the projected entry points run a layer of these sizes: matrix-coef bf16, sizes in multiples of 8 (any number
-    of tokens: activations beyond one launch's 2^29 elements are run in chunks of tokens by the library)."""
-    return linear_projection_bytes(tokens, in_f, out_f, k) > 0
+    of tokens: activations beyond one launch's 2^29 elements are run in chunks of tokens by the library).  Plain integer
+    arithmetic, the library's own rule restated (``rdb_linear_projection_bytes(desc) > 0``; a test holds the two together), so
+    that a tracing compiler can follow the choice of path without calling into the library."""
+    if min(tokens, in_f, out_f, k) <= 0 or k % 8 or in_f % 8 or out_f % 8:
+        return False
+    kpad, out64 = -(-k // 64) * 64, -(-out_f // 64) * 64
+    per_chunk = ((1 << 28) // max(in_f, out_f, kpad)) // 256 * 256   # tokens of one launch
+    if per_chunk < 256:
+        return False
+    nchunks = -(-tokens // per_chunk)
+    chunk = -(-(-(-tokens // nchunks)) // 256) * 256 if nchunks > 1 else tokens
+    tok64 = -(-chunk // 64) * 64
+    limit = 1 << 29   # elements one buffer descriptor addresses
+    return tok64 * kpad < limit and out64 * kpad < limit and chunk * k < limit and out_f * k < limit
 
 
 def linear_projection_preferred(tokens: int, in_f: int, out_f: int, k: int) -> bool:
