@@ -150,7 +150,8 @@ enum {
                              one more product with R hashed as an operand. */
 };
 
-enum { RDB_OP_LINEAR_FWD = 0, RDB_OP_LINEAR_BWD_DX = 1, RDB_OP_LINEAR_BWD_DCOEF = 2, RDB_OP_LINEAR_BWD_PROJECTED = 3 };
+enum { RDB_OP_LINEAR_FWD = 0, RDB_OP_LINEAR_BWD_DX = 1, RDB_OP_LINEAR_BWD_DCOEF = 2, RDB_OP_LINEAR_BWD_PROJECTED = 3,
+       RDB_OP_LINEAR_BWD_PROJECTED_TO = 4 };
 
 /* Device scratch (bytes) that entry point `op` can use for `desc`; 0 when it has no use for any.  A NULL or too small
  * workspace is never an error with RDB_ALGO_AUTO: the library then runs a kernel that needs none. */
@@ -271,6 +272,15 @@ int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, c
 int rdb_linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *state,
                              const void *coef, const rdb_linear_desc *desc, void *workspace,
                              int64_t workspace_bytes, void *stream);
+
+/* rdb_linear_bwd_projected with dcoef in the dtype the caller keeps its coefficients in: dcoef_dtype RDB_F32 (the call above)
+ * or RDB_BF16, [out_f x k], the fp32 sums rounded to bf16 once by the blocks that add them up; what
+ * RandumbTensorConstructor.backward does with `.to(ctx.dtype)` after materialize_bwd (R.py:986), without the extra pass over
+ * dcoef.  RDB_BF16 needs a workspace of rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_PROJECTED_TO, desc) bytes and a layer
+ * that runs as one chunk of tokens (rdb_linear_projection_chunks == 1); otherwise RDB_E_UNSUPPORTED and nothing is launched. */
+int rdb_linear_bwd_projected_to(void *dx, int64_t lddx, void *dcoef, int dcoef_dtype, const void *dy, int64_t lddy,
+                                const void *state, const void *coef, const rdb_linear_desc *desc, void *workspace,
+                                int64_t workspace_bytes, void *stream);
 
 /* Tuning switch without a counterpart in the reference.  Layers with k > 256 whose products have enough 256 x 256 output
  * tiles to give every compute unit one run rdb_linear_fwd_projected / rdb_linear_project_fwd / rdb_linear_bwd_projected on

@@ -14,7 +14,7 @@ SO_PATH = os.path.join(_HERE, "librandumb_hip.so")
 
 RDB_F32, RDB_BF16 = 0, 1
 RDB_ALGO_AUTO, RDB_ALGO_TILE, RDB_ALGO_STRIP, RDB_ALGO_FACTORED = 0, 1, 2, 3
-RDB_OP_LINEAR_FWD, RDB_OP_LINEAR_BWD_DX, RDB_OP_LINEAR_BWD_DCOEF, RDB_OP_LINEAR_BWD_PROJECTED = 0, 1, 2, 3
+RDB_OP_LINEAR_FWD, RDB_OP_LINEAR_BWD_DX, RDB_OP_LINEAR_BWD_DCOEF, RDB_OP_LINEAR_BWD_PROJECTED, RDB_OP_LINEAR_BWD_PROJECTED_TO = 0, 1, 2, 3, 4
 
 # every exported entry point, in header order; tests check the list against the built library
 EXPORTS = [
@@ -44,6 +44,7 @@ EXPORTS = [
     "rdb_linear_fwd_projected",
     "rdb_linear_bwd_dcoef_projected",
     "rdb_linear_bwd_projected",
+    "rdb_linear_bwd_projected_to",
     "rdb_set_big_tiles",
     "rdb_set_one_launch",
     "rdb_sync_giveups_async",
@@ -135,6 +136,7 @@ def load() -> ctypes.CDLL:
     L.rdb_linear_fwd_projected.argtypes = [vp, i64, vp, vp, vp, dp, vp]
     L.rdb_linear_bwd_dcoef_projected.argtypes = [vp, vp, i64, vp, dp, vp]
     L.rdb_linear_bwd_projected.argtypes = [vp, i64, vp, vp, i64, vp, vp, dp, vp, i64, vp]
+    L.rdb_linear_bwd_projected_to.argtypes = [vp, i64, vp, ci, vp, i64, vp, vp, dp, vp, i64, vp]
     L.rdb_set_big_tiles.argtypes = [ci]
     L.rdb_set_big_tiles.restype = ci
     L.rdb_set_one_launch.argtypes = [ci]
@@ -148,7 +150,7 @@ def load() -> ctypes.CDLL:
     for name in ("rdb_sq5_fill_2d", "rdb_sq5_fill_1d", "rdb_materialize_fwd", "rdb_materialize_bwd", "rdb_scale_bias_bwd",
                  "rdb_embed_fwd", "rdb_embed_bwd", "rdb_linear_fwd", "rdb_linear_bwd_dx", "rdb_linear_bwd_dcoef",
                  "rdb_linear_project", "rdb_linear_project_fwd", "rdb_linear_fwd_projected", "rdb_linear_bwd_dcoef_projected",
-                 "rdb_linear_bwd_projected"):
+                 "rdb_linear_bwd_projected", "rdb_linear_bwd_projected_to"):
         getattr(L, name).restype = ci
     _lib = L
     return L

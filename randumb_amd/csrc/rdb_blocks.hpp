@@ -122,6 +122,7 @@ struct RedParams {
     int64_t n;             // multiple of 4
     int splits;
     int accumulate;        // 0: out = sum of the splits; 1: out += that sum (a later chunk of tokens of the same layer)
+    int out_bf16;          // 1: out is bf16, the fp32 sum rounded once (not with accumulate)
 };
 
 __device__ __forceinline__ void red_block(const RedParams &p, int block, int nblocks)
@@ -145,7 +146,12 @@ __device__ __forceinline__ void red_block(const RedParams &p, int block, int nbl
             for (int j = 0; j < 8; ++j)
                 if (s0 + j < p.splits) v += u[j];
         }
-        reinterpret_cast<f32x4 *>(p.out)[e] = v;
+        if (p.out_bf16) {
+            const uint2 h = {f32x2_to_bf16x2(v[0], v[1]), f32x2_to_bf16x2(v[2], v[3])};
+            reinterpret_cast<uint2 *>(p.out)[e] = h;
+        } else {
+            reinterpret_cast<f32x4 *>(p.out)[e] = v;
+        }
     }
     RDB_STAMP(3);
 }

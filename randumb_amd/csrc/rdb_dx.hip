@@ -314,10 +314,14 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
 // Whole backward pass of the layer from the saved projection z: dx = (dy.C).N and dcoef = dy^T.z in two launches.
 // Returns RDB_E_UNSUPPORTED (without setting an error) when the request does not fit.
 // accumulate: dcoef += instead of dcoef = (a later chunk of tokens of a layer whose activations are passed in chunks).
+// dc_bf16: dcoef is bf16 [out_f x k], the fp32 sums rounded once by the blocks that add them up (needs the workspace with room
+// for the sums, linear_bwd_projected_workspace(d, num_cus, true), and is not combined with accumulate).
 int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z, const void *coef,
-                         const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, bool accumulate, hipStream_t s)
+                         const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, bool accumulate, bool dc_bf16,
+                         hipStream_t s)
 {
     if (!dx_factored_ok(d)) return RDB_E_UNSUPPORTED;
+    if (dc_bf16 && (accumulate || workspace_bytes < linear_bwd_projected_workspace(d, num_cus, true))) return RDB_E_UNSUPPORTED;
     if (!workspace || workspace_bytes < linear_dx_factored_workspace(d) || ((uintptr_t)workspace & 15)) return RDB_E_UNSUPPORTED;
     if (d->tokens * lddy >= (1ll << 29) || lddy % 8 || lddx % 8) return RDB_E_UNSUPPORTED;
     if (((uintptr_t)dy & 15) || ((uintptr_t)coef & 15) || ((uintptr_t)dx & 15) || ((uintptr_t)z & 15) || ((uintptr_t)dcoef & 15))
@@ -326,12 +330,12 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
     make_dyc_params(p1, dy, lddy, coef, workspace, d);
     const size_t smem_dc = engine_smem<KD_BO, KD_BM, X_BK, M_CONT, M_CONT>(), smem_tn = engine_smem<K2_BI, K2_BT, X_BK, K_CONT, K_CONT>();
     const size_t smem_dyc = engine_smem<K1_BC, K1_BT, X_BK, M_CONT, K_CONT>();
-    if (workspace_bytes >= linear_bwd_projected_workspace(d, num_cus, accumulate)) {
+    if (workspace_bytes >= linear_bwd_projected_workspace(d, num_cus, accumulate || dc_bf16)) {
         BwdAParams a;
         const int dc_items = make_dc_params(a.dc, dcoef, dy, lddy, d, num_cus);
         dc_params_from_state(a.dc, z, d);
         // one token range only: its sums are the result, stored straight into dcoef, and nothing is left to add up
-        const bool direct = a.dc.splits == 1 && !accumulate;
+        const bool direct = a.dc.splits == 1 && !accumulate && !dc_bf16;
         a.dc.partial = direct ? dcoef : reinterpret_cast<float *>(static_cast<char *>(workspace) + align256(linear_dx_factored_workspace(d)));
         a.dyc = p1;
         {   // the transposed coefficients, if the forward pass left them in the state (its header says so)
@@ -362,6 +366,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
         red.n = d->out_f * d->k;
         red.splits = red_splits;
         red.accumulate = accumulate ? 1 : 0;
+        red.out_bf16 = dc_bf16 ? 1 : 0;
         if (tn_stationary_ok(d, lddx)) {
             BwdBsParams bs;
             const int items = make_tns_params(bs.tn, dx, lddx, workspace, d, num_cus);

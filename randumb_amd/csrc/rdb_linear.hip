@@ -322,7 +322,8 @@ int linear_dcoef_f32(float *dcoef, float *d_scale_bias, const void *dy, int64_t 
                      void *workspace, int64_t workspace_bytes, hipStream_t s);
 // rdb_dx.hip
 int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z, const void *coef,
-                         const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, bool accumulate, hipStream_t s);
+                         const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, bool accumulate, bool dc_bf16,
+                         hipStream_t s);
 int64_t linear_dx_factored_workspace(const rdb_linear_desc *d);
 int64_t linear_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus, bool force_partial);
 int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias,
@@ -375,7 +376,7 @@ template <typename K> static int launch(K kernel, dim3 grid, size_t smem, hipStr
 
 using namespace rdb;
 
-static int64_t bwd_projected_workspace(const rdb_linear_desc *d);
+static int64_t bwd_projected_workspace(const rdb_linear_desc *d, bool force_partial);
 
 extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
 {
@@ -398,7 +399,8 @@ extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
         return linear_f32_workspace(op, &dd, num_compute_units());
     }
     if (op == RDB_OP_LINEAR_BWD_DX) return linear_dx_factored_workspace(d);
-    if (op == RDB_OP_LINEAR_BWD_PROJECTED) return bwd_projected_workspace(d);
+    if (op == RDB_OP_LINEAR_BWD_PROJECTED) return bwd_projected_workspace(d, false);
+    if (op == RDB_OP_LINEAR_BWD_PROJECTED_TO) return bwd_projected_workspace(d, true);
     if (op == RDB_OP_LINEAR_FWD) return d->coef_dtype == RDB_BF16 ? linear_projection_bytes(d) : 0;
     if (op == RDB_OP_LINEAR_BWD_DCOEF) return linear_projection_bytes(d);  // reads no coefficients: their dtype does not matter
     return 0;
@@ -843,38 +845,54 @@ extern "C" int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int6
 
 // workspace of rdb_linear_bwd_projected: that of the largest chunk; chunks after the first add to dcoef and so always keep
 // their sums in the workspace first
-static int64_t bwd_projected_workspace(const rdb_linear_desc *d)
+static int64_t bwd_projected_workspace(const rdb_linear_desc *d, bool force_partial)
 {
     const ChunkPlan pl = chunk_plan(d);
     if (pl.nchunks == 0) return 0;
     const rdb_linear_desc first = chunk_desc(d, pl, 0);
-    return linear_bwd_projected_workspace(&first, num_compute_units(), pl.nchunks > 1);
+    return linear_bwd_projected_workspace(&first, num_compute_units(), pl.nchunks > 1 || force_partial);
+}
+
+static int bwd_projected_entry(const char *who, void *dx, int64_t lddx, void *dcoef, int dcoef_dtype, const void *dy, int64_t lddy, const void *z,
+                               const void *coef, const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    ChunkPlan pl;
+    int rc = check_projected(who, d, &pl);
+    if (rc) return rc;
+    if (!dx || !dcoef || !dy || !z || !coef) return set_error(RDB_E_NULL, "%s: dx, dcoef, dy, z or coef is NULL", who);
+    if (lddy < d->out_f || lddx < d->in_f) return set_error(RDB_E_SHAPE, "%s: leading dimension smaller than the row", who);
+    if (dcoef_dtype != RDB_F32 && dcoef_dtype != RDB_BF16) return set_error(RDB_E_DTYPE, "%s: dcoef_dtype must be RDB_F32 or RDB_BF16", who);
+    const bool dc_bf16 = dcoef_dtype == RDB_BF16;
+    const rdb_linear_desc first = chunk_desc(d, pl, 0);
+    if (d->coef_dtype != RDB_BF16 || lddy % 8 || lddx % 8 || !aligned16(dy) || !aligned16(dx) || !aligned16(z) || !aligned16(coef) ||
+        !aligned16(dcoef) || !aligned16(workspace) || pl.chunk_tokens * lddy >= (1ll << 29) || pl.chunk_tokens * lddx >= (1ll << 29) || !workspace ||
+        workspace_bytes < linear_dx_factored_workspace(&first))
+        return set_error(RDB_E_UNSUPPORTED, "%s: coefficients must be bf16; all pointers 16-byte aligned; lddy, lddx multiples of 8 and below "
+                                            "twice the row; workspace of rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX) bytes at least", who);
+    if (dc_bf16 && (pl.nchunks > 1 || workspace_bytes < bwd_projected_workspace(d, true)))
+        return set_error(RDB_E_UNSUPPORTED, "%s: dcoef in bf16 needs a layer that runs as one chunk of tokens and a workspace of "
+                                            "rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_PROJECTED_TO) bytes", who);
+    for (int c = 0; c < pl.nchunks; ++c) {
+        const rdb_linear_desc dd = chunk_desc(d, pl, c);
+        rc = linear_bwd_projected(at_bytes(dx, c * pl.chunk_tokens * lddx * 2), lddx, static_cast<float *>(dcoef),
+                                  at_bytes(dy, c * pl.chunk_tokens * lddy * 2), lddy, at_bytes(z, c * pl.state_stride), coef, &dd,
+                                  num_compute_units(), workspace, workspace_bytes, c > 0, dc_bf16, (hipStream_t)stream);
+        if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "%s: internal: chunk %d of %d refused", who, c, pl.nchunks);
+        if (rc) return rc;
+    }
+    return RDB_OK;
 }
 
 extern "C" int rdb_linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z, const void *coef,
                                         const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
 {
-    ChunkPlan pl;
-    int rc = check_projected("rdb_linear_bwd_projected", d, &pl);
-    if (rc) return rc;
-    if (!dx || !dcoef || !dy || !z || !coef) return set_error(RDB_E_NULL, "rdb_linear_bwd_projected: dx, dcoef, dy, z or coef is NULL");
-    if (lddy < d->out_f || lddx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_projected: leading dimension smaller than the row");
-    const rdb_linear_desc first = chunk_desc(d, pl, 0);
-    if (d->coef_dtype != RDB_BF16 || lddy % 8 || lddx % 8 || !aligned16(dy) || !aligned16(dx) || !aligned16(z) || !aligned16(coef) ||
-        !aligned16(dcoef) || !aligned16(workspace) || pl.chunk_tokens * lddy >= (1ll << 29) || pl.chunk_tokens * lddx >= (1ll << 29) || !workspace ||
-        workspace_bytes < linear_dx_factored_workspace(&first))
-        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_projected: coefficients must be bf16; all pointers 16-byte aligned; lddy, lddx "
-                                            "multiples of 8 and below twice the row; workspace of rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX) "
-                                            "bytes at least");
-    for (int c = 0; c < pl.nchunks; ++c) {
-        const rdb_linear_desc dd = chunk_desc(d, pl, c);
-        rc = linear_bwd_projected(at_bytes(dx, c * pl.chunk_tokens * lddx * 2), lddx, dcoef, at_bytes(dy, c * pl.chunk_tokens * lddy * 2), lddy,
-                                  at_bytes(z, c * pl.state_stride), coef, &dd, num_compute_units(), workspace, workspace_bytes, c > 0,
-                                  (hipStream_t)stream);
-        if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_projected: internal: chunk %d of %d refused", c, pl.nchunks);
-        if (rc) return rc;
-    }
-    return RDB_OK;
+    return bwd_projected_entry("rdb_linear_bwd_projected", dx, lddx, dcoef, RDB_F32, dy, lddy, z, coef, d, workspace, workspace_bytes, stream);
+}
+
+extern "C" int rdb_linear_bwd_projected_to(void *dx, int64_t lddx, void *dcoef, int dcoef_dtype, const void *dy, int64_t lddy, const void *z,
+                                           const void *coef, const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    return bwd_projected_entry("rdb_linear_bwd_projected_to", dx, lddx, dcoef, dcoef_dtype, dy, lddy, z, coef, d, workspace, workspace_bytes, stream);
 }
 
 // rdb_factored.hip, rdb_smallk.hip

@@ -37,7 +37,25 @@ def _p(t: Optional[torch.Tensor]):
 
 
 def _stream(device) -> ctypes.c_void_p:
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    idx = device.index
+    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if idx is None else idx))
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on(device):
+    """Context in which ``device`` is the current device; no work when it already is (the usual case)."""
+    idx = device.index
+    return _NO_SWITCH if idx is None or idx == torch.cuda.current_device() else torch.cuda.device(idx)
 
 
 def _workspace(nbytes: int, device) -> Optional[torch.Tensor]:
@@ -143,7 +161,7 @@ def selftest_sync_giveup(y: torch.Tensor, scratch: torch.Tensor, coef: torch.Ten
     a tag nobody publishes; every block gives up after ``polls`` polls, ``y`` becomes NaN and the give-up counter grows."""
     _need_gpu("selftest_sync_giveup", y, scratch, coef)
     d = _desc(y.shape[0], in_f, coef.shape[0], coef, in_f, 1, seed, y.dtype, RDB_ALGO_AUTO)
-    with torch.cuda.device(y.device):
+    with _on(y.device):
         rc = _lib.load().rdb_selftest_sync_giveup(_p(y), y.stride(0), _p(scratch), scratch.numel() * scratch.element_size(), _p(coef),
                                                   ctypes.byref(d), int(polls), _stream(y.device))
     _lib.check(rc, "rdb_selftest_sync_giveup")
@@ -154,7 +172,7 @@ def sq5_fill_2d(N: int, M: int, seed: int, device="cuda") -> torch.Tensor:
     """Noise matrix ``(N, M)``, ``out[n, m] = noise(PRIME*n + m)``  (RandumbTensor.py:101-105)."""
     out = torch.empty((N, M), dtype=torch.float32, device=device)
     _need_gpu("sq5_fill_2d", out)
-    with torch.cuda.device(out.device):
+    with _on(out.device):
         _lib.check(_lib.load().rdb_sq5_fill_2d(_p(out), N, M, _seed(seed), _stream(out.device)), "rdb_sq5_fill_2d")
     return out
 
@@ -163,7 +181,7 @@ def sq5_fill_1d(N: int, seed: int, device="cuda") -> torch.Tensor:
     """1-D noise ``out[n] = noise(n)``  (RandumbTensor.py:122-126)."""
     out = torch.empty((N,), dtype=torch.float32, device=device)
     _need_gpu("sq5_fill_1d", out)
-    with torch.cuda.device(out.device):
+    with _on(out.device):
         _lib.check(_lib.load().rdb_sq5_fill_1d(_p(out), N, _seed(seed), _stream(out.device)), "rdb_sq5_fill_1d")
     return out
 
@@ -195,7 +213,7 @@ def materialize_fwd(coefs: torch.Tensor, size: Sequence[int], strides: Sequence[
             row_len = numel // rows
     else:
         raise ValueError("coefs must be 1-D or 2-D")
-    with torch.cuda.device(c.device):
+    with _on(c.device):
         rc = _lib.load().rdb_materialize_fwd(_p(output), _p(c), _DT[c.dtype], rows, k, row_len, size[0], size[1],
                                              strides[0], strides[1], _seed(seed), _p(sb), _stream(c.device))
     _lib.check(rc, "rdb_materialize_fwd")
@@ -213,7 +231,7 @@ def materialize_bwd(dout: torch.Tensor, dcoefs_size: int, seed: int, coef_rows: 
     row_len = 0 if coef_rows == 0 else Nw // max(coef_rows, 1)
     dcoefs = torch.empty(shape, dtype=torch.float32, device=d.device)
     L = _lib.load()
-    with torch.cuda.device(d.device):
+    with _on(d.device):
         ws_bytes = L.rdb_materialize_bwd_workspace_bytes(coef_rows, k, row_len, Nw)
         ws = _workspace(ws_bytes, d.device)
         rc = L.rdb_materialize_bwd(_p(dcoefs), _p(d), _DT[d.dtype], coef_rows, k, row_len, Nw, _seed(seed), _p(ws), ws_bytes,
@@ -229,7 +247,7 @@ def scale_bias_bwd(dout: torch.Tensor, seed: int) -> torch.Tensor:
     d = _native(dout)
     ds = torch.empty((1,), dtype=torch.float32, device=d.device)
     L = _lib.load()
-    with torch.cuda.device(d.device):
+    with _on(d.device):
         ws_bytes = L.rdb_scale_bias_bwd_workspace_bytes(d.numel())
         ws = _workspace(ws_bytes, d.device)
         rc = L.rdb_scale_bias_bwd(_p(ds), _p(d), _DT[d.dtype], d.numel(), _seed(seed), _p(ws), ws_bytes, _stream(d.device))
@@ -244,7 +262,7 @@ def embed_fwd(idx: torch.Tensor, coefs: torch.Tensor, rowsize: int, seed: int) -
     c = _native(coefs)
     ix = idx.to(torch.int64).contiguous()
     out = torch.empty((*idx.shape, rowsize), dtype=torch.float32, device=c.device)
-    with torch.cuda.device(c.device):
+    with _on(c.device):
         rc = _lib.load().rdb_embed_fwd(_p(out), _p(ix), ix.numel(), _p(c), _DT[c.dtype], c.numel(), int(rowsize), _seed(seed),
                                        _stream(c.device))
     _lib.check(rc, "rdb_embed_fwd")
@@ -259,7 +277,7 @@ def embed_bwd(idx: torch.Tensor, dout: torch.Tensor, dcoefs_size: int, rowsize: 
     k = int(dcoefs_size)
     dcoefs = torch.empty((k,), dtype=torch.float32, device=d.device)
     L = _lib.load()
-    with torch.cuda.device(d.device):
+    with _on(d.device):
         ws_bytes = L.rdb_embed_bwd_workspace_bytes(ix.numel(), int(rowsize), k)
         ws = _workspace(ws_bytes, d.device)
         rc = L.rdb_embed_bwd(_p(dcoefs), _p(ix), ix.numel(), _p(d), _DT[d.dtype], k, int(rowsize), _seed(seed), _p(ws), ws_bytes,
@@ -303,7 +321,7 @@ def linear_fwd(x: torch.Tensor, coef: torch.Tensor, in_f: int, out_f: int, sO: i
     y = torch.empty((x.shape[0], out_f), dtype=x.dtype, device=x.device)
     d = _desc(x.shape[0], in_f, out_f, c, sO, sI, seed, x.dtype, algo)
     L = _lib.load()
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_FWD, ctypes.byref(d))
         ws = _workspace(ws_bytes, x.device)
         st = _stream(x.device)
@@ -323,7 +341,7 @@ def linear_bwd_dx(dy: torch.Tensor, coef: torch.Tensor, in_f: int, out_f: int, s
     dx = torch.empty((dy.shape[0], in_f), dtype=dy.dtype, device=dy.device)
     d = _desc(dy.shape[0], in_f, out_f, c, sO, sI, seed, dy.dtype, algo)
     L = _lib.load()
-    with torch.cuda.device(dy.device):
+    with _on(dy.device):
         ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX, ctypes.byref(d))
         ws = _workspace(ws_bytes, dy.device)
         st = _stream(dy.device)
@@ -348,7 +366,7 @@ def linear_bwd_dcoef(dy: torch.Tensor, x: torch.Tensor, k: int, coef_rows: int, 
     d.sO, d.sI, d.seed = int(sO), int(sI), _seed(seed)
     d.act_dtype, d.coef_dtype, d.algo = _DT[dy.dtype], RDB_F32, int(algo)
     L = _lib.load()
-    with torch.cuda.device(dy.device):
+    with _on(dy.device):
         ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DCOEF, ctypes.byref(d))
         ws = _workspace(ws_bytes, dy.device)
         rc = L.rdb_linear_bwd_dcoef(_p(dcoef), _p(dsb), _p(dy), dy.stride(0), _p(x), x.stride(0), ctypes.byref(d), _p(ws), ws_bytes,
@@ -364,6 +382,34 @@ def _proj_desc(tokens, in_f, out_f, k, seed, coef_dtype=torch.bfloat16) -> Linea
     d.sO, d.sI, d.seed = int(in_f), 1, _seed(seed)
     d.act_dtype, d.coef_dtype, d.algo = RDB_BF16, _DT[coef_dtype], RDB_ALGO_AUTO
     return d
+
+
+class _ProjPlan:
+    """What the projected calls need to know about a layer and batch, asked of the library once per (sizes, seed)."""
+    __slots__ = ("desc", "ref", "state_bytes", "state_cols", "ws_bytes", "ws_bytes_to", "chunks")
+
+    def __init__(self, tokens, in_f, out_f, k, seed):
+        L = _lib.load()
+        self.desc = _proj_desc(tokens, in_f, out_f, k, seed)
+        self.ref = ctypes.byref(self.desc)
+        self.state_bytes = int(L.rdb_linear_projection_bytes(self.ref))
+        self.state_cols = -(-self.state_bytes // tokens) if self.state_bytes > 0 else 0
+        self.ws_bytes = int(L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_PROJECTED, self.ref))
+        self.ws_bytes_to = int(L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_PROJECTED_TO, self.ref))
+        self.chunks = int(L.rdb_linear_projection_chunks(self.ref, None)) if self.state_bytes > 0 else 0
+
+
+_plans: dict = {}
+
+
+def _plan(tokens: int, in_f: int, out_f: int, k: int, seed: int) -> _ProjPlan:
+    key = (tokens, in_f, out_f, k, seed)
+    p = _plans.get(key)
+    if p is None:
+        if len(_plans) > 4096:
+            _plans.clear()
+        p = _plans[key] = _ProjPlan(tokens, in_f, out_f, k, _seed(seed))
+    return p
 
 
 def linear_projection_bytes(tokens: int, in_f: int, out_f: int, k: int) -> int:
@@ -423,7 +469,7 @@ def linear_project(x: torch.Tensor, k: int, out_f: int, seed: int, coef: Optiona
         c = coef.contiguous()
         if tuple(c.shape) != (out_f, k):
             raise ValueError(f"coef must be ({out_f}, {k}), got {tuple(c.shape)}")
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = L.rdb_linear_project(_p(state), _p(x), x.stride(0), _p(c), ctypes.byref(d), _stream(x.device))
     _lib.check(rc, "rdb_linear_project")
     return state
@@ -432,25 +478,29 @@ def linear_project(x: torch.Tensor, k: int, out_f: int, seed: int, coef: Optiona
 def linear_project_fwd(x: torch.Tensor, coef: torch.Tensor, seed: int, bias: Optional[torch.Tensor] = None):
     """``(y, state)``: :func:`linear_project` (with ``coef``) and :func:`linear_fwd_projected` in one call, for k <= 256 in a
     single kernel launch; the forward pass of a training step, ``state`` being what it saves for backward."""
-    _need_gpu("linear_project_fwd", x, coef)
+    if not (x.is_cuda and coef.is_cuda):
+        _need_gpu("linear_project_fwd", x, coef)
     x = _act(x)
-    c = _native(coef)
+    c = coef if coef.is_contiguous() else coef.contiguous()
     if x.dtype != torch.bfloat16 or c.dtype != torch.bfloat16:
         raise ValueError("linear_project_fwd computes in bf16")
     out_f, k = c.shape
-    d = _proj_desc(x.shape[0], x.shape[1], out_f, k, seed)
+    tokens = x.shape[0]
+    pl = _plan(tokens, x.shape[1], out_f, k, seed)
     L = _lib.load()
-    nbytes = L.rdb_linear_projection_bytes(ctypes.byref(d))
-    if nbytes <= 0:
-        _lib.check(L.rdb_linear_project(None, None, x.stride(0), None, ctypes.byref(d), None), "rdb_linear_project")
-    state = torch.empty((x.shape[0], -(-nbytes // x.shape[0])), dtype=torch.uint8, device=x.device)
+    if pl.state_bytes <= 0:
+        _lib.check(L.rdb_linear_project(None, None, x.stride(0), None, pl.ref, None), "rdb_linear_project")
+    dev = x.device
+    state = torch.empty((tokens, pl.state_cols), dtype=torch.uint8, device=dev)
     b = None if bias is None else bias.to(torch.bfloat16).contiguous()
-    y = torch.empty((x.shape[0], out_f), dtype=torch.bfloat16, device=x.device)
-    with torch.cuda.device(x.device):
-        st = _stream(x.device)
-        rc = L.rdb_linear_project_fwd(_p(y), y.stride(0), _p(state), _p(x), x.stride(0), _p(c), _p(b), ctypes.byref(d), st)
-        _lib.check(rc, "rdb_linear_project_fwd")
-        _watch(x.device).tick(st)
+    y = torch.empty((tokens, out_f), dtype=torch.bfloat16, device=dev)
+    with _on(dev):
+        st = _stream(dev)
+        rc = L.rdb_linear_project_fwd(y.data_ptr(), out_f, state.data_ptr(), x.data_ptr(), x.stride(0), c.data_ptr(),
+                                      None if b is None else b.data_ptr(), pl.ref, st)
+        if rc:
+            _lib.check(rc, "rdb_linear_project_fwd")
+        _watch(dev).tick(st)
     return y, state
 
 
@@ -504,7 +554,7 @@ def linear_fwd_projected(state: torch.Tensor, coef: torch.Tensor, in_f: int, see
     _check_state(state, d, "linear_fwd_projected")
     b = None if bias is None else bias.to(torch.bfloat16).contiguous()
     y = torch.empty((tokens, out_f), dtype=torch.bfloat16, device=state.device)
-    with torch.cuda.device(state.device):
+    with _on(state.device):
         rc = _lib.load().rdb_linear_fwd_projected(_p(y), y.stride(0), _p(state), _p(c), _p(b), ctypes.byref(d), _stream(state.device))
     _lib.check(rc, "rdb_linear_fwd_projected")
     return y
@@ -518,7 +568,7 @@ def linear_bwd_dcoef_projected(dy: torch.Tensor, state: torch.Tensor, k: int, in
     d = _proj_desc(dy.shape[0], in_f, out_f, k, seed)
     _check_state(state, d, "linear_bwd_dcoef_projected")
     dcoef = torch.empty((out_f, k), dtype=torch.float32, device=dy.device)
-    with torch.cuda.device(dy.device):
+    with _on(dy.device):
         rc = _lib.load().rdb_linear_bwd_dcoef_projected(_p(dcoef), _p(dy), dy.stride(0), _p(state), ctypes.byref(d), _stream(dy.device))
     _lib.check(rc, "rdb_linear_bwd_dcoef_projected")
     return dcoef
@@ -541,29 +591,53 @@ def check_state_coef(state: torch.Tensor, coef: torch.Tensor, in_f: int) -> None
                                    "state; its copy of them is what the backward kernels would read")
 
 
-def linear_bwd_projected(dy: torch.Tensor, state: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int, ordered_sums: bool = True):
+def linear_bwd_projected(dy: torch.Tensor, state: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int, ordered_sums: bool = True,
+                         dcoef_dtype: torch.dtype = torch.float32):
     """Whole backward pass of a matrix-coef bf16 layer from the projection state: ``(dx, dcoef)`` with ``dx = dy @ W`` in
-    bf16 and ``dcoef = dy.T @ z`` in fp32, in two kernel launches.  ``ordered_sums`` gives the library room for the partial
-    sums of ``dcoef`` (added in a fixed order: bit-reproducible); without it they are combined with fp32 atomics."""
-    _need_gpu("linear_bwd_projected", dy, state, coef)
+    bf16 and ``dcoef = dy.T @ z``, in two kernel launches.  ``ordered_sums`` gives the library room for the partial sums of
+    ``dcoef`` (added in a fixed order: bit-reproducible); without it they are combined with fp32 atomics.  ``dcoef_dtype``:
+    fp32, or bf16 to have the sums rounded once by the kernel that adds them up (what ``.to(bfloat16)`` would give, without
+    the extra pass; layers whose tokens the library runs in several chunks get fp32 sums rounded by torch instead)."""
+    if not (dy.is_cuda and state.is_cuda and coef.is_cuda):
+        _need_gpu("linear_bwd_projected", dy, state, coef)
     dy = _act(dy)
     c = _native(coef)
     out_f, k = c.shape
-    d = _proj_desc(dy.shape[0], in_f, out_f, k, seed, c.dtype)
-    _check_state(state, d, "linear_bwd_projected")
+    tokens = dy.shape[0]
+    pl = _plan(tokens, in_f, out_f, k, seed)
+    if c.dtype != torch.bfloat16:
+        _check_state(state, _proj_desc(tokens, in_f, out_f, k, seed, c.dtype), "linear_bwd_projected")
+    elif state.dtype != torch.uint8 or state.dim() != 2 or state.numel() < pl.state_bytes or pl.state_bytes <= 0 or not state.is_contiguous():
+        _check_state(state, pl.desc, "linear_bwd_projected")
     if CHECK_STATE_COEF:
         check_state_coef(state, c, in_f)
-    z = state
-    dx = torch.empty((dy.shape[0], in_f), dtype=dy.dtype, device=dy.device)
-    dcoef = torch.empty((out_f, k), dtype=torch.float32, device=dy.device)
+    if dcoef_dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("dcoef_dtype must be float32 or bfloat16")
+    in_kernel = dcoef_dtype == torch.bfloat16 and ordered_sums and pl.chunks == 1 and c.dtype == torch.bfloat16
+    dev = dy.device
+    dx = torch.empty((tokens, in_f), dtype=dy.dtype, device=dev)
+    dcoef = torch.empty((out_f, k), dtype=torch.bfloat16 if in_kernel else torch.float32, device=dev)
     L = _lib.load()
-    with torch.cuda.device(dy.device):
-        ws_bytes = L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_PROJECTED if ordered_sums else RDB_OP_LINEAR_BWD_DX, ctypes.byref(d))
-        ws = _workspace(ws_bytes, dy.device)
-        rc = L.rdb_linear_bwd_projected(_p(dx), dx.stride(0), _p(dcoef), _p(dy), dy.stride(0), _p(z), _p(c), ctypes.byref(d), _p(ws),
-                                        ws_bytes, _stream(dy.device))
-    _lib.check(rc, "rdb_linear_bwd_projected")
-    return dx, dcoef
+    d = pl.desc if c.dtype == torch.bfloat16 else _proj_desc(tokens, in_f, out_f, k, seed, c.dtype)
+    ref = pl.ref if d is pl.desc else ctypes.byref(d)
+    with _on(dev):
+        if in_kernel:
+            ws_bytes = pl.ws_bytes_to
+        elif ordered_sums:
+            ws_bytes = pl.ws_bytes
+        else:
+            ws_bytes = int(L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX, ref))
+        ws = _workspace(ws_bytes, dev)
+        st = _stream(dev)
+        if in_kernel:
+            rc = L.rdb_linear_bwd_projected_to(dx.data_ptr(), in_f, dcoef.data_ptr(), RDB_BF16, dy.data_ptr(), dy.stride(0), state.data_ptr(),
+                                               c.data_ptr(), ref, _p(ws), ws_bytes, st)
+        else:
+            rc = L.rdb_linear_bwd_projected(dx.data_ptr(), in_f, dcoef.data_ptr(), dy.data_ptr(), dy.stride(0), state.data_ptr(), c.data_ptr(),
+                                            ref, _p(ws), ws_bytes, st)
+    if rc:
+        _lib.check(rc, "rdb_linear_bwd_projected")
+    return dx, (dcoef if dcoef.dtype == dcoef_dtype else dcoef.to(dcoef_dtype))
 
 
 def set_big_tiles(mode: int) -> int:

@@ -323,12 +323,16 @@ class _ProjectedLinear(torch.autograd.Function):
     def backward(ctx, dy):
         state, coefs = ctx.saved_tensors
         in_f, out_f, seed = ctx.meta
-        dy = dy.contiguous()
+        if dy.stride(-1) != 1 or dy.stride(0) < dy.shape[1] or dy.stride(0) % 8 or dy.data_ptr() % 16:
+            dy = dy.contiguous()   # the kernels read rows with a leading dimension; anything else is copied
         dx = dcoefs = dbias = None
         direct = not _tracing()
         if ctx.needs_input_grad[0] and ctx.needs_input_grad[1]:
-            dx, dc = hip.linear_bwd_projected(dy, state, coefs, in_f, seed) if direct else linear_bwd_projected(dy, state, coefs, in_f, seed)
-            dcoefs = dc.to(coefs.dtype)
+            if direct:   # the sums leave the kernel in the coefficients' dtype: no cast afterwards
+                dx, dcoefs = hip.linear_bwd_projected(dy, state, coefs, in_f, seed, dcoef_dtype=coefs.dtype)
+            else:
+                dx, dc = linear_bwd_projected(dy, state, coefs, in_f, seed)
+                dcoefs = dc.to(coefs.dtype)
         elif ctx.needs_input_grad[0]:
             dx = (hip.linear_bwd_dx(dy, coefs, in_f, out_f, in_f, 1, seed, None) if direct
                   else linear_bwd_dx(dy, coefs, in_f, out_f, in_f, 1, seed, None))
