@@ -16,6 +16,7 @@
 // Replaces materialize() + dense product (src/rten_cpp/RandumbTensor.py:942-946) and MmBackward's dW followed by
 // materialize_bwd (RandumbTensor.py:979-990, 304-359) for fp32 layers beyond the few-token regime of rdb_smallk.hip.
 #include "rdb_gemm.hpp"
+#include <algorithm>
 
 namespace rdb {
 
@@ -515,13 +516,17 @@ template <int ASRC, int BSRC> static int fg_launch_ranges(FgProduct q, FgPlan pl
     return fg_sum(out, part, q.M * q.N, stride, splits, s);
 }
 
-// z[T x k] = src[T x in_f] . N^T; the partial matrices of its ranges follow z in the workspace
-static int fg_project(float *z, const float *x, int64_t ldx, const rdb_linear_desc *d, int num_cus, hipStream_t s)
+// z[T x k] = src[T x in_f] . N^T; the partial matrices of its ranges go to `part` (room for max_ranges of them, up256(T k 4)
+// bytes apart; NULL: right behind z, as many as the plan wants)
+static int fg_project(float *z, const float *x, int64_t ldx, const rdb_linear_desc *d, int num_cus, hipStream_t s, float *part = nullptr,
+                      int max_ranges = 1 << 30)
 {
     FgProduct q = {x, ldx, (d->tokens - 1) * ldx + d->in_f, nullptr, 0, 0, z, d->k, nullptr, d->tokens, d->k, d->in_f, 128, 0, 0, d->seed};
     q.a_es = fg_es(d->act_dtype);
     const int64_t zt = up256(d->tokens * d->k * 4) / 4;
-    return fg_launch_ranges<FG_KCONT, FG_NOISE_M>(q, zt_plan(d, d->in_f, num_cus), z + zt, zt, num_cus, s, "f32_gemm_kernel (z = x . N^T)");
+    FgPlan plan = zt_plan(d, d->in_f, num_cus);
+    if (plan.ranges > max_ranges) plan.ranges = max_ranges < 1 ? 1 : max_ranges;
+    return fg_launch_ranges<FG_KCONT, FG_NOISE_M>(q, plan, part ? part : z + zt, zt, num_cus, s, "f32_gemm_kernel (z = x . N^T)");
 }
 
 // The three entry points return RDB_E_UNSUPPORTED, without setting an error, when the request does not fit.
@@ -610,6 +615,77 @@ int linear_dcoef_f32(float *dcoef, float *d_scale_bias, const void *dy, int64_t 
     const int nblocks = (int)(cdiv(d->tokens, qr.bm) * cdiv(d->out_f, FG_BN));
     f32_sum_scalars_kernel<<<1, 256, 0, s>>>(d_scale_bias, dots, nblocks);
     return check_launch("f32_sum_scalars_kernel");
+}
+
+// ----------------------------------------------------------------------------------------------- projected form in fp32
+// What a training step keeps from the forward to the backward pass in place of x: z = x . N^T in fp32, [tokens x k] row-major,
+// behind a 256-byte header (the same role as the bf16 state of rdb_direct.hpp; no fragment orders, no transposed copies: these
+// kernels stage both operands through LDS).  fp32 activations and coefficients, one launch's worth of tokens.
+static bool fg_state_ok(const rdb_linear_desc *d)
+{
+    return d->act_dtype == RDB_F32 && d->coef_dtype == RDB_F32 && fg_ok(d) && d->tokens * std::max(d->in_f, d->out_f) < (1ll << 28);
+}
+int64_t linear_f32_state_bytes(const rdb_linear_desc *d) { return fg_state_ok(d) ? 256 + up256(d->tokens * d->k * 4) : 0; }
+static float *fg_state_z(const void *state) { return reinterpret_cast<float *>(static_cast<char *>(const_cast<void *>(state)) + 256); }
+
+// workspace of the backward pass from the state: t = dy . C with the partial matrices of its ranges, then the partial matrices
+// of dC = dy^T . z
+int64_t linear_f32_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus)
+{
+    if (!fg_state_ok(d)) return 0;
+    const int r = dc_plan(d, num_cus).ranges;
+    return linear_f32_workspace(RDB_OP_LINEAR_BWD_DX, d, num_cus) + (r > 1 ? (int64_t)r * up256(d->out_f * d->k * 4) : 0);
+}
+
+static int fg_fwd_from_z(void *y, int64_t ldy, const float *z, const void *coef, const void *bias, const rdb_linear_desc *d, int num_cus, hipStream_t s)
+{
+    FgProduct q = {z, d->k, d->tokens * d->k, (const float *)coef, d->k, d->out_f * d->k, (float *)y, ldy, (const float *)bias,
+                   d->tokens, d->out_f, d->k, fg_plan(d->tokens, d->out_f, d->k, num_cus, d->k, 1).bm, 0, 0, d->seed};
+    return fg_launch<FG_KCONT, FG_KCONT>(q, num_cus, s, "f32_gemm_kernel (y = z . C^T)");
+}
+
+// state <- z.  The partial matrices of the projection's contraction ranges need scratch that this call is not given: with y
+// they lie in y's memory, which is written last (only when y is contiguous, and as many ranges as fit there); without y the
+// contraction runs in one range.
+int linear_project_f32(void *state, void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *bias, const rdb_linear_desc *d,
+                       int num_cus, hipStream_t s)
+{
+    if (!fg_state_ok(d) || !fg_aligned16(state) || d->tokens * ldx >= (1ll << 29)) return RDB_E_UNSUPPORTED;
+    if (y && (d->tokens * ldy >= (1ll << 29))) return RDB_E_UNSUPPORTED;
+    float *z = fg_state_z(state);
+    float *part = nullptr;
+    int max_ranges = 1;
+    if (y && ldy == d->out_f && fg_aligned16(y)) {
+        part = (float *)y;
+        max_ranges = (int)((d->tokens * d->out_f * 4) / up256(d->tokens * d->k * 4));
+    }
+    if (int rc = fg_project(z, (const float *)x, ldx, d, num_cus, s, part ? part : z, max_ranges)) return rc;
+    if (!y) return RDB_OK;
+    return fg_fwd_from_z(y, ldy, z, coef, bias, d, num_cus, s);
+}
+
+int linear_fwd_projected_f32(void *y, int64_t ldy, const void *state, const void *coef, const void *bias, const rdb_linear_desc *d, int num_cus,
+                             hipStream_t s)
+{
+    if (!fg_state_ok(d) || d->tokens * ldy >= (1ll << 29)) return RDB_E_UNSUPPORTED;
+    return fg_fwd_from_z(y, ldy, fg_state_z(state), coef, bias, d, num_cus, s);
+}
+
+// dx (NULL: not wanted) and dcoef from dy, the state and C.
+int linear_bwd_projected_f32(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *state, const void *coef,
+                             const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s)
+{
+    if (!fg_state_ok(d) || !workspace || !fg_aligned16(workspace) || workspace_bytes < linear_f32_bwd_projected_workspace(d, num_cus))
+        return RDB_E_UNSUPPORTED;
+    if (d->tokens * lddy >= (1ll << 29) || (dx && d->tokens * lddx >= (1ll << 29))) return RDB_E_UNSUPPORTED;
+    if (dx) {
+        if (int rc = linear_dx_f32(dx, lddx, dy, lddy, coef, nullptr, d, num_cus, workspace, workspace_bytes, s)) return rc;
+    }
+    float *part = reinterpret_cast<float *>(static_cast<char *>(workspace) + linear_f32_workspace(RDB_OP_LINEAR_BWD_DX, d, num_cus));
+    FgProduct q = {(const float *)dy, lddy, (d->tokens - 1) * lddy + d->out_f, fg_state_z(state), d->k, d->tokens * d->k, dcoef, d->k, nullptr,
+                   d->out_f, d->k, d->tokens, 128, 0, 0, d->seed};
+    return fg_launch_ranges<FG_MCONT, FG_MCONT>(q, dc_plan(d, num_cus), part, up256(d->out_f * d->k * 4) / 4, num_cus, s,
+                                                "f32_gemm_kernel (dC = dy^T . z)");
 }
 
 // ----------------------------------------------------------------------------------------------- materialise on the matrix cores

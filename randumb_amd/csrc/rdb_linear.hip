@@ -318,6 +318,14 @@ int linear_fwd_f32(void *y, int64_t ldy, const void *x, int64_t ldx, const void 
                    const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
 int linear_dx_f32(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias, const rdb_linear_desc *d,
                   int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
+int64_t linear_f32_state_bytes(const rdb_linear_desc *d);
+int64_t linear_f32_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus);
+int linear_project_f32(void *state, void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *bias, const rdb_linear_desc *d,
+                       int num_cus, hipStream_t s);
+int linear_fwd_projected_f32(void *y, int64_t ldy, const void *state, const void *coef, const void *bias, const rdb_linear_desc *d, int num_cus,
+                             hipStream_t s);
+int linear_bwd_projected_f32(void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *state, const void *coef,
+                             const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
 int linear_dcoef_f32(float *dcoef, float *d_scale_bias, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus,
                      void *workspace, int64_t workspace_bytes, hipStream_t s);
 // rdb_dx.hip
@@ -385,6 +393,7 @@ extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
     if (d->act_dtype == RDB_F32) {  // fp32: the small-k kernels, whose scratch is one [tokens x k] fp32 matrix
         rdb_linear_desc dd = *d;
         if (op == RDB_OP_LINEAR_BWD_DCOEF) dd.coef_dtype = RDB_F32;
+        if (op == RDB_OP_LINEAR_BWD_PROJECTED || op == RDB_OP_LINEAR_BWD_PROJECTED_TO) return linear_f32_bwd_projected_workspace(d, num_compute_units());
         if (op != RDB_OP_LINEAR_FWD && op != RDB_OP_LINEAR_BWD_DX && op != RDB_OP_LINEAR_BWD_DCOEF) return 0;
         // or the matrix-core kernels of rdb_f32.hip: a [tokens x k] matrix, and the coefficient gradient's token-range sums
         const int64_t a = linear_smallk_workspace(&dd), b = linear_f32_workspace(op, &dd, num_compute_units());
@@ -716,14 +725,36 @@ static int check_projected(const char *who, const rdb_linear_desc *d, ChunkPlan 
     return RDB_OK;
 }
 
+// fp32 layers: the state is z in fp32 (rdb_f32.hip), one chunk
+static bool f32_projected(const rdb_linear_desc *d) { return d && d->act_dtype == RDB_F32; }
+static int check_projected_f32(const char *who, const rdb_linear_desc *d)
+{
+    int rc = check_desc(who, d);
+    if (rc) return rc;
+    if (linear_f32_state_bytes(d) <= 0)
+        return set_error(RDB_E_UNSUPPORTED, "%s: the projected form in fp32 needs matrix-coef, fp32 activations and coefficients, non-empty sizes "
+                                            "and tokens * max(in_f, out_f) below 2^28", who);
+    return RDB_OK;
+}
+
 extern "C" int64_t rdb_linear_projection_bytes(const rdb_linear_desc *d)
 {
+    if (f32_projected(d)) return check_desc("rdb_linear_projection_bytes", d) ? 0 : linear_f32_state_bytes(d);
     const ChunkPlan pl = chunk_plan(d);
     return pl.nchunks * pl.state_stride;
 }
 
 extern "C" int rdb_linear_projection_layout(const rdb_linear_desc *d, int64_t *info)
 {
+    if (f32_projected(d)) {   // z row-major in fp32 behind the header: info[1] = 0
+        if (int rc = check_projected_f32("rdb_linear_projection_layout", d)) return rc;
+        if (!info) return set_error(RDB_E_NULL, "rdb_linear_projection_layout: info is NULL");
+        for (int i = 0; i < 8; ++i) info[i] = 0;
+        info[0] = 256;
+        info[4] = d->k;
+        info[5] = d->tokens;
+        return RDB_OK;
+    }
     ChunkPlan pl;
     int rc = check_projected("rdb_linear_projection_layout", d, &pl);
     if (rc) return rc;
@@ -746,6 +777,11 @@ extern "C" int rdb_linear_projection_layout(const rdb_linear_desc *d, int64_t *i
 // number of token chunks the projected entry points run `desc` in (1 for every layer whose activations fit one launch)
 extern "C" int rdb_linear_projection_chunks(const rdb_linear_desc *d, int64_t *chunk_tokens)
 {
+    if (f32_projected(d)) {
+        const bool ok = !check_desc("rdb_linear_projection_chunks", d) && linear_f32_state_bytes(d) > 0;
+        if (chunk_tokens) *chunk_tokens = ok ? d->tokens : 0;
+        return ok ? 1 : 0;
+    }
     const ChunkPlan pl = chunk_plan(d);
     if (chunk_tokens) *chunk_tokens = pl.chunk_tokens;
     return pl.nchunks;
@@ -755,6 +791,14 @@ static char *at_bytes(const void *p, int64_t bytes) { return static_cast<char *>
 
 extern "C" int rdb_linear_project(void *state, const void *x, int64_t ldx, const void *coef, const rdb_linear_desc *d, void *stream)
 {
+    if (f32_projected(d)) {
+        if (int rc = check_projected_f32("rdb_linear_project", d)) return rc;
+        if (!state || !x) return set_error(RDB_E_NULL, "rdb_linear_project: state or x is NULL");
+        if (ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_project: leading dimension smaller than the row");
+        int rc = linear_project_f32(state, nullptr, 0, x, ldx, nullptr, nullptr, d, num_compute_units(), (hipStream_t)stream);
+        if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_project: state must be 16-byte aligned and tokens * ldx below 2^29");
+        return rc;
+    }
     ChunkPlan pl;
     int rc = check_projected("rdb_linear_project", d, &pl);
     if (rc) return rc;
@@ -775,6 +819,14 @@ extern "C" int rdb_linear_project(void *state, const void *x, int64_t ldx, const
 extern "C" int rdb_linear_fwd_projected(void *y, int64_t ldy, const void *z, const void *coef, const void *bias, const rdb_linear_desc *d,
                                         void *stream)
 {
+    if (f32_projected(d)) {
+        if (int rc = check_projected_f32("rdb_linear_fwd_projected", d)) return rc;
+        if (!y || !z || !coef) return set_error(RDB_E_NULL, "rdb_linear_fwd_projected: y, z or coef is NULL");
+        if (ldy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_fwd_projected: leading dimension smaller than the row");
+        int rc = linear_fwd_projected_f32(y, ldy, z, coef, bias, d, num_compute_units(), (hipStream_t)stream);
+        if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd_projected: tokens * ldy must stay below 2^29");
+        return rc;
+    }
     ChunkPlan pl;
     int rc = check_projected("rdb_linear_fwd_projected", d, &pl);
     if (rc) return rc;
@@ -797,6 +849,15 @@ extern "C" int rdb_linear_fwd_projected(void *y, int64_t ldy, const void *z, con
 extern "C" int rdb_linear_project_fwd(void *y, int64_t ldy, void *state, const void *x, int64_t ldx, const void *coef, const void *bias,
                                       const rdb_linear_desc *d, void *stream)
 {
+    if (f32_projected(d)) {
+        if (int rc = check_projected_f32("rdb_linear_project_fwd", d)) return rc;
+        if (!y || !state || !x || !coef) return set_error(RDB_E_NULL, "rdb_linear_project_fwd: y, state, x or coef is NULL");
+        if (ldx < d->in_f || ldy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_project_fwd: leading dimension smaller than the row");
+        int rc = linear_project_f32(state, y, ldy, x, ldx, coef, bias, d, num_compute_units(), (hipStream_t)stream);
+        if (rc == RDB_E_UNSUPPORTED)
+            return set_error(RDB_E_UNSUPPORTED, "rdb_linear_project_fwd: state must be 16-byte aligned and tokens * ldx, tokens * ldy below 2^29");
+        return rc;
+    }
     ChunkPlan pl;
     int rc = check_projected("rdb_linear_project_fwd", d, &pl);
     if (rc) return rc;
@@ -818,6 +879,9 @@ extern "C" int rdb_linear_project_fwd(void *y, int64_t ldy, void *state, const v
 
 extern "C" int rdb_linear_bwd_dcoef_projected(float *dcoef, const void *dy, int64_t lddy, const void *z, const rdb_linear_desc *d, void *stream)
 {
+    if (f32_projected(d))
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_dcoef_projected: fp32 sums over token ranges need scratch: call "
+                                            "rdb_linear_bwd_projected with dx = NULL and a workspace");
     ChunkPlan pl;
     int rc = check_projected("rdb_linear_bwd_dcoef_projected", d, &pl);
     if (rc) return rc;
@@ -856,6 +920,18 @@ static int64_t bwd_projected_workspace(const rdb_linear_desc *d, bool force_part
 static int bwd_projected_entry(const char *who, void *dx, int64_t lddx, void *dcoef, int dcoef_dtype, const void *dy, int64_t lddy, const void *z,
                                const void *coef, const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
 {
+    if (f32_projected(d)) {   // dx may be NULL: the coefficient gradient alone
+        if (int rc = check_projected_f32(who, d)) return rc;
+        if (!dcoef || !dy || !z || (dx && !coef)) return set_error(RDB_E_NULL, "%s: dcoef, dy, z or coef is NULL", who);
+        if (lddy < d->out_f || (dx && lddx < d->in_f)) return set_error(RDB_E_SHAPE, "%s: leading dimension smaller than the row", who);
+        if (dcoef_dtype != RDB_F32) return set_error(RDB_E_DTYPE, "%s: fp32 layers return dcoef in fp32", who);
+        int rc = linear_bwd_projected_f32(dx, lddx, static_cast<float *>(dcoef), dy, lddy, z, coef, d, num_compute_units(), workspace, workspace_bytes,
+                                          (hipStream_t)stream);
+        if (rc == RDB_E_UNSUPPORTED)
+            return set_error(RDB_E_UNSUPPORTED, "%s: needs a 16-byte aligned workspace of rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_PROJECTED) "
+                                                "bytes and tokens * lddy, tokens * lddx below 2^29", who);
+        return rc;
+    }
     ChunkPlan pl;
     int rc = check_projected(who, d, &pl);
     if (rc) return rc;

@@ -376,11 +376,11 @@ def linear_bwd_dcoef(dy: torch.Tensor, x: torch.Tensor, k: int, coef_rows: int, 
 
 
 # ------------------------------------------------------------------------------------------------ fused linear, projected form
-def _proj_desc(tokens, in_f, out_f, k, seed, coef_dtype=torch.bfloat16) -> LinearDesc:
+def _proj_desc(tokens, in_f, out_f, k, seed, coef_dtype=torch.bfloat16, act_dtype=torch.bfloat16) -> LinearDesc:
     d = LinearDesc()
     d.tokens, d.in_f, d.out_f, d.k, d.coef_rows = int(tokens), int(in_f), int(out_f), int(k), int(out_f)
     d.sO, d.sI, d.seed = int(in_f), 1, _seed(seed)
-    d.act_dtype, d.coef_dtype, d.algo = RDB_BF16, _DT[coef_dtype], RDB_ALGO_AUTO
+    d.act_dtype, d.coef_dtype, d.algo = _DT[act_dtype], _DT[coef_dtype], RDB_ALGO_AUTO
     return d
 
 
@@ -388,9 +388,9 @@ class _ProjPlan:
     """What the projected calls need to know about a layer and batch, asked of the library once per (sizes, seed)."""
     __slots__ = ("desc", "ref", "state_bytes", "state_cols", "ws_bytes", "ws_bytes_to", "chunks")
 
-    def __init__(self, tokens, in_f, out_f, k, seed):
+    def __init__(self, tokens, in_f, out_f, k, seed, dtype):
         L = _lib.load()
-        self.desc = _proj_desc(tokens, in_f, out_f, k, seed)
+        self.desc = _proj_desc(tokens, in_f, out_f, k, seed, dtype, dtype)
         self.ref = ctypes.byref(self.desc)
         self.state_bytes = int(L.rdb_linear_projection_bytes(self.ref))
         self.state_cols = -(-self.state_bytes // tokens) if self.state_bytes > 0 else 0
@@ -402,26 +402,29 @@ class _ProjPlan:
 _plans: dict = {}
 
 
-def _plan(tokens: int, in_f: int, out_f: int, k: int, seed: int) -> _ProjPlan:
-    key = (tokens, in_f, out_f, k, seed)
+def _plan(tokens: int, in_f: int, out_f: int, k: int, seed: int, dtype=torch.bfloat16) -> _ProjPlan:
+    key = (tokens, in_f, out_f, k, seed, dtype)
     p = _plans.get(key)
     if p is None:
         if len(_plans) > 4096:
             _plans.clear()
-        p = _plans[key] = _ProjPlan(tokens, in_f, out_f, k, _seed(seed))
+        p = _plans[key] = _ProjPlan(tokens, in_f, out_f, k, _seed(seed), dtype)
     return p
 
 
-def linear_projection_bytes(tokens: int, in_f: int, out_f: int, k: int) -> int:
-    """Size of the projection state of a layer of these sizes; 0 when the projected form (matrix-coef, bf16) does not apply."""
-    return int(_lib.load().rdb_linear_projection_bytes(ctypes.byref(_proj_desc(tokens, in_f, out_f, k, 0))))
+def linear_projection_bytes(tokens: int, in_f: int, out_f: int, k: int, dtype=torch.bfloat16) -> int:
+    """Size of the projection state of a layer of these sizes; 0 when the projected form (matrix-coef, bf16 or fp32) does not apply."""
+    return int(_lib.load().rdb_linear_projection_bytes(ctypes.byref(_proj_desc(tokens, in_f, out_f, k, 0, dtype, dtype))))
 
 
-def linear_projection_supported(tokens: int, in_f: int, out_f: int, k: int) -> bool:
+def linear_projection_supported(tokens: int, in_f: int, out_f: int, k: int, dtype=torch.bfloat16) -> bool:
     """Whether the projected entry points run a layer of these sizes: matrix-coef bf16, sizes in multiples of 8 (any number
     of tokens: activations beyond one launch's 2^29 elements are run in chunks of tokens by the library).  Plain integer
     arithmetic, the library's own rule restated (``rdb_linear_projection_bytes(desc) > 0``; a test holds the two together), so
     that a tracing compiler can follow the choice of path without calling into the library."""
+    if dtype == torch.float32:   # z in fp32, one launch's worth of tokens, any sizes
+        return (min(tokens, in_f, out_f, k) > 0 and tokens * k < (1 << 29) and out_f * k < (1 << 29) and max(in_f, out_f) < (1 << 30)
+                and tokens * max(in_f, out_f) < (1 << 28))
     if min(tokens, in_f, out_f, k) <= 0 or k % 8 or in_f % 8 or out_f % 8:
         return False
     kpad, out64 = -(-k // 64) * 64, -(-out_f // 64) * 64
@@ -435,7 +438,7 @@ def linear_projection_supported(tokens: int, in_f: int, out_f: int, k: int) -> b
     return tok64 * kpad < limit and out64 * kpad < limit and chunk * k < limit and out_f * k < limit
 
 
-def linear_projection_preferred(tokens: int, in_f: int, out_f: int, k: int) -> bool:
+def linear_projection_preferred(tokens: int, in_f: int, out_f: int, k: int, dtype=torch.bfloat16) -> bool:
     """Whether a training step should save the projection state in place of ``x``.  Two conditions.  Speed: the factored
     products need 2*tokens*k*(in_f + out_f) flops per direction, a product on a stored weight 2*tokens*in_f*out_f; the kernels
     that form the weight on chip instead lose against the factored ones up to at least 8 times that (measured), so the bound
@@ -443,7 +446,11 @@ def linear_projection_preferred(tokens: int, in_f: int, out_f: int, k: int) -> b
     rounded up to 64, where the reference's autograd saves the 2 * in_f bytes of x (src/rten_cpp/RandumbTensor.py:942-946);
     the state may cost up to twice that, i.e. k rounded up to 64 must not exceed in_f (768 -> 3072, k = 256: 1024 against
     1536 bytes per token).  Layers that fail the second test still run the factored kernels, through ``rdb_linear_fwd`` and a
-    transient workspace, with x saved."""
+    transient workspace, with x saved.  fp32 layers: the state is z in fp32 (4 k bytes per token against 4 in_f)."""
+    if dtype == torch.float32:
+        # the state is z in fp32, 4 k bytes per token where x has 4 in_f: the same memory rule; and only beyond the few-token
+        # regime, whose vector-ALU kernels (k <= 64, up to 1024 tokens) have no projected form
+        return k <= 2 * in_f and (k > 64 or tokens > 1024) and linear_projection_supported(tokens, in_f, out_f, k, dtype)
     kpad = -(-k // 64) * 64
     return (k * (in_f + out_f) < 16 * in_f * out_f and kpad <= in_f
             and linear_projection_supported(tokens, in_f, out_f, k))
@@ -455,9 +462,9 @@ def linear_project(x: torch.Tensor, k: int, out_f: int, seed: int, coef: Optiona
     of ``x``) and, when ``coef`` (out_f, k) is given in bf16, the transposed coefficients for the input gradient."""
     _need_gpu("linear_project", x, coef)
     x = _act(x)
-    if x.dtype != torch.bfloat16:
-        raise ValueError("linear_project computes in bf16")
-    d = _proj_desc(x.shape[0], x.shape[1], out_f, k, seed)
+    if x.dtype not in _DT:
+        raise ValueError("linear_project computes in bf16 or fp32")
+    d = _proj_desc(x.shape[0], x.shape[1], out_f, k, seed, x.dtype, x.dtype)
     L = _lib.load()
     nbytes = L.rdb_linear_projection_bytes(ctypes.byref(d))
     if nbytes <= 0:
@@ -482,18 +489,18 @@ def linear_project_fwd(x: torch.Tensor, coef: torch.Tensor, seed: int, bias: Opt
         _need_gpu("linear_project_fwd", x, coef)
     x = _act(x)
     c = coef if coef.is_contiguous() else coef.contiguous()
-    if x.dtype != torch.bfloat16 or c.dtype != torch.bfloat16:
-        raise ValueError("linear_project_fwd computes in bf16")
+    if x.dtype != c.dtype or x.dtype not in _DT:
+        raise ValueError("linear_project_fwd computes in bf16 or in fp32: activations and coefficients in one of them")
     out_f, k = c.shape
     tokens = x.shape[0]
-    pl = _plan(tokens, x.shape[1], out_f, k, seed)
+    pl = _plan(tokens, x.shape[1], out_f, k, seed, x.dtype)
     L = _lib.load()
     if pl.state_bytes <= 0:
         _lib.check(L.rdb_linear_project(None, None, x.stride(0), None, pl.ref, None), "rdb_linear_project")
     dev = x.device
     state = torch.empty((tokens, pl.state_cols), dtype=torch.uint8, device=dev)
-    b = None if bias is None else bias.to(torch.bfloat16).contiguous()
-    y = torch.empty((tokens, out_f), dtype=torch.bfloat16, device=dev)
+    b = None if bias is None else bias.to(x.dtype).contiguous()
+    y = torch.empty((tokens, out_f), dtype=x.dtype, device=dev)
     with _on(dev):
         st = _stream(dev)
         rc = L.rdb_linear_project_fwd(y.data_ptr(), out_f, state.data_ptr(), x.data_ptr(), x.stride(0), c.data_ptr(),
@@ -504,11 +511,16 @@ def linear_project_fwd(x: torch.Tensor, coef: torch.Tensor, seed: int, bias: Opt
     return y, state
 
 
-def projection_unpack(state: torch.Tensor, in_f: int, out_f: int, k: int) -> dict:
+def projection_unpack(state: torch.Tensor, in_f: int, out_f: int, k: int, dtype=torch.bfloat16) -> dict:
     """The pieces of a projection state as ordinary row-major tensors, for tools and tests (a layout decode, no arithmetic):
     ``z`` (tokens, k) as the forward product reads it, ``z_t`` (k, tokens) as the coef gradient reads it, and ``coef_t``
     (k, out_f), the transposed coefficients, or ``None`` when the state was written without them."""
     tokens = state.shape[0]
+    if dtype == torch.float32:   # z row-major in fp32 behind the header; no transposed copies
+        d = _proj_desc(tokens, in_f, out_f, k, 0, dtype, dtype)
+        _check_state(state, d, "projection_unpack")
+        z = state.reshape(-1)[256:256 + 4 * tokens * k].view(torch.float32).view(tokens, k)
+        return {"z": z.clone(), "z_t": z.t().contiguous(), "coef_t": None}
     d = _proj_desc(tokens, in_f, out_f, k, 0)
     _check_state(state, d, "projection_unpack")
     info = (ctypes.c_int64 * 8)()
@@ -544,16 +556,18 @@ def _check_state(state: torch.Tensor, d: LinearDesc, who: str) -> None:
 
 
 def linear_fwd_projected(state: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int,
-                         bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``y = z @ coef.T (+ bias)`` for matrix-coef ``coef`` (out_f, k) in bf16; ``state`` from :func:`linear_project`."""
+                         bias: Optional[torch.Tensor] = None, f32_state: bool = False) -> torch.Tensor:
+    """``y = z @ coef.T (+ bias)`` for matrix-coef ``coef`` (out_f, k) in bf16; ``state`` from :func:`linear_project`.
+    ``f32_state``: the state is that of an fp32 layer (fp32 activations and coefficients)."""
     _need_gpu("linear_fwd_projected", state, coef)
     c = _native(coef)
     out_f, k = c.shape
     tokens = state.shape[0]
-    d = _proj_desc(tokens, in_f, out_f, k, seed, c.dtype)
+    act = torch.float32 if (f32_state and c.dtype == torch.float32) else torch.bfloat16
+    d = _proj_desc(tokens, in_f, out_f, k, seed, c.dtype, act)
     _check_state(state, d, "linear_fwd_projected")
-    b = None if bias is None else bias.to(torch.bfloat16).contiguous()
-    y = torch.empty((tokens, out_f), dtype=torch.bfloat16, device=state.device)
+    b = None if bias is None else bias.to(act).contiguous()
+    y = torch.empty((tokens, out_f), dtype=act, device=state.device)
     with _on(state.device):
         rc = _lib.load().rdb_linear_fwd_projected(_p(y), y.stride(0), _p(state), _p(c), _p(b), ctypes.byref(d), _stream(state.device))
     _lib.check(rc, "rdb_linear_fwd_projected")
@@ -592,38 +606,43 @@ def check_state_coef(state: torch.Tensor, coef: torch.Tensor, in_f: int) -> None
 
 
 def linear_bwd_projected(dy: torch.Tensor, state: torch.Tensor, coef: torch.Tensor, in_f: int, seed: int, ordered_sums: bool = True,
-                         dcoef_dtype: torch.dtype = torch.float32):
-    """Whole backward pass of a matrix-coef bf16 layer from the projection state: ``(dx, dcoef)`` with ``dx = dy @ W`` in
-    bf16 and ``dcoef = dy.T @ z``, in two kernel launches.  ``ordered_sums`` gives the library room for the partial sums of
-    ``dcoef`` (added in a fixed order: bit-reproducible); without it they are combined with fp32 atomics.  ``dcoef_dtype``:
-    fp32, or bf16 to have the sums rounded once by the kernel that adds them up (what ``.to(bfloat16)`` would give, without
-    the extra pass; layers whose tokens the library runs in several chunks get fp32 sums rounded by torch instead)."""
+                         dcoef_dtype: torch.dtype = torch.float32, want_dx: bool = True):
+    """Whole backward pass of a matrix-coef layer from the projection state: ``(dx, dcoef)`` with ``dx = dy @ W`` in the
+    activations' dtype and ``dcoef = dy.T @ z``, in two kernel launches for bf16.  ``ordered_sums`` gives the library room for
+    the partial sums of ``dcoef`` (added in a fixed order: bit-reproducible); without it (bf16 only) they are combined with
+    fp32 atomics.  ``dcoef_dtype``: fp32, or bf16 to have the sums rounded once by the kernel that adds them up (what
+    ``.to(bfloat16)`` would give, without the extra pass; layers whose tokens the library runs in several chunks get fp32 sums
+    rounded by torch instead).  fp32 layers (``dy`` and ``coef`` in fp32): sums in fp32 in a fixed order; ``want_dx=False``
+    returns ``(None, dcoef)``."""
     if not (dy.is_cuda and state.is_cuda and coef.is_cuda):
         _need_gpu("linear_bwd_projected", dy, state, coef)
     dy = _act(dy)
     c = _native(coef)
     out_f, k = c.shape
     tokens = dy.shape[0]
-    pl = _plan(tokens, in_f, out_f, k, seed)
-    if c.dtype != torch.bfloat16:
+    f32 = dy.dtype == torch.float32 and c.dtype == torch.float32
+    pl = _plan(tokens, in_f, out_f, k, seed, torch.float32 if f32 else torch.bfloat16)
+    if not f32 and c.dtype != torch.bfloat16:
         _check_state(state, _proj_desc(tokens, in_f, out_f, k, seed, c.dtype), "linear_bwd_projected")
     elif state.dtype != torch.uint8 or state.dim() != 2 or state.numel() < pl.state_bytes or pl.state_bytes <= 0 or not state.is_contiguous():
         _check_state(state, pl.desc, "linear_bwd_projected")
-    if CHECK_STATE_COEF:
+    if CHECK_STATE_COEF and not f32:
         check_state_coef(state, c, in_f)
     if dcoef_dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("dcoef_dtype must be float32 or bfloat16")
+    if not want_dx and not f32:
+        raise ValueError("want_dx=False is for fp32 layers; bf16 layers have linear_bwd_dcoef_projected")
     in_kernel = dcoef_dtype == torch.bfloat16 and ordered_sums and pl.chunks == 1 and c.dtype == torch.bfloat16
     dev = dy.device
-    dx = torch.empty((tokens, in_f), dtype=dy.dtype, device=dev)
+    dx = torch.empty((tokens, in_f), dtype=dy.dtype, device=dev) if want_dx else None
     dcoef = torch.empty((out_f, k), dtype=torch.bfloat16 if in_kernel else torch.float32, device=dev)
     L = _lib.load()
-    d = pl.desc if c.dtype == torch.bfloat16 else _proj_desc(tokens, in_f, out_f, k, seed, c.dtype)
+    d = pl.desc if (f32 or c.dtype == torch.bfloat16) else _proj_desc(tokens, in_f, out_f, k, seed, c.dtype)
     ref = pl.ref if d is pl.desc else ctypes.byref(d)
     with _on(dev):
         if in_kernel:
             ws_bytes = pl.ws_bytes_to
-        elif ordered_sums:
+        elif ordered_sums or f32:
             ws_bytes = pl.ws_bytes
         else:
             ws_bytes = int(L.rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX, ref))
@@ -633,8 +652,8 @@ def linear_bwd_projected(dy: torch.Tensor, state: torch.Tensor, coef: torch.Tens
             rc = L.rdb_linear_bwd_projected_to(dx.data_ptr(), in_f, dcoef.data_ptr(), RDB_BF16, dy.data_ptr(), dy.stride(0), state.data_ptr(),
                                                c.data_ptr(), ref, _p(ws), ws_bytes, st)
         else:
-            rc = L.rdb_linear_bwd_projected(dx.data_ptr(), in_f, dcoef.data_ptr(), dy.data_ptr(), dy.stride(0), state.data_ptr(), c.data_ptr(),
-                                            ref, _p(ws), ws_bytes, st)
+            rc = L.rdb_linear_bwd_projected(None if dx is None else dx.data_ptr(), in_f, dcoef.data_ptr(), dy.data_ptr(), dy.stride(0),
+                                            state.data_ptr(), c.data_ptr(), ref, _p(ws), ws_bytes, st)
     if rc:
         _lib.check(rc, "rdb_linear_bwd_projected")
     return dx, (dcoef if dcoef.dtype == dcoef_dtype else dcoef.to(dcoef_dtype))

@@ -211,18 +211,19 @@ def linear_project(x: Tensor, dcoefs_size: int, out_features: int, seed: int, co
 @linear_project.register_fake
 def _(x, dcoefs_size, out_features, seed, coefs):
     # the size is the library's business; a fake tensor only needs some 1-D byte shape
-    nbytes = hip.linear_projection_bytes(x.shape[0], x.shape[1], out_features, dcoefs_size)
+    nbytes = hip.linear_projection_bytes(x.shape[0], x.shape[1], out_features, dcoefs_size, x.dtype)
     return x.new_empty([x.shape[0], -(-nbytes // x.shape[0])], dtype=torch.uint8)
 
 
 @custom_op("rten::linear_fwd_projected", mutates_args=())
 def linear_fwd_projected(state: Tensor, coefs: Tensor, in_features: int, seed: int, bias: Optional[Tensor]) -> Tensor:
-    return hip.linear_fwd_projected(state, coefs, in_features, seed, bias)
+    """bf16 coefficients: the state of a bf16 layer; fp32 coefficients: that of an fp32 layer."""
+    return hip.linear_fwd_projected(state, coefs, in_features, seed, bias, f32_state=coefs.dtype == torch.float32)
 
 
 @linear_fwd_projected.register_fake
 def _(state, coefs, in_features, seed, bias):
-    return coefs.new_empty([state.shape[0], coefs.shape[0]], dtype=torch.bfloat16)
+    return coefs.new_empty([state.shape[0], coefs.shape[0]])
 
 
 @custom_op("rten::linear_project_fwd", mutates_args=())
@@ -235,8 +236,8 @@ def linear_project_fwd(x: Tensor, coefs: Tensor, seed: int, bias: Optional[Tenso
 
 @linear_project_fwd.register_fake
 def _(x, coefs, seed, bias):
-    nbytes = hip.linear_projection_bytes(x.shape[0], x.shape[1], coefs.shape[0], coefs.shape[1])
-    return [x.new_empty([x.shape[0], coefs.shape[0]], dtype=torch.bfloat16),
+    nbytes = hip.linear_projection_bytes(x.shape[0], x.shape[1], coefs.shape[0], coefs.shape[1], x.dtype)
+    return [x.new_empty([x.shape[0], coefs.shape[0]]),
             x.new_empty([x.shape[0], -(-nbytes // x.shape[0])], dtype=torch.uint8)]
 
 
@@ -337,9 +338,12 @@ class _ProjectedLinear(torch.autograd.Function):
             dx = (hip.linear_bwd_dx(dy, coefs, in_f, out_f, in_f, 1, seed, None) if direct
                   else linear_bwd_dx(dy, coefs, in_f, out_f, in_f, 1, seed, None))
         elif ctx.needs_input_grad[1]:
-            dc = (hip.linear_bwd_dcoef_projected(dy, state, coefs.shape[1], in_f, seed) if direct
-                  else linear_bwd_dcoef_projected(dy, state, coefs.shape[1], in_f, seed))
-            dcoefs = dc.to(coefs.dtype)
+            if coefs.dtype == torch.float32:   # fp32 sums over token ranges need the backward call's workspace
+                dcoefs = hip.linear_bwd_projected(dy, state, coefs, in_f, seed, want_dx=False)[1]
+            else:
+                dc = (hip.linear_bwd_dcoef_projected(dy, state, coefs.shape[1], in_f, seed) if direct
+                      else linear_bwd_dcoef_projected(dy, state, coefs.shape[1], in_f, seed))
+                dcoefs = dc.to(coefs.dtype)
         if ctx.bias_dtype is not None and ctx.needs_input_grad[5]:
             dbias = dy.sum(0).to(ctx.bias_dtype)
         return dx, dcoefs, None, None, None, dbias
@@ -347,12 +351,13 @@ class _ProjectedLinear(torch.autograd.Function):
 
 def linear(x: Tensor, coefs: Tensor, in_features: int, out_features: int, stride_o: int, stride_i: int, seed: int,
            scale_bias: Optional[Tensor], bias: Optional[Tensor]) -> Tensor:
-    """``x @ W.T (+ bias)`` with autograd, choosing the projected form when the layer qualifies (matrix-coef, bf16, no
-    fused random bias, sizes in multiples of 8) and ``rten::linear_fwd`` otherwise.  Same arguments as ``rten::linear_fwd``."""
+    """``x @ W.T (+ bias)`` with autograd, choosing the projected form when the layer qualifies (matrix-coef, no fused random
+    bias; bf16 with sizes in multiples of 8, or fp32 beyond the few-token regime) and ``rten::linear_fwd`` otherwise.  Same
+    arguments as ``rten::linear_fwd``."""
     if (scale_bias is None and coefs.dim() == 2 and coefs.shape[0] == out_features and stride_o == in_features and stride_i == 1
-            and x.is_cuda and x.dim() == 2 and x.dtype == torch.bfloat16 and coefs.dtype == torch.bfloat16
-            and (bias is None or bias.dtype == torch.bfloat16)
-            and hip.linear_projection_preferred(x.shape[0], in_features, out_features, coefs.shape[1])):
+            and x.is_cuda and x.dim() == 2 and x.dtype in (torch.bfloat16, torch.float32) and coefs.dtype == x.dtype
+            and (bias is None or bias.dtype == x.dtype)
+            and hip.linear_projection_preferred(x.shape[0], in_features, out_features, coefs.shape[1], x.dtype)):
         return _ProjectedLinear.apply(x, coefs, in_features, out_features, seed, bias)
     if x.is_cuda and not _tracing():
         return _EagerLinear.apply(x, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias, bias)

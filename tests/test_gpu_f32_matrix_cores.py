@@ -202,3 +202,70 @@ def test_materialise_on_the_matrix_cores(hip, oracle, rows, row_len, k):
     assert got.shape == (rows, k) and rel_l2(got.cpu().numpy(), want) < F32_TOL
     got2 = hip.materialize_bwd(dW.cuda(), k, 7, rows)
     assert torch.equal(got, got2)
+
+
+@pytest.mark.parametrize("T,in_f,out_f,k,seed", [s for s in SHAPES if s[0] != 4500] + [(2500, 200, 96, 160, 4)])
+def test_projected_form_in_fp32(hip, oracle, T, in_f, out_f, k, seed):
+    """The state-saving form of an fp32 layer: the forward call leaves z = x . N^T (fp32) in the state, the backward call takes
+    dx and dC from dy, the state and C without x.  Against the oracle at 1e-5; z itself against x @ Noise.T; the coefficient
+    gradient alone (dx not wanted) gives the bits of the full call; the same call twice gives the same bits.  The last shape
+    has k > out_f: the projection's contraction ranges find no room in y and run as one range."""
+    print(f"case f32 projected T={T} in={in_f} out={out_f} k={k}", flush=True)
+    x, dy, coef, bias = _inputs(T, in_f, out_f, k, seed)
+    xn, dyn, cn = x.numpy(), dy.numpy(), coef.numpy()
+    want_y = oracle.linear_fwd(xn, cn, in_f, out_f, seed, bias=bias.numpy())
+    want_dx, want_dc, _ = oracle.linear_bwd(xn, dyn, cn, in_f, out_f, seed)
+    xc, dyc, cc = x.cuda(), dy.cuda(), coef.cuda()
+    assert hip.linear_projection_supported(T, in_f, out_f, k, torch.float32)
+    y, state = hip.linear_project_fwd(xc, cc, seed, bias=bias.cuda())
+    assert y.dtype == torch.float32 and rel_l2(y.cpu().numpy(), want_y) < F32_TOL
+    z = hip.projection_unpack(state, in_f, out_f, k, torch.float32)["z"]
+    noise = oracle.noise_2d(in_f, k, seed).astype(np.float64)   # [i, m]
+    assert rel_l2(z.cpu().numpy(), xn.astype(np.float64) @ noise) < F32_TOL
+    dx, dc = hip.linear_bwd_projected(dyc, state, cc, in_f, seed)
+    assert dx.dtype == torch.float32 and rel_l2(dx.cpu().numpy(), want_dx) < F32_TOL
+    assert dc.dtype == torch.float32 and rel_l2(dc.cpu().numpy(), want_dc) < F32_TOL
+    none, dc_only = hip.linear_bwd_projected(dyc, state, cc, in_f, seed, want_dx=False)
+    assert none is None and torch.equal(dc_only, dc)
+    dx2, dc2 = hip.linear_bwd_projected(dyc, state, cc, in_f, seed)
+    assert torch.equal(dx2, dx) and torch.equal(dc2, dc)
+    # the state serves the separate forward call too, and the projection alone (one contraction range) agrees to rounding
+    y2 = hip.linear_fwd_projected(state, cc, in_f, seed, bias=bias.cuda(), f32_state=True)
+    assert torch.equal(y2, y)
+    state1 = hip.linear_project(xc, k, out_f, seed)
+    z1 = hip.projection_unpack(state1, in_f, out_f, k, torch.float32)["z"]
+    assert rel_l2(z1.cpu().numpy(), z.cpu().numpy()) < 1e-6
+
+
+def test_fp32_layer_takes_the_projected_form(hip, oracle):
+    """SillyLinear in fp32 beyond the few-token regime saves z instead of x (ops.linear's choice) and matches the oracle."""
+    import randumb_amd as ra
+    from randumb_amd import ops
+
+    T, in_f, out_f, k, seed = 1500, 264, 520, 136, 31
+    assert hip.linear_projection_preferred(T, in_f, out_f, k, torch.float32)
+    assert not hip.linear_projection_preferred(128, 784, 256, 64, torch.float32)   # the few-token regime keeps its own kernels
+    layer = ra.SillyLinear(in_f, out_f, [k, k], [seed, seed + 1], bias=False, matrix_coef=True).cuda()
+    x, dy, coef, _ = _inputs(T, in_f, out_f, k, seed)
+    with torch.no_grad():
+        layer.weight_coef.copy_(coef)
+        layer.weight_scale_bias.zero_()
+    seen = []
+    orig = ops._ProjectedLinear.apply
+    try:
+        ops._ProjectedLinear.apply = staticmethod(lambda *a: (seen.append(1), orig(*a))[1])
+        xg = x.cuda().requires_grad_()
+        y = layer(xg)
+        y.backward(dy.cuda())
+    finally:
+        ops._ProjectedLinear.apply = orig
+    assert seen, "the fp32 layer did not take the projected form"
+    want_y = oracle.linear_fwd(x.numpy(), coef.numpy(), in_f, out_f, seed)
+    want_dx, want_dc, _ = oracle.linear_bwd(x.numpy(), dy.numpy(), coef.numpy(), in_f, out_f, seed)
+    assert rel_l2(y.detach().cpu().numpy(), want_y) < F32_TOL
+    assert rel_l2(xg.grad.cpu().numpy(), want_dx) < F32_TOL
+    assert rel_l2(layer.weight_coef.grad.cpu().numpy(), want_dc) < F32_TOL
+    # the first layer of a network: its input needs no gradient
+    layer.zero_grad()
+    layer(x.cuda()).backward(dy.cuda())
+    assert rel_l2(layer.weight_coef.grad.cpu().numpy(), want_dc) < F32_TOL
