@@ -348,6 +348,13 @@ int linear_bwd_big(void *t, float *dc, const void *dy, int64_t lddy, const void 
 int linear_dx_rbias_add(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *scale_bias, const rdb_linear_desc *d, hipStream_t s);
 int linear_fwd_rbias_add(void *y, int64_t ldy, const void *x, int64_t ldx, const void *scale_bias, const rdb_linear_desc *d, hipStream_t s);
 
+// rdb_vecsplit.hip
+int64_t linear_vecsplit_workspace(int op, const rdb_linear_desc *d);
+int linear_fwd_vecsplit(void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *scale_bias, const void *bias,
+                        const rdb_linear_desc *d, int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
+int linear_dx_vecsplit(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias, const rdb_linear_desc *d,
+                       int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
+
 // rdb_dcoef.hip
 int linear_dcoef_fast(float *dcoef, float *dsb, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d,
                       int num_cus, hipStream_t s);
@@ -390,6 +397,7 @@ extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
 {
     if (!d) return 0;
     if (d->algo == RDB_ALGO_TILE || d->algo == RDB_ALGO_STRIP) return 0;
+    if (d->coef_rows == 0) return d->algo == RDB_ALGO_AUTO ? linear_vecsplit_workspace(op, d) : 0;   // vector-coef: the chunks' partial outputs
     if (d->act_dtype == RDB_F32) {  // fp32: the small-k kernels, whose scratch is one [tokens x k] fp32 matrix
         rdb_linear_desc dd = *d;
         if (op == RDB_OP_LINEAR_BWD_DCOEF) dd.coef_dtype = RDB_F32;
@@ -424,6 +432,11 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
     if (!y || (!x && d->in_f > 0) || (!coef && d->k > 0)) return set_error(RDB_E_NULL, "rdb_linear_fwd: y, x or coef is NULL");
     if (ldy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_fwd: leading dimension smaller than the row");
     hipStream_t s = (hipStream_t)stream;
+    if (d->algo == RDB_ALGO_AUTO && d->coef_rows == 0) {
+        // vector-coef, up to a few thousand tokens, with room for the partial outputs: W tiles spread over all compute units
+        rc = linear_fwd_vecsplit(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), workspace, workspace_bytes, s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
     if (d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) {
         rc = linear_fwd_factored(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
@@ -489,6 +502,10 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
     if (d->tokens == 0 || d->in_f == 0) return RDB_OK;
     if (!dx || (!dy && d->out_f > 0) || (!coef && d->k > 0)) return set_error(RDB_E_NULL, "rdb_linear_bwd_dx: dx, dy or coef is NULL");
     if (lddx < d->in_f || lddy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dx: leading dimension smaller than the row");
+    if (d->algo == RDB_ALGO_AUTO && d->coef_rows == 0) {
+        rc = linear_dx_vecsplit(dx, lddx, dy, lddy, coef, scale_bias, d, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
     if (d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) {
         if (scale_bias && d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16 && d->tokens * lddx < (1ll << 29)) {
             // W = C.N + s.R: the low-rank share through the factored kernels, then the random-bias share added on top

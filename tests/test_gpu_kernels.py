@@ -236,6 +236,32 @@ def test_linear_strided_weight_vector_coef(hip, oracle):
     assert rel_l2(cpu(got), mat1.double().numpy() @ W) < F32_TOL
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.bfloat16, 1e-2)])
+def test_vector_coef_split_form_against_the_general_kernel(hip, dtype, tol):
+    """The vector-coef forward and input gradient whose blocks own tiles of W (AUTO, with the workspace the library asks for)
+    against the general kernel that owns tiles of the output (RDB_ALGO_TILE): the same W bits, sums in another order.  Ragged
+    sizes, more than one token tile, fused random bias, bias; the same call twice gives the same bits."""
+    from randumb_amd._lib import RDB_ALGO_TILE
+
+    T, in_f, out_f, k, seed = 300, 200, 136, 72, 11
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(T, in_f, generator=g).to(dtype).cuda()
+    dy = torch.randn(T, out_f, generator=g).to(dtype).cuda()
+    c = (torch.randn(k, generator=g) * 0.05).to(dtype).cuda()
+    sb = torch.tensor([0.07]).to(dtype).cuda()
+    bias = torch.randn(out_f, generator=g).to(dtype).cuda()
+    rel = lambda a, b: float((a.float() - b.float()).norm() / b.float().norm())
+    for scale_bias in (None, sb):
+        y = hip.linear_fwd(x, c, in_f, out_f, in_f, 1, seed, scale_bias=scale_bias, bias=bias)
+        y_t = hip.linear_fwd(x, c, in_f, out_f, in_f, 1, seed, scale_bias=scale_bias, bias=bias, algo=RDB_ALGO_TILE)
+        assert rel(y, y_t) < tol
+        assert torch.equal(y, hip.linear_fwd(x, c, in_f, out_f, in_f, 1, seed, scale_bias=scale_bias, bias=bias))
+        dx = hip.linear_bwd_dx(dy, c, in_f, out_f, in_f, 1, seed, scale_bias=scale_bias)
+        dx_t = hip.linear_bwd_dx(dy, c, in_f, out_f, in_f, 1, seed, scale_bias=scale_bias, algo=RDB_ALGO_TILE)
+        assert rel(dx, dx_t) < tol
+        assert torch.equal(dx, hip.linear_bwd_dx(dy, c, in_f, out_f, in_f, 1, seed, scale_bias=scale_bias))
+
+
 def test_argument_errors(hip):
     from randumb_amd._lib import RandumbHipError
 

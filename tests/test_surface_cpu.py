@@ -244,8 +244,12 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     # bf16 sizes that are not multiples of 8 run on these kernels too (bf16 read value by value, z and t kept in fp32)
     odd16 = desc(16, 4096, 4094, 128)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(odd16)) == 16 * 128 * 4 * (1 + 32)
-    # vector-coef: the general kernel, no scratch
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(16, 4096, 4096, 128, rows=0, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 0
+    # vector-coef, up to 4096 tokens: one fp32 partial output per 32 values of the contraction; beyond: the general kernel, no scratch
+    vec = desc(16, 4096, 4096, 128, rows=0, act=_lib.RDB_F32, coef=_lib.RDB_F32)
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(vec)) == (4096 // 32) * 16 * 4096 * 4
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(vec)) == (4096 // 32) * 16 * 4096 * 4
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DCOEF, ctypes.byref(vec)) == 0
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(8192, 4096, 4096, 128, rows=0, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 0
 
     bad = ctypes.byref(desc(64, 100, 32, 16))
     assert L.rdb_linear_project(None, None, 100, None, bad, None) == -5  # RDB_E_UNSUPPORTED
