@@ -27,11 +27,14 @@ What the printed JSON line says, and with which clock:
   value                  F / ms_per_step with F = 6*T*in*out + 6*out*in*k, the flops of the algorithm the metric prescribes
                          (three dense products, the weight generation per direction, the dC contraction).  The kernels use
                          W = C N associatively and EXECUTE 2.65x fewer flops: executed_tflops and
-                         executed_frac_of_mfma_peak say how busy the matrix cores really are.
-  roofline               the slowest call (the backward pass: bwd_dc_dyc_kernel + bwd_tns_red_kernel), from HIP events:
-                         achieved / frac on the prescribed flops of dx and dC (2/3 of F), executed_frac on the flops the
-                         two kernels execute, hbm_frac = measured HBM bytes of the call / its duration / 8 TB/s; traffic is
-                         read from profiles/bench_c2_hbm_traffic.md (rocprofv3 FETCH_SIZE / WRITE_SIZE of this script)
+                         executed_frac_of_mfma_peak (and everything under `roofline`) say how busy the matrix cores really are.
+  roofline               the single slowest kernel of the step (bwd_dc_dyc_kernel: t = dy C and the partial sums of dC), timed alone
+                         between HIP events on the launch stream: achieved / frac on the flops the kernel EXECUTES against the
+                         dense bf16 MFMA peak; `kernels` gives the same for all three kernels of the step, `step.bound_time_us`
+                         the least the step could take (executed flops at the MFMA peak, or the bytes it must move at the HBM
+                         peak), `backward_call.frac_on_prescribed_flops` the dense-equivalent figure the metric's `value` is
+                         made of; traffic is read from profiles/bench_c2_hbm_traffic.md (rocprofv3 FETCH_SIZE / WRITE_SIZE of
+                         this script)
   cpu_baseline           the CPU restatement (materialise-then-matmul: oracle C + torch.matmul fp32) on all host cores
   compare, other_configs one-call entry points, kernels that form W on chip, materialise-to-HBM + dense GEMM, dense GEMM;
                          the small-k fp32 layer, the k = 1024 layer, the 12-layer model, the vector-coef (reference) form
@@ -60,8 +63,6 @@ F_STEP = 3.0 * F_PER_PRODUCT
 EXEC_FWD = 2.0 * T * K * (IN_F + OUT_F)
 EXEC_BWD = 2.0 * T * K * (OUT_F + IN_F) + 2.0 * T * K * OUT_F
 EXEC_STEP = EXEC_FWD + EXEC_BWD
-FWD_KERNELS = ("factored_zy_kernel",)
-BWD_KERNELS = ("bwd_dc_dyc_kernel", "bwd_tns_red_kernel")
 SETTLE_STEPS = 400   # untimed, before the warm-up steps: about 30 ms of continuous work
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_c2_hbm_traffic.md")
 
@@ -135,6 +136,11 @@ class LayerBuffers:
         p = self.p
         self._lib.check(self.L.rdb_linear_bwd_projected(p["dx"], IN_F, p["dC"], p["dy"], OUT_F, p["state"], p["C"], self.dref, p["ws"],
                                                         self.ws_bytes, self.stream), "rdb_linear_bwd_projected")
+
+    def bwd_part(self, part):
+        p = self.p
+        self._lib.check(self.L.rdb_linear_bwd_projected_part(part, p["dx"], IN_F, p["dC"], p["dy"], OUT_F, p["state"], p["C"], self.dref, p["ws"],
+                                                             self.ws_bytes, self.stream), "rdb_linear_bwd_projected_part")
 
     def dx_separate(self):
         p = self.p
@@ -378,7 +384,7 @@ def other_configs(event_ms, torch, L, _lib, dev):
         return yy, dxx, hip.materialize_bwd(dWW, K, SEED)
 
     vs_ms = event_ms(vec_step, 3)
-    # the fused kernel in this form regenerates the weight block of every 128-token block: one token block timed
+    # the fused forward in this form: blocks own tiles of W, all compute units share the hashes; 128 tokens timed
     x128 = xh[:128].contiguous()
     fused_ms = event_ms(lambda: hip.linear_fwd(x128, c1, IN_F, OUT_F, IN_F, 1, SEED), 3)
     out["vector_coef_reference_form_768x3072_k256_T8192"] = {
@@ -533,38 +539,61 @@ def main():
         "rdb_linear_project (separate call)": event_ms(main_set.project, iters),
         "rdb_linear_fwd_projected (separate call)": event_ms(main_set.fwd_projected, iters),
         "rdb_linear_bwd_projected": event_ms(main_set.bwd, iters),
+        "rdb_linear_bwd_projected, first launch alone": event_ms(lambda: main_set.bwd_part(1), iters),
+        "rdb_linear_bwd_projected, second launch alone": event_ms(lambda: main_set.bwd_part(2), iters),
         "rdb_linear_bwd_dx (separate call)": event_ms(main_set.dx_separate, iters),
         "rdb_linear_bwd_dcoef_projected (separate call)": event_ms(main_set.dcoef_separate, iters),
     }
-    fwd_ms = calls["rdb_linear_project_fwd"]
+    main_set.bwd()   # leave the outputs of a whole backward pass behind
+    # ---- roofline of the dominant kernel.  The step is three launches: factored_zy_kernel (forward call), bwd_dc_dyc_kernel
+    # and bwd_tns_red_kernel (backward call); each is timed alone between HIP events on the launch stream, back to back.
+    # What a kernel EXECUTES (the factored algorithm's flops) is what its share of the MFMA peak is taken on.
+    kernels = {
+        "factored_zy_kernel": {"ms": calls["rdb_linear_project_fwd"], "executed_flop": EXEC_FWD,
+                               "min_bytes": 2.0 * (T * IN_F + OUT_F * K + T * OUT_F) + 2.0 * 2 * T * K + 2.0 * OUT_F * K,
+                               "does": "z = x.N^T into the state, y = z.C^T"},
+        "bwd_dc_dyc_kernel": {"ms": calls["rdb_linear_bwd_projected, first launch alone"], "executed_flop": 2 * 2.0 * T * K * OUT_F,
+                              "min_bytes": 2.0 * (T * OUT_F + T * K + OUT_F * K + T * K),
+                              "does": "t = dy.C and the token ranges' sums of dC = dy^T.z"},
+        "bwd_tns_red_kernel": {"ms": calls["rdb_linear_bwd_projected, second launch alone"], "executed_flop": 2.0 * T * K * IN_F,
+                               "min_bytes": 2.0 * (T * K + T * IN_F) + 4.0 * OUT_F * K,
+                               "does": "dx = t.N and the ordered sum of dC"},
+    }
+    dom = max(kernels, key=lambda n: kernels[n]["ms"])
+    kd = kernels[dom]
+    achieved = kd["executed_flop"] / (kd["ms"] * 1e-3) / 1e12
+    traffic = profiled_traffic((dom,))
+    # the least a step can take on this chip: the flops it executes at the MFMA peak, or the bytes it must move (inputs once,
+    # outputs once, the state written and read) at the HBM peak, whichever is longer
+    step_min_bytes = 2.0 * (T * IN_F + T * OUT_F) * 2 + 2.0 * 2 * OUT_F * K + 4.0 * OUT_F * K + 2 * (2.0 * 2 * T * K + 2.0 * OUT_F * K)
+    bound_mfma_us, bound_hbm_us = EXEC_STEP / (MFMA_BF16_PEAK_TFLOPS * 1e12) * 1e6, step_min_bytes / (HBM_PEAK_TBPS * 1e12) * 1e6
     bwd_ms = calls["rdb_linear_bwd_projected"]
-    if bwd_ms >= fwd_ms:
-        dom, dom_ms, dom_flops, dom_exec, dom_kernels = "backward", bwd_ms, 2 * F_PER_PRODUCT, EXEC_BWD, BWD_KERNELS
-    else:
-        dom, dom_ms, dom_flops, dom_exec, dom_kernels = "forward", fwd_ms, F_PER_PRODUCT, EXEC_FWD, FWD_KERNELS
-    achieved = dom_flops / (dom_ms * 1e-3) / 1e12
-    traffic = profiled_traffic(dom_kernels)
-    executed_frac = dom_exec / (dom_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS
-    hbm_frac = None if traffic is None else traffic / (dom_ms * 1e-3) / 1e12 / HBM_PEAK_TBPS
-    # bytes the call has to move whatever the algorithm: its inputs once, its outputs once
-    min_bytes = 2.0 * (T * OUT_F + OUT_F * K + T * IN_F) + 4.0 * OUT_F * K if dom == "backward" else 2.0 * (T * IN_F + OUT_F * K + T * OUT_F)
-    hbm_min_frac = min_bytes / (dom_ms * 1e-3) / 1e12 / HBM_PEAK_TBPS
     roofline = {
-        # the roofline of the metric (share of the MFMA peak).  On the flops the factored algorithm executes the call is at
-        # `executed_frac` of that peak and, on the bytes it has to move, at `hbm_min_frac` of the HBM peak (`hbm_frac`: on the bytes
-        # the counters saw): the matrix cores are the nearer wall, neither is reached; the kernels are held by LDS /
-        # vector-memory issue and memory latency, see the SQ counters under profiles/
         "bound": "mfma",
-        "bound_observed": "neither pipe: waits on vector memory and LDS issue (profiles/bench_c2_sq_counters.md)",
-        "kernel": f"{dom} call ({' + '.join(dom_kernels)})",
+        "kernel": dom, "kernel_does": kd["does"],
         "achieved": round(achieved, 3), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 5),
+        "flops_counted": "the flops this kernel executes (factored algorithm)",
+        "executed_gflop_per_launch": round(kd["executed_flop"] / 1e9, 3),
+        "avg_kernel_ms": round(kd["ms"], 5),
+        "timed": f"HIP events on the launch stream around {iters} back-to-back launches of this kernel alone",
         "traffic": traffic, "traffic_source": "profiles/bench_c2_hbm_traffic.md" if traffic is not None else None,
-        "avg_kernel_ms": round(dom_ms, 5),
-        "algorithmic_gflop_per_launch": round(dom_flops / 1e9, 3),
-        "executed_gflop_per_launch": round(dom_exec / 1e9, 3),
-        "executed_achieved": round(dom_exec / (dom_ms * 1e-3) / 1e12, 3), "executed_frac": round(executed_frac, 5),
-        "hbm_frac": None if hbm_frac is None else round(hbm_frac, 5),
-        "hbm_min_bytes_per_launch": min_bytes, "hbm_min_frac": round(hbm_min_frac, 5),
+        "hbm_min_bytes_per_launch": kd["min_bytes"],
+        "hbm_frac_on_measured_traffic": None if traffic is None else round(traffic / (kd["ms"] * 1e-3) / 1e12 / HBM_PEAK_TBPS, 5),
+        "bound_observed": "neither pipe: waits on vector memory and LDS issue (profiles/bench_c2_sq_counters.md)",
+        "kernels": {n: {"ms": round(v["ms"], 5), "executed_gflop": round(v["executed_flop"] / 1e9, 3),
+                        "executed_tflops": round(v["executed_flop"] / (v["ms"] * 1e-3) / 1e12, 1),
+                        "frac": round(v["executed_flop"] / (v["ms"] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 5)} for n, v in kernels.items()},
+        # the same backward call on the flops the metric prescribes for it (dx and dC: two dense products, a weight generation and
+        # the dC contraction): what `value` is made of, not a utilisation of anything
+        "backward_call": {"ms": round(bwd_ms, 5), "prescribed_gflop": round(2 * F_PER_PRODUCT / 1e9, 3),
+                          "prescribed_tflops": round(2 * F_PER_PRODUCT / (bwd_ms * 1e-3) / 1e12, 1),
+                          "frac_on_prescribed_flops": round(2 * F_PER_PRODUCT / (bwd_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 5),
+                          "executed_gflop": round(EXEC_BWD / 1e9, 3),
+                          "executed_frac": round(EXEC_BWD / (bwd_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 5)},
+        "step": {"executed_gflop": round(EXEC_STEP / 1e9, 3), "min_bytes": step_min_bytes,
+                 "bound_time_us": round(max(bound_mfma_us, bound_hbm_us), 2), "bound_time_mfma_us": round(bound_mfma_us, 2),
+                 "bound_time_hbm_us": round(bound_hbm_us, 2), "measured_us": round(ms_per_step * 1e3, 2),
+                 "frac": round(EXEC_STEP / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 5)},
         "calls_ms": {n: round(v, 5) for n, v in calls.items()},
     }
 
@@ -629,8 +658,34 @@ def main():
             t["step"] = round(sum(t.values()), 4)
             return t
 
+        def python_surface_ms():
+            # the same layer through the drop-in surface: SillyLinear (autograd function, ctypes binding), host clock per forward +
+            # backward with the GPU kept busy; what a model built from the layer pays per layer when the host is the limit
+            from randumb_amd.SillyLayers import SillyLinear
+
+            lin = SillyLinear(IN_F, OUT_F, [K, K], [SEED, SEED + 1], bias=False, device=dev, dtype=torch.bfloat16, matrix_coef=True)
+            with torch.no_grad():
+                lin.weight_coef.copy_(C)
+                lin.weight_scale_bias.zero_()
+            xs = x.clone().requires_grad_()
+
+            def layer_step():
+                xs.grad = None
+                lin.weight_coef.grad = None
+                lin(xs).backward(dy)
+
+            for _ in range(100):
+                layer_step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(300):
+                layer_step()
+            torch.cuda.synchronize()
+            return round((time.perf_counter() - t0) * 1e3 / 300, 4)
+
         compare = {
             "one_call_entry_points_ms": onecall_ms(_lib.RDB_ALGO_AUTO),
+            "python_surface_SillyLinear_fwd_bwd_wall_ms": python_surface_ms(),
             "layer_with_fused_random_bias_ms": scale_bias_ms(),
             "w_tiles_formed_on_chip_ms": strip_ms(),
             "vendor_gemm_on_the_factored_shapes_ms": vendor_skinny(),

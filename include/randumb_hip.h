@@ -282,6 +282,14 @@ int rdb_linear_bwd_projected_to(void *dx, int64_t lddx, void *dcoef, int dcoef_d
                                 const void *state, const void *coef, const rdb_linear_desc *desc, void *workspace,
                                 int64_t workspace_bytes, void *stream);
 
+/* For tools that time the two kernel launches of rdb_linear_bwd_projected one by one (no counterpart in the reference):
+ * part 1 enqueues only the first launch (dy.C into the workspace and the partial sums of dcoef), part 2 only the second
+ * ((dy.C).N into dx and the ordered sum into dcoef, from what a first launch left in the workspace).  Same arguments and
+ * requirements as rdb_linear_bwd_projected, bf16 layers, workspace of the RDB_OP_LINEAR_BWD_PROJECTED amount. */
+int rdb_linear_bwd_projected_part(int part, void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy,
+                                  const void *state, const void *coef, const rdb_linear_desc *desc, void *workspace,
+                                  int64_t workspace_bytes, void *stream);
+
 /* Tuning switch without a counterpart in the reference.  Layers with k > 256 whose products have enough 256 x 256 output
  * tiles to give every compute unit one run rdb_linear_fwd_projected / rdb_linear_project_fwd / rdb_linear_bwd_projected on
  * 256-wide tiles with one persistent block per compute unit; all others on 128-wide tiles.  mode 0: never the 256-wide

@@ -45,6 +45,7 @@ EXPORTS = [
     "rdb_linear_bwd_dcoef_projected",
     "rdb_linear_bwd_projected",
     "rdb_linear_bwd_projected_to",
+    "rdb_linear_bwd_projected_part",
     "rdb_set_big_tiles",
     "rdb_set_one_launch",
     "rdb_sync_giveups_async",
@@ -137,6 +138,7 @@ def load() -> ctypes.CDLL:
     L.rdb_linear_bwd_dcoef_projected.argtypes = [vp, vp, i64, vp, dp, vp]
     L.rdb_linear_bwd_projected.argtypes = [vp, i64, vp, vp, i64, vp, vp, dp, vp, i64, vp]
     L.rdb_linear_bwd_projected_to.argtypes = [vp, i64, vp, ci, vp, i64, vp, vp, dp, vp, i64, vp]
+    L.rdb_linear_bwd_projected_part.argtypes = [ci, vp, i64, vp, vp, i64, vp, vp, dp, vp, i64, vp]
     L.rdb_set_big_tiles.argtypes = [ci]
     L.rdb_set_big_tiles.restype = ci
     L.rdb_set_one_launch.argtypes = [ci]
@@ -150,7 +152,7 @@ def load() -> ctypes.CDLL:
     for name in ("rdb_sq5_fill_2d", "rdb_sq5_fill_1d", "rdb_materialize_fwd", "rdb_materialize_bwd", "rdb_scale_bias_bwd",
                  "rdb_embed_fwd", "rdb_embed_bwd", "rdb_linear_fwd", "rdb_linear_bwd_dx", "rdb_linear_bwd_dcoef",
                  "rdb_linear_project", "rdb_linear_project_fwd", "rdb_linear_fwd_projected", "rdb_linear_bwd_dcoef_projected",
-                 "rdb_linear_bwd_projected", "rdb_linear_bwd_projected_to"):
+                 "rdb_linear_bwd_projected", "rdb_linear_bwd_projected_to", "rdb_linear_bwd_projected_part"):
         getattr(L, name).restype = ci
     _lib = L
     return L

@@ -311,6 +311,11 @@ int linear_dx_factored(void *dx, int64_t lddx, const void *dy, int64_t lddy, con
     return launch_engine(dx_tn_kernel, p2, items, engine_smem<K2_BI, K2_BT, X_BK, K_CONT, K_CONT>(), s, "dx_tn_kernel");
 }
 
+// Which of the two launches linear_bwd_projected enqueues: bit 0 the first, bit 1 the second (3: both).  Timing tools launch one
+// of them alone (rdb_linear_bwd_projected_part); the mask is the calling thread's.
+static thread_local int g_bwd_parts = 3;
+void set_bwd_projected_parts(int mask) { g_bwd_parts = mask & 3; }
+
 // Whole backward pass of the layer from the saved projection z: dx = (dy.C).N and dcoef = dy^T.z in two launches.
 // Returns RDB_E_UNSUPPORTED (without setting an error) when the request does not fit.
 // accumulate: dcoef += instead of dcoef = (a later chunk of tokens of a layer whose activations are passed in chunks).
@@ -347,8 +352,10 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
         }
         if (tn_stationary_ok(d, lddx)) a.dyc.frag_ksteps = (int)cdiv(d->k, 64) * 4;   // the t.N kernel below keeps t in registers
         a.dc_blocks = xcd_grid_size(dc_items);
-        int rc, red_splits = a.dc.splits;
-        if (big_bwd_applies(d, num_cus) && !a.dyc.frag_ksteps) {
+        int rc = RDB_OK, red_splits = a.dc.splits;
+        if (!(g_bwd_parts & 1)) {
+            if (big_bwd_applies(d, num_cus) && !a.dyc.frag_ksteps) red_splits = 1;
+        } else if (big_bwd_applies(d, num_cus) && !a.dyc.frag_ksteps) {
             // long coefficient dimension and many tiles: both products on 256-wide tiles; a dC tile contracts all tokens, so
             // there is one set of sums, stored where the first split's would go
             rc = linear_bwd_big(workspace, a.dc.partial, dy, lddy, z, coef, d, num_cus, true, true, s);
@@ -360,6 +367,7 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
             rc = check_launch("bwd_dc_dyc_kernel");
         }
         if (rc) return rc;
+        if (!(g_bwd_parts & 2)) return RDB_OK;
         RedParams red;
         red.partial = a.dc.partial;
         red.out = dcoef;

@@ -982,6 +982,23 @@ extern "C" int rdb_linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, co
     return bwd_projected_entry("rdb_linear_bwd_projected", dx, lddx, dcoef, RDB_F32, dy, lddy, z, coef, d, workspace, workspace_bytes, stream);
 }
 
+namespace rdb {
+void set_bwd_projected_parts(int mask);   // rdb_dx.hip
+}
+
+extern "C" int rdb_linear_bwd_projected_part(int part, void *dx, int64_t lddx, float *dcoef, const void *dy, int64_t lddy, const void *z,
+                                             const void *coef, const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    if (part != 1 && part != 2) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_projected_part: part must be 1 or 2");
+    if (d && d->act_dtype != RDB_BF16) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_bwd_projected_part: bf16 layers only");
+    if (d && workspace_bytes < bwd_projected_workspace(d, false))
+        return set_error(RDB_E_WORKSPACE, "rdb_linear_bwd_projected_part: needs the workspace of rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_PROJECTED)");
+    set_bwd_projected_parts(part);
+    const int rc = bwd_projected_entry("rdb_linear_bwd_projected_part", dx, lddx, dcoef, RDB_F32, dy, lddy, z, coef, d, workspace, workspace_bytes, stream);
+    set_bwd_projected_parts(3);
+    return rc;
+}
+
 extern "C" int rdb_linear_bwd_projected_to(void *dx, int64_t lddx, void *dcoef, int dcoef_dtype, const void *dy, int64_t lddy, const void *z,
                                            const void *coef, const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
 {
