@@ -646,16 +646,25 @@ def main():
 
         def scale_bias_ms():
             # the reference's default layer: W = C.N + s.noise1d (zero coefficients and a fused random bias at initialisation).
-            # forward: the strip kernel; dx: factored share + hashed random-bias share; dcoef and ds: dW tiles
+            # forward: the strip kernel; dx and d s: factored share + hashed random-bias share, reduced against x on the side;
+            # dcoef: factored (no dW).  Beside it the older split: dx alone, dcoef and d s from dW tiles.
             sb = torch.tensor([0.02], device=dev).bfloat16()
             ds = torch.empty(1, dtype=torch.float32, device=dev)
             psb, pds, r = ctypes.c_void_p(sb.data_ptr()), ctypes.c_void_p(ds.data_ptr()), main_set.dref
+            n_ds = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX_DSCALE, r)
+            ws_ds = torch.empty(max(n_ds, 16), dtype=torch.uint8, device=dev)
+            pws_ds = ctypes.c_void_p(ws_ds.data_ptr())
             fwd = lambda: _lib.check(L.rdb_linear_fwd(p["y"], OUT_F, p["x"], IN_F, p["C"], psb, None, r, p["ws"], ws_bytes, stream), "rdb_linear_fwd")
+            dxs = lambda: _lib.check(L.rdb_linear_bwd_dx_dscale(p["dx"], IN_F, pds, p["dy"], OUT_F, p["x"], IN_F, p["C"], psb, r, pws_ds, n_ds, stream),
+                                     "rdb_linear_bwd_dx_dscale")
+            dco = lambda: _lib.check(L.rdb_linear_bwd_dcoef(p["dC"], None, p["dy"], OUT_F, p["x"], IN_F, r, p["ws"], ws_bytes, stream),
+                                     "rdb_linear_bwd_dcoef")
             dxf = lambda: _lib.check(L.rdb_linear_bwd_dx(p["dx"], IN_F, p["dy"], OUT_F, p["C"], psb, r, p["ws"], ws_bytes, stream), "rdb_linear_bwd_dx")
             dcf = lambda: _lib.check(L.rdb_linear_bwd_dcoef(p["dC"], pds, p["dy"], OUT_F, p["x"], IN_F, r, p["ws"], ws_bytes, stream),
                                      "rdb_linear_bwd_dcoef")
-            t = {"fwd": round(event_ms(fwd, 20), 4), "dx": round(event_ms(dxf, 20), 4), "dcoef_and_dscale": round(event_ms(dcf, 20), 4)}
+            t = {"fwd": round(event_ms(fwd, 20), 4), "dx_and_dscale": round(event_ms(dxs, 20), 4), "dcoef": round(event_ms(dco, 20), 4)}
             t["step"] = round(sum(t.values()), 4)
+            t["with_dscale_from_dw_tiles"] = {"dx": round(event_ms(dxf, 20), 4), "dcoef_and_dscale": round(event_ms(dcf, 20), 4)}
             return t
 
         def python_surface_ms():

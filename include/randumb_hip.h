@@ -151,7 +151,7 @@ enum {
 };
 
 enum { RDB_OP_LINEAR_FWD = 0, RDB_OP_LINEAR_BWD_DX = 1, RDB_OP_LINEAR_BWD_DCOEF = 2, RDB_OP_LINEAR_BWD_PROJECTED = 3,
-       RDB_OP_LINEAR_BWD_PROJECTED_TO = 4 };
+       RDB_OP_LINEAR_BWD_PROJECTED_TO = 4, RDB_OP_LINEAR_BWD_DX_DSCALE = 5 };
 
 /* Device scratch (bytes) that entry point `op` can use for `desc`; 0 when it has no use for any.  A NULL or too small
  * workspace is never an error with RDB_ALGO_AUTO: the library then runs a kernel that needs none. */
@@ -180,6 +180,17 @@ int64_t rdb_linear_fwd_static_max_bytes(void);
 int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef,
                       const void *scale_bias, const rdb_linear_desc *desc, void *workspace,
                       int64_t workspace_bytes, void *stream);
+
+/* rdb_linear_bwd_dx for a layer with the fused random bias (W = C.N + s.R), and on the side the gradient of s:
+ *   dx[t, i] = sum_o dy[t, o] * W[o, i]        d_scale_bias[0] = sum_{o,i} (dy^T x)[o, i] * R[o, i] = <dy . R, x>   (fp32, overwritten)
+ * The random-bias share dy . R is a full-rank product that the input gradient forms anyway; reducing it against x in the same
+ * pass gives what scale_bias_bwd computes from a stored dW (R.py:399-420, 988), so that the coefficient gradient can come from
+ * rdb_linear_bwd_dcoef without d_scale_bias, i.e. from the factored kernels, and dW is never formed.  Partial sums are added in a
+ * fixed order.  Needs matrix-coef, bf16 activations and coefficients, sizes that are multiples of 8, a workspace of
+ * rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX_DSCALE, desc) bytes; otherwise RDB_E_UNSUPPORTED and nothing is launched. */
+int rdb_linear_bwd_dx_dscale(void *dx, int64_t lddx, float *d_scale_bias, const void *dy, int64_t lddy, const void *x,
+                             int64_t ldx, const void *coef, const void *scale_bias, const rdb_linear_desc *desc,
+                             void *workspace, int64_t workspace_bytes, void *stream);
 
 /* Replaces MmBackward's dW = dy^T x followed by RandumbTensorConstructor.backward ->
  * materialize_bwd (+ scale_bias_bwd) (R.py:979-990): dW is contracted with the regenerated noise tile

@@ -347,6 +347,9 @@ int linear_bwd_big(void *t, float *dc, const void *dy, int64_t lddy, const void 
 // rdb_rbias.hip
 int linear_dx_rbias_add(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *scale_bias, const rdb_linear_desc *d, hipStream_t s);
 int linear_fwd_rbias_add(void *y, int64_t ldy, const void *x, int64_t ldx, const void *scale_bias, const rdb_linear_desc *d, hipStream_t s);
+int64_t linear_dx_rbias_dot_floats(const rdb_linear_desc *d);
+int linear_dx_rbias_add_dscale(void *dx, int64_t lddx, float *dscale, float *dot_part, const void *dy, int64_t lddy, const void *x, int64_t ldx,
+                               const void *scale_bias, const rdb_linear_desc *d, hipStream_t s);
 
 // rdb_vecsplit.hip
 int64_t linear_vecsplit_workspace(int op, const rdb_linear_desc *d);
@@ -416,6 +419,10 @@ extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
         return linear_f32_workspace(op, &dd, num_compute_units());
     }
     if (op == RDB_OP_LINEAR_BWD_DX) return linear_dx_factored_workspace(d);
+    if (op == RDB_OP_LINEAR_BWD_DX_DSCALE) {   // dy.C, then one float per tile of the random-bias product
+        const int64_t t = linear_dx_factored_workspace(d);
+        return t > 0 ? (t + 255) / 256 * 256 + linear_dx_rbias_dot_floats(d) * 4 : 0;
+    }
     if (op == RDB_OP_LINEAR_BWD_PROJECTED) return bwd_projected_workspace(d, false);
     if (op == RDB_OP_LINEAR_BWD_PROJECTED_TO) return bwd_projected_workspace(d, true);
     if (op == RDB_OP_LINEAR_FWD) return d->coef_dtype == RDB_BF16 ? linear_projection_bytes(d) : 0;
@@ -568,6 +575,33 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
                    : launch(linear_dx_kernel<bf16_t, false>, grid, smem_fwd<bf16_t>(), s, p, "linear_dx_kernel<bf16,vector>");
     return mat ? launch(linear_dx_kernel<float, true>, grid, smem_fwd<float>(), s, p, "linear_dx_kernel<f32,matrix>")
                : launch(linear_dx_kernel<float, false>, grid, smem_fwd<float>(), s, p, "linear_dx_kernel<f32,vector>");
+}
+
+extern "C" int rdb_linear_bwd_dx_dscale(void *dx, int64_t lddx, float *d_scale_bias, const void *dy, int64_t lddy, const void *x, int64_t ldx,
+                                        const void *coef, const void *scale_bias, const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes,
+                                        void *stream)
+{
+    int rc = check_desc("rdb_linear_bwd_dx_dscale", d);
+    if (rc) return rc;
+    if (!dx || !d_scale_bias || !dy || !x || !coef || !scale_bias)
+        return set_error(RDB_E_NULL, "rdb_linear_bwd_dx_dscale: dx, d_scale_bias, dy, x, coef or scale_bias is NULL");
+    if (lddx < d->in_f || lddy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dx_dscale: leading dimension smaller than the row");
+    const int64_t need = rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX_DSCALE, d), t_bytes = (linear_dx_factored_workspace(d) + 255) / 256 * 256;
+    const char *why = "rdb_linear_bwd_dx_dscale: needs matrix-coef, bf16 activations and coefficients, sizes that are multiples of 8, 16-byte "
+                      "aligned rows and a workspace of rdb_linear_workspace_bytes(RDB_OP_LINEAR_BWD_DX_DSCALE) bytes";
+    if (d->act_dtype != RDB_BF16 || d->coef_dtype != RDB_BF16 || d->coef_rows == 0 || need <= 0 || !workspace || workspace_bytes < need ||
+        d->tokens * lddx >= (1ll << 29))
+        return set_error(RDB_E_UNSUPPORTED, "%s", why);
+    rdb_linear_desc df = *d;
+    df.algo = RDB_ALGO_FACTORED;   // the low-rank share through the factored kernels whatever the flop counts say
+    hipStream_t s = (hipStream_t)stream;
+    rc = linear_dx_factored(dx, lddx, dy, lddy, coef, nullptr, &df, num_compute_units(), workspace, workspace_bytes, s);
+    if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "%s", why);
+    if (rc) return rc;
+    float *dots = reinterpret_cast<float *>(static_cast<char *>(workspace) + t_bytes);
+    rc = linear_dx_rbias_add_dscale(dx, lddx, d_scale_bias, dots, dy, lddy, x, ldx, scale_bias, d, s);
+    if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "%s", why);
+    return rc;
 }
 
 extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const void *dy, int64_t lddy, const void *x, int64_t ldx,

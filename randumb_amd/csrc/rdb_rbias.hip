@@ -54,9 +54,14 @@ struct RBiasParams {
     int tiles_i, tiles_t;
     uint32_t sR, sK;
     uint32_t seed;
+    // DOT: the gradient of the scale on the side, d s = <src . R, other> = sum over the tile of the product (without s) times
+    // other[tokens x in_f columns]; one partial sum per work item, in work-item order
+    const bf16_t *other;
+    int64_t ld_other;
+    float *dot_part;
 };
 
-__global__ __launch_bounds__(256, 2) void rbias_add_kernel(RBiasParams p)
+template <bool DOT> __global__ __launch_bounds__(256, 2) void rbias_add_kernel(RBiasParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     bf16_t *lds = reinterpret_cast<bf16_t *>(smem_raw);
@@ -75,8 +80,10 @@ __global__ __launch_bounds__(256, 2) void rbias_add_kernel(RBiasParams p)
     // "B": src[tok][c]; contraction values past the end read as zeros, whatever the hash says there
     GlobalOperand<RB_BT, RB_BK, K_CONT> opdy = {p.dy, p.lddy, tok0, p.tokens, p.out_f, (int64_t)(p.tokens - 1) * p.lddy + p.out_f};
     gemm_mainloop<RB_BI, RB_BT, RB_BK, 1, 2, 1>(acc, lds, opr, opdy, 0, (p.out_f + RB_BK - 1) / RB_BK);
-    // dx += s * 2^-31 * acc, through LDS as fp32 so that every lane updates 8 consecutive features of a token's row
-    const float scale = bf16_to_f32(*p.scale_bias) * 4.656612873077392578125e-10f;
+    // dx += s * (2^-31 * acc), through LDS as fp32 so that every lane updates 8 consecutive features of a token's row
+    // (2^-31 * acc is exact, so the product with s is rounded once, as s * 2^-31 times acc would be)
+    const float sval = bf16_to_f32(*p.scale_bias);
+    constexpr float scale = 4.656612873077392578125e-10f;
     constexpr int LDF = RB_BI + 4;   // floats per token row of the staging tile
     float *stage = reinterpret_cast<float *>(smem_raw);
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5;
@@ -91,27 +98,78 @@ __global__ __launch_bounds__(256, 2) void rbias_add_kernel(RBiasParams p)
                                  acc[mi][ni][jq * 4 + 3] * scale};
                 *reinterpret_cast<f32x4 *>(stage + b * LDF + a) = v;
             }
-    __syncthreads();
+    // what the epilogue reads from memory (the old values of dx, and for DOT the other matrix) is requested before the barrier, so
+    // that the loads are in flight while the staging tile fills
+    constexpr int NP = RB_BI * RB_BT / 8 / 256;
+    Frag8 old[NP], ot[NP];
+    bool live[NP];
 #pragma unroll
-    for (int q = 0; q < RB_BI * RB_BT / 8 / 256; ++q) {
+    for (int q = 0; q < NP; ++q) {
         const int idx = q * 256 + t, b = idx / (RB_BI / 8), a = (idx % (RB_BI / 8)) * 8;
-        if (tok0 + b < p.tokens && i0 + a < p.in_f) {   // in_f is a multiple of 8: a piece lies inside or outside
-            bf16_t *dst = p.dx + (int64_t)(tok0 + b) * p.lddx + i0 + a;
-            Frag8 old;
-            old.f4 = *reinterpret_cast<const f32x4 *>(dst);
-            const f32x4 lo = *reinterpret_cast<const f32x4 *>(stage + b * LDF + a), hi = *reinterpret_cast<const f32x4 *>(stage + b * LDF + a + 4);
-            Frag8 nw;
-            nw.u[0] = f32x2_to_bf16x2(__uint_as_float(old.u[0] << 16) + lo[0], __uint_as_float(old.u[0] & 0xffff0000u) + lo[1]);
-            nw.u[1] = f32x2_to_bf16x2(__uint_as_float(old.u[1] << 16) + lo[2], __uint_as_float(old.u[1] & 0xffff0000u) + lo[3]);
-            nw.u[2] = f32x2_to_bf16x2(__uint_as_float(old.u[2] << 16) + hi[0], __uint_as_float(old.u[2] & 0xffff0000u) + hi[1]);
-            nw.u[3] = f32x2_to_bf16x2(__uint_as_float(old.u[3] << 16) + hi[2], __uint_as_float(old.u[3] & 0xffff0000u) + hi[3]);
-            *reinterpret_cast<f32x4 *>(dst) = nw.f4;
+        live[q] = tok0 + b < p.tokens && i0 + a < p.in_f;   // in_f is a multiple of 8: a piece lies inside or outside
+        if (live[q]) old[q].f4 = *reinterpret_cast<const f32x4 *>(p.dx + (int64_t)(tok0 + b) * p.lddx + i0 + a);
+    }
+    __syncthreads();
+    if (DOT) {   // the accumulators are in LDS now: their registers take the other matrix's pieces
+#pragma unroll
+        for (int q = 0; q < NP; ++q) {
+            const int idx = q * 256 + t, b = idx / (RB_BI / 8), a = (idx % (RB_BI / 8)) * 8;
+            if (live[q]) ot[q].f4 = *reinterpret_cast<const f32x4 *>(p.other + (int64_t)(tok0 + b) * p.ld_other + i0 + a);
         }
+    }
+    float dot = 0.0f;
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+        const int idx = q * 256 + t, b = idx / (RB_BI / 8), a = (idx % (RB_BI / 8)) * 8;
+        if (live[q]) {
+            const f32x4 lo = *reinterpret_cast<const f32x4 *>(stage + b * LDF + a), hi = *reinterpret_cast<const f32x4 *>(stage + b * LDF + a + 4);
+            if (DOT) {
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    dot = fmaf(lo[2 * e], __uint_as_float(ot[q].u[e] << 16), dot);
+                    dot = fmaf(lo[2 * e + 1], __uint_as_float(ot[q].u[e] & 0xffff0000u), dot);
+                    dot = fmaf(hi[2 * e], __uint_as_float(ot[q].u[2 + e] << 16), dot);
+                    dot = fmaf(hi[2 * e + 1], __uint_as_float(ot[q].u[2 + e] & 0xffff0000u), dot);
+                }
+            }
+            Frag8 nw;
+            nw.u[0] = f32x2_to_bf16x2(__uint_as_float(old[q].u[0] << 16) + sval * lo[0], __uint_as_float(old[q].u[0] & 0xffff0000u) + sval * lo[1]);
+            nw.u[1] = f32x2_to_bf16x2(__uint_as_float(old[q].u[1] << 16) + sval * lo[2], __uint_as_float(old[q].u[1] & 0xffff0000u) + sval * lo[3]);
+            nw.u[2] = f32x2_to_bf16x2(__uint_as_float(old[q].u[2] << 16) + sval * hi[0], __uint_as_float(old[q].u[2] & 0xffff0000u) + sval * hi[1]);
+            nw.u[3] = f32x2_to_bf16x2(__uint_as_float(old[q].u[3] << 16) + sval * hi[2], __uint_as_float(old[q].u[3] & 0xffff0000u) + sval * hi[3]);
+            *reinterpret_cast<f32x4 *>(p.dx + (int64_t)(tok0 + b) * p.lddx + i0 + a) = nw.f4;
+        }
+    }
+    if (DOT) {
+        // the block's share of <src . R, other>: lanes, then waves, in a fixed order
+        __shared__ float wsum[4];
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) dot += __shfl_xor(dot, off, 64);
+        if (lane == 0) wsum[wave] = dot;
+        __syncthreads();
+        if (t == 0) p.dot_part[w] = (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]);
     }
 }
 
+// out[0] = part[0] + ... + part[n - 1], in a fixed order (one block)
+__global__ __launch_bounds__(256) void rbias_sum_kernel(float *__restrict__ out, const float *__restrict__ part, int n)
+{
+    __shared__ float sh[256];
+    float v = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 256) v += part[i];
+    sh[threadIdx.x] = v;
+    __syncthreads();
+    for (int h = 128; h >= 1; h >>= 1) {
+        if ((int)threadIdx.x < h) sh[threadIdx.x] += sh[threadIdx.x + h];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = sh[0];
+}
+
+// other / dot_part / dscale: NULL, or the matrix the product is reduced against, room for one float per tile, and where the sum goes
 static int rbias_add(void *dst, int64_t ld_dst, int64_t cols, const void *src, int64_t ld_src, int64_t contraction, uint32_t sR, uint32_t sK,
-                     const void *scale_bias, const rdb_linear_desc *d, hipStream_t s)
+                     const void *scale_bias, const rdb_linear_desc *d, hipStream_t s, const void *other = nullptr, int64_t ld_other = 0,
+                     float *dot_part = nullptr, float *dscale = nullptr)
 {
     if (d->act_dtype != RDB_BF16 || d->coef_dtype != RDB_BF16 || d->coef_rows == 0 || !scale_bias) return RDB_E_UNSUPPORTED;
     if (d->in_f % 8 || d->out_f % 8 || d->tokens < 1 || d->in_f < 1 || d->out_f < 1) return RDB_E_UNSUPPORTED;
@@ -131,10 +189,27 @@ static int rbias_add(void *dst, int64_t ld_dst, int64_t cols, const void *src, i
     p.sR = sR;
     p.sK = sK;
     p.seed = d->seed;
+    p.other = (const bf16_t *)other;
+    p.ld_other = ld_other;
+    p.dot_part = dot_part;
     size_t smem = engine_smem<RB_BI, RB_BT, RB_BK, K_CONT, K_CONT>();
     const size_t stage = (size_t)RB_BT * (RB_BI + 4) * sizeof(float);
     if (smem < stage) smem = stage;
-    return launch_engine(rbias_add_kernel, p, p.tiles_i * p.tiles_t, smem, s, "rbias_add_kernel");
+    if (!other) return launch_engine(rbias_add_kernel<false>, p, p.tiles_i * p.tiles_t, smem, s, "rbias_add_kernel");
+    if (ld_other % 8 || ((uintptr_t)other & 15) || d->tokens * ld_other >= (1ll << 29) || !dot_part || !dscale) return RDB_E_UNSUPPORTED;
+    if (int rc = launch_engine(rbias_add_kernel<true>, p, p.tiles_i * p.tiles_t, smem, s, "rbias_add_kernel<dot>")) return rc;
+    rbias_sum_kernel<<<1, 256, 0, s>>>(dscale, dot_part, p.tiles_i * p.tiles_t);
+    return check_launch("rbias_sum_kernel");
+}
+
+// floats of scratch for the tiles' shares of the scale's gradient
+int64_t linear_dx_rbias_dot_floats(const rdb_linear_desc *d) { return cdiv(d->in_f, RB_BI) * cdiv(d->tokens, RB_BT); }
+
+// dx += s * dy . R and d s = <dy . R, x> in one pass over dy . R
+int linear_dx_rbias_add_dscale(void *dx, int64_t lddx, float *dscale, float *dot_part, const void *dy, int64_t lddy, const void *x, int64_t ldx,
+                               const void *scale_bias, const rdb_linear_desc *d, hipStream_t s)
+{
+    return rbias_add(dx, lddx, d->in_f, dy, lddy, d->out_f, 1u, (uint32_t)d->in_f, scale_bias, d, s, x, ldx, dot_part, dscale);
 }
 
 // dx += s * dy . R on the launch stream, after the kernels that wrote dx.  Returns RDB_E_UNSUPPORTED (without setting an

@@ -351,6 +351,35 @@ def linear_bwd_dx(dy: torch.Tensor, coef: torch.Tensor, in_f: int, out_f: int, s
     return dx
 
 
+def linear_bwd_dx_dscale(dy: torch.Tensor, x: torch.Tensor, coef: torch.Tensor, in_f: int, out_f: int, seed: int, scale_bias: torch.Tensor):
+    """``(dx, d_scale_bias)`` of a matrix-coef bf16 layer with the fused random bias: ``dx = dy @ W`` and the gradient of the
+    bias's scale, ``<dy @ R, x>`` (fp32, ``(1,)``), from one pass over the random-bias product.  ``None`` when the library has
+    no such kernel for the request (other dtypes or forms: the caller takes ``linear_bwd_dx`` and ``linear_bwd_dcoef``)."""
+    _need_gpu("linear_bwd_dx_dscale", dy, x, coef, scale_bias)
+    if dy.dtype != torch.bfloat16 or coef.dtype != torch.bfloat16 or coef.dim() != 2:
+        return None
+    dy, x = _act(dy), _act(x)
+    if x.dtype != dy.dtype:
+        x = x.to(dy.dtype)
+    c = _native(coef)
+    sb = _native(scale_bias).to(c.dtype)
+    d = _desc(dy.shape[0], in_f, out_f, c, in_f, 1, seed, dy.dtype, RDB_ALGO_AUTO)
+    L = _lib.load()
+    ws_bytes = int(L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX_DSCALE, ctypes.byref(d)))
+    if ws_bytes <= 0:
+        return None
+    dx = torch.empty((dy.shape[0], in_f), dtype=dy.dtype, device=dy.device)
+    ds = torch.empty((1,), dtype=torch.float32, device=dy.device)
+    with _on(dy.device):
+        ws = _workspace(ws_bytes, dy.device)
+        rc = L.rdb_linear_bwd_dx_dscale(_p(dx), dx.stride(0), _p(ds), _p(dy), dy.stride(0), _p(x), x.stride(0), _p(c), _p(sb), ctypes.byref(d),
+                                        _p(ws), ws_bytes, _stream(dy.device))
+    if rc == -5:   # RDB_E_UNSUPPORTED: nothing was launched
+        return None
+    _lib.check(rc, "rdb_linear_bwd_dx_dscale")
+    return dx, ds
+
+
 def linear_bwd_dcoef(dy: torch.Tensor, x: torch.Tensor, k: int, coef_rows: int, in_f: int, out_f: int, sO: int, sI: int,
                      seed: int, want_scale_bias_grad: bool = False, algo: int = RDB_ALGO_AUTO):
     """``(dcoef, d_scale_bias)`` in fp32: ``dcoef = (dy.T @ x) . Noise.T`` without storing ``dy.T @ x``."""

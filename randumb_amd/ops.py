@@ -289,9 +289,16 @@ class _EagerLinear(torch.autograd.Function):
         in_f, out_f, sO, sI, seed = ctx.meta
         dy = dy.contiguous()
         dx = dcoefs = dsb = dbias = None
-        if ctx.needs_input_grad[0]:
-            dx = hip.linear_bwd_dx(dy, coefs, in_f, out_f, sO, sI, seed, scale_bias)
         want_sb = scale_bias is not None and ctx.needs_input_grad[7]
+        if ctx.needs_input_grad[0] and want_sb and sO == in_f and sI == 1:
+            # the random-bias product dy.R that dx needs anyway also gives the gradient of the bias's scale (reduced against x in
+            # the same pass), so the coefficient gradient below comes from the factored kernels and dW is never formed
+            both = hip.linear_bwd_dx_dscale(dy, x, coefs, in_f, out_f, seed, scale_bias)
+            if both is not None:
+                dx, dsb = both[0], both[1].to(scale_bias.dtype)
+                want_sb = False
+        if ctx.needs_input_grad[0] and dx is None:
+            dx = hip.linear_bwd_dx(dy, coefs, in_f, out_f, sO, sI, seed, scale_bias)
         if ctx.needs_input_grad[1] or want_sb:
             dc, ds = hip.linear_bwd_dcoef(dy, x, coefs.shape[-1], 0 if coefs.dim() == 1 else coefs.shape[0], in_f, out_f, sO, sI, seed, want_sb)
             dcoefs = dc.to(coefs.dtype)

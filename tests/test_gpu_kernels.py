@@ -592,6 +592,15 @@ def test_default_layer_fast_path_with_scale_bias(hip, oracle, T, in_f, out_f, k)
         assert rel_l2(cpu(dx), want_dx) < BF16_TOL
         assert rel_l2(cpu(dc), want_dc) < BF16_TOL
         assert abs(float(ds) - want_ds) < BF16_TOL * max(abs(want_ds), float(np.linalg.norm(dW)))
+        # input gradient and the gradient of s from one pass over dy.R (what the layer's backward pass calls): the same dx bit
+        # for bit, d s = <dy.R, x> against the oracle and the same bits run to run; the coefficient gradient then needs no dW
+        both = hip.linear_bwd_dx_dscale(dyg, xg, cg, in_f, out_f, 9, sg)
+        assert both is not None and torch.equal(both[0], dx)
+        assert abs(float(both[1]) - want_ds) < BF16_TOL * max(abs(want_ds), float(np.linalg.norm(dW)))
+        # (the dW-tile kernel above rounds dW to bf16 before the contraction, this one reduces fp32 sums: it is the closer one)
+        assert torch.equal(hip.linear_bwd_dx_dscale(dyg, xg, cg, in_f, out_f, 9, sg)[1], both[1])
+        dc_only, none = hip.linear_bwd_dcoef(dyg, xg, k, out_f, in_f, out_f, in_f, 1, 9, want_scale_bias_grad=False)
+        assert none is None and rel_l2(cpu(dc_only), want_dc) < BF16_TOL
         # the same input gradient from the general kernel that forms the weight block by block
         from randumb_amd._lib import RDB_ALGO_TILE
         if T <= 256:
