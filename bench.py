@@ -303,6 +303,33 @@ def f32_layer_config(event_ms, torch, L, _lib, dev, g, compare=True):
     return res
 
 
+def smallk_config(event_ms, torch, L, _lib, dev, g):
+    """Small-k fp32 regime: 4096 -> 4096, k = 16, forward at batch 1 / 16 / 256.  "effective" = the bytes a stored-W product
+    would move (4*(out*in + B*in + B*out)) over the time; the fused kernel itself reads 4*(B*in + out*k) and writes 4*B*out."""
+    vp = ctypes.c_void_p
+    stream = vp(torch.cuda.current_stream().cuda_stream)
+    in_f = out_f = 4096
+    C = (torch.randn(out_f, 16, generator=g) / 64.0).to(dev)
+    small = {}
+    for B in (1, 16, 256):
+        x = torch.randn(B, in_f, generator=g).to(dev)
+        y = torch.empty(B, out_f, device=dev)
+        d = _lib.LinearDesc()
+        d.tokens, d.in_f, d.out_f, d.k, d.coef_rows, d.sO, d.sI, d.seed = B, in_f, out_f, 16, out_f, in_f, 1, 0
+        d.act_dtype, d.coef_dtype, d.algo = _lib.RDB_F32, _lib.RDB_F32, _lib.RDB_ALGO_AUTO
+        r = ctypes.byref(d)
+        n = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, r)
+        ws = torch.empty(max(n, 16), dtype=torch.uint8, device=dev)
+        args = (vp(y.data_ptr()), out_f, vp(x.data_ptr()), in_f, vp(C.data_ptr()), None, None, r, vp(ws.data_ptr()), n, stream)
+        _lib.check(L.rdb_linear_fwd(*args), "rdb_linear_fwd")
+        ms = event_ms(lambda: L.rdb_linear_fwd(*args), 200)
+        stored = 4.0 * (out_f * in_f + B * in_f + B * out_f)
+        actual = 4.0 * (B * in_f + out_f * 16 + B * out_f)
+        small[f"batch_{B}"] = {"fwd_ms": round(ms, 4), "effective_GBps_vs_stored_W": round(stored / ms / 1e6, 1),
+                               "actual_HBM_GBps": round(actual / ms / 1e6, 2)}
+    return small
+
+
 def gpt_step_config(event_ms, torch, dev, g):
     """GPT-2 small with random-backed linears: 12 layers, d = 768, 12 heads, vocab 50304, k = 256, seeds 0..47, bf16, batch
     8 x 1024 random token ids; one training step (forward + backward).  Attention, norms, embedding, head and loss are stock
@@ -333,28 +360,7 @@ def other_configs(event_ms, torch, L, _lib, dev):
     stream = vp(torch.cuda.current_stream().cuda_stream)
     g = torch.Generator().manual_seed(0)
 
-    # ---- small-k fp32 regime: 4096 -> 4096, k = 16, forward at batch 1 / 16 / 256.  "effective" = the bytes a stored-W product
-    # would move (4*(out*in + B*in + B*out)) over the time; the fused kernel itself reads 4*(B*in + out*k) and writes 4*B*out.
-    in_f = out_f = 4096
-    C = (torch.randn(out_f, 16, generator=g) / 64.0).to(dev)
-    small = {}
-    for B in (1, 16, 256):
-        x = torch.randn(B, in_f, generator=g).to(dev)
-        y = torch.empty(B, out_f, device=dev)
-        d = _lib.LinearDesc()
-        d.tokens, d.in_f, d.out_f, d.k, d.coef_rows, d.sO, d.sI, d.seed = B, in_f, out_f, 16, out_f, in_f, 1, 0
-        d.act_dtype, d.coef_dtype, d.algo = _lib.RDB_F32, _lib.RDB_F32, _lib.RDB_ALGO_AUTO
-        r = ctypes.byref(d)
-        n = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, r)
-        ws = torch.empty(max(n, 16), dtype=torch.uint8, device=dev)
-        args = (vp(y.data_ptr()), out_f, vp(x.data_ptr()), in_f, vp(C.data_ptr()), None, None, r, vp(ws.data_ptr()), n, stream)
-        _lib.check(L.rdb_linear_fwd(*args), "rdb_linear_fwd")
-        ms = event_ms(lambda: L.rdb_linear_fwd(*args), 200)
-        stored = 4.0 * (out_f * in_f + B * in_f + B * out_f)
-        actual = 4.0 * (B * in_f + out_f * 16 + B * out_f)
-        small[f"batch_{B}"] = {"fwd_ms": round(ms, 4), "effective_GBps_vs_stored_W": round(stored / ms / 1e6, 1),
-                               "actual_HBM_GBps": round(actual / ms / 1e6, 2)}
-    out["in4096_out4096_k16_fp32_matrix_coef"] = small
+    out["in4096_out4096_k16_fp32_matrix_coef"] = smallk_config(event_ms, torch, L, _lib, dev, g)
 
     out["in4096_out14336_k1024_T4096_bf16"] = llm_layer_config(event_ms, torch, L, _lib, dev, g)
     out["in768_out3072_k256_T8192_fp32"] = f32_layer_config(event_ms, torch, L, _lib, dev, g)
@@ -416,6 +422,8 @@ def main():
                          "(profiling runs)")
     ap.add_argument("--f32-layer-only", action="store_true",
                     help="time only the fp32 form of the headline layer (profiling runs)")
+    ap.add_argument("--smallk-only", action="store_true",
+                    help="run only the fp32 4096 -> 4096, k = 16 forward at batch 1 / 16 / 256 and exit (profiling runs)")
     ap.add_argument("--gpt-only", action="store_true",
                     help="run only the GPT-2 small training step with random-backed linears and exit (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -452,6 +460,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.smallk_only:
+        print(json.dumps({"in4096_out4096_k16_fp32_matrix_coef": smallk_config(make_event_ms(torch), torch, L, _lib, dev, g)}))
+        return
     if args.gpt_only:
         print(json.dumps({"gpt2_small_12L_k256_seeds0to47_bf16_8x1024": gpt_step_config(make_event_ms(torch), torch, dev, g)}))
         return
