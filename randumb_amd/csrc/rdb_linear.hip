@@ -10,6 +10,7 @@
 // (src/rten_cpp/RandumbTensor.py:942-952, 771-791), autograd's MmBackward on the dense weight, and
 // RandumbTensorConstructor.backward -> materialize_bwd / scale_bias_bwd (RandumbTensor.py:979-990).
 #include <algorithm>
+#include <cstdlib>
 
 #include "rdb_direct.hpp"
 #include "rdb_tile.hpp"
@@ -458,7 +459,8 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
                                                 "rdb_linear_workspace_bytes() bytes and either bf16 (activations and coef; sizes that are "
                                                 "multiples of 8; aligned rows) or fp32 (sizes that are multiples of 4; aligned rows)");
     }
-    if (d->algo != RDB_ALGO_TILE) {
+    static const int dev_fwd_rbias = getenv("RDB_FWD_RBIAS") ? atoi(getenv("RDB_FWD_RBIAS")) : 0;   // DEV
+    if (d->algo != RDB_ALGO_TILE && !(dev_fwd_rbias && d->algo == RDB_ALGO_AUTO && scale_bias)) {
         rc = linear_fwd_strip(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
         if (d->algo == RDB_ALGO_STRIP)
