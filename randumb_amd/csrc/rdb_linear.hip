@@ -10,7 +10,6 @@
 // (src/rten_cpp/RandumbTensor.py:942-952, 771-791), autograd's MmBackward on the dense weight, and
 // RandumbTensorConstructor.backward -> materialize_bwd / scale_bias_bwd (RandumbTensor.py:979-990).
 #include <algorithm>
-#include <cstdlib>
 
 #include "rdb_direct.hpp"
 #include "rdb_tile.hpp"
@@ -459,8 +458,20 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
                                                 "rdb_linear_workspace_bytes() bytes and either bf16 (activations and coef; sizes that are "
                                                 "multiples of 8; aligned rows) or fp32 (sizes that are multiples of 4; aligned rows)");
     }
-    static const int dev_fwd_rbias = getenv("RDB_FWD_RBIAS") ? atoi(getenv("RDB_FWD_RBIAS")) : 0;   // DEV
-    if (d->algo != RDB_ALGO_TILE && !(dev_fwd_rbias && d->algo == RDB_ALGO_AUTO && scale_bias)) {
+    if (d->algo == RDB_ALGO_AUTO && scale_bias && d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16) {
+        // W = C.N + s.R: the low-rank share through the factored kernels where AUTO would take them without the random bias,
+        // then the random-bias share (full rank: a product with R hashed as an operand) added on top.  Ahead of the kernel that
+        // forms weight strips on chip at every size measured (8192 tokens x 768 -> 768, k = 256: 41 against 74 us; 768 -> 3072:
+        // 118 against 121; 2048 tokens x 768 -> 3072: 43 against 74).
+        rdb_linear_desc df = *d;
+        rc = linear_fwd_factored(y, ldy, x, ldx, coef, nullptr, bias, &df, num_compute_units(), workspace, workspace_bytes, s);
+        if (rc == RDB_OK) {
+            rc = linear_fwd_rbias_add(y, ldy, x, ldx, scale_bias, d, s);
+            if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "rdb_linear_fwd: internal: the random-bias share refused a request the factored share took");
+        }
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
+    if (d->algo != RDB_ALGO_TILE) {
         rc = linear_fwd_strip(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
         if (d->algo == RDB_ALGO_STRIP)
@@ -468,8 +479,8 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
                                                 "16-byte aligned x rows and a weight strip that fits LDS");
     }
     if (d->algo == RDB_ALGO_AUTO && scale_bias && d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16) {
-        // W = C.N + s.R where no weight strip fits on chip (a long in_f): the low-rank share through the factored kernels, then
-        // the random-bias share added on top (3072 -> 768, k = 256, 8192 tokens: 3.0 ms for the general kernel below)
+        // the same two shares where the rule above did not take the factored form (k so long that it is not the cheaper one in
+        // flops) and no weight strip fits on chip: still far ahead of the general kernel below
         rdb_linear_desc df = *d;
         df.algo = RDB_ALGO_FACTORED;
         rc = linear_fwd_factored(y, ldy, x, ldx, coef, nullptr, bias, &df, num_compute_units(), workspace, workspace_bytes, s);

@@ -11,9 +11,10 @@
 // per compute unit so that one block's hashing runs under the other's matrix work.  R never exists in memory.
 #include "rdb_gemm.hpp"
 #include "rdb_tile.hpp"
-#include <cstdlib>
 
 namespace rdb {
+
+int num_compute_units();   // of the current device (rdb_error.hip)
 
 constexpr int RB_BI = 64, RB_BT = 256, RB_BK = 64;
 
@@ -182,9 +183,6 @@ __device__ __forceinline__ void rw_load_src(f32x4 (&rs)[RW_SP], const RwState &s
 
 __device__ __forceinline__ f32x4 rw_hash(const RwState &st, int stage)
 {
-#ifdef RW_NOHASH
-    return f32x4{1.0f, 1.0f, 1.0f, (float)stage};
-#else
     const uint32_t first = st.first0 + (uint32_t)stage * st.stage_step;
     uint32_t b[8];
 #pragma unroll
@@ -193,7 +191,6 @@ __device__ __forceinline__ f32x4 rw_hash(const RwState &st, int stage)
 #pragma unroll
     for (int e = 0; e < 4; ++e) f.u[e] = f32x2_to_bf16x2((float)(int32_t)b[2 * e], (float)(int32_t)b[2 * e + 1]);
     return f.f4;
-#endif
 }
 
 // One stage: the matrix instructions of LDS buffer `cur`; between them the registers (holding the next stage) go to the
@@ -212,7 +209,6 @@ __device__ __forceinline__ void rw_stage(f32x16 (&acc)[2][2], const bf16_t *__re
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const int c = ks & 1, n = c ^ 1;
-#ifndef RW_NOCOPY
 #pragma unroll
         for (int q = 0; q < RW_SP; ++q)
             if (q % KS == ks) {
@@ -222,7 +218,6 @@ __device__ __forceinline__ void rw_stage(f32x16 (&acc)[2][2], const bf16_t *__re
                     rs[q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(st.rs_src, (int)(st.soff[q] + adv), 0, 0));
                 }
             }
-#endif
         if (ks == 0) {
             if (STORE) *reinterpret_cast<f32x4 *>(oth + st.lds_r) = rr;
             if (RELOAD) rr = rw_hash(st, next);
@@ -233,17 +228,10 @@ __device__ __forceinline__ void rw_stage(f32x16 (&acc)[2][2], const bf16_t *__re
 #pragma unroll
             for (int ni = 0; ni < 2; ++ni) fb[n][ni] = RwTileS::frag(Ss, wave * 64 + ni * 32, ks + 1, lane);
         }
-#ifndef RW_NOMFMA
 #pragma unroll
         for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
             for (int ni = 0; ni < 2; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[c][mi], fb[c][ni], acc[mi][ni], 0, 0, 0);
-#else
-#pragma unroll
-        for (int mi = 0; mi < 2; ++mi)
-#pragma unroll
-            for (int ni = 0; ni < 2; ++ni) acc[mi][ni][0] += (float)fa[c][mi][0] * (float)fb[c][ni][0];
-#endif
     }
     __syncthreads();
 }
@@ -405,32 +393,30 @@ static int rbias_add(void *dst, int64_t ld_dst, int64_t cols, const void *src, i
     p.other = (const bf16_t *)other;
     p.ld_other = ld_other;
     p.dot_part = dot_part;
-    {   // DEV: wide kernel switch
-        static const int mode = getenv("RDB_RBIAS_WIDE") ? atoi(getenv("RDB_RBIAS_WIDE")) : 1;
-        const int wide_items = (int)(cdiv(cols, RW_BI) * cdiv(d->tokens, RW_BT));
-        if (mode == 2 || (mode == 1 && wide_items >= 128)) {
-            p.tiles_i = (int)cdiv(cols, RW_BI);
-            p.tiles_t = (int)cdiv(d->tokens, RW_BT);
-            const size_t wsmem = (size_t)2 * RW_STAGE * sizeof(bf16_t);
-            static_assert((size_t)RW_BT * (RW_BI + 4) * sizeof(float) <= (size_t)2 * RW_STAGE * sizeof(bf16_t), "the fp32 staging tile fits the pipeline's LDS");
-            if (other && (ld_other % 8 || ((uintptr_t)other & 15) || d->tokens * ld_other >= (1ll << 29) || !dot_part || !dscale)) return RDB_E_UNSUPPORTED;
-            if (!other) {
-                if (int rl = reserve_lds(reinterpret_cast<const void *>(rbias_wide_kernel<false>), wsmem, "rbias_wide_kernel")) return rl;
-                rbias_wide_kernel<false><<<xcd_grid_size(wide_items), RW_THREADS, wsmem, s>>>(p);
-                return check_launch("rbias_wide_kernel");
-            }
-            if (int rl = reserve_lds(reinterpret_cast<const void *>(rbias_wide_kernel<true>), wsmem, "rbias_wide_kernel<dot>")) return rl;
-            rbias_wide_kernel<true><<<xcd_grid_size(wide_items), RW_THREADS, wsmem, s>>>(p);
-            if (int rc = check_launch("rbias_wide_kernel<dot>")) return rc;
-            rbias_sum_kernel<<<1, 256, 0, s>>>(dscale, dot_part, wide_items);
-            return check_launch("rbias_sum_kernel");
+    if (other && (ld_other % 8 || ((uintptr_t)other & 15) || d->tokens * ld_other >= (1ll << 29) || !dot_part || !dscale)) return RDB_E_UNSUPPORTED;
+    // tiles of 512 tokens when they give at least every other compute unit a block (half the hashing per product: measured
+    // ahead from there on; 8192 tokens x 768 features, contraction 3072: 83 -> 67 us), tiles of 256 tokens otherwise
+    const int wide_items = (int)(cdiv(cols, RW_BI) * cdiv(d->tokens, RW_BT));
+    if (wide_items * 2 >= num_compute_units()) {
+        p.tiles_i = (int)cdiv(cols, RW_BI);
+        p.tiles_t = (int)cdiv(d->tokens, RW_BT);
+        const size_t wsmem = (size_t)2 * RW_STAGE * sizeof(bf16_t);
+        static_assert((size_t)RW_BT * (RW_BI + 4) * sizeof(float) <= (size_t)2 * RW_STAGE * sizeof(bf16_t), "the fp32 staging tile fits the pipeline's LDS");
+        if (!other) {
+            if (int rl = reserve_lds(reinterpret_cast<const void *>(rbias_wide_kernel<false>), wsmem, "rbias_wide_kernel")) return rl;
+            rbias_wide_kernel<false><<<xcd_grid_size(wide_items), RW_THREADS, wsmem, s>>>(p);
+            return check_launch("rbias_wide_kernel");
         }
+        if (int rl = reserve_lds(reinterpret_cast<const void *>(rbias_wide_kernel<true>), wsmem, "rbias_wide_kernel<dot>")) return rl;
+        rbias_wide_kernel<true><<<xcd_grid_size(wide_items), RW_THREADS, wsmem, s>>>(p);
+        if (int rc = check_launch("rbias_wide_kernel<dot>")) return rc;
+        rbias_sum_kernel<<<1, 256, 0, s>>>(dscale, dot_part, wide_items);
+        return check_launch("rbias_sum_kernel");
     }
     size_t smem = engine_smem<RB_BI, RB_BT, RB_BK, K_CONT, K_CONT>();
     const size_t stage = (size_t)RB_BT * (RB_BI + 4) * sizeof(float);
     if (smem < stage) smem = stage;
     if (!other) return launch_engine(rbias_add_kernel<false>, p, p.tiles_i * p.tiles_t, smem, s, "rbias_add_kernel");
-    if (ld_other % 8 || ((uintptr_t)other & 15) || d->tokens * ld_other >= (1ll << 29) || !dot_part || !dscale) return RDB_E_UNSUPPORTED;
     if (int rc = launch_engine(rbias_add_kernel<true>, p, p.tiles_i * p.tiles_t, smem, s, "rbias_add_kernel<dot>")) return rc;
     rbias_sum_kernel<<<1, 256, 0, s>>>(dscale, dot_part, p.tiles_i * p.tiles_t);
     return check_launch("rbias_sum_kernel");

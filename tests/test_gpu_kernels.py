@@ -570,6 +570,7 @@ def test_factored_dx_needs_what_it_says(hip):
     (200, 72, 136, 40),
     (1024, 3072, 768, 256),   # in_f too long for a weight strip on chip: factored forward + the random-bias share added on top
     (512, 1024, 1024, 512),   # k > 256 and the factored form not the cheaper one in flops: still the one that runs
+    (4000, 1032, 1048, 64),   # enough tiles of 512 tokens x 64 features for the eight-wave random-bias kernel in both directions, ragged against both
 ])
 def test_default_layer_fast_path_with_scale_bias(hip, oracle, T, in_f, out_f, k):
     """The reference's default layer starts from zero coefficients and a fused random bias (SillyLayers.py:122-133, 218-221):
