@@ -657,14 +657,28 @@ def main():
 
         def scale_bias_ms():
             # the reference's default layer: W = C.N + s.noise1d (zero coefficients and a fused random bias at initialisation).
-            # forward: the strip kernel; dx and d s: factored share + hashed random-bias share, reduced against x on the side;
-            # dcoef: factored (no dW).  Beside it the older split: dx alone, dcoef and d s from dW tiles.
+            # What SillyLinear runs: the low-rank share through the projected calls of the headline step (z = x.N^T formed once, by
+            # the forward pass), the full-rank random-bias share through kernels of its own on top (rdb_linear_rbias_fwd / _bwd,
+            # the latter also reducing d s = <dy.R, x>).  Beside it the one-call entry points (z formed by the forward and again
+            # by the coefficient gradient) and the older split with dcoef and d s from dW tiles.
             sb = torch.tensor([0.02], device=dev).bfloat16()
             ds = torch.empty(1, dtype=torch.float32, device=dev)
             psb, pds, r = ctypes.c_void_p(sb.data_ptr()), ctypes.c_void_p(ds.data_ptr()), main_set.dref
             n_ds = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX_DSCALE, r)
             ws_ds = torch.empty(max(n_ds, 16), dtype=torch.uint8, device=dev)
             pws_ds = ctypes.c_void_p(ws_ds.data_ptr())
+            n_rb = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_RBIAS_BWD, r)
+            ws_rb = torch.empty(max(n_rb, 16), dtype=torch.uint8, device=dev)
+            pws_rb = ctypes.c_void_p(ws_rb.data_ptr())
+
+            def fwd_projected():
+                main_set.project_fwd()
+                _lib.check(L.rdb_linear_rbias_fwd(p["y"], OUT_F, p["x"], IN_F, psb, r, stream), "rdb_linear_rbias_fwd")
+
+            def bwd_projected():
+                main_set.bwd()
+                _lib.check(L.rdb_linear_rbias_bwd(p["dx"], IN_F, pds, p["dy"], OUT_F, p["x"], IN_F, psb, r, pws_rb, n_rb, stream), "rdb_linear_rbias_bwd")
+
             fwd = lambda: _lib.check(L.rdb_linear_fwd(p["y"], OUT_F, p["x"], IN_F, p["C"], psb, None, r, p["ws"], ws_bytes, stream), "rdb_linear_fwd")
             dxs = lambda: _lib.check(L.rdb_linear_bwd_dx_dscale(p["dx"], IN_F, pds, p["dy"], OUT_F, p["x"], IN_F, p["C"], psb, r, pws_ds, n_ds, stream),
                                      "rdb_linear_bwd_dx_dscale")
@@ -673,8 +687,11 @@ def main():
             dxf = lambda: _lib.check(L.rdb_linear_bwd_dx(p["dx"], IN_F, p["dy"], OUT_F, p["C"], psb, r, p["ws"], ws_bytes, stream), "rdb_linear_bwd_dx")
             dcf = lambda: _lib.check(L.rdb_linear_bwd_dcoef(p["dC"], pds, p["dy"], OUT_F, p["x"], IN_F, r, p["ws"], ws_bytes, stream),
                                      "rdb_linear_bwd_dcoef")
-            t = {"fwd": round(event_ms(fwd, 20), 4), "dx_and_dscale": round(event_ms(dxs, 20), 4), "dcoef": round(event_ms(dco, 20), 4)}
+            t = {"fwd": round(event_ms(fwd_projected, 20), 4), "bwd_with_dscale": round(event_ms(bwd_projected, 20), 4)}
             t["step"] = round(sum(t.values()), 4)
+            o = {"fwd": round(event_ms(fwd, 20), 4), "dx_and_dscale": round(event_ms(dxs, 20), 4), "dcoef": round(event_ms(dco, 20), 4)}
+            o["step"] = round(sum(o.values()), 4)
+            t["one_call_entry_points"] = o
             t["with_dscale_from_dw_tiles"] = {"dx": round(event_ms(dxf, 20), 4), "dcoef_and_dscale": round(event_ms(dcf, 20), 4)}
             return t
 

@@ -151,7 +151,7 @@ enum {
 };
 
 enum { RDB_OP_LINEAR_FWD = 0, RDB_OP_LINEAR_BWD_DX = 1, RDB_OP_LINEAR_BWD_DCOEF = 2, RDB_OP_LINEAR_BWD_PROJECTED = 3,
-       RDB_OP_LINEAR_BWD_PROJECTED_TO = 4, RDB_OP_LINEAR_BWD_DX_DSCALE = 5 };
+       RDB_OP_LINEAR_BWD_PROJECTED_TO = 4, RDB_OP_LINEAR_BWD_DX_DSCALE = 5, RDB_OP_LINEAR_RBIAS_BWD = 6 };
 
 /* Device scratch (bytes) that entry point `op` can use for `desc`; 0 when it has no use for any.  A NULL or too small
  * workspace is never an error with RDB_ALGO_AUTO: the library then runs a kernel that needs none. */
@@ -191,6 +191,23 @@ int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t lddy, cons
 int rdb_linear_bwd_dx_dscale(void *dx, int64_t lddx, float *d_scale_bias, const void *dy, int64_t lddy, const void *x,
                              int64_t ldx, const void *coef, const void *scale_bias, const rdb_linear_desc *desc,
                              void *workspace, int64_t workspace_bytes, void *stream);
+
+/* The random-bias share of a layer with W = C.N + s.R (R[o, i] = noise1d(o*in_f + i), the term materialize adds at
+ * R.py:286-289) on its own, ADDED to a matrix that already holds the low-rank share; for callers that run that share through
+ * the projected entry points below (projection state saved by the forward pass, so that the backward pass forms x.N^T only
+ * once).  desc->k and the coefficients play no part.
+ *   rdb_linear_rbias_fwd:  y[t, o]  += s * sum_i x[t, i]  * R[o, i]
+ *   rdb_linear_rbias_bwd:  dx[t, i] += s * sum_o dy[t, o] * R[o, i];  when d_scale_bias != NULL also
+ *                          d_scale_bias[0] = <dy . R, x> (fp32, overwritten; what scale_bias_bwd computes from a stored dW,
+ *                          R.py:399-420), from the same pass; x and a workspace of
+ *                          rdb_linear_workspace_bytes(RDB_OP_LINEAR_RBIAS_BWD, desc) bytes are needed then only.
+ * bf16 activations and scale (one bf16 value), matrix-coef descriptor, sizes that are multiples of 8, 16-byte aligned rows;
+ * RDB_E_UNSUPPORTED and nothing launched otherwise.  Sums in a fixed order: the same bits from run to run. */
+int rdb_linear_rbias_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, const void *scale_bias,
+                         const rdb_linear_desc *desc, void *stream);
+int rdb_linear_rbias_bwd(void *dx, int64_t lddx, float *d_scale_bias, const void *dy, int64_t lddy, const void *x,
+                         int64_t ldx, const void *scale_bias, const rdb_linear_desc *desc, void *workspace,
+                         int64_t workspace_bytes, void *stream);
 
 /* Replaces MmBackward's dW = dy^T x followed by RandumbTensorConstructor.backward ->
  * materialize_bwd (+ scale_bias_bwd) (R.py:979-990): dW is contracted with the regenerated noise tile

@@ -16,6 +16,7 @@ RDB_F32, RDB_BF16 = 0, 1
 RDB_ALGO_AUTO, RDB_ALGO_TILE, RDB_ALGO_STRIP, RDB_ALGO_FACTORED = 0, 1, 2, 3
 RDB_OP_LINEAR_FWD, RDB_OP_LINEAR_BWD_DX, RDB_OP_LINEAR_BWD_DCOEF, RDB_OP_LINEAR_BWD_PROJECTED, RDB_OP_LINEAR_BWD_PROJECTED_TO = 0, 1, 2, 3, 4
 RDB_OP_LINEAR_BWD_DX_DSCALE = 5
+RDB_OP_LINEAR_RBIAS_BWD = 6
 
 # every exported entry point, in header order; tests check the list against the built library
 EXPORTS = [
@@ -37,6 +38,8 @@ EXPORTS = [
     "rdb_linear_fwd_static_max_bytes",
     "rdb_linear_bwd_dx",
     "rdb_linear_bwd_dx_dscale",
+    "rdb_linear_rbias_fwd",
+    "rdb_linear_rbias_bwd",
     "rdb_linear_bwd_dcoef",
     "rdb_linear_projection_bytes",
     "rdb_linear_projection_chunks",
@@ -55,7 +58,7 @@ EXPORTS = [
     "rdb_selftest_sync_giveup",
 ]
 
-ABI_VERSION = 7   # what this binding was written against (rdb_abi_version)
+ABI_VERSION = 8   # what this binding was written against (rdb_abi_version)
 
 
 class LinearDesc(ctypes.Structure):
@@ -129,6 +132,8 @@ def load() -> ctypes.CDLL:
     L.rdb_linear_bwd_dx.argtypes = [vp, i64, vp, i64, vp, vp, dp, vp, i64, vp]
     L.rdb_linear_bwd_dcoef.argtypes = [vp, vp, vp, i64, vp, i64, dp, vp, i64, vp]
     L.rdb_linear_bwd_dx_dscale.argtypes = [vp, i64, vp, vp, i64, vp, i64, vp, vp, dp, vp, i64, vp]
+    L.rdb_linear_rbias_fwd.argtypes = [vp, i64, vp, i64, vp, dp, vp]
+    L.rdb_linear_rbias_bwd.argtypes = [vp, i64, vp, vp, i64, vp, i64, vp, dp, vp, i64, vp]
     L.rdb_linear_projection_bytes.argtypes = [dp]
     L.rdb_linear_projection_bytes.restype = i64
     L.rdb_linear_projection_chunks.argtypes = [dp, ctypes.POINTER(i64)]
@@ -153,7 +158,8 @@ def load() -> ctypes.CDLL:
     L.rdb_selftest_sync_giveup.argtypes = [vp, i64, vp, i64, vp, dp, ci, vp]
     L.rdb_selftest_sync_giveup.restype = ci
     for name in ("rdb_sq5_fill_2d", "rdb_sq5_fill_1d", "rdb_materialize_fwd", "rdb_materialize_bwd", "rdb_scale_bias_bwd",
-                 "rdb_embed_fwd", "rdb_embed_bwd", "rdb_linear_fwd", "rdb_linear_bwd_dx", "rdb_linear_bwd_dx_dscale", "rdb_linear_bwd_dcoef",
+                 "rdb_embed_fwd", "rdb_embed_bwd", "rdb_linear_fwd", "rdb_linear_bwd_dx", "rdb_linear_bwd_dx_dscale", "rdb_linear_rbias_fwd",
+                 "rdb_linear_rbias_bwd", "rdb_linear_bwd_dcoef",
                  "rdb_linear_project", "rdb_linear_project_fwd", "rdb_linear_fwd_projected", "rdb_linear_bwd_dcoef_projected",
                  "rdb_linear_bwd_projected", "rdb_linear_bwd_projected_to", "rdb_linear_bwd_projected_part"):
         getattr(L, name).restype = ci

@@ -123,7 +123,7 @@ int one_launch_mode() { return __atomic_load_n(&g_one_launch, __ATOMIC_RELAXED);
 
 }  // namespace rdb
 
-extern "C" int rdb_abi_version(void) { return 7; }
+extern "C" int rdb_abi_version(void) { return 8; }
 
 extern "C" int rdb_set_one_launch(int mode)
 {

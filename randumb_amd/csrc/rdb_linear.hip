@@ -423,6 +423,8 @@ extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
         const int64_t t = linear_dx_factored_workspace(d);
         return t > 0 ? (t + 255) / 256 * 256 + linear_dx_rbias_dot_floats(d) * 4 : 0;
     }
+    if (op == RDB_OP_LINEAR_RBIAS_BWD)   // one float per tile of the random-bias product (the gradient of the scale)
+        return (d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16 && d->in_f % 8 == 0 && d->out_f % 8 == 0) ? linear_dx_rbias_dot_floats(d) * 4 : 0;
     if (op == RDB_OP_LINEAR_BWD_PROJECTED) return bwd_projected_workspace(d, false);
     if (op == RDB_OP_LINEAR_BWD_PROJECTED_TO) return bwd_projected_workspace(d, true);
     if (op == RDB_OP_LINEAR_FWD) return d->coef_dtype == RDB_BF16 ? linear_projection_bytes(d) : 0;
@@ -615,6 +617,51 @@ extern "C" int rdb_linear_bwd_dx_dscale(void *dx, int64_t lddx, float *d_scale_b
     rc = linear_dx_rbias_add_dscale(dx, lddx, d_scale_bias, dots, dy, lddy, x, ldx, scale_bias, d, s);
     if (rc == RDB_E_UNSUPPORTED) return set_error(RDB_E_UNSUPPORTED, "%s", why);
     return rc;
+}
+
+// The random-bias share on its own, on top of a result that holds the low-rank share already.
+static int rbias_request_ok(const char *who, const rdb_linear_desc *d)
+{
+    if (d->act_dtype != RDB_BF16 || d->coef_dtype != RDB_BF16 || d->coef_rows == 0 || d->in_f % 8 || d->out_f % 8)
+        return set_error(RDB_E_UNSUPPORTED, "%s: needs matrix-coef, bf16 activations and coefficients, and sizes that are multiples of 8", who);
+    return RDB_OK;
+}
+
+extern "C" int rdb_linear_rbias_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, const void *scale_bias, const rdb_linear_desc *d, void *stream)
+{
+    int rc = check_desc("rdb_linear_rbias_fwd", d);
+    if (rc) return rc;
+    if (!y || !x || !scale_bias) return set_error(RDB_E_NULL, "rdb_linear_rbias_fwd: y, x or scale_bias is NULL");
+    if (ldy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_rbias_fwd: leading dimension smaller than the row");
+    if ((rc = rbias_request_ok("rdb_linear_rbias_fwd", d))) return rc;
+    rc = linear_fwd_rbias_add(y, ldy, x, ldx, scale_bias, d, (hipStream_t)stream);
+    if (rc == RDB_E_UNSUPPORTED)
+        return set_error(RDB_E_UNSUPPORTED, "rdb_linear_rbias_fwd: needs 16-byte aligned rows (pointers and leading dimensions) and fewer than "
+                                            "2^29 elements per matrix");
+    return rc;
+}
+
+extern "C" int rdb_linear_rbias_bwd(void *dx, int64_t lddx, float *d_scale_bias, const void *dy, int64_t lddy, const void *x, int64_t ldx,
+                                    const void *scale_bias, const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    int rc = check_desc("rdb_linear_rbias_bwd", d);
+    if (rc) return rc;
+    if (!dx || !dy || !scale_bias) return set_error(RDB_E_NULL, "rdb_linear_rbias_bwd: dx, dy or scale_bias is NULL");
+    if (lddx < d->in_f || lddy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_rbias_bwd: leading dimension smaller than the row");
+    if ((rc = rbias_request_ok("rdb_linear_rbias_bwd", d))) return rc;
+    const char *why = "rdb_linear_rbias_bwd: needs 16-byte aligned rows (pointers and leading dimensions) and fewer than 2^29 elements per matrix";
+    hipStream_t s = (hipStream_t)stream;
+    if (!d_scale_bias) {
+        rc = linear_dx_rbias_add(dx, lddx, dy, lddy, scale_bias, d, s);
+        return rc == RDB_E_UNSUPPORTED ? set_error(RDB_E_UNSUPPORTED, "%s", why) : rc;
+    }
+    if (!x) return set_error(RDB_E_NULL, "rdb_linear_rbias_bwd: the gradient of the scale needs x");
+    if (ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_rbias_bwd: leading dimension smaller than the row");
+    const int64_t need = rdb_linear_workspace_bytes(RDB_OP_LINEAR_RBIAS_BWD, d);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 3))
+        return set_error(RDB_E_WORKSPACE, "rdb_linear_rbias_bwd: the gradient of the scale needs a workspace of %lld bytes", (long long)need);
+    rc = linear_dx_rbias_add_dscale(dx, lddx, d_scale_bias, static_cast<float *>(workspace), dy, lddy, x, ldx, scale_bias, d, s);
+    return rc == RDB_E_UNSUPPORTED ? set_error(RDB_E_UNSUPPORTED, "%s", why) : rc;
 }
 
 extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const void *dy, int64_t lddy, const void *x, int64_t ldx,

@@ -380,6 +380,54 @@ def linear_bwd_dx_dscale(dy: torch.Tensor, x: torch.Tensor, coef: torch.Tensor, 
     return dx, ds
 
 
+def _rbias_desc(tokens: int, in_f: int, out_f: int, seed: int) -> LinearDesc:
+    d = LinearDesc()
+    d.tokens, d.in_f, d.out_f, d.k, d.coef_rows, d.sO, d.sI, d.seed = int(tokens), int(in_f), int(out_f), 8, int(out_f), int(in_f), 1, _seed(seed)
+    d.act_dtype, d.coef_dtype, d.algo = _lib.RDB_BF16, _lib.RDB_BF16, RDB_ALGO_AUTO
+    return d
+
+
+def linear_rbias_supported(in_f: int, out_f: int, dtype) -> bool:
+    """Whether the random-bias share has kernels of its own for the layer (bf16, sizes in multiples of 8)."""
+    return dtype == torch.bfloat16 and in_f % 8 == 0 and out_f % 8 == 0
+
+
+def linear_rbias_fwd_(y: torch.Tensor, x: torch.Tensor, scale_bias: torch.Tensor, in_f: int, out_f: int, seed: int) -> torch.Tensor:
+    """In place: ``y += scale_bias * x @ R.T`` with ``R[o, i] = noise1d(o * in_f + i)``, the fused random bias of a weight
+    ``W = C.N + s.R`` (src/rten_cpp/RandumbTensor.py:286-289), on top of a ``y`` that holds the low-rank share.  bf16."""
+    _need_gpu("linear_rbias_fwd_", y, x, scale_bias)
+    x = _act(x)
+    sb = _native(scale_bias).to(torch.bfloat16)
+    d = _rbias_desc(x.shape[0], in_f, out_f, seed)
+    with _on(x.device):
+        _lib.check(_lib.load().rdb_linear_rbias_fwd(_p(y), y.stride(0), _p(x), x.stride(0), _p(sb), ctypes.byref(d), _stream(x.device)),
+                   "rdb_linear_rbias_fwd")
+    return y
+
+
+def linear_rbias_bwd_(dx: torch.Tensor, dy: torch.Tensor, x: Optional[torch.Tensor], scale_bias: torch.Tensor, in_f: int, out_f: int,
+                      seed: int, want_scale_bias_grad: bool = False) -> Optional[torch.Tensor]:
+    """In place: ``dx += scale_bias * dy @ R``; returns the gradient of the scale, ``<dy @ R, x>`` (fp32, ``(1,)``), from the same
+    pass when asked for (``x`` is needed then only)."""
+    _need_gpu("linear_rbias_bwd_", dx, dy, scale_bias)
+    dy = _act(dy)
+    sb = _native(scale_bias).to(torch.bfloat16)
+    d = _rbias_desc(dy.shape[0], in_f, out_f, seed)
+    L = _lib.load()
+    with _on(dy.device):
+        if not want_scale_bias_grad:
+            _lib.check(L.rdb_linear_rbias_bwd(_p(dx), dx.stride(0), None, _p(dy), dy.stride(0), None, 0, _p(sb), ctypes.byref(d), None, 0,
+                                              _stream(dy.device)), "rdb_linear_rbias_bwd")
+            return None
+        x = _act(x)
+        ws_bytes = int(L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_RBIAS_BWD, ctypes.byref(d)))
+        ws = _workspace(ws_bytes, dy.device)
+        ds = torch.empty((1,), dtype=torch.float32, device=dy.device)
+        _lib.check(L.rdb_linear_rbias_bwd(_p(dx), dx.stride(0), _p(ds), _p(dy), dy.stride(0), _p(x), x.stride(0), _p(sb), ctypes.byref(d),
+                                          _p(ws), ws_bytes, _stream(dy.device)), "rdb_linear_rbias_bwd")
+    return ds
+
+
 def linear_bwd_dcoef(dy: torch.Tensor, x: torch.Tensor, k: int, coef_rows: int, in_f: int, out_f: int, sO: int, sI: int,
                      seed: int, want_scale_bias_grad: bool = False, algo: int = RDB_ALGO_AUTO):
     """``(dcoef, d_scale_bias)`` in fp32: ``dcoef = (dy.T @ x) . Noise.T`` without storing ``dy.T @ x``."""

@@ -310,38 +310,48 @@ class _EagerLinear(torch.autograd.Function):
 
 
 class _ProjectedLinear(torch.autograd.Function):
-    """``y = x @ W.T (+ bias)`` for a matrix-coef weight in bf16.  The forward pass computes the projection state
-    (``z = x @ Noise.T`` in the two element orders its consumers read, and the transposed coefficients) once and saves it for
-    the backward pass in place of ``x``; the reference's autograd saves ``x`` and materialises ``W`` again
-    (RandumbTensor.py:942-946, 979-990).  Per token the state holds 4 bytes per coefficient (k rounded up to 64) where x holds
-    2 per input feature, plus once per layer a copy of the coefficients; ``linear`` takes this function only while that is at
-    most twice the size of x (``hip.linear_projection_preferred``)."""
+    """``y = x @ W.T (+ bias)`` for a matrix-coef weight in bf16 or fp32.  The forward pass computes the projection state
+    (``z = x @ Noise.T`` in the element orders its consumers read, and for bf16 the transposed coefficients) once and saves it
+    for the backward pass, which then needs nothing else of ``x``; the reference's autograd saves ``x`` and materialises ``W``
+    again (RandumbTensor.py:942-946, 979-990).  Per token the bf16 state holds 4 bytes per coefficient (k rounded up to 64)
+    where x holds 2 per input feature, plus once per layer a copy of the coefficients; ``x`` itself usually stays alive too
+    (its producer saved it), so ``linear`` takes this function only while the state is at most twice the size of x
+    (``hip.linear_projection_preferred``).  With the fused random bias (``scale_bias``, bf16, eager only) the full-rank share
+    ``s.R`` is added by kernels of its own in both directions and ``x`` is saved as well: the gradient of ``s`` is
+    ``<dy @ R, x>``."""
 
     @staticmethod
-    def forward(ctx, x, coefs, in_features, out_features, seed, bias):
+    def forward(ctx, x, coefs, in_features, out_features, seed, bias, scale_bias=None):
         # eagerly: straight to the library (the operator wrappers of torch.library cost more host time than the layer's
         # kernels take); under torch.compile: through the registered operators, which it can trace
         y, state = linear_project_fwd(x, coefs, seed, bias) if _tracing() else hip.linear_project_fwd(x, coefs, seed, _dense(bias))
-        ctx.save_for_backward(state, coefs)
+        if scale_bias is not None:
+            hip.linear_rbias_fwd_(y, x, scale_bias, in_features, out_features, seed)
+            ctx.save_for_backward(state, coefs, scale_bias, x)
+        else:
+            ctx.save_for_backward(state, coefs)
         ctx.meta = (in_features, out_features, seed)
         ctx.bias_dtype = None if bias is None else bias.dtype
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        state, coefs = ctx.saved_tensors
+        state, coefs = ctx.saved_tensors[:2]
+        scale_bias, x = ctx.saved_tensors[2:] if len(ctx.saved_tensors) == 4 else (None, None)
         in_f, out_f, seed = ctx.meta
         if dy.stride(-1) != 1 or dy.stride(0) < dy.shape[1] or dy.stride(0) % 8 or dy.data_ptr() % 16:
             dy = dy.contiguous()   # the kernels read rows with a leading dimension; anything else is copied
-        dx = dcoefs = dbias = None
+        dx = dcoefs = dbias = dsb = None
         direct = not _tracing()
-        if ctx.needs_input_grad[0] and ctx.needs_input_grad[1]:
+        want_sb = scale_bias is not None and ctx.needs_input_grad[6]
+        want_dx = ctx.needs_input_grad[0] or want_sb   # the gradient of the scale comes out of the random-bias share of dx
+        if want_dx and ctx.needs_input_grad[1]:
             if direct:   # the sums leave the kernel in the coefficients' dtype: no cast afterwards
                 dx, dcoefs = hip.linear_bwd_projected(dy, state, coefs, in_f, seed, dcoef_dtype=coefs.dtype)
             else:
                 dx, dc = linear_bwd_projected(dy, state, coefs, in_f, seed)
                 dcoefs = dc.to(coefs.dtype)
-        elif ctx.needs_input_grad[0]:
+        elif want_dx:
             dx = (hip.linear_bwd_dx(dy, coefs, in_f, out_f, in_f, 1, seed, None) if direct
                   else linear_bwd_dx(dy, coefs, in_f, out_f, in_f, 1, seed, None))
         elif ctx.needs_input_grad[1]:
@@ -351,21 +361,29 @@ class _ProjectedLinear(torch.autograd.Function):
                 dc = (hip.linear_bwd_dcoef_projected(dy, state, coefs.shape[1], in_f, seed) if direct
                       else linear_bwd_dcoef_projected(dy, state, coefs.shape[1], in_f, seed))
                 dcoefs = dc.to(coefs.dtype)
+        if scale_bias is not None and dx is not None:
+            ds = hip.linear_rbias_bwd_(dx, dy, x, scale_bias, in_f, out_f, seed, want_scale_bias_grad=want_sb)
+            if want_sb:
+                dsb = ds.to(scale_bias.dtype)
+        if not ctx.needs_input_grad[0]:
+            dx = None
         if ctx.bias_dtype is not None and ctx.needs_input_grad[5]:
             dbias = dy.sum(0).to(ctx.bias_dtype)
-        return dx, dcoefs, None, None, None, dbias
+        return dx, dcoefs, None, None, None, dbias, dsb
 
 
 def linear(x: Tensor, coefs: Tensor, in_features: int, out_features: int, stride_o: int, stride_i: int, seed: int,
            scale_bias: Optional[Tensor], bias: Optional[Tensor]) -> Tensor:
-    """``x @ W.T (+ bias)`` with autograd, choosing the projected form when the layer qualifies (matrix-coef, no fused random
-    bias; bf16 with sizes in multiples of 8, or fp32 beyond the few-token regime) and ``rten::linear_fwd`` otherwise.  Same
-    arguments as ``rten::linear_fwd``."""
-    if (scale_bias is None and coefs.dim() == 2 and coefs.shape[0] == out_features and stride_o == in_features and stride_i == 1
+    """``x @ W.T (+ bias)`` with autograd, choosing the projected form when the layer qualifies (matrix-coef; bf16 with sizes in
+    multiples of 8, or fp32 beyond the few-token regime; the fused random bias in bf16 when run eagerly) and
+    ``rten::linear_fwd`` otherwise.  Same arguments as ``rten::linear_fwd``."""
+    rbias_ok = scale_bias is None or (x.dtype == torch.bfloat16 and scale_bias.numel() == 1 and not _tracing()
+                                      and hip.linear_rbias_supported(in_features, out_features, x.dtype))
+    if (rbias_ok and coefs.dim() == 2 and coefs.shape[0] == out_features and stride_o == in_features and stride_i == 1
             and x.is_cuda and x.dim() == 2 and x.dtype in (torch.bfloat16, torch.float32) and coefs.dtype == x.dtype
             and (bias is None or bias.dtype == x.dtype)
             and hip.linear_projection_preferred(x.shape[0], in_features, out_features, coefs.shape[1], x.dtype)):
-        return _ProjectedLinear.apply(x, coefs, in_features, out_features, seed, bias)
+        return _ProjectedLinear.apply(x, coefs, in_features, out_features, seed, bias, scale_bias)
     if x.is_cuda and not _tracing():
         return _EagerLinear.apply(x, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias, bias)
     return linear_fwd(x, coefs, in_features, out_features, stride_o, stride_i, seed, scale_bias, bias)

@@ -600,6 +600,18 @@ def test_default_layer_fast_path_with_scale_bias(hip, oracle, T, in_f, out_f, k)
         assert abs(float(both[1]) - want_ds) < BF16_TOL * max(abs(want_ds), float(np.linalg.norm(dW)))
         # (the dW-tile kernel above rounds dW to bf16 before the contraction, this one reduces fp32 sums: it is the closer one)
         assert torch.equal(hip.linear_bwd_dx_dscale(dyg, xg, cg, in_f, out_f, 9, sg)[1], both[1])
+        # the random-bias share as calls of its own on top of the projected entry points (what the layer runs: z = x.N^T is formed
+        # once, by the forward pass): the same kernels in the same order as inside rdb_linear_fwd / rdb_linear_bwd_dx_dscale
+        if hip.linear_projection_supported(T, in_f, out_f, k):
+            y2, state = hip.linear_project_fwd(xg, cg, 9, None)
+            hip.linear_rbias_fwd_(y2, xg, sg, in_f, out_f, 9)
+            assert rel_l2(cpu(y2), want_y) < BF16_TOL
+            dx2, dc2 = hip.linear_bwd_projected(dyg, state, cg, in_f, 9)
+            ds2 = hip.linear_rbias_bwd_(dx2, dyg, xg, sg, in_f, out_f, 9, want_scale_bias_grad=True)
+            assert rel_l2(cpu(dx2), want_dx) < BF16_TOL and rel_l2(cpu(dc2), want_dc) < BF16_TOL
+            assert torch.equal(ds2, both[1]), "the gradient of the scale does not depend on what dx held"
+            dx3, _ = hip.linear_bwd_projected(dyg, state, cg, in_f, 9)
+            assert hip.linear_rbias_bwd_(dx3, dyg, None, sg, in_f, out_f, 9) is None and torch.equal(dx3, dx2)
         dc_only, none = hip.linear_bwd_dcoef(dyg, xg, k, out_f, in_f, out_f, in_f, 1, 9, want_scale_bias_grad=False)
         assert none is None and rel_l2(cpu(dc_only), want_dc) < BF16_TOL
         # the same input gradient from the general kernel that forms the weight block by block

@@ -204,6 +204,37 @@ def test_bf16_layer_matches_oracle(ra, oracle):
     assert l.weight_coef.grad.dtype == torch.bfloat16 and rel_l2(cpu(l.weight_coef.grad), dC) < BF16_TOL
 
 
+def test_bf16_layer_with_fused_random_bias_takes_the_projected_form(ra, oracle):
+    """The reference's default layer (fused random bias s.R on the weight, SillyLayers.py:122-133) in bf16 with non-zero
+    coefficients: the low-rank share through the projected entry points (z saved by the forward pass), the random-bias share
+    through kernels of its own in both directions, the gradient of s from the input gradient's pass; all against the oracle."""
+    print("case bf16 layer with scale_bias", flush=True)
+    g = torch.Generator().manual_seed(8)
+    in_f, out_f, k, seed, T = 512, 384, 128, 5, 640
+    l = ra.SillyLinear(in_f, out_f, [k, k], [seed, 1], bias=False, rt_bias=True, matrix_coef=True)
+    with torch.no_grad():
+        l.weight_coef.copy_(torch.randn(out_f, k, generator=g) * 0.02)
+        l.weight_scale_bias.fill_(0.0625)
+    l = l.to(torch.bfloat16).cuda()
+    x = torch.randn(T, in_f, generator=g).bfloat16().cuda().requires_grad_()
+    dy = torch.randn(T, out_f, generator=g).bfloat16().cuda()
+    y = l(x)
+    assert "ProjectedLinear" in str(y.grad_fn) or "ProjectedLinear" in str(y.grad_fn.next_functions[0][0])
+    y.backward(dy)
+    xn, dyn, Cn = cpu(x), cpu(dy), cpu(l.weight_coef)
+    assert rel_l2(cpu(y), oracle.linear_fwd(xn, Cn, in_f, out_f, seed, scale_bias=0.0625)) < BF16_TOL
+    dx, dC, dW = oracle.linear_bwd(xn, dyn, Cn, in_f, out_f, seed, scale_bias=0.0625)
+    assert rel_l2(cpu(x.grad), dx) < BF16_TOL
+    assert rel_l2(cpu(l.weight_coef.grad), dC) < BF16_TOL
+    want_ds = float(oracle.scale_bias_bwd(dW.astype(np.float32), seed)[0])
+    assert abs(float(l.weight_scale_bias.grad) - want_ds) < BF16_TOL * max(abs(want_ds), float(np.linalg.norm(dW)))
+    # only the scale wants a gradient: still computed (from the random-bias share of an input gradient nobody asked for)
+    l.zero_grad(set_to_none=True)
+    l.weight_coef.requires_grad_(False)
+    l(x.detach()).backward(dy)
+    assert abs(float(l.weight_scale_bias.grad) - want_ds) < BF16_TOL * max(abs(want_ds), float(np.linalg.norm(dW)))
+
+
 def test_conv2d_layers_match_a_dense_autograd_graph(ra, oracle):
     """Two convolution layers with pseudorandom kernels (the front of the reference's MNIST net, mnist.py:55-84) against the
     same convolutions on dense kernels built from the oracle, in fp64 on the CPU: output, input gradient, and the gradient

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_lib.SO_PATH)
     for name in declared:
         assert hasattr(lib, name), name
-    assert _lib.load().rdb_abi_version() == _lib.ABI_VERSION == 7
+    assert _lib.load().rdb_abi_version() == _lib.ABI_VERSION == 8
     assert ctypes.sizeof(_lib.LinearDesc) == 7 * 8 + 4 * 4
 
 
@@ -34,11 +34,11 @@ def test_loader_refuses_a_library_of_another_abi_version(monkeypatch):
     from randumb_amd import _lib
 
     monkeypatch.setattr(_lib, "_lib", None)
-    monkeypatch.setattr(_lib, "ABI_VERSION", 6)
-    with pytest.raises(_lib.RandumbHipError, match="ABI version 7"):
-        _lib.load()
     monkeypatch.setattr(_lib, "ABI_VERSION", 7)
-    assert _lib.load().rdb_abi_version() == 7
+    with pytest.raises(_lib.RandumbHipError, match="ABI version 8"):
+        _lib.load()
+    monkeypatch.setattr(_lib, "ABI_VERSION", 8)
+    assert _lib.load().rdb_abi_version() == 8
 
 
 def test_one_launch_switch_without_a_gpu():
