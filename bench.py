@@ -7,7 +7,7 @@ activations with fp32 accumulation, x ~ N(0,1), dy ~ N(0,1), C ~ N(0, 3*0.02^2/k
 
 A "step" is one pass of the hot path, y = x W^T, dx = dy W, dC = (dy^T x) N^T with W = C N never stored, through
 the C ABI of librandumb_hip.so with inputs already resident in HBM, the way a training step calls it:
-  forward   rdb_linear_project_fwd (z = x N^T and the transposed coefficients, kept for the backward pass in place of x,
+  forward   rdb_linear_project_fwd (z = x N^T and the transposed coefficients, kept for the backward pass,
             and y = z C^T, in one launch)
   backward  rdb_linear_bwd_projected (dx and dC from dy, the projection state and C, in two launches)
 Every buffer (inputs, outputs, projection state, workspace) is allocated before the timed region.

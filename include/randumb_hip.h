@@ -226,7 +226,8 @@ int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const void *dy, int6
  * noise directions of this layer's weight) is all that the forward product and the coefficient gradient need of x:
  *   y = z . C^T (+ bias)        dcoef = dy^T . z
  * rdb_linear_fwd and rdb_linear_bwd_dcoef compute z into their workspace on every call.  A training step can instead
- * compute it once, keep it from the forward to the backward pass in place of x and call the consumers below.  Replaces,
+ * compute it once, keep it from the forward to the backward pass (the backward pass then needs nothing else of x; whether x
+ * itself can be freed depends on who else holds it) and call the consumers below.  fp32 layers likewise, with z in fp32.  Replaces,
  * like rdb_linear_fwd / rdb_linear_bwd_dcoef, materialize() + dense product (R.py:942-952) and MmBackward's dW followed by
  * materialize_bwd (R.py:979-990, 304-359); the tensor autograd saves for the backward pass (there: x, with W
  * re-materialised) becomes the projection state.

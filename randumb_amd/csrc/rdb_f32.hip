@@ -618,7 +618,7 @@ int linear_dcoef_f32(float *dcoef, float *d_scale_bias, const void *dy, int64_t 
 }
 
 // ----------------------------------------------------------------------------------------------- projected form in fp32
-// What a training step keeps from the forward to the backward pass in place of x: z = x . N^T in fp32, [tokens x k] row-major,
+// What a training step keeps from the forward to the backward pass (all that the latter needs of x): z = x . N^T in fp32, [tokens x k] row-major,
 // behind a 256-byte header (the same role as the bf16 state of rdb_direct.hpp; no fragment orders, no transposed copies: these
 // kernels stage both operands through LDS).  fp32 activations and coefficients, one launch's worth of tokens.
 static bool fg_state_ok(const rdb_linear_desc *d)

@@ -516,7 +516,7 @@ def linear_projection_supported(tokens: int, in_f: int, out_f: int, k: int, dtyp
 
 
 def linear_projection_preferred(tokens: int, in_f: int, out_f: int, k: int, dtype=torch.bfloat16) -> bool:
-    """Whether a training step should save the projection state in place of ``x``.  Two conditions.  Speed: the factored
+    """Whether a training step should save the projection state for its backward pass.  Two conditions.  Speed: the factored
     products need 2*tokens*k*(in_f + out_f) flops per direction, a product on a stored weight 2*tokens*in_f*out_f; the kernels
     that form the weight on chip instead lose against the factored ones up to at least 8 times that (measured), so the bound
     is 16 times, as in the library.  Memory: the state holds z twice (two element orders), 2 * 2 * k bytes per token with k

@@ -238,7 +238,7 @@ def test_projected_form_in_fp32(hip, oracle, T, in_f, out_f, k, seed):
 
 
 def test_fp32_layer_takes_the_projected_form(hip, oracle):
-    """SillyLinear in fp32 beyond the few-token regime saves z instead of x (ops.linear's choice) and matches the oracle."""
+    """SillyLinear in fp32 beyond the few-token regime saves z for the backward pass (ops.linear's choice) and matches the oracle."""
     import randumb_amd as ra
     from randumb_amd import ops
 

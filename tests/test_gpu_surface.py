@@ -194,7 +194,7 @@ def test_bf16_layer_matches_oracle(ra, oracle):
     dy = torch.randn(4, T // 4, out_f, generator=g).bfloat16().cuda()
     y = l(x)
     assert y.shape == (4, T // 4, out_f) and y.dtype == torch.bfloat16
-    # a matrix-coef bf16 layer without the fused random bias takes the projected form: z = x.N^T saved instead of x
+    # a matrix-coef bf16 layer without the fused random bias takes the projected form: z = x.N^T saved for the backward pass
     assert "ProjectedLinear" in str(y.grad_fn.next_functions[0][0])
     y.backward(dy)
     xn, dyn, Cn = cpu(x).reshape(T, in_f), cpu(dy).reshape(T, out_f), cpu(l.weight_coef)
