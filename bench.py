@@ -407,6 +407,48 @@ def other_configs(event_ms, torch, L, _lib, dev):
     return out
 
 
+def rbias_layer_config(event_ms, torch, L, _lib, dev, main_set):
+    # the reference's default layer: W = C.N + s.noise1d (zero coefficients and a fused random bias at initialisation).
+    # What SillyLinear runs: the low-rank share through the projected calls of the headline step (z = x.N^T formed once, by
+    # the forward pass), the full-rank random-bias share through kernels of its own on top (rdb_linear_rbias_fwd / _bwd,
+    # the latter also reducing d s = <dy.R, x>).  Beside it the one-call entry points (z formed by the forward and again
+    # by the coefficient gradient) and the older split with dcoef and d s from dW tiles.
+    p, ws_bytes, stream = main_set.p, main_set.ws_bytes, main_set.stream
+    sb = torch.tensor([0.02], device=dev).bfloat16()
+    ds = torch.empty(1, dtype=torch.float32, device=dev)
+    psb, pds, r = ctypes.c_void_p(sb.data_ptr()), ctypes.c_void_p(ds.data_ptr()), main_set.dref
+    n_ds = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX_DSCALE, r)
+    ws_ds = torch.empty(max(n_ds, 16), dtype=torch.uint8, device=dev)
+    pws_ds = ctypes.c_void_p(ws_ds.data_ptr())
+    n_rb = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_RBIAS_BWD, r)
+    ws_rb = torch.empty(max(n_rb, 16), dtype=torch.uint8, device=dev)
+    pws_rb = ctypes.c_void_p(ws_rb.data_ptr())
+
+    def fwd_projected():
+        main_set.project_fwd()
+        _lib.check(L.rdb_linear_rbias_fwd(p["y"], OUT_F, p["x"], IN_F, psb, r, stream), "rdb_linear_rbias_fwd")
+
+    def bwd_projected():
+        main_set.bwd()
+        _lib.check(L.rdb_linear_rbias_bwd(p["dx"], IN_F, pds, p["dy"], OUT_F, p["x"], IN_F, psb, r, pws_rb, n_rb, stream), "rdb_linear_rbias_bwd")
+
+    fwd = lambda: _lib.check(L.rdb_linear_fwd(p["y"], OUT_F, p["x"], IN_F, p["C"], psb, None, r, p["ws"], ws_bytes, stream), "rdb_linear_fwd")
+    dxs = lambda: _lib.check(L.rdb_linear_bwd_dx_dscale(p["dx"], IN_F, pds, p["dy"], OUT_F, p["x"], IN_F, p["C"], psb, r, pws_ds, n_ds, stream),
+                             "rdb_linear_bwd_dx_dscale")
+    dco = lambda: _lib.check(L.rdb_linear_bwd_dcoef(p["dC"], None, p["dy"], OUT_F, p["x"], IN_F, r, p["ws"], ws_bytes, stream),
+                             "rdb_linear_bwd_dcoef")
+    dxf = lambda: _lib.check(L.rdb_linear_bwd_dx(p["dx"], IN_F, p["dy"], OUT_F, p["C"], psb, r, p["ws"], ws_bytes, stream), "rdb_linear_bwd_dx")
+    dcf = lambda: _lib.check(L.rdb_linear_bwd_dcoef(p["dC"], pds, p["dy"], OUT_F, p["x"], IN_F, r, p["ws"], ws_bytes, stream),
+                             "rdb_linear_bwd_dcoef")
+    t = {"fwd": round(event_ms(fwd_projected, 100), 4), "bwd_with_dscale": round(event_ms(bwd_projected, 100), 4)}
+    t["step"] = round(sum(t.values()), 4)
+    o = {"fwd": round(event_ms(fwd, 20), 4), "dx_and_dscale": round(event_ms(dxs, 20), 4), "dcoef": round(event_ms(dco, 20), 4)}
+    o["step"] = round(sum(o.values()), 4)
+    t["one_call_entry_points"] = o
+    t["with_dscale_from_dw_tiles"] = {"dx": round(event_ms(dxf, 20), 4), "dcoef_and_dscale": round(event_ms(dcf, 20), 4)}
+    return t
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -422,6 +464,8 @@ def main():
                          "(profiling runs)")
     ap.add_argument("--f32-layer-only", action="store_true",
                     help="time only the fp32 form of the headline layer (profiling runs)")
+    ap.add_argument("--rbias-layer-only", action="store_true",
+                    help="run only the headline layer with the fused random bias (projected calls + random-bias share) and exit")
     ap.add_argument("--smallk-only", action="store_true",
                     help="run only the fp32 4096 -> 4096, k = 16 forward at batch 1 / 16 / 256 and exit (profiling runs)")
     ap.add_argument("--gpt-only", action="store_true",
@@ -473,6 +517,11 @@ def main():
         print(json.dumps({"in4096_out14336_k1024_T4096_bf16": llm_layer_config(make_event_ms(torch), torch, L, _lib, dev, g, vendor=False)}))
         return
     main_set = LayerBuffers(L, _lib, torch, dev, g)
+    if args.rbias_layer_only:
+        for _ in range(SETTLE_STEPS):   # clocks settle
+            main_set.step()
+        print(json.dumps({"layer_with_fused_random_bias_ms": rbias_layer_config(make_event_ms(torch), torch, L, _lib, dev, main_set)}))
+        return
     sets = [main_set] + [LayerBuffers(L, _lib, torch, dev, g, share_inputs_of=main_set) for _ in range(2)]
     set_mb = sum(t.numel() * t.element_size() for t in (main_set.x, main_set.dy, main_set.y, main_set.dx, main_set.dC, main_set.ws,
                                                        main_set.state, main_set.C)) / 1e6
@@ -655,46 +704,6 @@ def main():
             return {"fwd_strip": t["fwd"], "dx_noise_strip": t["dx"], "dcoef_dw_tile": t["dcoef"],
                     "step": round(t["fwd"] + t["dx"] + t["dcoef"], 4), "dx_tile": onecall_ms(_lib.RDB_ALGO_TILE)["dx"]}
 
-        def scale_bias_ms():
-            # the reference's default layer: W = C.N + s.noise1d (zero coefficients and a fused random bias at initialisation).
-            # What SillyLinear runs: the low-rank share through the projected calls of the headline step (z = x.N^T formed once, by
-            # the forward pass), the full-rank random-bias share through kernels of its own on top (rdb_linear_rbias_fwd / _bwd,
-            # the latter also reducing d s = <dy.R, x>).  Beside it the one-call entry points (z formed by the forward and again
-            # by the coefficient gradient) and the older split with dcoef and d s from dW tiles.
-            sb = torch.tensor([0.02], device=dev).bfloat16()
-            ds = torch.empty(1, dtype=torch.float32, device=dev)
-            psb, pds, r = ctypes.c_void_p(sb.data_ptr()), ctypes.c_void_p(ds.data_ptr()), main_set.dref
-            n_ds = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX_DSCALE, r)
-            ws_ds = torch.empty(max(n_ds, 16), dtype=torch.uint8, device=dev)
-            pws_ds = ctypes.c_void_p(ws_ds.data_ptr())
-            n_rb = L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_RBIAS_BWD, r)
-            ws_rb = torch.empty(max(n_rb, 16), dtype=torch.uint8, device=dev)
-            pws_rb = ctypes.c_void_p(ws_rb.data_ptr())
-
-            def fwd_projected():
-                main_set.project_fwd()
-                _lib.check(L.rdb_linear_rbias_fwd(p["y"], OUT_F, p["x"], IN_F, psb, r, stream), "rdb_linear_rbias_fwd")
-
-            def bwd_projected():
-                main_set.bwd()
-                _lib.check(L.rdb_linear_rbias_bwd(p["dx"], IN_F, pds, p["dy"], OUT_F, p["x"], IN_F, psb, r, pws_rb, n_rb, stream), "rdb_linear_rbias_bwd")
-
-            fwd = lambda: _lib.check(L.rdb_linear_fwd(p["y"], OUT_F, p["x"], IN_F, p["C"], psb, None, r, p["ws"], ws_bytes, stream), "rdb_linear_fwd")
-            dxs = lambda: _lib.check(L.rdb_linear_bwd_dx_dscale(p["dx"], IN_F, pds, p["dy"], OUT_F, p["x"], IN_F, p["C"], psb, r, pws_ds, n_ds, stream),
-                                     "rdb_linear_bwd_dx_dscale")
-            dco = lambda: _lib.check(L.rdb_linear_bwd_dcoef(p["dC"], None, p["dy"], OUT_F, p["x"], IN_F, r, p["ws"], ws_bytes, stream),
-                                     "rdb_linear_bwd_dcoef")
-            dxf = lambda: _lib.check(L.rdb_linear_bwd_dx(p["dx"], IN_F, p["dy"], OUT_F, p["C"], psb, r, p["ws"], ws_bytes, stream), "rdb_linear_bwd_dx")
-            dcf = lambda: _lib.check(L.rdb_linear_bwd_dcoef(p["dC"], pds, p["dy"], OUT_F, p["x"], IN_F, r, p["ws"], ws_bytes, stream),
-                                     "rdb_linear_bwd_dcoef")
-            t = {"fwd": round(event_ms(fwd_projected, 20), 4), "bwd_with_dscale": round(event_ms(bwd_projected, 20), 4)}
-            t["step"] = round(sum(t.values()), 4)
-            o = {"fwd": round(event_ms(fwd, 20), 4), "dx_and_dscale": round(event_ms(dxs, 20), 4), "dcoef": round(event_ms(dco, 20), 4)}
-            o["step"] = round(sum(o.values()), 4)
-            t["one_call_entry_points"] = o
-            t["with_dscale_from_dw_tiles"] = {"dx": round(event_ms(dxf, 20), 4), "dcoef_and_dscale": round(event_ms(dcf, 20), 4)}
-            return t
-
         def python_surface_ms():
             # the same layer through the drop-in surface: SillyLinear (autograd function, ctypes binding), host clock per forward +
             # backward with the GPU kept busy; what a model built from the layer pays per layer when the host is the limit
@@ -723,7 +732,7 @@ def main():
         compare = {
             "one_call_entry_points_ms": onecall_ms(_lib.RDB_ALGO_AUTO),
             "python_surface_SillyLinear_fwd_bwd_wall_ms": python_surface_ms(),
-            "layer_with_fused_random_bias_ms": scale_bias_ms(),
+            "layer_with_fused_random_bias_ms": rbias_layer_config(event_ms, torch, L, _lib, dev, main_set),
             "w_tiles_formed_on_chip_ms": strip_ms(),
             "vendor_gemm_on_the_factored_shapes_ms": vendor_skinny(),
             "materialize_then_gemm_ms": round(event_ms(mat_gemm_step, 10), 4),
