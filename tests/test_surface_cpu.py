@@ -194,6 +194,17 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     # operand size limit: then it stays [tokens x k]
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(desc(1000, 200, 328, 72))) == 1024 * 128 * 2
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(desc((1 << 26) - 8, 768, 3072, 8))) == ((1 << 26) - 8) * 8 * 2
+    # the random-bias share on its own: one float per tile of 64 features x 256 tokens for the scale's gradient; argument checks
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_RBIAS_BWD, r) == (768 // 64) * (8192 // 256) * 4
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_RBIAS_BWD, ctypes.byref(desc(8192, 768, 3072, 256, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 0
+    assert L.rdb_linear_rbias_fwd(None, 3072, None, 768, None, r, None) == -1
+    fake = ctypes.c_void_p(256)   # never dereferenced: the calls below are refused before any launch
+    assert L.rdb_linear_rbias_fwd(fake, 3071, fake, 768, fake, r, None) == -2
+    assert L.rdb_linear_rbias_fwd(fake, 3072, fake, 768, fake, ctypes.byref(desc(8192, 768, 3072, 256, act=_lib.RDB_F32, coef=_lib.RDB_F32)), None) == -5
+    assert L.rdb_linear_rbias_bwd(fake, 776, None, fake, 3072, None, 0, fake, ctypes.byref(desc(8192, 772, 3072, 256)), None, 0, None) == -5
+    ds = ctypes.c_void_p(512)
+    assert L.rdb_linear_rbias_bwd(fake, 768, ds, fake, 3072, None, 0, fake, r, None, 0, None) == -1          # d s needs x
+    assert L.rdb_linear_rbias_bwd(fake, 768, ds, fake, 3072, fake, 768, fake, r, None, 0, None) == -6    # ... and scratch
     # kernels that form W tiles need no scratch; neither does a layer the factored form does not apply to
     for algo in (_lib.RDB_ALGO_TILE, _lib.RDB_ALGO_STRIP):
         assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(8192, 768, 3072, 256, algo=algo))) == 0
@@ -407,3 +418,8 @@ def test_projected_form_is_chosen_only_where_it_runs_and_pays():
     assert hip.linear_projection_preferred(4096, 4096, 14336, 1024) and hip.linear_projection_preferred(300, 1032, 2056, 512)
     assert hip.linear_projection_supported(512, 256, 1024, 512) and not hip.linear_projection_preferred(512, 256, 1024, 512)
     assert not hip.linear_projection_preferred(64, 8, 8, 8)
+    # the fused random bias has kernels of its own beside the projected calls in bf16 with sizes in multiples of 8 only
+    import torch
+
+    assert hip.linear_rbias_supported(768, 3072, torch.bfloat16) and not hip.linear_rbias_supported(768, 3072, torch.float32)
+    assert not hip.linear_rbias_supported(772, 3072, torch.bfloat16) and not hip.linear_rbias_supported(768, 3076, torch.bfloat16)
