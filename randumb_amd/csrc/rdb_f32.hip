@@ -65,13 +65,35 @@ struct FgParams {
     float *dot_part;            // FG_DOT: one value per block, in block order (x fastest, then y)
 };
 
+// fp32 products on the bf16 matrix cores.  v = h + m + l exactly, each part a bf16 (the top 8 bits of what is left: truncation,
+// so every difference is exact); a product a . b is then the sum of the nine products of the parts, each exact in the matrix
+// core's fp32 accumulation, and the six largest of them, ah bh + ah bm + am bh + ah bl + al bh + am bm, leave out less than
+// 2^-23 |a b|: an fp32 product's own rounding.  Six bf16 matrix instructions of 32 x 32 x 16 do the work of eight fp32 ones of
+// 32 x 32 x 2 in 3/8 of the time.  (An infinite input becomes NaN: inf - inf.)  The parts come back as fp32 bit patterns with
+// the low half zero.
+__device__ __forceinline__ void fg_split3(float v, uint32_t &h, uint32_t &m, uint32_t &l)
+{
+    h = __float_as_uint(v) & 0xffff0000u;
+    const float r1 = v - __uint_as_float(h);
+    m = __float_as_uint(r1) & 0xffff0000u;
+    const float r2 = r1 - __uint_as_float(m);
+    l = __float_as_uint(r2) & 0xffff0000u;
+}
+
 // One operand's way from its source into LDS: load(stage) requests / hashes the stage's values into registers, store() puts
 // them into a tile.  Rows past `rows` and contraction values past `kend` are zeros.
 // VEC: the matrix is read in 16-byte pieces (16-byte aligned base, leading dimension a multiple of 4, and the extent that
 // runs along a piece a multiple of 4, so that a piece lies inside or outside as a whole); otherwise value by value.
-template <int ROWS, int SRC, bool VEC> struct FgOperand {
+// SPLIT: the tile goes to LDS as three bf16 planes (see fg_split3): planes of [2 halves of the stage's 16 contraction values]
+// [rows][8] for the sources read along the contraction (a lane's MFMA operand is 16 consecutive bytes), of [16][rows + 32] for
+// FG_MCONT (read back with the LDS transpose read).  The noise sources then give a thread consecutive contraction values.
+template <int ROWS, int SRC, bool VEC, bool SPLIT = false> struct FgOperand {
     static constexpr int LD = ROWS + 4, TILE = FG_BK * LD, NV = ROWS * FG_BK / FG_THREADS / 4;   // float4 per thread and stage
     static_assert(NV >= 1, "a stage is at least one float4 per thread");
+    static constexpr int LDM = ROWS + 32;                                            // FG_MCONT plane: elements per contraction value
+    static constexpr int PLANE = SRC == FG_MCONT ? FG_BK * LDM : 2 * ROWS * 8;       // bf16 elements of one plane
+    static constexpr int TILE_BYTES = SPLIT ? 3 * PLANE * 2 : TILE * 4;
+    static constexpr int KPT = NV * 4;                                               // SPLIT, noise: consecutive contraction values per thread
     __amdgpu_buffer_rsrc_t rs;
     uint32_t off[NV];   // byte offset of the thread's pieces at stage 0
     bool ok[NV];        // ... and whether the piece's (first) row exists
@@ -121,7 +143,7 @@ template <int ROWS, int SRC, bool VEC> struct FgOperand {
             kk0 = t / (ROWS / 4);
         } else {
             const int row = t % ROWS;
-            kk0 = t / ROWS;
+            kk0 = SPLIT ? (t / ROWS) * KPT : t / ROWS;
             row_ok = row0 + row < rows;
             if (SRC == FG_NOISE_1D) {
                 first = ((uint32_t)(row0 + row) * sR + (uint32_t)(k_begin + kk0) * sK) * SQ5_N1 + seed;
@@ -170,7 +192,7 @@ template <int ROWS, int SRC, bool VEC> struct FgOperand {
     static constexpr bool HASHED = SRC == FG_NOISE_M || SRC == FG_NOISE_I || SRC == FG_NOISE_1D;
     __device__ __forceinline__ void hash_piece(int stage, int j)
     {
-        constexpr int KSTEP = FG_THREADS / ROWS;
+        constexpr int KSTEP = SPLIT ? 1 : FG_THREADS / ROWS;
         const uint32_t f = first + (uint32_t)(stage * FG_BK + j * KSTEP) * inc;
         const bool in = row_ok && k_begin + stage * FG_BK + kk0 + j * KSTEP < kend;
         r[j >> 2][j & 3] = in ? sq5_unit(sq5_tail(f)) : 0.0f;
@@ -198,16 +220,65 @@ template <int ROWS, int SRC, bool VEC> struct FgOperand {
             for (int j = 0; j < NV * 4; ++j) tile[(kk0 + j * KSTEP) * LD + row] = r[j >> 2][j & 3];
         }
     }
+    // SPLIT: four of the thread's values into the three planes, 8 bytes each, at element offset `at` of a plane
+    __device__ __forceinline__ void put4(bf16_t *__restrict__ tile, int at, const f32x4 &v) const
+    {
+        uint32_t h[4], m[4], l[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) fg_split3(v[j], h[j], m[j], l[j]);
+        *reinterpret_cast<uint2 *>(tile + at) = make_uint2(h[1] | (h[0] >> 16), h[3] | (h[2] >> 16));
+        *reinterpret_cast<uint2 *>(tile + PLANE + at) = make_uint2(m[1] | (m[0] >> 16), m[3] | (m[2] >> 16));
+        *reinterpret_cast<uint2 *>(tile + 2 * PLANE + at) = make_uint2(l[1] | (l[0] >> 16), l[3] | (l[2] >> 16));
+    }
+    __device__ __forceinline__ void store_split(bf16_t *__restrict__ tile) const
+    {
+        const int t = threadIdx.x;
+        if (SRC == FG_KCONT) {
+#pragma unroll
+            for (int h = 0; h < NV; ++h) {   // contraction values 4 kq .. 4 kq + 3 of a row
+                const int idx = h * FG_THREADS + t, row = idx >> 2, kq = idx & 3;
+                put4(tile, ((kq >> 1) * ROWS + row) * 8 + (kq & 1) * 4, r[h]);
+            }
+        } else if (SRC == FG_MCONT) {
+#pragma unroll
+            for (int h = 0; h < NV; ++h) {   // four consecutive rows at one contraction value
+                const int idx = h * FG_THREADS + t, kk = idx / (ROWS / 4), r4 = (idx % (ROWS / 4)) * 4;
+                put4(tile, kk * LDM + r4, r[h]);
+            }
+        } else {
+            const int row = t % ROWS;
+#pragma unroll
+            for (int h = 0; h < NV; ++h) {   // contraction values kk0 + 4 h .. + 3 of a row
+                const int kk = kk0 + 4 * h;
+                put4(tile, ((kk >> 3) * ROWS + row) * 8 + (kk & 7), r[h]);
+            }
+        }
+    }
+    // SPLIT: the MFMA operand of the 32 rows from rb of one plane: lane (r, g) gets contraction values 8 g .. 8 g + 7 of row rb + r
+    __device__ static __forceinline__ bf16x8 frag(const bf16_t *__restrict__ plane, int rb, int lane)
+    {
+        const int r = lane & 31, g = lane >> 5;
+        if (SRC != FG_MCONT) return *reinterpret_cast<const bf16x8 *>(plane + (g * ROWS + rb + r) * 8);
+        // 16-lane group q covers rows rb + 16 q .. + 15; source lane s of the group addresses contraction value 8 g + s / 4,
+        // rows 4 (s % 4) .. + 3; result lane c receives the rows' column c for four contraction values
+        Frag8 f;
+        const int sl = lane & 15, q = (lane >> 4) & 1;
+        const bf16_t *src = plane + (g * 8 + (sl >> 2)) * LDM + rb + q * 16 + (sl & 3) * 4;
+        f.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(src));
+        f.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(src + 4 * LDM));
+        return f.v;
+    }
 };
 
 // out[M x N] (+)= A . B^T over one split of the contraction.  Block: BM x 128 of the output, four waves as 2 x 2, a wave owns
 // (BM / 2) x 64 in BM / 64 x 2 accumulator tiles.  Two LDS buffers, one barrier per stage: while a stage is multiplied the
 // next one is on its way from memory (or being hashed) in registers.
-template <int BM, int ASRC, int BSRC, int EPI, bool VEC> __global__ __launch_bounds__(FG_THREADS, 2) void f32_gemm_kernel(FgParams p)
+template <int BM, int ASRC, int BSRC, int EPI, bool VEC, bool SPLIT = false>
+__global__ __launch_bounds__(FG_THREADS, 2) void f32_gemm_kernel(FgParams p)
 {
-    typedef FgOperand<BM, ASRC, VEC> PA;
-    typedef FgOperand<FG_BN, BSRC, VEC> PB;
-    constexpr int MI = BM / 64, NI = 2, STAGE = PA::TILE + PB::TILE;
+    typedef FgOperand<BM, ASRC, VEC, SPLIT> PA;
+    typedef FgOperand<FG_BN, BSRC, VEC, SPLIT> PB;
+    constexpr int MI = BM / 64, NI = 2, STAGE = (PA::TILE_BYTES + PB::TILE_BYTES) / 4;   // floats
     __shared__ __align__(16) float lds[2 * STAGE];
     const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 31, g = lane >> 5, wm = wave >> 1, wn = wave & 1;
     const int m0 = blockIdx.x * BM, n0 = blockIdx.y * FG_BN;   // the long extent (tokens, as a rule) on the grid's x
@@ -227,14 +298,57 @@ template <int BM, int ASRC, int BSRC, int EPI, bool VEC> __global__ __launch_bou
     pa.load(0);
     pb.load(0);
     for (int s = 0; s < nstage; ++s) {
-        float *As = lds + (s & 1) * STAGE, *Bs = As + PA::TILE;
-        pa.store(As);
-        pb.store(Bs);
+        float *As = lds + (s & 1) * STAGE, *Bs = As + PA::TILE_BYTES / 4;
+        if (SPLIT) {
+            pa.store_split(reinterpret_cast<bf16_t *>(As));
+            pb.store_split(reinterpret_cast<bf16_t *>(Bs));
+        } else {
+            pa.store(As);
+            pb.store(Bs);
+        }
         __syncthreads();   // also: every wave is done reading the other buffer (the stage before this one)
         const bool more = s + 1 < nstage;
         if (more) {
             if (!PA::HASHED) pa.load(s + 1);
             if (!PB::HASHED) pb.load(s + 1);
+        }
+        if (SPLIT) {
+            // the stage is one k-step of the bf16 matrix instruction: three planes a side, six products a tile pair, the small
+            // ones first; the next stage's noise values are hashed between the tile pairs
+            const bf16_t *ap = reinterpret_cast<const bf16_t *>(As), *bp = reinterpret_cast<const bf16_t *>(Bs);
+            bf16x8 fa[MI][3], fb[NI][3];
+#pragma unroll
+            for (int pl = 0; pl < 3; ++pl) {
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi) fa[mi][pl] = PA::frag(ap + pl * PA::PLANE, wm * (BM / 2) + mi * 32, lane);
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni) fb[ni][pl] = PB::frag(bp + pl * PB::PLANE, wn * 64 + ni * 32, lane);
+            }
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni) {
+                    f32x16 c = acc[mi][ni];
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][1], fb[ni][1], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][2], fb[ni][0], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][0], fb[ni][2], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][1], fb[ni][0], c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][0], fb[ni][1], c, 0, 0, 0);
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][0], fb[ni][0], c, 0, 0, 0);
+                    constexpr int GROUPS = MI * NI;
+                    const int grp = mi * NI + ni;
+                    if (PB::HASHED && more) {
+                        constexpr int PER = (PB::NV * 4 + GROUPS - 1) / GROUPS;
+#pragma unroll
+                        for (int j = grp * PER; j < (grp + 1) * PER && j < PB::NV * 4; ++j) pb.hash_piece(s + 1, j);
+                    }
+                    if (PA::HASHED && more) {
+                        constexpr int PER = (PA::NV * 4 + GROUPS - 1) / GROUPS;
+#pragma unroll
+                        for (int j = grp * PER; j < (grp + 1) * PER && j < PA::NV * 4; ++j) pa.hash_piece(s + 1, j);
+                    }
+                }
+            continue;
         }
         const float *ap = As + g * PA::LD + wm * (BM / 2) + r, *bp = Bs + g * PB::LD + wn * 64 + r;
 #pragma unroll
@@ -395,6 +509,17 @@ int64_t linear_f32_workspace(int op, const rdb_linear_desc *d, int num_cus)
     return with_parts(d->in_f) + (r > 1 ? (int64_t)r * up256(d->out_f * d->k * 4) : 0) + up256(cdiv(d->tokens, 64) * cdiv(d->out_f, FG_BN) * 4);
 }
 
+// 1 (default): the linear layers' products run as six bf16 matrix instructions on three-way splits of their operands
+// (fg_split3); 0: as fp32 matrix instructions.  Process-wide (rdb_set_f32_split).
+static int g_f32_split = 1;
+int f32_split_mode() { return g_f32_split; }
+int set_f32_split_mode(int mode)
+{
+    const int old = g_f32_split;
+    g_f32_split = mode ? 1 : 0;
+    return old;
+}
+
 struct FgProduct {
     const float *a;
     int64_t lda, a_elems;
@@ -416,12 +541,18 @@ struct FgProduct {
     float *dot_part;
     // bytes per element of the A and B matrices (2: bf16), and whether out / bias / dotm and scale are bf16
     int a_es = 4, b_es = 4, out_bf16 = 0, scale_bf16 = 0;
+    // the products as six bf16 matrix instructions on three-way splits of the operands (fg_split3); materialising stays on the
+    // fp32 matrix instructions (its unit-coefficient results are compared bit for bit)
+    bool split = f32_split_mode() != 0;
 };
 
-#define FG_LAUNCH(BM_, EPI_)                                                                      \
-    do {                                                                                          \
-        if (vec) f32_gemm_kernel<BM_, ASRC, BSRC, EPI_, true><<<grid, FG_THREADS, 0, s>>>(p);     \
-        else f32_gemm_kernel<BM_, ASRC, BSRC, EPI_, false><<<grid, FG_THREADS, 0, s>>>(p);        \
+#define FG_LAUNCH(BM_, EPI_)                                                                                  \
+    do {                                                                                                      \
+        if (q.split) {                                                                                        \
+            if (vec) f32_gemm_kernel<BM_, ASRC, BSRC, EPI_, true, true><<<grid, FG_THREADS, 0, s>>>(p);       \
+            else f32_gemm_kernel<BM_, ASRC, BSRC, EPI_, false, true><<<grid, FG_THREADS, 0, s>>>(p);          \
+        } else if (vec) f32_gemm_kernel<BM_, ASRC, BSRC, EPI_, true><<<grid, FG_THREADS, 0, s>>>(p);          \
+        else f32_gemm_kernel<BM_, ASRC, BSRC, EPI_, false><<<grid, FG_THREADS, 0, s>>>(p);                    \
     } while (0)
 template <int ASRC, int BSRC> static int fg_launch(const FgProduct &q, int num_cus, hipStream_t s, const char *name)
 {
@@ -712,7 +843,7 @@ int materialize_mat_f32(float *out, const void *coef, int coef_dtype, int64_t co
                        fg_plan(coef_rows, row_len, k, num_cus, k, 1).bm, 0, 0, seed, (uint32_t)row_len, 1u, (const float *)scale_bias, nullptr, 0, nullptr};
         q.a_es = fg_es(coef_dtype);
         q.scale_bf16 = coef_dtype == RDB_BF16;
-        return fg_launch<FG_KCONT, FG_NOISE_I>(q, num_cus, s, "f32_gemm_kernel (W = C . N)");
+            return fg_launch<FG_KCONT, FG_NOISE_I>(q, num_cus, s, "f32_gemm_kernel (W = C . N)");
     }
     // W^T[i, o]: rows = i hashed, columns = o from C; the random bias at index o * row_len + i
     FgProduct q = {nullptr, 0, 0, C, k, coef_rows * k, out, coef_rows, nullptr, row_len, coef_rows, k,
