@@ -233,9 +233,11 @@ def llm_layer_config(event_ms, torch, L, _lib, dev, g, vendor=True):
 
 
 def f32_layer_config(event_ms, torch, L, _lib, dev, g, compare=True):
-    """The headline layer in fp32 (768 -> 3072, k = 256, 8192 tokens): the three one-call entry points on the fp32 matrix cores,
-    every buffer allocated beforehand.  Fractions are on the flops the kernels execute (each call forms its own z or t),
-    against the fp32 matrix peak."""
+    """The headline layer in fp32 (768 -> 3072, k = 256, 8192 tokens) through the projected calls and through the three one-call
+    entry points, every buffer allocated beforehand.  The products run on the bf16 matrix cores on exact three-way splits of
+    their fp32 operands (six bf16 matrix instructions for an fp32 product, rdb_set_f32_split); beside them the same calls on
+    the fp32 matrix instructions.  "executed" flops are the fp32 products the calls perform; the matrix cores execute six
+    times as many bf16 flops."""
     vp = ctypes.c_void_p
     stream = vp(torch.cuda.current_stream().cuda_stream)
     Tl, in_f, out_f, k = T, IN_F, OUT_F, K
@@ -277,18 +279,27 @@ def f32_layer_config(event_ms, torch, L, _lib, dev, g, compare=True):
     p_bwd = lambda: _lib.check(L.rdb_linear_bwd_projected(pdx, in_f, pdC, pdy, out_f, pst, pC, r, pws, wsb, stream), "rdb_linear_bwd_projected")
     tp_fwd, tp_bwd = event_ms(p_fwd, 50), event_ms(p_bwd, 50)
     ms = tp_fwd + tp_bwd
+    before = L.rdb_set_f32_split(0)   # the same two calls on the fp32 matrix instructions
+    tf_fwd, tf_bwd = event_ms(p_fwd, 50), event_ms(p_bwd, 50)
+    L.rdb_set_f32_split(before)
     executed = 2 * proj + 3 * prod
     ms_one = t_fwd + t_dx + t_dc
     res = {
         "calls_ms": {"rdb_linear_project_fwd": round(tp_fwd, 4), "rdb_linear_bwd_projected": round(tp_bwd, 4)},
         "fwd_bwd_ms": round(ms, 4), "executed_gflop": round(executed / 1e9, 1), "executed_TFLOPs": round(executed / ms / 1e9, 1),
-        "executed_frac_of_f32_mfma_peak": round(executed / ms / 1e9 / MFMA_F32_PEAK_TFLOPS, 4),
+        "ratio_to_f32_matrix_instruction_peak": round(executed / ms / 1e9 / MFMA_F32_PEAK_TFLOPS, 4),
+        "bf16_matrix_instruction_TFLOPs": round(6 * executed / ms / 1e9, 1),
+        "bf16_matrix_instruction_frac_of_peak": round(6 * executed / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4),
         "prescribed_TFLOPs_equivalent": round(F_STEP / ms / 1e9, 1),
+        "on_fp32_matrix_instructions_ms": {"rdb_linear_project_fwd": round(tf_fwd, 4), "rdb_linear_bwd_projected": round(tf_bwd, 4),
+                                           "fwd_bwd_ms": round(tf_fwd + tf_bwd, 4),
+                                           "frac_of_f32_mfma_peak": round(executed / (tf_fwd + tf_bwd) / 1e9 / MFMA_F32_PEAK_TFLOPS, 4)},
         "one_call_entry_points_ms": {"rdb_linear_fwd": round(t_fwd, 4), "rdb_linear_bwd_dx": round(t_dx, 4), "rdb_linear_bwd_dcoef": round(t_dc, 4),
                                      "sum": round(ms_one, 4), "executed_gflop": round(3 * (proj + prod) / 1e9, 1)},
-        "kernels": "f32_gemm_kernel (v_mfma_f32_32x32x2_f32) for the five products, noise hashed into the operand tiles",
-        "note": "fp32 activations, coefficients and sums; z = x.N^T is formed once and kept (fp32) in the projection state; the one-call "
-                "entry points form it twice"}
+        "kernels": "f32_gemm_kernel for the five products, noise hashed into the operand tiles; operands split into three bf16 parts "
+                   "(exact) on their way into LDS, six v_mfma_f32_32x32x16_bf16 per 16 contraction values of a tile pair, fp32 sums",
+        "note": "fp32 activations, coefficients and results at fp32 accuracy (parity 1e-5 against the fp64 oracle, as the fp32 matrix "
+                "instructions); z = x.N^T is formed once and kept (fp32) in the projection state; the one-call entry points form it twice"}
     del keep
     if compare:
         gf, gdx, gdc, keep = calls(_lib.RDB_ALGO_TILE)

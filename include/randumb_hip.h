@@ -328,6 +328,15 @@ int rdb_linear_bwd_projected_part(int part, void *dx, int64_t lddx, float *dcoef
  * mode. */
 int rdb_set_big_tiles(int mode);
 
+/* Tuning switch without a counterpart in the reference, for the products of fp32 layers (and of bf16 layers whose sizes are not
+ * multiples of 8) and for the matrix-coef materialise products that run on the matrix cores.  mode 1 (default): every operand
+ * value is split exactly into three bf16 parts (v = h + m + l, each the top 8 bits of what is left) on its way into LDS and a
+ * product runs as six bf16 matrix instructions (ah bh + ah bm + am bh + ah bl + al bh + am bm, fp32 accumulation): the terms
+ * left out are below 2^-23 of a product, an fp32 multiplication's own rounding, and the 32 x 32 x 16 bf16 instruction does in
+ * 3/8 of the time what eight 32 x 32 x 2 fp32 ones do.  mode 0: fp32 matrix instructions.  Results agree to fp32 rounding;
+ * with mode 1 an infinite input gives NaN where mode 0 gives an infinity.  Process-wide; returns the previous mode. */
+int rdb_set_f32_split(int mode);
+
 /* ------------------------------------------------------------------------------- one-launch forms and their bounded waits
  * No counterpart in the reference (its kernels are one launch per product).  rdb_linear_project_fwd / rdb_linear_fwd with
  * bf16 and k <= 256, and rdb_linear_fwd / rdb_linear_bwd_dx with fp32, k <= 64 and few tokens, run producer and consumer

@@ -52,6 +52,7 @@ EXPORTS = [
     "rdb_linear_bwd_projected_to",
     "rdb_linear_bwd_projected_part",
     "rdb_set_big_tiles",
+    "rdb_set_f32_split",
     "rdb_set_one_launch",
     "rdb_sync_giveups_async",
     "rdb_sync_giveups",
@@ -149,6 +150,8 @@ def load() -> ctypes.CDLL:
     L.rdb_linear_bwd_projected_part.argtypes = [ci, vp, i64, vp, vp, i64, vp, vp, dp, vp, i64, vp]
     L.rdb_set_big_tiles.argtypes = [ci]
     L.rdb_set_big_tiles.restype = ci
+    L.rdb_set_f32_split.argtypes = [ci]
+    L.rdb_set_f32_split.restype = ci
     L.rdb_set_one_launch.argtypes = [ci]
     L.rdb_set_one_launch.restype = ci
     L.rdb_sync_giveups_async.argtypes = [vp, vp]

@@ -1,5 +1,8 @@
-// Fused linear layer, matrix-coef + fp32, any coefficient dimension and many tokens: the factored algorithm on the fp32
-// matrix cores (v_mfma_f32_32x32x2_f32).
+// Fused linear layer, matrix-coef + fp32, any coefficient dimension and many tokens: the factored algorithm on the matrix
+// cores at fp32 accuracy.  By default every operand value is split exactly into three bf16 parts on its way into LDS and a
+// product runs as six bf16 matrix instructions (v_mfma_f32_32x32x16_bf16; see fg_split3): gfx950's bf16 matrix rate is 16 times
+// its fp32 one, so six of them cost 3/8 of the eight fp32 instructions (v_mfma_f32_32x32x2_f32) they replace; the fp32
+// instructions remain as the other mode of rdb_set_f32_split.
 //
 //   forward  z = x . N^T [T x k],  y = z . C^T (+ bias)
 //   dx       t = dy . C  [T x k],  dx = t . N
@@ -7,7 +10,7 @@
 //
 // N[m, i] = noise(PRIME*i + m) is hashed into the pipeline's LDS tiles and never stored; W = C . N is never formed.  All
 // five products run on one kernel template that differs in where its two operands come from (a row-major matrix read along
-// or across its rows, or the hash).  Everything is fp32: operands, products and sums.  (bf16 layers whose sizes keep them off
+// or across its rows, or the hash).  Operands, intermediate matrices and sums are fp32 in memory and in the accumulators.  (bf16 layers whose sizes keep them off
 // the bf16 kernels, which want multiples of 8, run here too: bf16 matrices are read value by value and widened, z and t stay
 // fp32, y and dx are rounded to bf16 once.)
 // With scale_bias (W = C . N + s . R, R[o, i] = noise1d(o*in_f + i), full rank: src/rten_cpp/RandumbTensor.py:286-289) the

@@ -1127,6 +1127,11 @@ extern "C" int rdb_selftest_sync_giveup(void *y, int64_t ldy, void *scratch, int
     return rc;
 }
 
+namespace rdb {
+int set_f32_split_mode(int mode);   // rdb_f32.hip
+}
+extern "C" int rdb_set_f32_split(int mode) { return rdb::set_f32_split_mode(mode); }
+
 extern "C" int rdb_set_big_tiles(int mode)
 {
     const int before = big_tiles_mode();

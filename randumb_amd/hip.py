@@ -736,6 +736,13 @@ def linear_bwd_projected(dy: torch.Tensor, state: torch.Tensor, coef: torch.Tens
     return dx, (dcoef if dcoef.dtype == dcoef_dtype else dcoef.to(dcoef_dtype))
 
 
+def set_f32_split(mode: int) -> int:
+    """Process-wide switch of the fp32 products that run on the matrix cores: 1 (default) = three-way bf16 splits of the operands
+    and six bf16 matrix instructions per product (fp32 accuracy at 3/8 of the matrix-core time), 0 = fp32 matrix instructions.
+    Returns the previous mode."""
+    return int(_lib.load().rdb_set_f32_split(int(mode)))
+
+
 def set_big_tiles(mode: int) -> int:
     """Process-wide switch of the projected entry points' kernels for k > 256: 0 = 128-wide tiles only, 1 = 256-wide tiles
     (one persistent block per compute unit) when the layer has a tile for every other compute unit at least (default),

@@ -1,5 +1,7 @@
-"""fp32 matrix-coef layers on the fp32 matrix cores (the factored algorithm, any k, many tokens) against the CPU oracle, at the
-fp32 tolerance of the path (rel-L2 1e-5), and against the general kernel.
+"""fp32 matrix-coef layers on the matrix cores (the factored algorithm, any k, many tokens) against the CPU oracle, at the
+fp32 tolerance of the path (rel-L2 1e-5), and against the general kernel.  By default the products run as six bf16 matrix
+instructions on exact three-way splits of the operands; test_split_products_are_as_accurate_as_fp32_instructions runs the fp32
+matrix instructions beside them.
 
 Asking for RDB_ALGO_FACTORED makes the library refuse rather than fall back to the general kernel, so a call that succeeds
 with k > 64 (beyond the vector-ALU kernels for few tokens) ran these kernels."""
@@ -269,3 +271,39 @@ def test_fp32_layer_takes_the_projected_form(hip, oracle):
     layer.zero_grad()
     layer(x.cuda()).backward(dy.cuda())
     assert rel_l2(layer.weight_coef.grad.cpu().numpy(), want_dc) < F32_TOL
+
+
+@pytest.mark.parametrize("T,in_f,out_f,k,seed", [(512, 768, 1024, 128, 3), (333, 777, 555, 99, 8), (2100, 516, 132, 100, 77)])
+def test_split_products_are_as_accurate_as_fp32_instructions(hip, oracle, T, in_f, out_f, k, seed):
+    """rdb_set_f32_split: the same calls with the operands split three ways onto the bf16 matrix instructions (default) and on
+    the fp32 matrix instructions.  Both within the fp32 tolerance of the fp64 oracle, the split products no further from it than
+    1.5 times the fp32 instructions' own error (plus a floor), and the two a few fp32 roundings apart.  Inputs with a wide
+    range of magnitudes, so that the low parts matter."""
+    from randumb_amd._lib import RDB_ALGO_FACTORED
+
+    print(f"case f32 split vs fp32 instructions T={T} in={in_f} out={out_f} k={k}", flush=True)
+    x, dy, coef, bias = _inputs(T, in_f, out_f, k, seed)
+    g = torch.Generator().manual_seed(seed + 100)
+    x = x * torch.exp(3.0 * torch.randn(T, 1, generator=g))          # rows of very different sizes
+    coef = coef * torch.exp(2.0 * torch.randn(1, k, generator=g))
+    xn, dyn, cn = x.numpy(), dy.numpy(), coef.numpy()
+    want_y = oracle.linear_fwd(xn, cn, in_f, out_f, seed, bias=bias.numpy())
+    want_dx, want_dc, _ = oracle.linear_bwd(xn, dyn, cn, in_f, out_f, seed)
+    xg, dyg, cg, bg = x.cuda(), dy.cuda(), coef.cuda(), bias.cuda()
+    got = {}
+    before = hip.set_f32_split(1)
+    try:
+        for mode in (1, 0):
+            hip.set_f32_split(mode)
+            y = hip.linear_fwd(xg, cg, in_f, out_f, in_f, 1, seed, bias=bg, algo=RDB_ALGO_FACTORED)
+            dx = hip.linear_bwd_dx(dyg, cg, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+            dc, _ = hip.linear_bwd_dcoef(dyg, xg, k, out_f, in_f, out_f, in_f, 1, seed, algo=RDB_ALGO_FACTORED)
+            got[mode] = [t.cpu().numpy() for t in (y, dx, dc)]
+    finally:
+        hip.set_f32_split(before)
+    for name, i, want in (("y", 0, want_y), ("dx", 1, want_dx), ("dcoef", 2, want_dc)):
+        e_split, e_f32 = rel_l2(got[1][i], want), rel_l2(got[0][i], want)
+        print(f"  {name}: split {e_split:.2e}  fp32 instructions {e_f32:.2e}  between them {rel_l2(got[1][i], got[0][i]):.2e}", flush=True)
+        assert e_split < F32_TOL and e_f32 < F32_TOL, name
+        assert e_split < 1.5 * e_f32 + 2e-7, name
+        assert rel_l2(got[1][i], got[0][i]) < 2e-6, name

@@ -132,6 +132,20 @@ def test_big_tiles_switch_without_a_gpu():
     assert L.rdb_set_big_tiles(first) == first
 
 
+def test_f32_split_switch_without_a_gpu():
+    """rdb_set_f32_split returns the previous mode and starts at 1 (fp32 products as three-way bf16 splits)."""
+    from randumb_amd import _lib
+
+    L = _lib.load()
+    first = L.rdb_set_f32_split(0)
+    try:
+        assert first == 1
+        assert L.rdb_set_f32_split(5) == 0 and L.rdb_set_f32_split(0) == 1
+    finally:
+        L.rdb_set_f32_split(first)
+    assert L.rdb_set_f32_split(first) == first
+
+
 def test_argument_errors_come_back_as_codes_without_a_gpu():
     from randumb_amd import _lib
 
