@@ -211,7 +211,10 @@ int rdb_linear_rbias_bwd(void *dx, int64_t lddx, float *d_scale_bias, const void
 
 /* Replaces MmBackward's dW = dy^T x followed by RandumbTensorConstructor.backward ->
  * materialize_bwd (+ scale_bias_bwd) (R.py:979-990): dW is contracted with the regenerated noise tile
- * as it is produced and never written to memory.
+ * as it is produced and never written to memory.  (One exception, the reference's own data flow: a vector-coef layer whose
+ * weight is contiguous, under RDB_ALGO_AUTO with the workspace rdb_linear_workspace_bytes asks for, forms dW in fp32 in that
+ * workspace once and contracts it once, every element with its k hashed values, at the rate of the hash; without the
+ * workspace the general kernel repeats those k hashes per element for every block of tokens.  Sums in a fixed order.)
  * dcoef (fp32, [k] or [out_f x k]) and, when d_scale_bias != NULL, d_scale_bias (fp32 [1]) are
  * OVERWRITTEN.  fp32 activations: partial sums are added in a fixed order, the result is the same bit for
  * bit from run to run.  bf16 activations: partial sums from different tiles are combined with fp32 atomics

@@ -751,6 +751,28 @@ int linear_dcoef_f32(float *dcoef, float *d_scale_bias, const void *dy, int64_t 
     return check_launch("f32_sum_scalars_kernel");
 }
 
+// ----------------------------------------------------------------------------------------------- dW = dy^T . x on its own
+// For the vector-coef coefficient gradient: every element of dW meets k hashed values, so that gradient is bound by the hash
+// whatever is fused into it, and a kernel that forms dW tile by tile per block of tokens repeats the k hashes per element for
+// every block.  With room for dW (fp32, [out_f x in_f]) in the caller's workspace it is formed once, by this product, and
+// contracted once by the kernels of rdb_materialize_bwd.  Scratch behind dW: one more [out_f x in_f] matrix per token range.
+static FgPlan dw_plan(const rdb_linear_desc *d, int num_cus) { return fg_plan(d->out_f, d->in_f, d->tokens, num_cus, 256, 64); }
+int64_t linear_dw_f32_workspace(const rdb_linear_desc *d, int num_cus)
+{
+    if (d->out_f * d->in_f >= (1ll << 29) || d->tokens <= 0) return 0;
+    const int r = dw_plan(d, num_cus).ranges;
+    return up256(d->out_f * d->in_f * 4) * (1 + (r > 1 ? r : 0));
+}
+int linear_dw_f32(float *dW, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus, hipStream_t s)
+{
+    if (d->tokens * lddy >= (1ll << 29) || d->tokens * ldx >= (1ll << 29) || d->out_f * d->in_f >= (1ll << 29)) return RDB_E_UNSUPPORTED;
+    FgProduct q = {(const float *)dy, lddy, (d->tokens - 1) * lddy + d->out_f, (const float *)x, ldx, (d->tokens - 1) * ldx + d->in_f, dW, d->in_f, nullptr,
+                   d->out_f, d->in_f, d->tokens, 128, 0, 0, d->seed};
+    q.a_es = q.b_es = fg_es(d->act_dtype);
+    const int64_t stride = up256(d->out_f * d->in_f * 4) / 4;
+    return fg_launch_ranges<FG_MCONT, FG_MCONT>(q, dw_plan(d, num_cus), dW + stride, stride, num_cus, s, "f32_gemm_kernel (dW = dy^T . x)");
+}
+
 // ----------------------------------------------------------------------------------------------- projected form in fp32
 // What a training step keeps from the forward to the backward pass (all that the latter needs of x): z = x . N^T in fp32, [tokens x k] row-major,
 // behind a 256-byte header (the same role as the bf16 state of rdb_direct.hpp; no fragment orders, no transposed copies: these

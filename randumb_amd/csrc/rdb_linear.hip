@@ -320,6 +320,8 @@ int linear_dx_f32(void *dx, int64_t lddx, const void *dy, int64_t lddy, const vo
                   int num_cus, void *workspace, int64_t workspace_bytes, hipStream_t s);
 int64_t linear_f32_state_bytes(const rdb_linear_desc *d);
 int64_t linear_f32_bwd_projected_workspace(const rdb_linear_desc *d, int num_cus);
+int64_t linear_dw_f32_workspace(const rdb_linear_desc *d, int num_cus);
+int linear_dw_f32(float *dW, const void *dy, int64_t lddy, const void *x, int64_t ldx, const rdb_linear_desc *d, int num_cus, hipStream_t s);
 int linear_project_f32(void *state, void *y, int64_t ldy, const void *x, int64_t ldx, const void *coef, const void *bias, const rdb_linear_desc *d,
                        int num_cus, hipStream_t s);
 int linear_fwd_projected_f32(void *y, int64_t ldy, const void *state, const void *coef, const void *bias, const rdb_linear_desc *d, int num_cus,
@@ -396,11 +398,32 @@ using namespace rdb;
 
 static int64_t bwd_projected_workspace(const rdb_linear_desc *d, bool force_partial);
 
+// vector-coef coefficient gradient in two passes: dW = dy^T . x into the workspace (and the partial matrices of its token
+// ranges), then the contraction of rdb_materialize_bwd and, for the scale's gradient, of rdb_scale_bias_bwd, with their scratch
+// behind it.  Only for a weight that is contiguous in memory (element (o, i) at o * in_f + i).
+static bool vec_dcoef_two_pass_ok(const rdb_linear_desc *d)
+{
+    return d->coef_rows == 0 && d->sO == d->in_f && d->sI == 1 && d->k > 0 && d->tokens > 0 && d->out_f * d->in_f < (1ll << 29) &&
+           (d->act_dtype == RDB_F32 || d->act_dtype == RDB_BF16);
+}
+static int64_t vec_dcoef_workspace(const rdb_linear_desc *d)
+{
+    if (!vec_dcoef_two_pass_ok(d)) return 0;
+    const int64_t dw = linear_dw_f32_workspace(d, num_compute_units());
+    if (dw <= 0) return 0;
+    const int64_t nw = d->out_f * d->in_f;
+    return dw + (rdb_materialize_bwd_workspace_bytes(0, d->k, 0, nw) + 255) / 256 * 256 + (rdb_scale_bias_bwd_workspace_bytes(nw) + 255) / 256 * 256;
+}
+
 extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
 {
     if (!d) return 0;
     if (d->algo == RDB_ALGO_TILE || d->algo == RDB_ALGO_STRIP) return 0;
-    if (d->coef_rows == 0) return d->algo == RDB_ALGO_AUTO ? linear_vecsplit_workspace(op, d) : 0;   // vector-coef: the chunks' partial outputs
+    if (d->coef_rows == 0) {   // vector-coef: the chunks' partial outputs; for the coefficient gradient dW and what its contraction needs
+        if (d->algo != RDB_ALGO_AUTO) return 0;
+        if (op == RDB_OP_LINEAR_BWD_DCOEF) return vec_dcoef_workspace(d);
+        return linear_vecsplit_workspace(op, d);
+    }
     if (d->act_dtype == RDB_F32) {  // fp32: the small-k kernels, whose scratch is one [tokens x k] fp32 matrix
         rdb_linear_desc dd = *d;
         if (op == RDB_OP_LINEAR_BWD_DCOEF) dd.coef_dtype = RDB_F32;
@@ -676,6 +699,25 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
     if (!empty) {
         if (!dy || !x) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef: dy or x is NULL");
         if (lddy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dcoef: leading dimension smaller than the row");
+    }
+    if (!empty && d->algo == RDB_ALGO_AUTO && ncoef > 0 && vec_dcoef_two_pass_ok(d)) {
+        // vector-coef with room for dW in the workspace: dW formed once (on the matrix cores at fp32 accuracy), then every element
+        // of it contracted once with its k hashed values, at the rate of the hash (the general kernel below repeats the k hashes
+        // per element for every block of tokens: 1.5 ms against 0.35 ms at 128 tokens x 768 -> 3072, k = 256)
+        const int64_t need = vec_dcoef_workspace(d);
+        if (need > 0 && workspace && workspace_bytes >= need && ((uintptr_t)workspace & 15) == 0) {
+            float *dW = static_cast<float *>(workspace);
+            rc = linear_dw_f32(dW, dy, lddy, x, ldx, d, num_compute_units(), s);
+            if (rc == RDB_OK) {
+                const int64_t nw = d->out_f * d->in_f, mb = (rdb_materialize_bwd_workspace_bytes(0, d->k, 0, nw) + 255) / 256 * 256;
+                char *after = static_cast<char *>(workspace) + linear_dw_f32_workspace(d, num_compute_units());
+                rc = rdb_materialize_bwd(dcoef, dW, RDB_F32, 0, d->k, 0, nw, d->seed, after, mb, stream);
+                if (rc == RDB_OK && d_scale_bias)
+                    rc = rdb_scale_bias_bwd(d_scale_bias, dW, RDB_F32, nw, d->seed, after + mb, rdb_scale_bias_bwd_workspace_bytes(nw), stream);
+                return rc;
+            }
+            if (rc != RDB_E_UNSUPPORTED) return rc;
+        }
     }
     if (!empty && d->act_dtype == RDB_F32 && (d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED)) {
         // The fp32 factored kernels overwrite their outputs: nothing to clear first.  The matrix-core kernels also return the

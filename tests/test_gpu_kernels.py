@@ -260,6 +260,16 @@ def test_vector_coef_split_form_against_the_general_kernel(hip, dtype, tol):
         dx_t = hip.linear_bwd_dx(dy, c, in_f, out_f, in_f, 1, seed, scale_bias=scale_bias, algo=RDB_ALGO_TILE)
         assert rel(dx, dx_t) < tol
         assert torch.equal(dx, hip.linear_bwd_dx(dy, c, in_f, out_f, in_f, 1, seed, scale_bias=scale_bias))
+        # the coefficient gradient with room for dW in the workspace (dW formed once, contracted once with its k hashed values per
+        # element) against the general kernel, with and without the gradient of the random bias's scale
+        want_ds = scale_bias is not None
+        dc, ds = hip.linear_bwd_dcoef(dy, x, k, 0, in_f, out_f, in_f, 1, seed, want_scale_bias_grad=want_ds)
+        dc_t, ds_t = hip.linear_bwd_dcoef(dy, x, k, 0, in_f, out_f, in_f, 1, seed, want_scale_bias_grad=want_ds, algo=RDB_ALGO_TILE)
+        assert rel(dc, dc_t) < max(tol, 1e-5)
+        again = hip.linear_bwd_dcoef(dy, x, k, 0, in_f, out_f, in_f, 1, seed, want_scale_bias_grad=want_ds)
+        assert torch.equal(dc, again[0])
+        if want_ds:
+            assert abs(float(ds) - float(ds_t)) < max(tol, 1e-5) * max(1.0, abs(float(ds_t))) and torch.equal(ds, again[1])
 
 
 def test_argument_errors(hip):

@@ -273,7 +273,18 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     vec = desc(16, 4096, 4096, 128, rows=0, act=_lib.RDB_F32, coef=_lib.RDB_F32)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(vec)) == (4096 // 32) * 16 * 4096 * 4
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(vec)) == (4096 // 32) * 16 * 4096 * 4
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DCOEF, ctypes.byref(vec)) == 0
+    # its coefficient gradient: room for dW = dy^T.x (fp32; here one range of tokens) and for what contracting it needs
+    up256 = lambda n: -(-n // 256) * 256
+    L.rdb_materialize_bwd_workspace_bytes.restype = ctypes.c_int64
+    L.rdb_scale_bias_bwd_workspace_bytes.restype = ctypes.c_int64
+    nw = 4096 * 4096
+    want = nw * 4 + up256(L.rdb_materialize_bwd_workspace_bytes(ctypes.c_int64(0), ctypes.c_int64(128), ctypes.c_int64(0), ctypes.c_int64(nw))) \
+        + up256(L.rdb_scale_bias_bwd_workspace_bytes(ctypes.c_int64(nw)))
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DCOEF, ctypes.byref(vec)) == want
+    # ... only for a weight that is contiguous in memory
+    tr = desc(16, 4096, 4096, 128, rows=0, act=_lib.RDB_F32, coef=_lib.RDB_F32)
+    tr.sO, tr.sI = 1, 4096
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DCOEF, ctypes.byref(tr)) == 0
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(8192, 4096, 4096, 128, rows=0, act=_lib.RDB_F32, coef=_lib.RDB_F32))) == 0
 
     bad = ctypes.byref(desc(64, 100, 32, 16))
