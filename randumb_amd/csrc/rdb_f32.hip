@@ -85,8 +85,9 @@ __device__ __forceinline__ void fg_split3(float v, uint32_t &h, uint32_t &m, uin
 
 // One operand's way from its source into LDS: load(stage) requests / hashes the stage's values into registers, store() puts
 // them into a tile.  Rows past `rows` and contraction values past `kend` are zeros.
-// VEC: the matrix is read in 16-byte pieces (16-byte aligned base, leading dimension a multiple of 4, and the extent that
-// runs along a piece a multiple of 4, so that a piece lies inside or outside as a whole); otherwise value by value.
+// VEC: the matrix is read in pieces of four values (16 bytes of fp32, 8 bytes of bf16; 16-byte aligned base, leading dimension a
+// multiple of 4, and the extent that runs along a piece a multiple of 4, so that a piece lies inside or outside as a whole);
+// otherwise value by value.
 // SPLIT: the tile goes to LDS as three bf16 planes (see fg_split3): planes of [2 halves of the stage's 16 contraction values]
 // [rows][8] for the sources read along the contraction (a lane's MFMA operand is 16 consecutive bytes), of [16][rows + 32] for
 // FG_MCONT (read back with the LDS transpose read).  The noise sources then give a thread consecutive contraction values.
@@ -115,6 +116,16 @@ template <int ROWS, int SRC, bool VEC, bool SPLIT = false> struct FgOperand {
             return bf16_to_f32(h);
         }
         return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, in ? (int)(o + 4 * j) : (int)FG_OOB, 0, 0));
+    }
+    // VEC: four consecutive elements at byte offset o (fp32: 16 bytes; bf16: 8 bytes, widened), zeros when outside
+    __device__ __forceinline__ f32x4 load4(uint32_t o, bool in) const
+    {
+        if (es == 2) {
+            const f32x2 h = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(rs, in ? (int)o : (int)FG_OOB, 0, 0));
+            const uint32_t lo = __float_as_uint(h[0]), hi = __float_as_uint(h[1]);
+            return f32x4{__uint_as_float(lo << 16), __uint_as_float(lo & 0xffff0000u), __uint_as_float(hi << 16), __uint_as_float(hi & 0xffff0000u)};
+        }
+        return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, in ? (int)o : (int)FG_OOB, 0, 0));
     }
     __device__ __forceinline__ void init(const float *src, int64_t ld, int64_t bytes, int row0, int rows, int k_begin_, int kend_, uint32_t seed,
                                          uint32_t sR, uint32_t sK, int es_)
@@ -167,7 +178,7 @@ template <int ROWS, int SRC, bool VEC, bool SPLIT = false> struct FgOperand {
             for (int h = 0; h < NV; ++h) {
                 const uint32_t o = off[h] + (uint32_t)stage * step;
                 if (VEC) {   // all inside or all outside
-                    r[h] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (ok[h] && kk < kend) ? (int)o : (int)FG_OOB, 0, 0));
+                    r[h] = load4(o, ok[h] && kk < kend);
                 } else {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) r[h][j] = load1(o, ok[h] && kk + j < kend, j);
@@ -179,7 +190,7 @@ template <int ROWS, int SRC, bool VEC, bool SPLIT = false> struct FgOperand {
                 const bool in = ok[h] && k_begin + stage * FG_BK + kk0 + h * (FG_THREADS / (ROWS / 4)) < kend;
                 const uint32_t o = off[h] + (uint32_t)stage * step;
                 if (VEC) {
-                    r[h] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, in ? (int)o : (int)FG_OOB, 0, 0));
+                    r[h] = load4(o, in);
                 } else {   // a thread's four values are consecutive rows: rows_left of them exist
 #pragma unroll
                     for (int j = 0; j < 4; ++j) r[h][j] = load1(o, in && j < rows_left[h], j);
@@ -593,7 +604,7 @@ template <int ASRC, int BSRC> static int fg_launch(const FgProduct &q, int num_c
         if (src != FG_KCONT && src != FG_MCONT) return true;
         return fg_aligned16(m) && ld % 4 == 0 && (src == FG_KCONT ? q.K % 4 == 0 : rows % 4 == 0);
     };
-    const bool vec = vec_ok(ASRC, q.a, q.lda, q.M) && vec_ok(BSRC, q.b, q.ldb, q.N) && q.a_es == 4 && q.b_es == 4;   // bf16: value by value
+    const bool vec = vec_ok(ASRC, q.a, q.lda, q.M) && vec_ok(BSRC, q.b, q.ldb, q.N);   // bf16 matrices: 8-byte pieces of four values
     if (cdiv(q.N, FG_BN) > 65535) return RDB_E_UNSUPPORTED;   // the grid's y
     const dim3 grid((unsigned)cdiv(q.M, q.bm), (unsigned)cdiv(q.N, FG_BN), (unsigned)splits);
     if (BSRC == FG_NOISE_1D) {   // the random-bias products: added on top of an output, or reduced against a matrix
