@@ -20,6 +20,7 @@
 // materialize_bwd (RandumbTensor.py:979-990, 304-359) for fp32 layers beyond the few-token regime of rdb_smallk.hip.
 #include "rdb_gemm.hpp"
 #include <algorithm>
+#include <type_traits>
 
 namespace rdb {
 
@@ -234,9 +235,16 @@ template <int ROWS, int SRC, bool VEC, bool SPLIT = false> struct FgOperand {
             for (int j = 0; j < NV * 4; ++j) tile[(kk0 + j * KSTEP) * LD + row] = r[j >> 2][j & 3];
         }
     }
-    // SPLIT: four of the thread's values into the three planes, 8 bytes each, at element offset `at` of a plane
-    __device__ __forceinline__ void put4(bf16_t *__restrict__ tile, int at, const f32x4 &v) const
+    // SPLIT: four of the thread's values into the planes, 8 bytes each, at element offset `at` of a plane.  Values that come from a
+    // bf16 matrix are their own first part and the other two are zero: only the first plane is written (and read, see the kernel).
+    __device__ __forceinline__ bool one_plane() const { return !HASHED && es == 2; }
+    template <bool ONE> __device__ __forceinline__ void put4(bf16_t *__restrict__ tile, int at, const f32x4 &v) const
     {
+        if (ONE) {
+            *reinterpret_cast<uint2 *>(tile + at) = make_uint2((__float_as_uint(v[1]) & 0xffff0000u) | (__float_as_uint(v[0]) >> 16),
+                                                               (__float_as_uint(v[3]) & 0xffff0000u) | (__float_as_uint(v[2]) >> 16));
+            return;
+        }
         uint32_t h[4], m[4], l[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) fg_split3(v[j], h[j], m[j], l[j]);
@@ -244,27 +252,27 @@ template <int ROWS, int SRC, bool VEC, bool SPLIT = false> struct FgOperand {
         *reinterpret_cast<uint2 *>(tile + PLANE + at) = make_uint2(m[1] | (m[0] >> 16), m[3] | (m[2] >> 16));
         *reinterpret_cast<uint2 *>(tile + 2 * PLANE + at) = make_uint2(l[1] | (l[0] >> 16), l[3] | (l[2] >> 16));
     }
-    __device__ __forceinline__ void store_split(bf16_t *__restrict__ tile) const
+    template <bool ONE> __device__ __forceinline__ void store_split(bf16_t *__restrict__ tile) const
     {
         const int t = threadIdx.x;
         if (SRC == FG_KCONT) {
 #pragma unroll
             for (int h = 0; h < NV; ++h) {   // contraction values 4 kq .. 4 kq + 3 of a row
                 const int idx = h * FG_THREADS + t, row = idx >> 2, kq = idx & 3;
-                put4(tile, ((kq >> 1) * ROWS + row) * 8 + (kq & 1) * 4, r[h]);
+                put4<ONE>(tile, ((kq >> 1) * ROWS + row) * 8 + (kq & 1) * 4, r[h]);
             }
         } else if (SRC == FG_MCONT) {
 #pragma unroll
             for (int h = 0; h < NV; ++h) {   // four consecutive rows at one contraction value
                 const int idx = h * FG_THREADS + t, kk = idx / (ROWS / 4), r4 = (idx % (ROWS / 4)) * 4;
-                put4(tile, kk * LDM + r4, r[h]);
+                put4<ONE>(tile, kk * LDM + r4, r[h]);
             }
         } else {
             const int row = t % ROWS;
 #pragma unroll
             for (int h = 0; h < NV; ++h) {   // contraction values kk0 + 4 h .. + 3 of a row
                 const int kk = kk0 + 4 * h;
-                put4(tile, ((kk >> 3) * ROWS + row) * 8 + (kk & 7), r[h]);
+                put4<ONE>(tile, ((kk >> 3) * ROWS + row) * 8 + (kk & 7), r[h]);
             }
         }
     }
@@ -287,7 +295,7 @@ template <int ROWS, int SRC, bool VEC, bool SPLIT = false> struct FgOperand {
 // out[M x N] (+)= A . B^T over one split of the contraction.  Block: BM x 128 of the output, four waves as 2 x 2, a wave owns
 // (BM / 2) x 64 in BM / 64 x 2 accumulator tiles.  Two LDS buffers, one barrier per stage: while a stage is multiplied the
 // next one is on its way from memory (or being hashed) in registers.
-template <int BM, int ASRC, int BSRC, int EPI, bool VEC, bool SPLIT = false>
+template <int BM, int ASRC, int BSRC, int EPI, bool VEC, bool SPLIT = false, bool ANY16 = false>
 __global__ __launch_bounds__(FG_THREADS, 2) void f32_gemm_kernel(FgParams p)
 {
     typedef FgOperand<BM, ASRC, VEC, SPLIT> PA;
@@ -311,82 +319,106 @@ __global__ __launch_bounds__(FG_THREADS, 2) void f32_gemm_kernel(FgParams p)
             for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.0f;
     pa.load(0);
     pb.load(0);
-    for (int s = 0; s < nstage; ++s) {
-        float *As = lds + (s & 1) * STAGE, *Bs = As + PA::TILE_BYTES / 4;
-        if (SPLIT) {
-            pa.store_split(reinterpret_cast<bf16_t *>(As));
-            pb.store_split(reinterpret_cast<bf16_t *>(Bs));
-        } else {
-            pa.store(As);
-            pb.store(Bs);
-        }
-        __syncthreads();   // also: every wave is done reading the other buffer (the stage before this one)
-        const bool more = s + 1 < nstage;
-        if (more) {
-            if (!PA::HASHED) pa.load(s + 1);
-            if (!PB::HASHED) pb.load(s + 1);
-        }
-        if (SPLIT) {
-            // the stage is one k-step of the bf16 matrix instruction: three planes a side, six products a tile pair, the small
-            // ones first; the next stage's noise values are hashed between the tile pairs
-            const bf16_t *ap = reinterpret_cast<const bf16_t *>(As), *bp = reinterpret_cast<const bf16_t *>(Bs);
-            bf16x8 fa[MI][3], fb[NI][3];
-#pragma unroll
-            for (int pl = 0; pl < 3; ++pl) {
-#pragma unroll
-                for (int mi = 0; mi < MI; ++mi) fa[mi][pl] = PA::frag(ap + pl * PA::PLANE, wm * (BM / 2) + mi * 32, lane);
-#pragma unroll
-                for (int ni = 0; ni < NI; ++ni) fb[ni][pl] = PB::frag(bp + pl * PB::PLANE, wn * 64 + ni * 32, lane);
+    // The stage loop, once per number of planes of the two sides (known per launch, not per kernel: a side that comes from a
+    // bf16 matrix has one plane), so that each copy is straight-line code between its barriers.
+    auto stages = [&](auto a_one, auto b_one) __attribute__((always_inline)) {
+        constexpr int AP = decltype(a_one)::value ? 1 : 3, BP = decltype(b_one)::value ? 1 : 3;
+        for (int s = 0; s < nstage; ++s) {
+            float *As = lds + (s & 1) * STAGE, *Bs = As + PA::TILE_BYTES / 4;
+            if (SPLIT) {
+                pa.template store_split<AP == 1>(reinterpret_cast<bf16_t *>(As));
+                pb.template store_split<BP == 1>(reinterpret_cast<bf16_t *>(Bs));
+            } else {
+                pa.store(As);
+                pb.store(Bs);
             }
+            __syncthreads();   // also: every wave is done reading the other buffer (the stage before this one)
+            const bool more = s + 1 < nstage;
+            if (more) {
+                if (!PA::HASHED) pa.load(s + 1);
+                if (!PB::HASHED) pb.load(s + 1);
+            }
+            if (SPLIT) {
+                // the stage is one k-step of the bf16 matrix instruction: three planes a side, six products a tile pair, the small
+                // ones first (a side that comes from a bf16 matrix has one plane: three products, or one); the next stage's noise
+                // values are hashed between the tile pairs
+                const bf16_t *ap = reinterpret_cast<const bf16_t *>(As), *bp = reinterpret_cast<const bf16_t *>(Bs);
+                {
+                    bf16x8 fa[MI][AP], fb[NI][BP];
 #pragma unroll
-            for (int mi = 0; mi < MI; ++mi)
+                    for (int pl = 0; pl < 3; ++pl) {
 #pragma unroll
-                for (int ni = 0; ni < NI; ++ni) {
-                    f32x16 c = acc[mi][ni];
-                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][1], fb[ni][1], c, 0, 0, 0);
-                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][2], fb[ni][0], c, 0, 0, 0);
-                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][0], fb[ni][2], c, 0, 0, 0);
-                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][1], fb[ni][0], c, 0, 0, 0);
-                    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][0], fb[ni][1], c, 0, 0, 0);
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][0], fb[ni][0], c, 0, 0, 0);
-                    constexpr int GROUPS = MI * NI;
-                    const int grp = mi * NI + ni;
-                    if (PB::HASHED && more) {
-                        constexpr int PER = (PB::NV * 4 + GROUPS - 1) / GROUPS;
+                        for (int mi = 0; mi < MI; ++mi)
+                            if (pl < AP) fa[mi][pl] = PA::frag(ap + pl * PA::PLANE, wm * (BM / 2) + mi * 32, lane);
 #pragma unroll
-                        for (int j = grp * PER; j < (grp + 1) * PER && j < PB::NV * 4; ++j) pb.hash_piece(s + 1, j);
+                        for (int ni = 0; ni < NI; ++ni)
+                            if (pl < BP) fb[ni][pl] = PB::frag(bp + pl * PB::PLANE, wn * 64 + ni * 32, lane);
                     }
-                    if (PA::HASHED && more) {
-                        constexpr int PER = (PA::NV * 4 + GROUPS - 1) / GROUPS;
 #pragma unroll
-                        for (int j = grp * PER; j < (grp + 1) * PER && j < PA::NV * 4; ++j) pa.hash_piece(s + 1, j);
-                    }
+                    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                        for (int ni = 0; ni < NI; ++ni) {
+                            f32x16 c = acc[mi][ni];
+                            if constexpr (AP == 3 && BP == 3) c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][1], fb[ni][1], c, 0, 0, 0);
+                            if constexpr (AP == 3) c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][2], fb[ni][0], c, 0, 0, 0);
+                            if constexpr (BP == 3) c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][0], fb[ni][2], c, 0, 0, 0);
+                            if constexpr (AP == 3) c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][1], fb[ni][0], c, 0, 0, 0);
+                            if constexpr (BP == 3) c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][0], fb[ni][1], c, 0, 0, 0);
+                            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[mi][0], fb[ni][0], c, 0, 0, 0);
+                            constexpr int GROUPS = MI * NI;
+                            const int grp = mi * NI + ni;
+                            if (PB::HASHED && more) {
+                                constexpr int PER = (PB::NV * 4 + GROUPS - 1) / GROUPS;
+#pragma unroll
+                                for (int j = grp * PER; j < (grp + 1) * PER && j < PB::NV * 4; ++j) pb.hash_piece(s + 1, j);
+                            }
+                            if (PA::HASHED && more) {
+                                constexpr int PER = (PA::NV * 4 + GROUPS - 1) / GROUPS;
+#pragma unroll
+                                for (int j = grp * PER; j < (grp + 1) * PER && j < PA::NV * 4; ++j) pa.hash_piece(s + 1, j);
+                            }
+                        }
                 }
-            continue;
+                continue;
+            }
+            const float *ap = As + g * PA::LD + wm * (BM / 2) + r, *bp = Bs + g * PB::LD + wn * 64 + r;
+#pragma unroll
+            for (int ks = 0; ks < FG_BK / 2; ++ks) {
+                float fa[MI], fb[NI];
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi) fa[mi] = ap[ks * 2 * PA::LD + mi * 32];
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni) fb[ni] = bp[ks * 2 * PB::LD + ni * 32];
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi], fb[ni], acc[mi][ni], 0, 0, 0);
+                // the next stage's noise values are hashed in the shadow of these matrix instructions, a share per k-step
+                if (PB::HASHED && more) {
+                    constexpr int PER = (PB::NV * 4 + FG_BK / 2 - 1) / (FG_BK / 2);
+#pragma unroll
+                    for (int j = ks * PER; j < (ks + 1) * PER && j < PB::NV * 4; ++j) pb.hash_piece(s + 1, j);
+                }
+                if (PA::HASHED && more) {
+                    constexpr int PER = (PA::NV * 4 + FG_BK / 2 - 1) / (FG_BK / 2);
+#pragma unroll
+                    for (int j = ks * PER; j < (ks + 1) * PER && j < PA::NV * 4; ++j) pa.hash_piece(s + 1, j);
+                }
+            }
         }
-        const float *ap = As + g * PA::LD + wm * (BM / 2) + r, *bp = Bs + g * PB::LD + wn * 64 + r;
-#pragma unroll
-        for (int ks = 0; ks < FG_BK / 2; ++ks) {
-            float fa[MI], fb[NI];
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi) fa[mi] = ap[ks * 2 * PA::LD + mi * 32];
-#pragma unroll
-            for (int ni = 0; ni < NI; ++ni) fb[ni] = bp[ks * 2 * PB::LD + ni * 32];
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-                for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[mi], fb[ni], acc[mi][ni], 0, 0, 0);
-            // the next stage's noise values are hashed in the shadow of these matrix instructions, a share per k-step
-            if (PB::HASHED && more) {
-                constexpr int PER = (PB::NV * 4 + FG_BK / 2 - 1) / (FG_BK / 2);
-#pragma unroll
-                for (int j = ks * PER; j < (ks + 1) * PER && j < PB::NV * 4; ++j) pb.hash_piece(s + 1, j);
-            }
-            if (PA::HASHED && more) {
-                constexpr int PER = (PA::NV * 4 + FG_BK / 2 - 1) / (FG_BK / 2);
-#pragma unroll
-                for (int j = ks * PER; j < (ks + 1) * PER && j < PA::NV * 4; ++j) pa.hash_piece(s + 1, j);
-            }
+    };
+    typedef std::integral_constant<bool, true> One;
+    typedef std::integral_constant<bool, false> Three;
+    if (!SPLIT || !ANY16) {   // ANY16: one of the matrices is bf16 (only then is the choice compiled in)
+        stages(Three{}, Three{});
+    } else {
+        const bool a1 = pa.one_plane(), b1 = pb.one_plane();
+        if (PA::HASHED || !a1) {
+            if (PB::HASHED || !b1) stages(Three{}, Three{});
+            else stages(Three{}, One{});
+        } else {
+            if (PB::HASHED || !b1) stages(One{}, Three{});
+            else stages(One{}, One{});
         }
     }
     // accumulator j of lane (r, g): row 8 (j / 4) + 4 g + j % 4 of the A side, column r of the B side
@@ -562,7 +594,10 @@ struct FgProduct {
 
 #define FG_LAUNCH(BM_, EPI_)                                                                                  \
     do {                                                                                                      \
-        if (q.split) {                                                                                        \
+        if (q.split && any16) {                                                                               \
+            if (vec) f32_gemm_kernel<BM_, ASRC, BSRC, EPI_, true, true, true><<<grid, FG_THREADS, 0, s>>>(p); \
+            else f32_gemm_kernel<BM_, ASRC, BSRC, EPI_, false, true, true><<<grid, FG_THREADS, 0, s>>>(p);    \
+        } else if (q.split) {                                                                                 \
             if (vec) f32_gemm_kernel<BM_, ASRC, BSRC, EPI_, true, true><<<grid, FG_THREADS, 0, s>>>(p);       \
             else f32_gemm_kernel<BM_, ASRC, BSRC, EPI_, false, true><<<grid, FG_THREADS, 0, s>>>(p);          \
         } else if (vec) f32_gemm_kernel<BM_, ASRC, BSRC, EPI_, true><<<grid, FG_THREADS, 0, s>>>(p);          \
@@ -605,6 +640,7 @@ template <int ASRC, int BSRC> static int fg_launch(const FgProduct &q, int num_c
         return fg_aligned16(m) && ld % 4 == 0 && (src == FG_KCONT ? q.K % 4 == 0 : rows % 4 == 0);
     };
     const bool vec = vec_ok(ASRC, q.a, q.lda, q.M) && vec_ok(BSRC, q.b, q.ldb, q.N);   // bf16 matrices: 8-byte pieces of four values
+    const bool any16 = q.a_es == 2 || ((BSRC == FG_KCONT || BSRC == FG_MCONT) && q.b_es == 2);   // the A side is always a matrix
     if (cdiv(q.N, FG_BN) > 65535) return RDB_E_UNSUPPORTED;   // the grid's y
     const dim3 grid((unsigned)cdiv(q.M, q.bm), (unsigned)cdiv(q.N, FG_BN), (unsigned)splits);
     if (BSRC == FG_NOISE_1D) {   // the random-bias products: added on top of an output, or reduced against a matrix
