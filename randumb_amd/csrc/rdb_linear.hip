@@ -483,6 +483,12 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
                                                 "rdb_linear_workspace_bytes() bytes and either bf16 (activations and coef; sizes that are "
                                                 "multiples of 8; aligned rows) or fp32 (sizes that are multiples of 4; aligned rows)");
     }
+    if (d->algo == RDB_ALGO_AUTO && d->act_dtype == RDB_BF16 && d->coef_rows != 0 && (d->in_f % 8 || d->out_f % 8 || d->k % 8)) {
+        // bf16 sizes the bf16 factored kernels do not take (not multiples of 8): the fp32-accurate matrix-core kernels reading the
+        // bf16 matrices, ahead of the kernel that forms weight strips on chip (4096 tokens x 1000 -> 1000, k = 100: 31 against 133 us)
+        rc = linear_fwd_f32(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), workspace, workspace_bytes, s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
     if (d->algo == RDB_ALGO_AUTO && scale_bias && d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16) {
         // W = C.N + s.R: the low-rank share through the factored kernels where AUTO would take them without the random bias,
         // then the random-bias share (full rank: a product with R hashed as an operand) added on top.  Ahead of the kernel that
@@ -516,7 +522,8 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
         if (rc != RDB_E_UNSUPPORTED) return rc;
     }
     if (d->algo == RDB_ALGO_AUTO && d->act_dtype == RDB_BF16) {
-        // bf16 sizes that kept every kernel above away (not multiples of 8): the fp32 matrix cores, reading bf16 value by value
+        // bf16 requests that kept every kernel above away (rows that are not 16-byte aligned, ...): the same kernels, reading bf16
+        // value by value
         rc = linear_fwd_f32(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
     }
