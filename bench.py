@@ -341,6 +341,31 @@ def smallk_config(event_ms, torch, L, _lib, dev, g):
     return small
 
 
+def few_token_config(event_ms, torch, L, _lib, dev, g):
+    """Few tokens with the headline k: 4096 -> 4096, k = 256, bf16, 1 / 16 / 64 tokens, the three one-call entry points (the
+    vector-ALU kernels of the few-token regime), and the same calls forced onto the matrix-core kernels (algo FACTORED)."""
+    from randumb_amd import hip
+
+    in_f = out_f = 4096
+    k = 256
+    C = (torch.randn(out_f, k, generator=g) * 0.01).bfloat16().to(dev)
+    res = {}
+    for B in (1, 16, 64):
+        x = torch.randn(B, in_f, generator=g).bfloat16().to(dev)
+        dy = torch.randn(B, out_f, generator=g).bfloat16().to(dev)
+        if B == 1:
+            for _ in range(300):   # clocks settle
+                hip.linear_fwd(x, C, in_f, out_f, in_f, 1, 0)
+        row = {}
+        for name, algo in (("", _lib.RDB_ALGO_AUTO), ("matrix_core_kernels_", _lib.RDB_ALGO_FACTORED)):
+            row[name + "fwd_ms"] = round(event_ms(lambda: hip.linear_fwd(x, C, in_f, out_f, in_f, 1, 0, algo=algo), 100), 4)
+            row[name + "dx_ms"] = round(event_ms(lambda: hip.linear_bwd_dx(dy, C, in_f, out_f, in_f, 1, 0, algo=algo), 100), 4)
+            row[name + "dcoef_ms"] = round(event_ms(lambda: hip.linear_bwd_dcoef(dy, x, k, out_f, in_f, out_f, in_f, 1, 0, algo=algo), 100), 4)
+        res[f"batch_{B}"] = row
+    res["note"] = "through the Python wrappers (an allocation of the result and of the workspace per call included)"
+    return res
+
+
 def gpt_step_config(event_ms, torch, dev, g):
     """GPT-2 small with random-backed linears: 12 layers, d = 768, 12 heads, vocab 50304, k = 256, seeds 0..47, bf16, batch
     8 x 1024 random token ids; one training step (forward + backward).  Attention, norms, embedding, head and loss are stock
@@ -372,6 +397,7 @@ def other_configs(event_ms, torch, L, _lib, dev):
     g = torch.Generator().manual_seed(0)
 
     out["in4096_out4096_k16_fp32_matrix_coef"] = smallk_config(event_ms, torch, L, _lib, dev, g)
+    out["in4096_out4096_k256_bf16_few_tokens"] = few_token_config(event_ms, torch, L, _lib, dev, g)
 
     out["in4096_out14336_k1024_T4096_bf16"] = llm_layer_config(event_ms, torch, L, _lib, dev, g)
     out["in768_out3072_k256_T8192_fp32"] = f32_layer_config(event_ms, torch, L, _lib, dev, g)
@@ -479,6 +505,8 @@ def main():
                     help="run only the headline layer with the fused random bias (projected calls + random-bias share) and exit")
     ap.add_argument("--smallk-only", action="store_true",
                     help="run only the fp32 4096 -> 4096, k = 16 forward at batch 1 / 16 / 256 and exit (profiling runs)")
+    ap.add_argument("--few-tokens-only", action="store_true",
+                    help="run only the bf16 4096 -> 4096, k = 256 calls at 1 / 16 / 64 tokens and exit (profiling runs)")
     ap.add_argument("--gpt-only", action="store_true",
                     help="run only the GPT-2 small training step with random-backed linears and exit (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -517,6 +545,9 @@ def main():
         del src, dst
     if args.smallk_only:
         print(json.dumps({"in4096_out4096_k16_fp32_matrix_coef": smallk_config(make_event_ms(torch), torch, L, _lib, dev, g)}))
+        return
+    if args.few_tokens_only:
+        print(json.dumps({"in4096_out4096_k256_bf16_few_tokens": few_token_config(make_event_ms(torch), torch, L, _lib, dev, g)}))
         return
     if args.gpt_only:
         print(json.dumps({"gpt2_small_12L_k256_seeds0to47_bf16_8x1024": gpt_step_config(make_event_ms(torch), torch, dev, g)}))

@@ -415,9 +415,25 @@ static int64_t vec_dcoef_workspace(const rdb_linear_desc *d)
     return dw + (rdb_materialize_bwd_workspace_bytes(0, d->k, 0, nw) + 255) / 256 * 256 + (rdb_scale_bias_bwd_workspace_bytes(nw) + 255) / 256 * 256;
 }
 
+static int64_t linear_workspace_bytes_main(int op, const rdb_linear_desc *d);
+
 extern "C" int64_t rdb_linear_workspace_bytes(int op, const rdb_linear_desc *d)
 {
     if (!d) return 0;
+    int64_t need = linear_workspace_bytes_main(op, d);
+    if (d->algo == RDB_ALGO_AUTO && d->act_dtype == RDB_BF16 && d->coef_rows != 0 &&
+        (op == RDB_OP_LINEAR_FWD || op == RDB_OP_LINEAR_BWD_DX || op == RDB_OP_LINEAR_BWD_DCOEF)) {
+        // bf16 with a few tokens: the vector-ALU kernels of rdb_smallk.hip come first (their scratch: partial [tokens x k] matrices)
+        rdb_linear_desc dd = *d;
+        if (op == RDB_OP_LINEAR_BWD_DCOEF) dd.coef_dtype = RDB_BF16;
+        const int64_t few = linear_smallk_workspace(&dd);
+        if (few > need) need = few;
+    }
+    return need;
+}
+
+static int64_t linear_workspace_bytes_main(int op, const rdb_linear_desc *d)
+{
     if (d->algo == RDB_ALGO_TILE || d->algo == RDB_ALGO_STRIP) return 0;
     if (d->coef_rows == 0) {   // vector-coef: the chunks' partial outputs; for the coefficient gradient dW and what its contraction needs
         if (d->algo != RDB_ALGO_AUTO) return 0;
@@ -467,6 +483,12 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
     if (d->algo == RDB_ALGO_AUTO && d->coef_rows == 0) {
         // vector-coef, up to a few thousand tokens, with room for the partial outputs: W tiles spread over all compute units
         rc = linear_fwd_vecsplit(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), workspace, workspace_bytes, s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
+    if (d->algo == RDB_ALGO_AUTO && d->act_dtype == RDB_BF16 && d->tokens <= 64) {
+        // a few tokens: the matrix-core kernels below would run a handful of blocks, each alone with a contraction over all of
+        // in_f; the vector-ALU kernels spread it over the chip (16 tokens x 4096 -> 4096, k = 256: 39 us against 12)
+        rc = linear_fwd_smallk(y, ldy, x, ldx, coef, scale_bias, bias, d, workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
     }
     if (d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) {
@@ -556,6 +578,10 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
     if (lddx < d->in_f || lddy < d->out_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dx: leading dimension smaller than the row");
     if (d->algo == RDB_ALGO_AUTO && d->coef_rows == 0) {
         rc = linear_dx_vecsplit(dx, lddx, dy, lddy, coef, scale_bias, d, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
+    }
+    if (d->algo == RDB_ALGO_AUTO && d->act_dtype == RDB_BF16 && d->tokens <= 64) {   // a few tokens: as in rdb_linear_fwd
+        rc = linear_dx_smallk(dx, lddx, dy, lddy, coef, scale_bias, d, workspace, workspace_bytes, (hipStream_t)stream);
         if (rc != RDB_E_UNSUPPORTED) return rc;
     }
     if (d->algo == RDB_ALGO_AUTO || d->algo == RDB_ALGO_FACTORED) {
@@ -706,6 +732,11 @@ extern "C" int rdb_linear_bwd_dcoef(float *dcoef, float *d_scale_bias, const voi
     if (!empty) {
         if (!dy || !x) return set_error(RDB_E_NULL, "rdb_linear_bwd_dcoef: dy or x is NULL");
         if (lddy < d->out_f || ldx < d->in_f) return set_error(RDB_E_SHAPE, "rdb_linear_bwd_dcoef: leading dimension smaller than the row");
+    }
+    if (!empty && d->algo == RDB_ALGO_AUTO && d->act_dtype == RDB_BF16 && d->coef_rows != 0 && d->tokens <= 64 && !d_scale_bias) {
+        // a few tokens: as in rdb_linear_fwd (dcoef is overwritten)
+        rc = linear_dcoef_smallk(dcoef, dy, lddy, x, ldx, d, workspace, workspace_bytes, s);
+        if (rc != RDB_E_UNSUPPORTED) return rc;
     }
     if (!empty && d->algo == RDB_ALGO_AUTO && ncoef > 0 && vec_dcoef_two_pass_ok(d)) {
         // vector-coef with room for dW in the workspace: dW formed once (on the matrix cores at fp32 accuracy), then every element

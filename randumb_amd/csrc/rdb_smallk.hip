@@ -1,7 +1,9 @@
-// Fused linear layer, matrix-coef + fp32, small coefficient dimension and few tokens (the GEMV-like regime): factored
-// algorithm on the vector ALU.
+// Fused linear layer, matrix-coef, few tokens (the GEMV-like regime): factored algorithm on the vector ALU, in fp32 whatever the
+// dtype of the operands (fp32, or bf16 activations and coefficients).  Two ranges: k <= 64 with up to 1024 tokens (fp32), and
+// k <= 256 with up to 64 tokens (both dtypes), where the matrix-core kernels would run a handful of blocks, each alone with a
+// long contraction.
 //
-// With k <= 64 and a handful of tokens the layer moves almost no data (x, C, y) and does almost no arithmetic once W = C . N
+// With a handful of tokens the layer moves almost no data (x, C, y) and does almost no arithmetic once W = C . N
 // is used associatively; what remains is the hash of N, in_f * k values per token tile:
 //   forward  z = x . N^T [T x k],  y = z . C^T (+ bias)
 //   dx       t = dy . C  [T x k],  dx = t . N
@@ -15,7 +17,9 @@ namespace rdb {
 
 constexpr int SK_TT = 8;    // tokens per block of the contracting kernel
 constexpr int SK_ET = 16;   // tokens per block of the expanding kernel
-constexpr int SK_MAX_K = 64;
+constexpr int SK_MAX_K = 64;      // the range with many tokens
+constexpr int SK_BIG_K = 256;     // the range with few tokens
+constexpr int SK_FEW_TOKENS = 64;
 
 // sum over the partial matrices p[ch][idx], ch = 0 .. nchunk-1, in chunk order; loads issued eight at a time
 __device__ __forceinline__ float sum_partials(const float *__restrict__ p, int64_t stride, int nchunk)
@@ -38,23 +42,25 @@ __device__ __forceinline__ float sum_partials(const float *__restrict__ p, int64
 // expanding kernel adds the chunks up in chunk order while it loads them.
 struct SkContract {
     float *out;          // [chunks][T][k] partial sums
-    const float *src;    // [T x J], leading dimension ld_src
+    const void *src;     // [T x J], leading dimension ld_src (elements of the kernel's type E)
     int64_t ld_src;
-    const float *coef;   // [J x k] (not HASH)
+    const void *coef;    // [J x k] (not HASH; E)
     int T, J, k;
     uint32_t seed;
 };
 
 // bx: token tile, by: chunk of 256 values of j.  The partial sums are stored at device scope: blocks of the same launch on
 // another die may be the ones that read them (smallk_fused_kernel).
-template <bool HASH> __device__ __forceinline__ void smallk_contract_block(const SkContract &p, int bx, int by)
+// MB: coefficients per block (m0 .. m0 + MB - 1; accumulators per thread: MB / 16 x 8 tokens): 64 where k <= 64, 32 where the
+// grid's z spreads a larger k over more blocks; E: float or bf16_t.
+template <int MB, typename E, bool HASH> __device__ __forceinline__ void smallk_contract_block(const SkContract &p, int bx, int by, int m0)
 {
-    constexpr int JC = 256, MC = SK_MAX_K / 16;
+    constexpr int JC = 256, MC = MB / 16;
     __shared__ float xs[SK_TT][JC];
     __shared__ float red[16][SK_TT][16];
     float *__restrict__ out = p.out;
-    const float *__restrict__ src = p.src;
-    const float *__restrict__ coef = p.coef;
+    const E *__restrict__ src = static_cast<const E *>(p.src);
+    const E *__restrict__ coef = static_cast<const E *>(p.coef);
     const int64_t lds_src = p.ld_src;
     const int T = p.T, J = p.J, k = p.k;
     const uint32_t seed = p.seed;
@@ -68,17 +74,17 @@ template <bool HASH> __device__ __forceinline__ void smallk_contract_block(const
     {
         const int jc = by * JC;
 #pragma unroll
-        for (int tt = 0; tt < SK_TT; ++tt) xs[tt][tid] = (t0 + tt < T && jc + tid < J) ? src[(int64_t)(t0 + tt) * lds_src + jc + tid] : 0.0f;
+        for (int tt = 0; tt < SK_TT; ++tt) xs[tt][tid] = (t0 + tt < T && jc + tid < J) ? elem<E>::load(src + (int64_t)(t0 + tt) * lds_src + jc + tid) : 0.0f;
         __syncthreads();
 #pragma unroll
         for (int c = 0; c < MC; ++c) {
-            const int m = c * 16 + m16;
-            if (c * 16 < k) {  // uniform
+            const int m = m0 + c * 16 + m16;
+            if (m0 + c * 16 < k) {  // uniform
                 uint32_t first = sq5_first((uint32_t)(jc + slice), (uint32_t)m, seed);
                 for (int jj = 0; jj < JC / 16; ++jj, first += 16u * PN1) {
                     const int j = jc + slice + 16 * jj;
                     // no branches in here: out-of-range (j, m) read a valid address and are zeroed by a select
-                    float b = HASH ? sq5_unit(sq5_tail(first)) : coef[(int64_t)(j < J ? j : J - 1) * k + (m < k ? m : k - 1)];
+                    float b = HASH ? sq5_unit(sq5_tail(first)) : elem<E>::load(coef + (int64_t)(j < J ? j : J - 1) * k + (m < k ? m : k - 1));
                     b = (m < k && j < J) ? b : 0.0f;
 #pragma unroll
                     for (int tt = 0; tt < SK_TT; ++tt) acc[c][tt] = fmaf(xs[tt][slice + 16 * jj], b, acc[c][tt]);
@@ -89,12 +95,12 @@ template <bool HASH> __device__ __forceinline__ void smallk_contract_block(const
     }
 #pragma unroll
     for (int c = 0; c < MC; ++c) {
-        if (c * 16 >= k) break;
+        if (m0 + c * 16 >= k) break;
 #pragma unroll
         for (int tt = 0; tt < SK_TT; ++tt) red[slice][tt][m16] = acc[c][tt];
         __syncthreads();
         if (tid < SK_TT * 16) {
-            const int tt = tid >> 4, m = c * 16 + m16;
+            const int tt = tid >> 4, m = m0 + c * 16 + m16;
             float s = 0.0f;
 #pragma unroll
             for (int sl = 0; sl < 16; ++sl) s += red[sl][tt][m16];
@@ -104,18 +110,21 @@ template <bool HASH> __device__ __forceinline__ void smallk_contract_block(const
     }
 }
 
-template <bool HASH> __global__ __launch_bounds__(256) void smallk_contract_kernel(SkContract p) { smallk_contract_block<HASH>(p, blockIdx.x, blockIdx.y); }
+template <int MB, typename E, bool HASH> __global__ __launch_bounds__(256) void smallk_contract_kernel(SkContract p)
+{
+    smallk_contract_block<MB, E, HASH>(p, blockIdx.x, blockIdx.y, blockIdx.z * MB);
+}
 
 // out[t, c] = sum_m src[t, m] * B(c, m) (+ bias[c]),  B(c, m) = noise(PRIME*c + m) (HASH) or coef[c, m]; c runs over the
 // cols = in_f or out_f.  Block = 256 columns x 16 tokens; a thread owns one column and keeps its 16 B values in registers.
 // src holds `nchunk` partial matrices [T x k] (from the contracting kernel), added up here in chunk order.
 struct SkExpand {
-    float *out;          // [T x cols], leading dimension ld_out
+    void *out;           // [T x cols], leading dimension ld_out (E)
     int64_t ld_out;
     const float *src;    // [nchunk][T][k] partial sums
     int nchunk;
-    const float *coef;   // [cols x k] (not HASH)
-    const float *bias;   // [cols] or NULL
+    const void *coef;    // [cols x k] (not HASH; E)
+    const void *bias;    // [cols] or NULL (E)
     int T, cols, k;
     uint32_t seed;
     // NULL, or slots [token tiles of SK_TT][nchunk] that contracting blocks of the same launch set to sync_tag; sync_count: one
@@ -128,13 +137,13 @@ struct SkExpand {
 };
 
 // bx: block of 256 columns, by: block of SK_ET tokens.
-template <bool HASH> __device__ __forceinline__ void smallk_expand_block(const SkExpand &p, int bx, int by)
+template <int KMAX, typename E, bool HASH> __device__ __forceinline__ void smallk_expand_block(const SkExpand &p, int bx, int by)
 {
-    __shared__ __align__(16) float s[SK_ET][SK_MAX_K];
-    float *__restrict__ out = p.out;
+    __shared__ __align__(16) float s[SK_ET][KMAX];
+    E *__restrict__ out = static_cast<E *>(p.out);
     const float *__restrict__ src = p.src;
-    const float *__restrict__ coef = p.coef;
-    const float *__restrict__ bias = p.bias;
+    const E *__restrict__ coef = static_cast<const E *>(p.coef);
+    const E *__restrict__ bias = static_cast<const E *>(p.bias);
     const int64_t ld_out = p.ld_out;
     const int nchunk = p.nchunk, T = p.T, cols = p.cols, k = p.k;
     const uint32_t seed = p.seed;
@@ -146,7 +155,7 @@ template <bool HASH> __device__ __forceinline__ void smallk_expand_block(const S
         const int cc = c < cols ? c : cols - 1;
 #pragma unroll
         for (int m = 0; m < 16; ++m) {  // branch-free: a column from k on reads a valid address and becomes 0
-            const float v = HASH ? sq5_unit(sq5_tail(sq5_first((uint32_t)cc, (uint32_t)m, seed))) : coef[(int64_t)cc * k + ((m < k) ? m : k - 1)];
+            const float v = HASH ? sq5_unit(sq5_tail(sq5_first((uint32_t)cc, (uint32_t)m, seed))) : elem<E>::load(coef + (int64_t)cc * k + ((m < k) ? m : k - 1));
             b0[m] = (m < k) ? v : 0.0f;
         }
     }
@@ -164,14 +173,14 @@ template <bool HASH> __device__ __forceinline__ void smallk_expand_block(const S
         if (verdict == 0) {   // gave up: the block's share of the output becomes NaN, never a sum of whatever is in memory
             if (c < cols)
                 for (int tt = 0; tt < SK_ET; ++tt)
-                    if (t0 + tt < T) out[(int64_t)(t0 + tt) * ld_out + c] = __uint_as_float(0x7fc00000u);
+                    if (t0 + tt < T) elem<E>::store(out + (int64_t)(t0 + tt) * ld_out + c, __uint_as_float(0x7fc00000u));
             return;
         }
     }
     // s = sum of the partial matrices in chunk order; columns from k on take part as zeros.  A thread owns up to 4 entries
     // and keeps the loads of 8 chunks of all of them in flight at once: the kernel is a chain of memory latencies otherwise.
     {
-        constexpr int PER = SK_ET * SK_MAX_K / 256;
+        constexpr int PER = SK_ET * KMAX / 256, CB = KMAX <= SK_MAX_K ? 8 : 4;
         float v[PER];
         const float *ptr[PER];
         bool ok[PER];
@@ -183,19 +192,19 @@ template <bool HASH> __device__ __forceinline__ void smallk_expand_block(const S
             ptr[i] = ok[i] ? src + (int64_t)(t0 + tt) * k + m : src;   // always a valid address
         }
         const int64_t stride = (int64_t)T * k;
-        for (int c0 = 0; c0 < nchunk; c0 += 8) {
-            float l[PER][8];
+        for (int c0 = 0; c0 < nchunk; c0 += CB) {
+            float l[PER][CB];
 #pragma unroll
             for (int i = 0; i < PER; ++i)
 #pragma unroll
-                for (int u = 0; u < 8; ++u)   // device scope: possibly written by another die during this launch
+                for (int u = 0; u < CB; ++u)   // device scope: possibly written by another die during this launch
                     l[i][u] = __hip_atomic_load(ptr[i] + (int64_t)((c0 + u < nchunk) ? c0 + u : nchunk - 1) * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
             for (int i = 0; i < PER; ++i)
 #pragma unroll
-                for (int u = 0; u < 8; ++u) v[i] += (ok[i] && c0 + u < nchunk) ? l[i][u] : 0.0f;
+                for (int u = 0; u < CB; ++u) v[i] += (ok[i] && c0 + u < nchunk) ? l[i][u] : 0.0f;
         }
-        for (int e = tid; e < SK_ET * SK_MAX_K; e += 256) s[e / SK_MAX_K][e % SK_MAX_K] = 0.0f;
+        for (int e = tid; e < SK_ET * KMAX; e += 256) s[e / KMAX][e % KMAX] = 0.0f;
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
@@ -217,11 +226,11 @@ template <bool HASH> __device__ __forceinline__ void smallk_expand_block(const S
 #pragma unroll
             for (int m = 0; m < 16; ++m) {
                 const float v = HASH ? sq5_unit(sq5_tail(sq5_first((uint32_t)c, (uint32_t)(mc + m), seed)))
-                                     : coef[(int64_t)c * k + ((mc + m < k) ? mc + m : k - 1)];
+                                     : elem<E>::load(coef + (int64_t)c * k + ((mc + m < k) ? mc + m : k - 1));
                 b[m] = (mc + m < k) ? v : 0.0f;
             }
         }
-        // mc <= 48 and m <= 15: always inside the 64 columns of s
+        // mc <= KMAX - 16 and m <= 15: always inside the KMAX columns of s
 #pragma unroll
         for (int tt = 0; tt < SK_ET; ++tt) {
             const f32x4 *row = reinterpret_cast<const f32x4 *>(&s[tt][mc]);
@@ -235,13 +244,118 @@ template <bool HASH> __device__ __forceinline__ void smallk_expand_block(const S
             }
         }
     }
-    const float bv = bias ? bias[c] : 0.0f;
+    const float bv = bias ? elem<E>::load(bias + c) : 0.0f;
 #pragma unroll
     for (int tt = 0; tt < SK_ET; ++tt)
-        if (t0 + tt < T) out[(int64_t)(t0 + tt) * ld_out + c] = acc[tt] + bv;
+        if (t0 + tt < T) elem<E>::store(out + (int64_t)(t0 + tt) * ld_out + c, acc[tt] + bv);
 }
 
-template <bool HASH> __global__ __launch_bounds__(256) void smallk_expand_kernel(SkExpand p) { smallk_expand_block<HASH>(p, blockIdx.x, blockIdx.y); }
+template <int KMAX, typename E, bool HASH> __global__ __launch_bounds__(256) void smallk_expand_kernel(SkExpand p)
+{
+    smallk_expand_block<KMAX, E, HASH>(p, blockIdx.x, blockIdx.y);
+}
+
+// The same for k up to 256 and few tokens, where one thread per column would leave the chip empty and every thread alone with
+// k values of B: block = 32 columns x 16 tokens, thread = (column, one of eight ranges of 32 coefficients); the ranges of a
+// column meet in LDS in range order.  The block's rows of C pass through LDS (read from memory along the rows, by the threads
+// along the columns).  A launch of its own, after the contracting kernel's.
+constexpr int SKW_COLS = 32, SKW_RANGES = 8;
+template <typename E, bool HASH> __global__ __launch_bounds__(256) void smallk_expand_wide_kernel(SkExpand p)
+{
+    constexpr int KW = SK_BIG_K, RANGE = KW / SKW_RANGES, CLD = KW + 1;
+    static_assert(SKW_COLS * SKW_RANGES == 256 && SK_ET % SKW_RANGES == 0 && RANGE % 16 == 0, "thread layout of the wide expansion");
+    __shared__ __align__(16) float s[SK_ET][KW];
+    __shared__ float cs[SKW_COLS * CLD];   // C rows, stride CLD (conflict-free down a column); later the ranges' sums [range][token][column]
+    static_assert(SKW_RANGES * SK_ET * SKW_COLS <= SKW_COLS * CLD, "the ranges' sums fit where the C rows were");
+    E *__restrict__ out = static_cast<E *>(p.out);
+    const float *__restrict__ src = p.src;
+    const E *__restrict__ coef = static_cast<const E *>(p.coef);
+    const E *__restrict__ bias = static_cast<const E *>(p.bias);
+    const int64_t ld_out = p.ld_out;
+    const int nchunk = p.nchunk, T = p.T, cols = p.cols, k = p.k;
+    const uint32_t seed = p.seed;
+    const int tid = threadIdx.x, col = tid % SKW_COLS, g = tid / SKW_COLS;
+    const int c0 = blockIdx.x * SKW_COLS, c = c0 + col, t0 = blockIdx.y * SK_ET;
+    const int cc = c < cols ? c : cols - 1;
+    if (!HASH) {   // rows c0 .. c0 + 31 of C are consecutive in memory: nrow * k values, thread after thread
+        const int nrow = (cols - c0 < SKW_COLS) ? cols - c0 : SKW_COLS;
+        const E *base = coef + (int64_t)c0 * k;
+        for (int e = tid; e < nrow * k; e += 256) cs[(e / k) * CLD + e % k] = elem<E>::load(base + e);
+    }
+    // s = sum of the partial matrices in chunk order; columns from k on take part as zeros
+    {
+        constexpr int PER = SK_ET * KW / 256, CB = 4;
+        float v[PER];
+        const float *ptr[PER];
+        bool ok[PER];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int e = tid + 256 * i, tt = e / k, m = e % k;   // entries e < SK_ET * k, row-major over (tt, m < k)
+            v[i] = 0.0f;
+            ok[i] = e < SK_ET * k && t0 + tt < T;
+            ptr[i] = ok[i] ? src + (int64_t)(t0 + tt) * k + m : src;   // always a valid address
+        }
+        const int64_t stride = (int64_t)T * k;
+        for (int q0 = 0; q0 < nchunk; q0 += CB) {
+            float l[PER][CB];
+#pragma unroll
+            for (int i = 0; i < PER; ++i)
+#pragma unroll
+                for (int u = 0; u < CB; ++u) l[i][u] = ptr[i][(int64_t)((q0 + u < nchunk) ? q0 + u : nchunk - 1) * stride];
+#pragma unroll
+            for (int i = 0; i < PER; ++i)
+#pragma unroll
+                for (int u = 0; u < CB; ++u) v[i] += (ok[i] && q0 + u < nchunk) ? l[i][u] : 0.0f;
+        }
+        for (int e = tid; e < SK_ET * KW; e += 256) s[e / KW][e % KW] = 0.0f;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int e = tid + 256 * i;
+            if (e < SK_ET * k) s[e / k][e % k] = v[i];
+        }
+    }
+    __syncthreads();
+    float acc[SK_ET];
+#pragma unroll
+    for (int tt = 0; tt < SK_ET; ++tt) acc[tt] = 0.0f;
+    const float *crow = cs + (c < cols ? col : 0) * CLD;
+    for (int mc = g * RANGE; mc < (g + 1) * RANGE && mc < k; mc += 16) {
+        float b[16];
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {   // branch-free: a coefficient from k on reads a valid address and becomes 0
+            const float v = HASH ? sq5_unit(sq5_tail(sq5_first((uint32_t)cc, (uint32_t)(mc + m), seed))) : crow[(mc + m < k) ? mc + m : k - 1];
+            b[m] = (mc + m < k) ? v : 0.0f;
+        }
+#pragma unroll
+        for (int tt = 0; tt < SK_ET; ++tt) {
+            const f32x4 *row = reinterpret_cast<const f32x4 *>(&s[tt][mc]);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const f32x4 sv = row[q];
+                acc[tt] = fmaf(sv[0], b[4 * q], acc[tt]);
+                acc[tt] = fmaf(sv[1], b[4 * q + 1], acc[tt]);
+                acc[tt] = fmaf(sv[2], b[4 * q + 2], acc[tt]);
+                acc[tt] = fmaf(sv[3], b[4 * q + 3], acc[tt]);
+            }
+        }
+    }
+    __syncthreads();   // everybody is done with the C rows
+    float *red = cs;
+#pragma unroll
+    for (int tt = 0; tt < SK_ET; ++tt) red[(g * SK_ET + tt) * SKW_COLS + col] = acc[tt];
+    __syncthreads();
+    if (c >= cols) return;
+    const float bv = bias ? elem<E>::load(bias + c) : 0.0f;
+#pragma unroll
+    for (int q = 0; q < SK_ET / SKW_RANGES; ++q) {   // this thread finishes two of the column's tokens
+        const int tt = g * (SK_ET / SKW_RANGES) + q;
+        float v = red[tt * SKW_COLS + col];
+#pragma unroll
+        for (int r = 1; r < SKW_RANGES; ++r) v += red[(r * SK_ET + tt) * SKW_COLS + col];
+        if (t0 + tt < T) elem<E>::store(out + (int64_t)(t0 + tt) * ld_out + c, v + bv);
+    }
+}
 
 // Both in one launch: the contracting blocks first, each publishing a tag when its partial sums are in memory, then the
 // expanding blocks, each waiting for the tags of its 16 tokens' tiles.  At a few tokens the two launches are most of the
@@ -254,7 +368,7 @@ struct SkFused {
     int c_tiles, c_blocks, e_colblocks;
 };
 
-template <bool CHASH> __global__ __launch_bounds__(256) void smallk_fused_kernel(SkFused p)
+template <int KMAX, typename E, bool CHASH> __global__ __launch_bounds__(256) void smallk_fused_kernel(SkFused p)
 {
     const int b = blockIdx.x;
     if (b < p.c_blocks) {
@@ -262,19 +376,20 @@ template <bool CHASH> __global__ __launch_bounds__(256) void smallk_fused_kernel
         // a replayed launch carries the tag it was recorded with: should a consumer of an earlier replay have given up, the slot
         // may still hold it (the consumers clear the slots only when all of them got past their wait)
         if (threadIdx.x == 0) __hip_atomic_store(p.slots + (int64_t)bx * p.e.nchunk + by, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        smallk_contract_block<CHASH>(p.c, bx, by);
+        smallk_contract_block<KMAX, E, CHASH>(p.c, bx, by, 0);
         if (by == 0 && bx % (SK_ET / SK_TT) == 0 && threadIdx.x == 0)
             __hip_atomic_store(p.counters + bx / (SK_ET / SK_TT), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         publish_tag(p.slots + (int64_t)bx * p.e.nchunk + by, p.e.sync_tag);
     } else {
         const int e = b - p.c_blocks;
-        smallk_expand_block<!CHASH>(p.e, e % p.e_colblocks, e / p.e_colblocks);
+        smallk_expand_block<KMAX, E, !CHASH>(p.e, e % p.e_colblocks, e / p.e_colblocks);
     }
 }
 
 // dC[o, m] = sum_t dy[t, o] * z[t, m].  Block = 256 output rows x one chunk of 16 coefficients; z goes through LDS in tiles
 // of 64 tokens; a thread owns one output row and walks the tokens in order.
-__global__ __launch_bounds__(256) void smallk_dcoef_kernel(float *__restrict__ dcoef, const float *__restrict__ dy, int64_t lddy,
+template <typename E>
+__global__ __launch_bounds__(256) void smallk_dcoef_kernel(float *__restrict__ dcoef, const E *__restrict__ dy, int64_t lddy,
                                                            const float *__restrict__ z, int nchunk, int T, int out_f, int k)
 {
     __shared__ __align__(16) float zs[64][16];
@@ -292,7 +407,7 @@ __global__ __launch_bounds__(256) void smallk_dcoef_kernel(float *__restrict__ d
         if (o < out_f) {
             const int n = (T - t0 < 64) ? T - t0 : 64;
             for (int tt = 0; tt < n; ++tt) {
-                const float g = dy[(int64_t)(t0 + tt) * lddy + o];
+                const float g = elem<E>::load(dy + (int64_t)(t0 + tt) * lddy + o);
 #pragma unroll
                 for (int m = 0; m < 16; ++m) acc[m] = fmaf(g, zs[tt][m], acc[m]);
             }
@@ -307,15 +422,35 @@ __global__ __launch_bounds__(256) void smallk_dcoef_kernel(float *__restrict__ d
 }
 
 // ----------------------------------------------------------------------------------------------- host side
-// The regime this file is for; AUTO additionally wants it to be the cheaper way.
+// The regimes this file is for; AUTO additionally wants the factored form to be the cheaper way.
 static bool smallk_ok(const rdb_linear_desc *d)
 {
-    return d->act_dtype == RDB_F32 && d->coef_dtype == RDB_F32 && d->coef_rows != 0 && d->k > 0 && d->k <= SK_MAX_K && d->tokens > 0 &&
-           d->tokens <= 4096 && d->in_f > 0 && d->out_f > 0 && d->in_f < (1 << 30) && d->out_f < (1 << 30);
+    const bool f32 = d->act_dtype == RDB_F32 && d->coef_dtype == RDB_F32, b16 = d->act_dtype == RDB_BF16 && d->coef_dtype == RDB_BF16;
+    if (!(f32 || b16) || d->coef_rows == 0 || d->k <= 0 || d->tokens <= 0 || d->in_f <= 0 || d->out_f <= 0 || d->in_f >= (1 << 30) ||
+        d->out_f >= (1 << 30))
+        return false;
+    if (f32 && d->k <= SK_MAX_K && d->tokens <= 4096) return true;
+    return d->k <= SK_BIG_K && d->tokens <= SK_FEW_TOKENS;
 }
-static bool smallk_wanted(const rdb_linear_desc *d)
+enum SkDirection { SK_FWD, SK_DX, SK_DCOEF };
+static bool smallk_wanted(const rdb_linear_desc *d, int dir)
 {
-    return d->algo == RDB_ALGO_FACTORED || (d->tokens <= 1024 && d->k * (d->in_f + d->out_f) < d->in_f * d->out_f);
+    const bool cheaper = d->k * (d->in_f + d->out_f) < d->in_f * d->out_f;
+    if (d->act_dtype == RDB_F32 && d->k <= SK_MAX_K) return d->algo == RDB_ALGO_FACTORED || (d->tokens <= 1024 && cheaper);
+    if (d->tokens > SK_FEW_TOKENS || !cheaper) return false;
+    if (d->k <= SK_MAX_K || dir == SK_DCOEF) return true;
+    // k beyond 64, forward and input gradient (contraction over J, expansion to cols).  Every expanding block adds up the
+    // partial matrices of its 16 tokens itself: beyond some 160 MB of such reads the matrix-core kernels are ahead again
+    // (64 tokens x 4096 -> 11008, k = 256: 55 us against 40; 4096 -> 4096: 27 against 39).  And in bf16 their time grows with the
+    // contraction (a few blocks, each alone with all of it): below about 1536 values they are ahead (768 -> 3072: 15 us
+    // against 17), beyond it behind (4096: 39 against 21).
+    const int64_t J = dir == SK_FWD ? d->in_f : d->out_f, cols = dir == SK_FWD ? d->out_f : d->in_f;
+    const int64_t resum = cdiv(cols, SKW_COLS) * cdiv(d->tokens, SK_ET) * cdiv(J, 256) * SK_ET * d->k * (int64_t)sizeof(float);
+    // (the bf16 input gradient's alternative is so slow on a long contraction that the bound is higher there: 64 tokens x
+    // 4096 -> 11008: 41 us against 72)
+    const int64_t cap = (dir == SK_DX && d->act_dtype == RDB_BF16) ? (400ll << 20) : (160ll << 20);
+    if (resum > cap) return false;
+    return d->act_dtype == RDB_F32 || J >= 1536;
 }
 
 // scratch: one partial [tokens x k] fp32 matrix per 256-chunk of the longer of in_f and out_f, then the tag slots of the
@@ -337,9 +472,9 @@ static bool ws_ok(const rdb_linear_desc *d, const void *ws, int64_t bytes) { ret
 
 // Contraction over J (the rows of src) then expansion to `cols` columns: one launch when an expanding block's tags fit one
 // wave's lanes (J <= 8192), two otherwise.
-template <bool CHASH>
-static int contract_expand(float *out, int64_t ld_out, int cols, const float *src, int64_t ld_src, int J, const float *coef, const float *bias,
-                           const rdb_linear_desc *d, void *workspace, hipStream_t s)
+template <int KMAX, typename E, bool CHASH>
+static int contract_expand_as(void *out, int64_t ld_out, int cols, const void *src, int64_t ld_src, int J, const void *coef, const void *bias,
+                              const rdb_linear_desc *d, void *workspace, hipStream_t s)
 {
     const int T = (int)d->tokens, k = (int)d->k;
     const int nchunk = (int)cdiv(J, 256), tiles = (int)cdiv(T, SK_TT);
@@ -358,13 +493,41 @@ static int contract_expand(float *out, int64_t ld_out, int cols, const float *sr
         f.counters = reinterpret_cast<unsigned int *>(f.slots + (int64_t)tiles * nchunk) + 2;
         f.e.sync_count = f.counters;
         f.e.sync_consumers = f.e_colblocks;
-        smallk_fused_kernel<CHASH><<<f.c_blocks + e_blocks, 256, 0, s>>>(f);
+        smallk_fused_kernel<KMAX, E, CHASH><<<f.c_blocks + e_blocks, 256, 0, s>>>(f);
         return check_launch("smallk_fused_kernel");
     }
-    smallk_contract_kernel<CHASH><<<dim3((unsigned)tiles, nchunk), 256, 0, s>>>(f.c);
+    smallk_contract_kernel<KMAX, E, CHASH><<<dim3((unsigned)tiles, nchunk), 256, 0, s>>>(f.c);
     if (int rc = check_launch("smallk_contract_kernel")) return rc;
-    smallk_expand_kernel<!CHASH><<<dim3((unsigned)f.e_colblocks, (unsigned)cdiv(T, SK_ET)), 256, 0, s>>>(f.e);
+    smallk_expand_kernel<KMAX, E, !CHASH><<<dim3((unsigned)f.e_colblocks, (unsigned)cdiv(T, SK_ET)), 256, 0, s>>>(f.e);
     return check_launch("smallk_expand_kernel");
+}
+// the instance for the request's k and dtype (activations and coefficients have the same one: smallk_ok)
+// k beyond 64 (few tokens): the contraction spread over the grid's z in ranges of SK_MB coefficients, then the wide expansion;
+// two launches
+constexpr int SK_MB = 32;
+template <typename E, bool CHASH>
+static int contract_expand_wide(void *out, int64_t ld_out, int cols, const void *src, int64_t ld_src, int J, const void *coef, const void *bias,
+                                const rdb_linear_desc *d, void *workspace, hipStream_t s)
+{
+    const int T = (int)d->tokens, k = (int)d->k, nchunk = (int)cdiv(J, 256);
+    if (nchunk > 65535) return RDB_E_UNSUPPORTED;   // the grid's y
+    const SkContract c = {(float *)workspace, src, ld_src, coef, T, J, k, d->seed};
+    const SkExpand e = {out, ld_out, (const float *)workspace, nchunk, coef, bias, T, cols, k, d->seed, nullptr, 0, {nullptr, nullptr, 0}, nullptr, 0};
+    smallk_contract_kernel<SK_MB, E, CHASH><<<dim3((unsigned)cdiv(T, SK_TT), nchunk, (unsigned)cdiv(k, SK_MB)), 256, 0, s>>>(c);
+    if (int rc = check_launch("smallk_contract_kernel")) return rc;
+    smallk_expand_wide_kernel<E, !CHASH><<<dim3((unsigned)cdiv(cols, SKW_COLS), (unsigned)cdiv(T, SK_ET)), 256, 0, s>>>(e);
+    return check_launch("smallk_expand_wide_kernel");
+}
+template <bool CHASH>
+static int contract_expand(void *out, int64_t ld_out, int cols, const void *src, int64_t ld_src, int J, const void *coef, const void *bias,
+                           const rdb_linear_desc *d, void *workspace, hipStream_t s)
+{
+    const bool b16 = d->act_dtype == RDB_BF16;
+    if (d->k <= SK_MAX_K)
+        return b16 ? contract_expand_as<SK_MAX_K, bf16_t, CHASH>(out, ld_out, cols, src, ld_src, J, coef, bias, d, workspace, s)
+                   : contract_expand_as<SK_MAX_K, float, CHASH>(out, ld_out, cols, src, ld_src, J, coef, bias, d, workspace, s);
+    return b16 ? contract_expand_wide<bf16_t, CHASH>(out, ld_out, cols, src, ld_src, J, coef, bias, d, workspace, s)
+               : contract_expand_wide<float, CHASH>(out, ld_out, cols, src, ld_src, J, coef, bias, d, workspace, s);
 }
 
 // Test hook: only the expanding blocks of the one-launch form, waiting (at most `polls` polls each) for a tag that nobody
@@ -372,17 +535,17 @@ static int contract_expand(float *out, int64_t ld_out, int cols, const float *sr
 int selftest_giveup_smallk(void *y, int64_t ldy, const void *coef, const rdb_linear_desc *d, void *workspace, int64_t workspace_bytes, int polls,
                            hipStream_t s)
 {
-    if (!smallk_ok(d) || !ws_ok(d, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    if (!smallk_ok(d) || d->act_dtype != RDB_F32 || d->k > SK_MAX_K || !ws_ok(d, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
     const int T = (int)d->tokens, k = (int)d->k, nchunk = (int)cdiv(d->in_f, 256), tiles = (int)cdiv(T, SK_TT);
     if (nchunk * (SK_ET / SK_TT) > 64) return RDB_E_UNSUPPORTED;
-    SkExpand e = {(float *)y, ldy, (const float *)workspace, nchunk, (const float *)coef, nullptr, T, (int)d->out_f, k, d->seed, nullptr, 0,
+    SkExpand e = {y, ldy, (const float *)workspace, nchunk, coef, nullptr, T, (int)d->out_f, k, d->seed, nullptr, 0,
                   {nullptr, nullptr, polls}, nullptr, 0};
     e.sync = reinterpret_cast<unsigned long long *>(static_cast<char *>(workspace) + partial_bytes(d));
     e.sync_tag = next_sync_tag();
     if (int rc = sync_giveups_ptr(&e.sync_wait.giveups)) return rc;
     e.sync_count = reinterpret_cast<unsigned int *>(e.sync + (int64_t)tiles * nchunk) + 2;
     e.sync_consumers = (int)cdiv(d->out_f, 256);
-    smallk_expand_kernel<false><<<dim3((unsigned)cdiv(d->out_f, 256), (unsigned)cdiv(T, SK_ET)), 256, 0, s>>>(e);
+    smallk_expand_kernel<SK_MAX_K, float, false><<<dim3((unsigned)cdiv(d->out_f, 256), (unsigned)cdiv(T, SK_ET)), 256, 0, s>>>(e);
     return check_launch("smallk_expand_kernel (self-test)");
 }
 
@@ -393,20 +556,18 @@ int linear_fwd_smallk(void *y, int64_t ldy, const void *x, int64_t ldx, const vo
     // a layer with a handful of output features (a classifier head) gives the kernel that forms W tiles one column of blocks,
     // each hashing all of N: the factored form wins there whatever the flop counts say (256 -> 10, k = 64, 128 tokens: 19 us
     // against 57)
-    const bool few_outputs = d->tokens <= 1024 && d->out_f <= 32;
-    if (!smallk_ok(d) || scale_bias || !(smallk_wanted(d) || few_outputs) || !ws_ok(d, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    const bool few_outputs = d->act_dtype == RDB_F32 && d->k <= SK_MAX_K && d->tokens <= 1024 && d->out_f <= 32;
+    if (!smallk_ok(d) || scale_bias || !(smallk_wanted(d, SK_FWD) || few_outputs) || !ws_ok(d, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
     // z = x . N^T (hashed), y = z . C^T + bias
-    return contract_expand<true>((float *)y, ldy, (int)d->out_f, (const float *)x, ldx, (int)d->in_f, (const float *)coef, (const float *)bias, d,
-                                 workspace, s);
+    return contract_expand<true>(y, ldy, (int)d->out_f, x, ldx, (int)d->in_f, coef, bias, d, workspace, s);
 }
 
 int linear_dx_smallk(void *dx, int64_t lddx, const void *dy, int64_t lddy, const void *coef, const void *scale_bias, const rdb_linear_desc *d,
                      void *workspace, int64_t workspace_bytes, hipStream_t s)
 {
-    if (!smallk_ok(d) || scale_bias || !smallk_wanted(d) || !ws_ok(d, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    if (!smallk_ok(d) || scale_bias || !smallk_wanted(d, SK_DX) || !ws_ok(d, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
     // t = dy . C, dx = t . N (hashed)
-    return contract_expand<false>((float *)dx, lddx, (int)d->in_f, (const float *)dy, lddy, (int)d->out_f, (const float *)coef, nullptr, d,
-                                  workspace, s);
+    return contract_expand<false>(dx, lddx, (int)d->in_f, dy, lddy, (int)d->out_f, coef, nullptr, d, workspace, s);
 }
 
 // dcoef is overwritten (no zero fill needed).
@@ -414,17 +575,27 @@ int linear_dcoef_smallk(float *dcoef, const void *dy, int64_t lddy, const void *
                         int64_t workspace_bytes, hipStream_t s)
 {
     rdb_linear_desc dd = *d;
-    dd.coef_dtype = RDB_F32;  // no coefficients are read here
-    if (!smallk_ok(&dd) || !smallk_wanted(&dd) || !ws_ok(&dd, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
+    dd.coef_dtype = d->act_dtype;  // no coefficients are read here
+    if (!smallk_ok(&dd) || !smallk_wanted(&dd, SK_DCOEF) || !ws_ok(&dd, workspace, workspace_bytes)) return RDB_E_UNSUPPORTED;
     const int T = (int)d->tokens, k = (int)d->k;
+    const bool b16 = d->act_dtype == RDB_BF16;
     float *z = (float *)workspace;
     const int nchunk = (int)cdiv(d->in_f, 256);
-    const SkContract c = {z, (const float *)x, ldx, nullptr, T, (int)d->in_f, k, d->seed};
-    smallk_contract_kernel<true><<<dim3((unsigned)cdiv(T, SK_TT), nchunk), 256, 0, s>>>(c);
+    const SkContract c = {z, x, ldx, nullptr, T, (int)d->in_f, k, d->seed};
+    const dim3 cgrid((unsigned)cdiv(T, SK_TT), nchunk);
+    if (k <= SK_MAX_K) {
+        if (b16) smallk_contract_kernel<SK_MAX_K, bf16_t, true><<<cgrid, 256, 0, s>>>(c);
+        else smallk_contract_kernel<SK_MAX_K, float, true><<<cgrid, 256, 0, s>>>(c);
+    } else {
+        const dim3 wgrid(cgrid.x, cgrid.y, (unsigned)cdiv(k, SK_MB));
+        if (b16) smallk_contract_kernel<SK_MB, bf16_t, true><<<wgrid, 256, 0, s>>>(c);
+        else smallk_contract_kernel<SK_MB, float, true><<<wgrid, 256, 0, s>>>(c);
+    }
     int rc = check_launch("smallk_contract_kernel<hash>");
     if (rc) return rc;
     dim3 grid((unsigned)cdiv(d->out_f, 256), (unsigned)cdiv(k, 16));
-    smallk_dcoef_kernel<<<grid, 256, 0, s>>>(dcoef, (const float *)dy, lddy, z, nchunk, T, (int)d->out_f, k);
+    if (b16) smallk_dcoef_kernel<bf16_t><<<grid, 256, 0, s>>>(dcoef, (const bf16_t *)dy, lddy, z, nchunk, T, (int)d->out_f, k);
+    else smallk_dcoef_kernel<float><<<grid, 256, 0, s>>>(dcoef, (const float *)dy, lddy, z, nchunk, T, (int)d->out_f, k);
     return check_launch("smallk_dcoef_kernel");
 }
 

@@ -240,6 +240,67 @@ def test_small_k_fp32_ragged_shapes(hip, oracle):
     assert rel_l2(cpu(dx), want_dx) < F32_TOL and rel_l2(cpu(dC), want_dC) < F32_TOL
 
 
+FEW_TOKEN_CASES = [(1, 2048, 1024, 256, False), (16, 1024, 2048, 256, True), (64, 1024, 768, 128, False), (33, 777, 555, 99, True),
+                   (5, 8448, 512, 72, False)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,in_f,out_f,k,with_bias", FEW_TOKEN_CASES)
+def test_few_token_regime_up_to_k_256(hip, oracle, dtype, T, in_f, out_f, k, with_bias):
+    """Up to 64 tokens with k up to 256, both dtypes: the vector-ALU kernels compute in fp32 whatever the operands' dtype, so on
+    bf16 operands y and dx carry one rounding to bf16 (rel-L2 about 1e-3; the bf16 matrix-core kernels, which also round z and
+    t, are near 3e-3: the threshold between them shows which kernels ran) and the coefficient gradient, an fp32 result, meets
+    the fp32 tolerance.  The last case contracts over
+    more than 8192 features (two launches), the odd one divides nothing."""
+    print(f"case few tokens: {dtype} T={T} {in_f}->{out_f} k={k} bias={with_bias}", flush=True)
+    seed = 31
+    g = torch.Generator().manual_seed(T + k)
+    x = torch.randn(T, in_f, generator=g).to(dtype)
+    dy = torch.randn(T, out_f, generator=g).to(dtype)
+    C = (torch.randn(out_f, k, generator=g) * (3.0 / k) ** 0.5 / 32.0).to(dtype)
+    bias = torch.randn(out_f, generator=g).to(dtype) if with_bias else None
+    y = hip.linear_fwd(x.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, bias=None if bias is None else bias.cuda())
+    dx = hip.linear_bwd_dx(dy.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed)
+    dC, _ = hip.linear_bwd_dcoef(dy.cuda(), x.cuda(), k, out_f, in_f, out_f, in_f, 1, seed)
+    assert y.dtype == dtype and dx.dtype == dtype and dC.dtype == torch.float32
+    xn, dyn, Cn = x.float().numpy(), dy.float().numpy(), C.float().numpy()
+    want_y = oracle.linear_fwd(xn, Cn, in_f, out_f, seed, bias=None if bias is None else bias.float().numpy())
+    want_dx, want_dC, _ = oracle.linear_bwd(xn, dyn, Cn, in_f, out_f, seed)
+    # in bf16 the library takes these kernels for a direction whose contraction is long enough (1536 values) to leave the
+    # matrix-core kernels behind; the coefficient gradient always
+    tol_y = F32_TOL if dtype == torch.float32 else 2e-3 if in_f >= 1536 else BF16_TOL
+    tol_dx = F32_TOL if dtype == torch.float32 else 2e-3 if out_f >= 1536 else BF16_TOL
+    assert rel_l2(cpu(y), want_y) < tol_y
+    assert rel_l2(cpu(dx), want_dx) < tol_dx
+    assert rel_l2(cpu(dC), want_dC) < F32_TOL
+    # bit for bit run to run (fixed summation order, no atomics)
+    assert torch.equal(y, hip.linear_fwd(x.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, bias=None if bias is None else bias.cuda()))
+    assert torch.equal(dC, hip.linear_bwd_dcoef(dy.cuda(), x.cuda(), k, out_f, in_f, out_f, in_f, 1, seed)[0])
+
+
+def test_few_token_layer_through_the_surface(ra, hip, oracle):
+    """A bf16 SillyLinear-shaped call with 8 tokens through ops.linear (autograd): takes the one-call entry points, not the
+    projected form, and agrees with the oracle."""
+    print("case few tokens through the surface", flush=True)
+    from randumb_amd import ops
+
+    T, in_f, out_f, k, seed = 8, 2048, 1536, 256, 5
+    assert not hip.linear_projection_preferred(T, in_f, out_f, k, torch.bfloat16)
+    assert hip.linear_projection_preferred(T, 1024, 1024, k, torch.bfloat16)   # short contractions: the matrix-core kernels
+    assert hip.linear_projection_preferred(4096, in_f, out_f, k, torch.bfloat16)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(T, in_f, generator=g).bfloat16().cuda().requires_grad_(True)
+    C = (torch.randn(out_f, k, generator=g) * 0.01).bfloat16().cuda().requires_grad_(True)
+    dy = torch.randn(T, out_f, generator=g).bfloat16().cuda()
+    y = ops.linear(x, C, in_f, out_f, in_f, 1, seed, None, None)
+    y.backward(dy)
+    xn, dyn, Cn = cpu(x), cpu(dy), cpu(C)
+    want_dx, want_dC, _ = oracle.linear_bwd(xn, dyn, Cn, in_f, out_f, seed)
+    assert rel_l2(cpu(y), oracle.linear_fwd(xn, Cn, in_f, out_f, seed)) < 2e-3
+    assert rel_l2(cpu(x.grad), want_dx) < 2e-3
+    assert rel_l2(cpu(C.grad), want_dC) < 4e-3   # the gradient leaves in the coefficients' dtype
+
+
 GPT2_SHAPES = [("qkv", 768, 2304), ("proj", 768, 768), ("fc", 768, 3072), ("mlp_proj", 3072, 768)]
 
 
