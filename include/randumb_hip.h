@@ -145,8 +145,9 @@ enum {
     RDB_ALGO_FACTORED = 3 /* matrix-coef only: use W = C.N associatively so that no weight tile is formed:
                              y = (x.N^T).C^T, dx = (dy.C).N, dcoef = dy^T.(x.N^T); the [tokens x k] intermediate lives in
                              the caller's workspace.  bf16 activations and coef (sizes multiples of 8): bf16 matrix cores;
-                             fp32, or bf16 with other sizes: fp32 matrix cores, or the vector ALU for k <= 64 and few
-                             tokens; partial sums are added in a fixed order.  With scale_bias the full-rank share s.R is
+                             fp32, or bf16 with other sizes: fp32 matrix cores; a few tokens (k <= 64 in fp32 up to 1024
+                             tokens; under AUTO also k <= 256 up to 64 tokens in either dtype): the vector ALU, in fp32;
+                             partial sums are added in a fixed order.  With scale_bias the full-rank share s.R is
                              one more product with R hashed as an operand. */
 };
 

@@ -273,9 +273,15 @@ def test_few_token_regime_up_to_k_256(hip, oracle, dtype, T, in_f, out_f, k, wit
     assert rel_l2(cpu(y), want_y) < tol_y
     assert rel_l2(cpu(dx), want_dx) < tol_dx
     assert rel_l2(cpu(dC), want_dC) < F32_TOL
-    # bit for bit run to run (fixed summation order, no atomics)
+    # bit for bit run to run (fixed summation order, no atomics), and as separate launches
     assert torch.equal(y, hip.linear_fwd(x.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, bias=None if bias is None else bias.cuda()))
     assert torch.equal(dC, hip.linear_bwd_dcoef(dy.cuda(), x.cuda(), k, out_f, in_f, out_f, in_f, 1, seed)[0])
+    before = hip.set_one_launch(0)
+    try:
+        assert torch.equal(y, hip.linear_fwd(x.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, bias=None if bias is None else bias.cuda()))
+        assert torch.equal(dx, hip.linear_bwd_dx(dy.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed))
+    finally:
+        hip.set_one_launch(before)
 
 
 def test_few_token_layer_through_the_surface(ra, hip, oracle):
