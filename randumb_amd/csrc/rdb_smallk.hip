@@ -180,16 +180,19 @@ template <int KMAX, typename E, bool HASH> __device__ __forceinline__ void small
     // s = sum of the partial matrices in chunk order; columns from k on take part as zeros.  A thread owns up to 4 entries
     // and keeps the loads of 8 chunks of all of them in flight at once: the kernel is a chain of memory latencies otherwise.
     {
-        constexpr int PER = SK_ET * KMAX / 256, CB = KMAX <= SK_MAX_K ? 8 : 4;
+        // entry i of a thread: token (tid / KMAX) + (256 / KMAX) i, coefficient tid % KMAX (no division by k)
+        constexpr int PER = SK_ET * KMAX / 256, CB = 8, TSTEP = 256 / KMAX;
+        static_assert(256 % KMAX == 0 && SK_ET % TSTEP == 0, "the tile's entries split evenly over the threads");
+        const int em = tid % KMAX, et = tid / KMAX;
         float v[PER];
         const float *ptr[PER];
         bool ok[PER];
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int e = tid + 256 * i, tt = e / k, m = e % k;   // entries e < SK_ET * k, row-major over (tt, m < k)
+            const int tt = et + TSTEP * i;
             v[i] = 0.0f;
-            ok[i] = e < SK_ET * k && t0 + tt < T;
-            ptr[i] = ok[i] ? src + (int64_t)(t0 + tt) * k + m : src;   // always a valid address
+            ok[i] = em < k && t0 + tt < T;
+            ptr[i] = ok[i] ? src + (int64_t)(t0 + tt) * k + em : src;   // always a valid address
         }
         const int64_t stride = (int64_t)T * k;
         for (int c0 = 0; c0 < nchunk; c0 += CB) {
@@ -204,13 +207,8 @@ template <int KMAX, typename E, bool HASH> __device__ __forceinline__ void small
 #pragma unroll
                 for (int u = 0; u < CB; ++u) v[i] += (ok[i] && c0 + u < nchunk) ? l[i][u] : 0.0f;
         }
-        for (int e = tid; e < SK_ET * KMAX; e += 256) s[e / KMAX][e % KMAX] = 0.0f;
-        __syncthreads();
 #pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            const int e = tid + 256 * i;
-            if (e < SK_ET * k) s[e / k][e % k] = v[i];
-        }
+        for (int i = 0; i < PER; ++i) s[et + TSTEP * i][em] = ok[i] ? v[i] : 0.0f;   // every entry of s is somebody's
     }
     __syncthreads();
     if (c >= cols) return;
@@ -255,10 +253,28 @@ template <int KMAX, typename E, bool HASH> __global__ __launch_bounds__(256) voi
     smallk_expand_block<KMAX, E, HASH>(p, blockIdx.x, blockIdx.y);
 }
 
+// zsum[e] = part[0][e] + part[1][e] + ... in chunk order, one entry [token, coefficient] per thread: k beyond 64, where many
+// expanding blocks share a token's partial matrices and each of them adding them up again costs more than this launch
+__global__ __launch_bounds__(256) void smallk_sum_chunks_kernel(float *__restrict__ zsum, const float *__restrict__ part, int64_t n, int nchunk)
+{
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= n) return;
+    float v = 0.0f;
+    for (int c0 = 0; c0 < nchunk; c0 += 16) {
+        float l[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) l[u] = part[(int64_t)((c0 + u < nchunk) ? c0 + u : nchunk - 1) * n + e];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) v += (c0 + u < nchunk) ? l[u] : 0.0f;
+    }
+    zsum[e] = v;
+}
+
 // The same for k up to 256 and few tokens, where one thread per column would leave the chip empty and every thread alone with
 // k values of B: block = 32 columns x 16 tokens, thread = (column, one of eight ranges of 32 coefficients); the ranges of a
 // column meet in LDS in range order.  The block's rows of C pass through LDS (read from memory along the rows, by the threads
-// along the columns).  A launch of its own, after the contracting kernel's.
+// along the columns).  A launch of its own, after the contracting kernel's and smallk_sum_chunks_kernel's (src = the sum,
+// nchunk = 1).
 constexpr int SKW_COLS = 32, SKW_RANGES = 8;
 template <typename E, bool HASH> __global__ __launch_bounds__(256) void smallk_expand_wide_kernel(SkExpand p)
 {
@@ -277,43 +293,58 @@ template <typename E, bool HASH> __global__ __launch_bounds__(256) void smallk_e
     const int tid = threadIdx.x, col = tid % SKW_COLS, g = tid / SKW_COLS;
     const int c0 = blockIdx.x * SKW_COLS, c = c0 + col, t0 = blockIdx.y * SK_ET;
     const int cc = c < cols ? c : cols - 1;
-    if (!HASH) {   // rows c0 .. c0 + 31 of C are consecutive in memory: nrow * k values, thread after thread
-        const int nrow = (cols - c0 < SKW_COLS) ? cols - c0 : SKW_COLS;
-        const E *base = coef + (int64_t)c0 * k;
-        for (int e = tid; e < nrow * k; e += 256) cs[(e / k) * CLD + e % k] = elem<E>::load(base + e);
+    if (!HASH) {
+        // the block's rows of C: a wave reads 64 consecutive values of one row at a time; all of a thread's 32 loads are in
+        // flight before the first is stored (rows past cols and coefficients past k: zeros)
+        const int r0 = tid >> 6, m0 = tid & 63;
+        float cv[SKW_COLS / 4][KW / 64];
+#pragma unroll
+        for (int r = 0; r < SKW_COLS / 4; ++r)
+#pragma unroll
+            for (int j = 0; j < KW / 64; ++j) {
+                const int row = r0 + 4 * r, m = m0 + 64 * j;
+                const bool in = c0 + row < cols && m < k;   // (a valid address either way; the select makes the zero)
+                const float x = elem<E>::load(coef + (int64_t)(c0 + row < cols ? c0 + row : cols - 1) * k + (m < k ? m : k - 1));
+                cv[r][j] = in ? x : 0.0f;
+            }
+#pragma unroll
+        for (int r = 0; r < SKW_COLS / 4; ++r)
+#pragma unroll
+            for (int j = 0; j < KW / 64; ++j) cs[(r0 + 4 * r) * CLD + m0 + 64 * j] = cv[r][j];
     }
-    // s = sum of the partial matrices in chunk order; columns from k on take part as zeros
+    // s = sum of the partial matrices in chunk order (as a rule one: smallk_sum_chunks_kernel ran first); thread = coefficient,
+    // one entry per token; coefficients from k on and tokens past the end take part as zeros
     {
-        constexpr int PER = SK_ET * KW / 256, CB = 4;
-        float v[PER];
-        const float *ptr[PER];
-        bool ok[PER];
-#pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            const int e = tid + 256 * i, tt = e / k, m = e % k;   // entries e < SK_ET * k, row-major over (tt, m < k)
-            v[i] = 0.0f;
-            ok[i] = e < SK_ET * k && t0 + tt < T;
-            ptr[i] = ok[i] ? src + (int64_t)(t0 + tt) * k + m : src;   // always a valid address
-        }
+        static_assert(KW == 256, "one coefficient per thread");
+        constexpr int CB = 4;
+        // no branches around the loads: an entry that does not exist reads a valid address and becomes 0 by a select
+        const int m = tid < k ? tid : k - 1;
+        float v[SK_ET];
+        const float *ptr[SK_ET];
         const int64_t stride = (int64_t)T * k;
-        for (int q0 = 0; q0 < nchunk; q0 += CB) {
-            float l[PER][CB];
 #pragma unroll
-            for (int i = 0; i < PER; ++i)
-#pragma unroll
-                for (int u = 0; u < CB; ++u) l[i][u] = ptr[i][(int64_t)((q0 + u < nchunk) ? q0 + u : nchunk - 1) * stride];
-#pragma unroll
-            for (int i = 0; i < PER; ++i)
-#pragma unroll
-                for (int u = 0; u < CB; ++u) v[i] += (ok[i] && q0 + u < nchunk) ? l[i][u] : 0.0f;
+        for (int i = 0; i < SK_ET; ++i) {
+            v[i] = 0.0f;
+            ptr[i] = src + (int64_t)(t0 + i < T ? t0 + i : T - 1) * k + m;
         }
-        for (int e = tid; e < SK_ET * KW; e += 256) s[e / KW][e % KW] = 0.0f;
-        __syncthreads();
+        if (nchunk == 1) {
 #pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            const int e = tid + 256 * i;
-            if (e < SK_ET * k) s[e / k][e % k] = v[i];
+            for (int i = 0; i < SK_ET; ++i) v[i] = ptr[i][0];
+        } else {
+            for (int q0 = 0; q0 < nchunk; q0 += CB) {
+                float l[SK_ET][CB];
+#pragma unroll
+                for (int i = 0; i < SK_ET; ++i)
+#pragma unroll
+                    for (int u = 0; u < CB; ++u) l[i][u] = ptr[i][(int64_t)((q0 + u < nchunk) ? q0 + u : nchunk - 1) * stride];
+#pragma unroll
+                for (int i = 0; i < SK_ET; ++i)
+#pragma unroll
+                    for (int u = 0; u < CB; ++u) v[i] += (q0 + u < nchunk) ? l[i][u] : 0.0f;
+            }
         }
+#pragma unroll
+        for (int i = 0; i < SK_ET; ++i) s[i][tid] = (tid < k && t0 + i < T) ? v[i] : 0.0f;
     }
     __syncthreads();
     float acc[SK_ET];
@@ -324,7 +355,7 @@ template <typename E, bool HASH> __global__ __launch_bounds__(256) void smallk_e
         float b[16];
 #pragma unroll
         for (int m = 0; m < 16; ++m) {   // branch-free: a coefficient from k on reads a valid address and becomes 0
-            const float v = HASH ? sq5_unit(sq5_tail(sq5_first((uint32_t)cc, (uint32_t)(mc + m), seed))) : crow[(mc + m < k) ? mc + m : k - 1];
+            const float v = HASH ? sq5_unit(sq5_tail(sq5_first((uint32_t)cc, (uint32_t)(mc + m), seed))) : crow[mc + m];   // zeros from k on
             b[m] = (mc + m < k) ? v : 0.0f;
         }
 #pragma unroll
@@ -439,17 +470,10 @@ static bool smallk_wanted(const rdb_linear_desc *d, int dir)
     if (d->act_dtype == RDB_F32 && d->k <= SK_MAX_K) return d->algo == RDB_ALGO_FACTORED || (d->tokens <= 1024 && cheaper);
     if (d->tokens > SK_FEW_TOKENS || !cheaper) return false;
     if (d->k <= SK_MAX_K || dir == SK_DCOEF) return true;
-    // k beyond 64, forward and input gradient (contraction over J, expansion to cols).  Every expanding block adds up the
-    // partial matrices of its 16 tokens itself: beyond some 160 MB of such reads the matrix-core kernels are ahead again
-    // (64 tokens x 4096 -> 11008, k = 256: 55 us against 40; 4096 -> 4096: 27 against 39).  And in bf16 their time grows with the
-    // contraction (a few blocks, each alone with all of it): below about 1536 values they are ahead (768 -> 3072: 15 us
-    // against 17), beyond it behind (4096: 39 against 21).
-    const int64_t J = dir == SK_FWD ? d->in_f : d->out_f, cols = dir == SK_FWD ? d->out_f : d->in_f;
-    const int64_t resum = cdiv(cols, SKW_COLS) * cdiv(d->tokens, SK_ET) * cdiv(J, 256) * SK_ET * d->k * (int64_t)sizeof(float);
-    // (the bf16 input gradient's alternative is so slow on a long contraction that the bound is higher there: 64 tokens x
-    // 4096 -> 11008: 41 us against 72)
-    const int64_t cap = (dir == SK_DX && d->act_dtype == RDB_BF16) ? (400ll << 20) : (160ll << 20);
-    if (resum > cap) return false;
+    // k beyond 64, forward and input gradient (contraction over J): in bf16 the matrix-core kernels' time grows with the
+    // contraction (a few blocks, each alone with all of it): below about 1536 values they are ahead (768 -> 3072: 15 us against
+    // 17), beyond it behind (4096: 39 against 17)
+    const int64_t J = dir == SK_FWD ? d->in_f : d->out_f;
     return d->act_dtype == RDB_F32 || J >= 1536;
 }
 
@@ -461,9 +485,12 @@ static int64_t partial_bytes(const rdb_linear_desc *d)
     const int64_t longer = d->in_f > d->out_f ? d->in_f : d->out_f;
     return (cdiv(longer, 256) * d->tokens * d->k * (int64_t)sizeof(float) + 7) / 8 * 8;
 }
+// k beyond 64: behind the partial matrices their sum [tokens x k]
+static int64_t zsum_bytes(const rdb_linear_desc *d) { return (d->tokens * d->k * (int64_t)sizeof(float) + 7) / 8 * 8; }
 int64_t linear_smallk_workspace(const rdb_linear_desc *d)
 {
     if (!smallk_ok(d)) return 0;
+    if (d->k > SK_MAX_K) return partial_bytes(d) + zsum_bytes(d);
     const int64_t longer = d->in_f > d->out_f ? d->in_f : d->out_f;
     return partial_bytes(d) + cdiv(d->tokens, SK_TT) * cdiv(longer, 256) * 8 + 8 + cdiv(d->tokens, SK_ET) * 8;
 }
@@ -502,9 +529,15 @@ static int contract_expand_as(void *out, int64_t ld_out, int cols, const void *s
     return check_launch("smallk_expand_kernel");
 }
 // the instance for the request's k and dtype (activations and coefficients have the same one: smallk_ok)
-// k beyond 64 (few tokens): the contraction spread over the grid's z in ranges of SK_MB coefficients, then the wide expansion;
-// two launches
+// k beyond 64 (few tokens): the contraction spread over the grid's z in ranges of SK_MB coefficients, the sum of its chunks,
+// then the wide expansion; three launches
 constexpr int SK_MB = 32;
+static int sum_chunks(float *zsum, const float *part, const rdb_linear_desc *d, int nchunk, hipStream_t s)
+{
+    const int64_t n = d->tokens * d->k;
+    smallk_sum_chunks_kernel<<<(unsigned)cdiv(n, 256), 256, 0, s>>>(zsum, part, n, nchunk);
+    return check_launch("smallk_sum_chunks_kernel");
+}
 template <typename E, bool CHASH>
 static int contract_expand_wide(void *out, int64_t ld_out, int cols, const void *src, int64_t ld_src, int J, const void *coef, const void *bias,
                                 const rdb_linear_desc *d, void *workspace, hipStream_t s)
@@ -512,9 +545,11 @@ static int contract_expand_wide(void *out, int64_t ld_out, int cols, const void 
     const int T = (int)d->tokens, k = (int)d->k, nchunk = (int)cdiv(J, 256);
     if (nchunk > 65535) return RDB_E_UNSUPPORTED;   // the grid's y
     const SkContract c = {(float *)workspace, src, ld_src, coef, T, J, k, d->seed};
-    const SkExpand e = {out, ld_out, (const float *)workspace, nchunk, coef, bias, T, cols, k, d->seed, nullptr, 0, {nullptr, nullptr, 0}, nullptr, 0};
+    float *zsum = reinterpret_cast<float *>(static_cast<char *>(workspace) + partial_bytes(d));
+    const SkExpand e = {out, ld_out, zsum, 1, coef, bias, T, cols, k, d->seed, nullptr, 0, {nullptr, nullptr, 0}, nullptr, 0};
     smallk_contract_kernel<SK_MB, E, CHASH><<<dim3((unsigned)cdiv(T, SK_TT), nchunk, (unsigned)cdiv(k, SK_MB)), 256, 0, s>>>(c);
     if (int rc = check_launch("smallk_contract_kernel")) return rc;
+    if (int rc = sum_chunks(zsum, (const float *)workspace, d, nchunk, s)) return rc;
     smallk_expand_wide_kernel<E, !CHASH><<<dim3((unsigned)cdiv(cols, SKW_COLS), (unsigned)cdiv(T, SK_ET)), 256, 0, s>>>(e);
     return check_launch("smallk_expand_wide_kernel");
 }
@@ -593,9 +628,17 @@ int linear_dcoef_smallk(float *dcoef, const void *dy, int64_t lddy, const void *
     }
     int rc = check_launch("smallk_contract_kernel<hash>");
     if (rc) return rc;
+    const float *zz = z;
+    int zchunks = nchunk;
+    if (k > SK_MAX_K) {   // every block of the kernel below would add the chunks up again
+        float *zsum = reinterpret_cast<float *>(static_cast<char *>(workspace) + partial_bytes(&dd));
+        if ((rc = sum_chunks(zsum, z, &dd, nchunk, s))) return rc;
+        zz = zsum;
+        zchunks = 1;
+    }
     dim3 grid((unsigned)cdiv(d->out_f, 256), (unsigned)cdiv(k, 16));
-    if (b16) smallk_dcoef_kernel<bf16_t><<<grid, 256, 0, s>>>(dcoef, (const bf16_t *)dy, lddy, z, nchunk, T, (int)d->out_f, k);
-    else smallk_dcoef_kernel<float><<<grid, 256, 0, s>>>(dcoef, (const float *)dy, lddy, z, nchunk, T, (int)d->out_f, k);
+    if (b16) smallk_dcoef_kernel<bf16_t><<<grid, 256, 0, s>>>(dcoef, (const bf16_t *)dy, lddy, zz, zchunks, T, (int)d->out_f, k);
+    else smallk_dcoef_kernel<float><<<grid, 256, 0, s>>>(dcoef, (const float *)dy, lddy, zz, zchunks, T, (int)d->out_f, k);
     return check_launch("smallk_dcoef_kernel");
 }
 

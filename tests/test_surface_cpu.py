@@ -255,9 +255,9 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     k128 = desc(16, 4096, 4096, 128, act=_lib.RDB_F32, coef=_lib.RDB_F32)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(k128)) == 16 * 128 * 4 * (1 + 32)
     # bf16 with a few tokens (up to 64, k up to 256): the vector-ALU kernels' scratch where it is the larger need (16 chunks of
-    # 256 features, a [16 x 256] fp32 matrix each, their tags and one counter): for the input gradient, whose matrix-core form
+    # 256 features, a [16 x 256] fp32 matrix each, and their sum): for the input gradient, whose matrix-core form
     # needs only t; the other two calls' need stays the projection state's.  One token more and the few-token kernels are out.
-    few16 = 16 * 16 * 256 * 4 + 2 * 16 * 8 + 8 + 8
+    few16 = 16 * 16 * 256 * 4 + 16 * 256 * 4   # the chunks' partial matrices and their sum
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(desc(16, 4096, 4096, 256))) == few16
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(desc(65, 4096, 4096, 256))) == 96 * 256 * 2
     for op in (_lib.RDB_OP_LINEAR_FWD, _lib.RDB_OP_LINEAR_BWD_DCOEF):
