@@ -469,11 +469,12 @@ static bool smallk_wanted(const rdb_linear_desc *d, int dir)
     const bool cheaper = d->k * (d->in_f + d->out_f) < d->in_f * d->out_f;
     if (d->act_dtype == RDB_F32 && d->k <= SK_MAX_K) return d->algo == RDB_ALGO_FACTORED || (d->tokens <= 1024 && cheaper);
     if (d->tokens > SK_FEW_TOKENS || !cheaper) return false;
-    if (d->k <= SK_MAX_K || dir == SK_DCOEF) return true;
-    // k beyond 64, forward and input gradient (contraction over J): in bf16 the matrix-core kernels' time grows with the
-    // contraction (a few blocks, each alone with all of it): below about 1536 values they are ahead (768 -> 3072: 15 us against
-    // 17), beyond it behind (4096: 39 against 17)
-    const int64_t J = dir == SK_FWD ? d->in_f : d->out_f;
+    if (d->k <= SK_MAX_K) return true;
+    // k beyond 64 (contraction over J: in_f for the forward and the coefficient gradient's z, out_f for the input gradient): in
+    // bf16 the matrix-core kernels' time grows with the contraction (a few blocks, each alone with all of it): below about
+    // 1536 values they are ahead (768 -> 3072, 16 tokens: forward 15 us against 16, coefficient gradient 17 against 17-24),
+    // beyond it behind (4096 -> 4096: 39 against 16, 41 against 18)
+    const int64_t J = dir == SK_DX ? d->out_f : d->in_f;
     return d->act_dtype == RDB_F32 || J >= 1536;
 }
 

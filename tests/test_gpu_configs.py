@@ -267,12 +267,14 @@ def test_few_token_regime_up_to_k_256(hip, oracle, dtype, T, in_f, out_f, k, wit
     want_y = oracle.linear_fwd(xn, Cn, in_f, out_f, seed, bias=None if bias is None else bias.float().numpy())
     want_dx, want_dC, _ = oracle.linear_bwd(xn, dyn, Cn, in_f, out_f, seed)
     # in bf16 the library takes these kernels for a direction whose contraction is long enough (1536 values) to leave the
-    # matrix-core kernels behind; the coefficient gradient always
+    # matrix-core kernels behind (the coefficient gradient's is z = x.N^T, over in_f)
     tol_y = F32_TOL if dtype == torch.float32 else 2e-3 if in_f >= 1536 else BF16_TOL
     tol_dx = F32_TOL if dtype == torch.float32 else 2e-3 if out_f >= 1536 else BF16_TOL
     assert rel_l2(cpu(y), want_y) < tol_y
     assert rel_l2(cpu(dx), want_dx) < tol_dx
-    assert rel_l2(cpu(dC), want_dC) < F32_TOL
+    # (sizes that are not multiples of 8 never take the bf16 matrix-core kernels: fp32-accurate either way)
+    odd = in_f % 8 != 0 or out_f % 8 != 0 or k % 8 != 0
+    assert rel_l2(cpu(dC), want_dC) < (F32_TOL if dtype == torch.float32 or in_f >= 1536 or odd else BF16_TOL)
     # bit for bit run to run (fixed summation order, no atomics), and as separate launches
     assert torch.equal(y, hip.linear_fwd(x.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, bias=None if bias is None else bias.cuda()))
     assert torch.equal(dC, hip.linear_bwd_dcoef(dy.cuda(), x.cuda(), k, out_f, in_f, out_f, in_f, 1, seed)[0])
