@@ -382,6 +382,9 @@ int linear_bwd_projected(void *dx, int64_t lddx, float *dcoef, const void *dy, i
             bs.tn_blocks = xcd_grid_size(items);
             int rblocks = (int)cdiv(red.n / 4 * red.splits, ST_THREADS * 16);   // about 16 loads of 16 bytes a thread
             if (rblocks > num_cus / 2) rblocks = num_cus / 2;
+            // a block of this kernel has a compute unit to itself: where the product's blocks leave units free, no more reduction
+            // blocks than those, so that the launch is one round of blocks
+            if (bs.tn_blocks < num_cus && rblocks > num_cus - bs.tn_blocks) rblocks = num_cus - bs.tn_blocks;
             if (rblocks < 1) rblocks = 1;
             if (direct) rblocks = 0;
             const int kg = (int)cdiv(d->k, 64);
