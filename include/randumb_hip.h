@@ -146,7 +146,7 @@ enum {
                              y = (x.N^T).C^T, dx = (dy.C).N, dcoef = dy^T.(x.N^T); the [tokens x k] intermediate lives in
                              the caller's workspace.  bf16 activations and coef (sizes multiples of 8): bf16 matrix cores;
                              fp32, or bf16 with other sizes: fp32 matrix cores; a few tokens (k <= 64 in fp32 up to 1024
-                             tokens; under AUTO also k <= 256 up to 64 tokens in either dtype): the vector ALU, in fp32;
+                             tokens; under AUTO also k <= 256 up to 96 tokens in either dtype): the vector ALU, in fp32;
                              partial sums are added in a fixed order.  With scale_bias the full-rank share s.R is
                              one more product with R hashed as an operand. */
 };

@@ -485,7 +485,7 @@ extern "C" int rdb_linear_fwd(void *y, int64_t ldy, const void *x, int64_t ldx, 
         rc = linear_fwd_vecsplit(y, ldy, x, ldx, coef, scale_bias, bias, d, num_compute_units(), workspace, workspace_bytes, s);
         if (rc != RDB_E_UNSUPPORTED) return rc;
     }
-    if (d->algo == RDB_ALGO_AUTO && d->act_dtype == RDB_BF16 && d->tokens <= 64) {
+    if (d->algo == RDB_ALGO_AUTO && d->act_dtype == RDB_BF16 && d->tokens <= 96) {
         // a few tokens: the matrix-core kernels below would run a handful of blocks, each alone with a contraction over all of
         // in_f; the vector-ALU kernels spread it over the chip (16 tokens x 4096 -> 4096, k = 256: 39 us against 12)
         rc = linear_fwd_smallk(y, ldy, x, ldx, coef, scale_bias, bias, d, workspace, workspace_bytes, s);
@@ -580,7 +580,7 @@ extern "C" int rdb_linear_bwd_dx(void *dx, int64_t lddx, const void *dy, int64_t
         rc = linear_dx_vecsplit(dx, lddx, dy, lddy, coef, scale_bias, d, num_compute_units(), workspace, workspace_bytes, (hipStream_t)stream);
         if (rc != RDB_E_UNSUPPORTED) return rc;
     }
-    if (d->algo == RDB_ALGO_AUTO && d->act_dtype == RDB_BF16 && d->tokens <= 64) {   // a few tokens: as in rdb_linear_fwd
+    if (d->algo == RDB_ALGO_AUTO && d->act_dtype == RDB_BF16 && d->tokens <= 96) {   // a few tokens: as in rdb_linear_fwd
         rc = linear_dx_smallk(dx, lddx, dy, lddy, coef, scale_bias, d, workspace, workspace_bytes, (hipStream_t)stream);
         if (rc != RDB_E_UNSUPPORTED) return rc;
     }

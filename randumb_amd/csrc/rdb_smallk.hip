@@ -1,6 +1,6 @@
 // Fused linear layer, matrix-coef, few tokens (the GEMV-like regime): factored algorithm on the vector ALU, in fp32 whatever the
 // dtype of the operands (fp32, or bf16 activations and coefficients).  Two ranges: k <= 64 with up to 1024 tokens (fp32), and
-// k <= 256 with up to 64 tokens (both dtypes), where the matrix-core kernels would run a handful of blocks, each alone with a
+// k <= 256 with up to 96 tokens (both dtypes; 64 for the coefficient gradient), where the matrix-core kernels would run a handful of blocks, each alone with a
 // long contraction.
 //
 // With a handful of tokens the layer moves almost no data (x, C, y) and does almost no arithmetic once W = C . N
@@ -19,7 +19,8 @@ constexpr int SK_TT = 8;    // tokens per block of the contracting kernel
 constexpr int SK_ET = 16;   // tokens per block of the expanding kernel
 constexpr int SK_MAX_K = 64;      // the range with many tokens
 constexpr int SK_BIG_K = 256;     // the range with few tokens
-constexpr int SK_FEW_TOKENS = 64;
+constexpr int SK_FEW_TOKENS = 96;         // forward and input gradient
+constexpr int SK_FEW_TOKENS_DCOEF = 64;   // coefficient gradient (its second kernel walks the tokens one by one)
 
 // sum over the partial matrices p[ch][idx], ch = 0 .. nchunk-1, in chunk order; loads issued eight at a time
 __device__ __forceinline__ float sum_partials(const float *__restrict__ p, int64_t stride, int nchunk)
@@ -468,7 +469,7 @@ static bool smallk_wanted(const rdb_linear_desc *d, int dir)
 {
     const bool cheaper = d->k * (d->in_f + d->out_f) < d->in_f * d->out_f;
     if (d->act_dtype == RDB_F32 && d->k <= SK_MAX_K) return d->algo == RDB_ALGO_FACTORED || (d->tokens <= 1024 && cheaper);
-    if (d->tokens > SK_FEW_TOKENS || !cheaper) return false;
+    if (d->tokens > (dir == SK_DCOEF ? SK_FEW_TOKENS_DCOEF : SK_FEW_TOKENS) || !cheaper) return false;
     if (d->k <= SK_MAX_K) return true;
     // k beyond 64 (contraction over J: in_f for the forward and the coefficient gradient's z, out_f for the input gradient): in
     // bf16 the matrix-core kernels' time grows with the contraction (a few blocks, each alone with all of it): below about

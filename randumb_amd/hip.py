@@ -524,10 +524,10 @@ def linear_projection_preferred(tokens: int, in_f: int, out_f: int, k: int, dtyp
     the state may cost up to twice that, i.e. k rounded up to 64 must not exceed in_f (768 -> 3072, k = 256: 1024 against
     1536 bytes per token).  Layers that fail the second test still run the factored kernels, through ``rdb_linear_fwd`` and a
     transient workspace, with x saved.  fp32 layers: the state is z in fp32 (4 k bytes per token against 4 in_f)."""
-    # not in the few-token regimes, whose vector-ALU kernels (k <= 256 up to 64 tokens; in fp32 also k <= 64 up to 1024 tokens)
+    # not in the few-token regimes, whose vector-ALU kernels (k <= 256 up to 96 tokens; in fp32 also k <= 64 up to 1024 tokens)
     # have no projected form: rdb_linear_fwd and the two gradient calls take them
     few = k * (in_f + out_f) < in_f * out_f and ((dtype == torch.float32 and k <= 64 and tokens <= 1024) or (
-        k <= 256 and tokens <= 64 and (k <= 64 or dtype == torch.float32 or max(in_f, out_f) >= 1536)))
+        k <= 256 and tokens <= 96 and (k <= 64 or dtype == torch.float32 or max(in_f, out_f) >= 1536)))
     if dtype == torch.float32:
         # the state is z in fp32, 4 k bytes per token where x has 4 in_f: the same memory rule
         return k <= 2 * in_f and not few and (k > 64 or tokens > 1024) and linear_projection_supported(tokens, in_f, out_f, k, dtype)

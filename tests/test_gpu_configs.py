@@ -241,13 +241,13 @@ def test_small_k_fp32_ragged_shapes(hip, oracle):
 
 
 FEW_TOKEN_CASES = [(1, 2048, 1024, 256, False), (16, 1024, 2048, 256, True), (64, 1024, 768, 128, False), (33, 777, 555, 99, True),
-                   (5, 8448, 512, 72, False)]
+                   (5, 8448, 512, 72, False), (80, 2048, 1536, 256, False)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T,in_f,out_f,k,with_bias", FEW_TOKEN_CASES)
 def test_few_token_regime_up_to_k_256(hip, oracle, dtype, T, in_f, out_f, k, with_bias):
-    """Up to 64 tokens with k up to 256, both dtypes: the vector-ALU kernels compute in fp32 whatever the operands' dtype, so on
+    """Up to 96 tokens (64 for the coefficient gradient) with k up to 256, both dtypes: the vector-ALU kernels compute in fp32 whatever the operands' dtype, so on
     bf16 operands y and dx carry one rounding to bf16 (rel-L2 about 1e-3; the bf16 matrix-core kernels, which also round z and
     t, are near 3e-3: the threshold between them shows which kernels ran) and the coefficient gradient, an fp32 result, meets
     the fp32 tolerance.  The last case contracts over
@@ -274,7 +274,7 @@ def test_few_token_regime_up_to_k_256(hip, oracle, dtype, T, in_f, out_f, k, wit
     assert rel_l2(cpu(dx), want_dx) < tol_dx
     # (sizes that are not multiples of 8 never take the bf16 matrix-core kernels: fp32-accurate either way)
     odd = in_f % 8 != 0 or out_f % 8 != 0 or k % 8 != 0
-    assert rel_l2(cpu(dC), want_dC) < (F32_TOL if dtype == torch.float32 or in_f >= 1536 or odd else BF16_TOL)
+    assert rel_l2(cpu(dC), want_dC) < (F32_TOL if dtype == torch.float32 or (in_f >= 1536 and T <= 64) or odd else BF16_TOL)
     # bit for bit run to run (fixed summation order, no atomics), and as separate launches
     assert torch.equal(y, hip.linear_fwd(x.cuda(), C.cuda(), in_f, out_f, in_f, 1, seed, bias=None if bias is None else bias.cuda()))
     assert torch.equal(dC, hip.linear_bwd_dcoef(dy.cuda(), x.cuda(), k, out_f, in_f, out_f, in_f, 1, seed)[0])

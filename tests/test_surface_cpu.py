@@ -254,15 +254,15 @@ def test_workspace_queries_and_projected_argument_checks_without_a_gpu():
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(f32)) == max(small_k, 1024 * (1 + 32))
     k128 = desc(16, 4096, 4096, 128, act=_lib.RDB_F32, coef=_lib.RDB_F32)
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(k128)) == 16 * 128 * 4 * (1 + 32)
-    # bf16 with a few tokens (up to 64, k up to 256): the vector-ALU kernels' scratch where it is the larger need (16 chunks of
+    # bf16 with a few tokens (up to 96, k up to 256): the vector-ALU kernels' scratch where it is the larger need (16 chunks of
     # 256 features, a [16 x 256] fp32 matrix each, and their sum): for the input gradient, whose matrix-core form
-    # needs only t; the other two calls' need stays the projection state's.  One token more and the few-token kernels are out.
+    # needs only t; the other two calls' need stays the projection state's.  Beyond 96 tokens the few-token kernels are out.
     few16 = 16 * 16 * 256 * 4 + 16 * 256 * 4   # the chunks' partial matrices and their sum
     assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(desc(16, 4096, 4096, 256))) == few16
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(desc(65, 4096, 4096, 256))) == 96 * 256 * 2
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_BWD_DX, ctypes.byref(desc(97, 4096, 4096, 256))) == 128 * 256 * 2
     for op in (_lib.RDB_OP_LINEAR_FWD, _lib.RDB_OP_LINEAR_BWD_DCOEF):
         assert L.rdb_linear_workspace_bytes(op, ctypes.byref(desc(16, 4096, 4096, 256))) == state_bytes(16, 4096, 4096, 256) > few16
-    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(65, 4096, 4096, 256))) == state_bytes(65, 4096, 4096, 256)
+    assert L.rdb_linear_workspace_bytes(_lib.RDB_OP_LINEAR_FWD, ctypes.byref(desc(97, 4096, 4096, 256))) == state_bytes(97, 4096, 4096, 256)
     # 8192 tokens x 256 coefficients are 128 tiles of 128 x 128: four ranges; the coefficient gradient's 48 tiles: ten ranges of
     # tokens, one [out_f x k] matrix each
     c2 = desc(8192, 768, 3072, 256, act=_lib.RDB_F32, coef=_lib.RDB_F32)
