@@ -431,9 +431,33 @@ __global__ __launch_bounds__(256) void smallk_dcoef_kernel(float *__restrict__ d
 #pragma unroll
     for (int m = 0; m < 16; ++m) acc[m] = 0.0f;
     for (int t0 = 0; t0 < T; t0 += 64) {
-        for (int e = tid; e < 64 * 16; e += 256) {
-            const int tt = e >> 4, m = e & 15;
-            zs[tt][m] = (t0 + tt < T && mc + m < k) ? sum_partials(z + (int64_t)(t0 + tt) * k + mc + m, (int64_t)T * k, nchunk) : 0.0f;
+        {   // a thread's four entries of the z tile, the loads of eight chunks of all four in flight together (an entry that does
+            // not exist reads a valid address and becomes 0 by a select)
+            const float *at[4];
+            float zv[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int e = tid + 256 * q, tt = e >> 4, m = e & 15;
+                at[q] = z + (int64_t)(t0 + tt < T ? t0 + tt : T - 1) * k + (mc + m < k ? mc + m : k - 1);
+                zv[q] = 0.0f;
+            }
+            const int64_t stride = (int64_t)T * k;
+            for (int c0 = 0; c0 < nchunk; c0 += 8) {
+                float l[4][8];
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) l[q][u] = at[q][(int64_t)((c0 + u < nchunk) ? c0 + u : nchunk - 1) * stride];
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) zv[q] += (c0 + u < nchunk) ? l[q][u] : 0.0f;
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int e = tid + 256 * q, tt = e >> 4, m = e & 15;
+                zs[tt][m] = (t0 + tt < T && mc + m < k) ? zv[q] : 0.0f;
+            }
         }
         __syncthreads();
         if (o < out_f) {
