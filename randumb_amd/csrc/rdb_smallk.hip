@@ -22,20 +22,6 @@ constexpr int SK_BIG_K = 256;     // the range with few tokens
 constexpr int SK_FEW_TOKENS = 96;         // forward and input gradient
 constexpr int SK_FEW_TOKENS_DCOEF = 64;   // coefficient gradient (its second kernel walks the tokens one by one)
 
-// sum over the partial matrices p[ch][idx], ch = 0 .. nchunk-1, in chunk order; loads issued eight at a time
-__device__ __forceinline__ float sum_partials(const float *__restrict__ p, int64_t stride, int nchunk)
-{
-    float v = 0.0f;
-    for (int c0 = 0; c0 < nchunk; c0 += 8) {
-        float l[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) l[u] = p[(int64_t)((c0 + u < nchunk) ? c0 + u : nchunk - 1) * stride];  // always a valid address
-#pragma unroll
-        for (int u = 0; u < 8; ++u) v += (c0 + u < nchunk) ? l[u] : 0.0f;
-    }
-    return v;
-}
-
 // out[t, m] = sum_j src[t, j] * B(j, m),  B(j, m) = noise(PRIME*j + m) (HASH) or coef[j, m]; j runs over J = in_f or out_f.
 // Block = 8 tokens x one chunk of 256 values of j (blockIdx.y), so that even a single token spreads the hash over many
 // compute units; thread = (m % 16, one of 16 interleaved slices of the chunk); the source rows go through LDS (coalesced
